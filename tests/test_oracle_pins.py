@@ -1,0 +1,298 @@
+"""
+Pins for the CPU oracle (no GPU needed).
+
+The reference holds no golden vectors for this path (all of its tests draw inputs at run time on
+"cuda"), so every oracle function is pinned here against something its own formula does not
+contain: closed-form exact cases, brute force in Python integers, fp64 library routines
+(``torch.nn.functional.gelu/silu/rms_norm``, complex multiplication for RoPE), mutual inverses
+written from two different statements of a layout, and the independently written scalar C
+restatement.  A dropped term, a wrong sign or nibble order, or a transposed operand fails at
+least one of them.
+"""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import c_oracle
+from oracle import svdq_oracle as O
+
+
+# ----------------------------------------------------------------------------- nibbles
+def test_unpack_hand_bytes():
+    # byte 0xA3: element 0 = low nibble 3, element 1 = high nibble 0xA (= -6 signed)
+    # byte 0x8F: element 2 = 0xF (= -1), element 3 = 8 (= -8)
+    p = torch.tensor([[0xA3, 0x8F]], dtype=torch.uint8)
+    assert O.unpack_int4(p, signed=False).tolist() == [[3, 10, 15, 8]]
+    assert O.unpack_int4(p, signed=True).tolist() == [[3, -6, -1, -8]]
+    assert O.pack_int4(torch.tensor([[3, -6, -1, -8]])).tolist() == [[0xA3, 0x8F]]
+
+
+def test_pack_unpack_round_trip():
+    g = torch.Generator().manual_seed(0)
+    c = torch.randint(-8, 8, (5, 128), generator=g, dtype=torch.int32)
+    assert torch.equal(O.unpack_int4(O.pack_int4(c), True), c)
+    u = torch.randint(0, 16, (5, 128), generator=g, dtype=torch.int32)
+    assert torch.equal(O.unpack_int4(O.pack_int4(u), False), u)
+
+
+# ----------------------------------------------------------------------------- quantizer
+def _pow2_grid_case(unsigned: bool, seed: int):
+    """x = s * c / (1/smooth) on power-of-two grids: every fp32 op is exact, so the answer is known."""
+    g = torch.Generator().manual_seed(seed)
+    M, K = 7, 256
+    lo, hi = (0, 15) if unsigned else (-7, 7)
+    c = torch.randint(lo, hi + 1, (M, K), generator=g, dtype=torch.int32)
+    c.view(M, K // 64, 64)[:, :, 5] = hi  # the group maximum is exactly qmax * s
+    e = torch.randint(-6, 3, (M, K // 64), generator=g)
+    s = torch.pow(2.0, e.float())
+    smooth = torch.pow(2.0, torch.randint(-1, 3, (K,), generator=g).float())
+    x = (c.float().view(M, K // 64, 64) * s[:, :, None]).view(M, K) * smooth[None, :]
+    return x.to(torch.bfloat16), smooth.to(torch.bfloat16), c, s
+
+
+@pytest.mark.parametrize("unsigned", [False, True])
+def test_quantizer_exact_on_power_of_two_grid(unsigned):
+    x, smooth, c, s = _pow2_grid_case(unsigned, 3)
+    assert torch.equal(x.float(), x.float().to(torch.bfloat16).float())  # the inputs are exact in bf16
+    packed, scales, _, codes = O.quantize_act(x, None, smooth, unsigned=unsigned)
+    assert torch.equal(codes, c)
+    assert torch.equal(scales.float().t(), s)
+    assert torch.equal(O.unpack_int4(packed, not unsigned), c)
+
+
+def test_quantizer_ties_round_half_to_even():
+    # one group, scale exactly 1 (max 7): values k + 0.5 must round like Python's round()
+    vals = [-6.5, -5.5, -2.5, -1.5, -0.5, 0.5, 1.5, 2.5, 3.5, 4.5, 5.5, 6.5, 7.0, 0.25, -0.75]
+    x = torch.zeros(1, 64)
+    x[0, : len(vals)] = torch.tensor(vals)
+    _, scales, _, codes = O.quantize_act(x.to(torch.bfloat16))
+    assert scales.float().item() == 1.0
+    assert codes[0, : len(vals)].tolist() == [int(round(v)) for v in vals]
+
+
+def test_quantizer_zero_and_nonpositive_groups():
+    x = torch.zeros(2, 128, dtype=torch.bfloat16)
+    x[0, 64:] = -3.0  # unsigned: all-non-positive group -> scale 0, codes clamp to 0
+    x[1, :64] = 2.0
+    _, s_u, _, c_u = O.quantize_act(x, unsigned=True)
+    assert s_u.float()[1, 0].item() == 0.0 and c_u[0, 64:].abs().sum() == 0
+    assert c_u[1, :64].eq(15).all()
+    _, s_s, _, c_s = O.quantize_act(x, unsigned=False)
+    assert s_s.float()[0, 0].item() == 0.0 and c_s[0, :64].abs().sum() == 0
+    assert c_s[0, 64:].eq(-7).all() and c_s[1, :64].eq(7).all()
+
+
+@pytest.mark.parametrize("unsigned", [False, True])
+def test_quantizer_half_step_bound_and_lora(unsigned):
+    x = O.make_activations(48, 512, seed=11)
+    if unsigned:
+        x = x.abs()
+    lin = O.make_svdq_linear(512, 64, R=32, seed=12)
+    packed, scales, lora, codes = O.quantize_act(x, lin["proj_down"], lin["smooth_factor"], unsigned=unsigned)
+    lo, hi = (0, 15) if unsigned else (-8, 7)
+    assert codes.min() >= lo and codes.max() <= hi
+    # dequantised with the *unrounded* scale the error is at most half a step (fp64 arithmetic here)
+    v = x.double() / lin["smooth_factor"].double()[None, :]
+    vg = v.view(48, 8, 64)
+    gmax = vg.amax(-1) if unsigned else vg.abs().amax(-1)
+    step = gmax / (15 if unsigned else 7)
+    err = (codes.double().view(48, 8, 64) * step[..., None] - vg).abs()
+    assert (err <= 0.5 * step[..., None] * (1 + 1e-5) + 1e-12).all()
+    # stored scale = bf16(step)
+    assert ((scales.float().t().double() - step).abs() <= step * 2**-8).all()
+    # LoRA-down is the plain product on the un-smoothed input
+    ref = x.double() @ lin["proj_down"].double()
+    assert (lora.double() - ref).abs().max() <= 1e-5 * ref.abs().max()
+
+
+@pytest.mark.parametrize("unsigned,shift", [(False, 0.0), (True, 0.171875)])
+def test_quantizer_matches_c_restatement_bit_exact(unsigned, shift):
+    x = O.make_activations(40, 384, seed=21)
+    if unsigned:
+        x = (x.float().abs() * 0.1 - 0.1).to(torch.bfloat16)
+    lin = O.make_svdq_linear(384, 64, R=16, seed=22)
+    packed, scales, lora, _ = O.quantize_act(x, lin["proj_down"], lin["smooth_factor"], unsigned=unsigned, shift=shift)
+    c_packed, c_scales, c_lora = c_oracle.quantize_act(x, lin["smooth_factor"], lin["proj_down"], unsigned, shift)
+    assert torch.equal(packed, c_packed)
+    assert torch.equal(scales.view(torch.int16), c_scales.view(torch.int16))
+    assert (lora - c_lora).abs().max() <= 1e-5 * lora.abs().max()
+
+
+# ----------------------------------------------------------------------------- integer group dots, GEMM
+@pytest.mark.parametrize("act_unsigned", [False, True])
+def test_group_acc_brute_force(act_unsigned):
+    g = torch.Generator().manual_seed(5)
+    M, N, K = 3, 4, 128
+    act = torch.randint(0, 256, (M, K // 2), generator=g, dtype=torch.uint8)
+    wgt = torch.randint(0, 256, (N, K // 2), generator=g, dtype=torch.uint8)
+    p = O.group_acc_i32(act, wgt, act_unsigned)
+
+    def nib(row, k, signed):
+        v = (int(row[k // 2]) >> (4 * (k % 2))) & 0xF
+        return v - 16 if signed and v >= 8 else v
+
+    for gi in range(K // 64):
+        for m in range(M):
+            for n in range(N):
+                s = sum(nib(act[m], k, not act_unsigned) * nib(wgt[n], k, True) for k in range(gi * 64, gi * 64 + 64))
+                assert p[gi, m, n].item() == s
+        assert torch.equal(c_oracle.group_acc_i32(act, wgt, gi, act_unsigned), p[gi])
+
+
+@pytest.mark.parametrize("act_unsigned", [False, True])
+def test_gemm_unit_scales_is_exact_integer_gemm(act_unsigned):
+    g = torch.Generator().manual_seed(6)
+    M, N, K = 16, 24, 256
+    act = torch.randint(0, 256, (M, K // 2), generator=g, dtype=torch.uint8)
+    wgt = torch.randint(0, 256, (N, K // 2), generator=g, dtype=torch.uint8)
+    one_a = torch.ones(K // 64, M, dtype=torch.bfloat16)
+    one_w = torch.ones(K // 64, N, dtype=torch.bfloat16)
+    out = O.gemm_w4a4(act, wgt, one_a, one_w, act_unsigned=act_unsigned)
+    a = O.unpack_int4(act, not act_unsigned).numpy().astype(np.int64)
+    w = O.unpack_int4(wgt, True).numpy().astype(np.int64)
+    assert np.array_equal(out.numpy().astype(np.int64), a @ w.T)
+
+
+def test_gemm_fp64_closed_form_and_c_restatement():
+    g = torch.Generator().manual_seed(7)
+    M, N, K, R = 20, 12, 256, 16
+    act = torch.randint(0, 256, (M, K // 2), generator=g, dtype=torch.uint8)
+    wgt = torch.randint(0, 256, (N, K // 2), generator=g, dtype=torch.uint8)
+    asc = (torch.rand(K // 64, M, generator=g) * 0.05 + 0.01).to(torch.bfloat16)
+    wsc = (torch.rand(K // 64, N, generator=g) * 0.05 + 0.01).to(torch.bfloat16)
+    bias = torch.randn(N, generator=g).to(torch.bfloat16)
+    la = torch.randn(M, R, generator=g)
+    lu = (torch.randn(N, R, generator=g) * 0.1).to(torch.bfloat16)
+    out = O.gemm_w4a4(act, wgt, asc, wsc, bias, la, lu)
+    # dense fp64: dequantise both operands element by element, one big matmul
+    grp = torch.arange(K) // 64
+    a = O.unpack_int4(act, True).double() * asc.double()[grp].t()
+    w = O.unpack_int4(wgt, True).double() * wsc.double()[grp].t()
+    ref = a @ w.t() + la.to(torch.bfloat16).double() @ lu.double().t() + bias.double()
+    assert (out.double() - ref).abs().max() <= 2e-6 * ref.abs().max()
+    # without LoRA the torch and C restatements perform the same fp32 ops in the same order
+    o1 = O.gemm_w4a4(act, wgt, asc, wsc, bias)
+    o2 = c_oracle.gemm_w4a4(act, wgt, asc, wsc, bias)
+    assert torch.equal(o1, o2)
+    o3 = c_oracle.gemm_w4a4(act, wgt, asc, wsc, bias, la, lu)
+    assert (o3 - out).abs().max() <= 1e-5 * out.abs().max()
+
+
+# ----------------------------------------------------------------------------- epilogues
+def test_gelu_and_silu_match_library_fp64():
+    x = torch.linspace(-8, 8, 4001)
+    ref = torch.nn.functional.gelu(x.double(), approximate="tanh")
+    assert (O.gelu_tanh(x).double() - ref).abs().max() < 2e-6
+    assert (O.silu(x).double() - torch.nn.functional.silu(x.double())).abs().max() < 2e-6
+
+
+def test_qk_norm_rope_against_complex_rotation():
+    g = torch.Generator().manual_seed(8)
+    M, H = 9, 2
+    N = 3 * H * 128
+    lin = torch.randn(M, N, generator=g)
+    nq = (torch.rand(128, generator=g) + 0.5).to(torch.bfloat16)
+    nk = (torch.rand(128, generator=g) + 0.5).to(torch.bfloat16)
+    theta = torch.rand(M, 64, generator=g, dtype=torch.float64) * 6.28
+    rot = torch.stack([torch.sin(theta), torch.cos(theta)], -1).float().reshape(M, 128)
+    out = O.qk_norm_rope(lin, nq, nk, rot)
+    x = lin.double().view(M, 3, H, 128)
+    for part, w in ((0, nq), (1, nk)):
+        h = torch.nn.functional.rms_norm(x[:, part], (128,), w.double(), eps=1e-6)
+        z = torch.view_as_complex(h.reshape(M, H, 64, 2).contiguous())
+        rz = z * torch.polar(torch.ones_like(theta), theta)[:, None]
+        ref = torch.view_as_real(rz).reshape(M, H, 128)
+        assert (out.view(M, 3, H, 128)[:, part].double() - ref).abs().max() < 2e-5
+    assert torch.equal(out.view(M, 3, H * 128)[:, 2], lin.view(M, 3, H * 128)[:, 2])
+
+
+def test_gelu_quant_is_quantizer_of_library_gelu():
+    g = torch.Generator().manual_seed(9)
+    M, N, R2 = 12, 256, 16
+    lin = torch.randn(M, N, generator=g) * 2
+    smooth = (torch.rand(N, generator=g) + 0.5).to(torch.bfloat16)
+    ld = (torch.randn(N, R2, generator=g) * 0.1).to(torch.bfloat16)
+    packed, scales, lora, codes = O.gelu_quant(lin, smooth, ld, torch.bfloat16)
+    gl = torch.nn.functional.gelu(lin.double(), approximate="tanh")
+    v = (gl + 0.171875) / smooth.double()
+    step = v.view(M, N // 64, 64).amax(-1).clamp_min(0) / 15
+    ref = torch.round(v.view(M, N // 64, 64) / step[..., None]).clamp(0, 15).view(M, N)
+    diff = (codes.double() - ref).abs()
+    assert diff.max() <= 1 and (diff > 0).double().mean() < 1e-3
+    assert ((scales.float().t().double() - step).abs() <= step * 2**-8 + 1e-12).all()
+    refl = gl.float().to(torch.bfloat16).double() @ ld.double()
+    assert (lora.double() - refl).abs().max() <= 1e-4 * refl.abs().max()
+    assert codes.min() >= 0  # gelu >= -0.17 so the shifted value is positive
+
+
+def test_swiglu_interleave_and_quant():
+    n = 128
+    idx = O.interleave_swiglu(n)
+    assert sorted(idx.tolist()) == list(range(n))
+    cols = torch.arange(n).float()[idx].view(n // 32, 2, 16)  # what out.view(M, n//32, 2, 16) sees
+    assert torch.equal(cols[:, 0].flatten(), torch.arange(n // 2).float())  # gate rows in order
+    assert torch.equal(cols[:, 1].flatten(), torch.arange(n // 2, n).float())  # up rows in order
+    g = torch.Generator().manual_seed(10)
+    M = 6
+    lin = torch.randn(M, n, generator=g)  # [gate | up]
+    smooth = (torch.rand(n // 2, generator=g) + 0.5).to(torch.bfloat16)
+    _, scales, _, codes = O.swiglu_quant(lin[:, idx], smooth, None, torch.bfloat16)
+    y = torch.nn.functional.silu(lin[:, : n // 2].double()) * lin[:, n // 2 :].double() / smooth.double()
+    step = y.abs().view(M, 1, 64).amax(-1) / 7
+    ref = torch.round(y.view(M, 1, 64) / step[..., None]).clamp(-8, 7).view(M, 64)
+    assert (codes.double() - ref).abs().max() <= 1 and (codes.double() != ref).double().mean() < 1e-2
+
+
+# ----------------------------------------------------------------------------- AWQ
+def test_awq_pack_decode_inverse_and_gemv_kernel_statement():
+    g = torch.Generator().manual_seed(13)
+    N, K = 16, 128
+    q = torch.randint(0, 16, (N, K), generator=g, dtype=torch.int32)
+    packed = O.awq_pack(q)
+    assert packed.shape == (N // 4, K) and packed.dtype == torch.int16
+    assert torch.equal(O.awq_decode(packed, N, K), q)
+    # third statement of the layout (the streaming GEMV's, nunchaku/ops/triton/awq.py:137-144):
+    # stored column e = 64c + 16b + d of packed row a, nibble m <-> (n, k) = (4a + b, 64c + 32(d//8) + 8m + d%8)
+    pu = packed.to(torch.int32) & 0xFFFF
+    for a in range(N // 4):
+        for e in range(K):
+            c, b, d = e // 64, (e % 64) // 16, e % 16
+            for m in range(4):
+                assert ((pu[a, e].item() >> (4 * m)) & 0xF) == q[4 * a + b, 64 * c + 32 * (d // 8) + 8 * m + d % 8].item()
+    pk = packed.contiguous()
+    lib = c_oracle.lib()
+    for n in range(N):
+        for k in range(0, K, 7):
+            assert lib.oracle_awq_nibble(c_oracle._p(pk), K, n, k) == q[n, k].item()
+
+
+@pytest.mark.parametrize("m", [1, 3])
+def test_awq_gemv_fp64_dense(m):
+    lin = O.make_awq_linear(256, 64, seed=14)
+    g = torch.Generator().manual_seed(15)
+    x = torch.randn(m, 256, generator=g).to(torch.bfloat16)
+    packed = lin["qweight"].view(torch.int16).reshape(16, 256)
+    out = O.awq_gemv(x, packed, lin["wscales"], lin["wzeros"])
+    grp = torch.arange(256) // 64
+    w = lin["codes"].double() * lin["wscales"].double()[grp].t() + lin["wzeros"].double()[grp].t()
+    ref = x.double() @ w.t()
+    assert (out.double() - ref).abs().max() <= 1e-5 * ref.abs().max()
+    out_c = c_oracle.awq_gemv(x, packed, lin["wscales"], lin["wzeros"])
+    assert (out_c - out).abs().max() <= 1e-5 * ref.abs().max()
+
+
+# ----------------------------------------------------------------------------- FLUX rotary table
+def test_flux_rotary_closed_form():
+    ids = O.flux_ids(4, 3, 5)
+    assert ids.shape == (4 + 15, 3) and ids[:4].abs().sum() == 0
+    assert ids[4 + 1 * 5 + 2].tolist() == [0.0, 1.0, 2.0]
+    rot = O.flux_rotary(ids)
+    assert rot.shape == (19, 64, 1, 2) and rot.dtype == torch.float32
+    t = 4 + 2 * 5 + 3  # h = 2, w = 3
+    for pair, (axis_pos, d, i) in {0: (0.0, 16, 0), 8 + 5: (2.0, 56, 5), 8 + 28 + 27: (3.0, 56, 27)}.items():
+        ang = axis_pos * 10000.0 ** (-(2 * i) / d)
+        assert abs(rot[t, pair, 0, 0].item() - math.sin(ang)) < 1e-6
+        assert abs(rot[t, pair, 0, 1].item() - math.cos(ang)) < 1e-6
