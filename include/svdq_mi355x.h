@@ -1,0 +1,152 @@
+/*
+ * svdq_mi355x.h -- C ABI of the MI355X (gfx950) SVDQuant kernel library (libsvdq_mi355x.so).
+ *
+ * Plain pointers and sizes only; every pointer is a device pointer unless stated otherwise, every
+ * buffer is owned by the caller, and the library allocates nothing.  All launches are asynchronous on the
+ * given stream (a hipStream_t passed as void*; NULL = the default stream).  Functions return 0 on success or a
+ * negative SVDQ_E_* code; svdq_last_error() gives the message for the calling thread.
+ *
+ * "T" below is bfloat16 (dtype code SVDQ_BF16) or float16 (SVDQ_FP16); one T per call.
+ *
+ * Each entry point replaces one binding of the reference (paths relative to the reference checkout):
+ *   svdq_quantize_act        nunchaku/ops/quantize.py:82-87      (_C.ops.quantize_w4a4_act_fuse_lora /
+ *                                                                 ops/triton/gemm_w4a4.py:1521 quantize_w4a4_act_fuse_lora)
+ *   svdq_gemm_w4a4           nunchaku/ops/gemm.py:151-207        (_C.ops.gemm_w4a4 / ops/triton/gemm_w4a4.py:1003 gemm_w4a4),
+ *                            kernel-argument structs modelled on ops/triton/native/w4a4.py:80-124
+ *   svdq_awq_gemv_w4a16      nunchaku/ops/dispatch.py:19-34      (_C.ops.gemv_awq / ops/triton/awq.py:186 awq_gemv_w4a16)
+ *   svdq_transpose_lora_down no counterpart: one-time re-layout of a LoRA-down weight, see below
+ *   svdq_group_acc_i32       no counterpart: debug read-out of the exact int32 group accumulators
+ */
+#ifndef SVDQ_MI355X_H
+#define SVDQ_MI355X_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SVDQ_ABI_VERSION 1
+
+enum { SVDQ_BF16 = 0, SVDQ_FP16 = 1 };
+
+enum {
+    SVDQ_OK = 0,
+    SVDQ_E_INVALID = -1,     /* bad shape / alignment / combination of arguments */
+    SVDQ_E_UNSUPPORTED = -2, /* valid in the reference, not implemented here      */
+    SVDQ_E_LAUNCH = -3       /* HIP reported an error for the launch              */
+};
+
+/* Epilogue of svdq_gemm_w4a4 (reference: ops/triton/gemm_w4a4.py:1151-1205 dispatch). */
+enum {
+    SVDQ_EPI_PLAIN = 0,        /* bias + LoRA-up, store T                                             */
+    SVDQ_EPI_QK_NORM_ROPE = 1, /* + per-head RMSNorm and RoPE on the Q and K thirds (gemm_w4a4.py:499) */
+    SVDQ_EPI_GELU_QUANT = 2,   /* + GELU, next layer's LoRA-down, +shift, unsigned int4 requantization  */
+    SVDQ_EPI_SWIGLU_QUANT = 3  /* + silu(gate)*up on 16-interleaved columns, signed int4 requantization */
+};
+
+/*
+ * Activation quantizer: per-channel smooth divide, per-group-64 absmax int4 quantization, fused LoRA-down.
+ * Reference arithmetic: ops/triton/gemm_w4a4.py:1397-1455 (int4 branches).  Rows >= M of out/scales/lora_act
+ * are never written.
+ */
+typedef struct {
+    const void *x;           /* (M, K) T, row stride ld_x elements                                          */
+    const void *smooth;      /* (K,) T or NULL                                                              */
+    const void *lora_down_t; /* (R, K) T: the (K, R) LoRA-down weight transposed, row stride K; NULL iff R=0 */
+    void *out;               /* (>= M, K/2) uint8, low nibble = even k, row stride ld_out bytes             */
+    void *scales;            /* (K/64, >= M) T, element [g, m] at g*ld_scales + m                           */
+    float *lora_act;         /* (>= M, R) fp32, row stride ld_lora_act elements; NULL iff R=0               */
+    int32_t M, K, R;         /* K % 64 == 0, R % 16 == 0                                                    */
+    int32_t ld_x, ld_out, ld_scales, ld_lora_act;
+    int32_t dtype;           /* SVDQ_BF16 / SVDQ_FP16                                                       */
+    int32_t is_unsigned;     /* 0: codes in [-8, 7], absmax / 7;  1: codes in [0, 15], max / 15             */
+    int32_t fuse_glu;        /* 1: x is (M, 2K) and the quantized value is x[:, :K] * silu(x[:, K:])        */
+    float shift;             /* added before smoothing (0.171875 after GELU, else 0)                        */
+} svdq_quantize_args;
+
+int svdq_quantize_act(const svdq_quantize_args *args, void *stream);
+
+/* (K, R) row-major T  ->  (R, K) row-major T.  Done once per weight; the quantizer and the fused
+ * requantizing epilogues read the transposed form so their MFMA operands are K-contiguous. */
+int svdq_transpose_lora_down(const void *lora_down, void *lora_down_t, int32_t K, int32_t R, int32_t ld_in,
+                             void *stream);
+
+/*
+ * W4A4 GEMM: out[m, n] = sum_g as[g, m] * ws[g, n] * (sum_{k in g} a[m, k] w[n, k])  (int8 MFMA, exact int32 per group)
+ *                        + T(lora_act[m, :]) . lora_up[n, :] + bias[n],  then the epilogue.
+ * Reference arithmetic: ops/triton/gemm_w4a4.py:447-488 (main loop), 156-209 (epilogue), 499-521 (QK), 730-778
+ * (GELU + requantization), 998-1000 (SwiGLU semantics).
+ */
+typedef struct {
+    const void *act;        /* (M, K/2) packed int4, row stride ld_act bytes (multiple of 16, base 16-B aligned) */
+    const void *wgt;        /* (N, K/2) packed signed int4, row stride ld_wgt bytes (same alignment)            */
+    const void *ascales;    /* (K/64, >= M) T, group stride ld_ascales elements                                 */
+    const void *wscales;    /* (K/64, >= N) T, group stride ld_wscales elements                                 */
+    const void *bias;       /* (N,) T or NULL                                                                   */
+    const float *lora_act;  /* (>= M, R) fp32, row stride ld_lora_act; NULL iff R = 0                           */
+    const void *lora_up;    /* (N, R) T, row stride ld_lora_up; NULL iff R = 0                                  */
+    void *out;              /* (actual_m, N) T, row stride ld_out; may be NULL for the requantizing epilogues   */
+    int32_t M, N, K, R;     /* K % 128 == 0, N % 8 == 0, R % 16 == 0                                            */
+    int32_t actual_m;       /* rows of out that exist (<= M); rows beyond are computed but never written       */
+    int32_t ld_act, ld_wgt, ld_ascales, ld_wscales, ld_lora_act, ld_lora_up, ld_out;
+    int32_t dtype;
+    int32_t act_unsigned;   /* activation nibbles are [0, 15] instead of two's complement                       */
+    int32_t epilogue;       /* SVDQ_EPI_*                                                                       */
+    /* SVDQ_EPI_QK_NORM_ROPE: N = 3 * heads * 128 */
+    const void *norm_q;     /* (128,) T  */
+    const void *norm_k;     /* (128,) T  */
+    const float *rotary;    /* (actual_m, 128) fp32 rows of (sin, cos) pairs, row stride ld_rotary elements     */
+    int32_t ld_rotary;
+    float eps;
+    /* SVDQ_EPI_GELU_QUANT / SVDQ_EPI_SWIGLU_QUANT: NQ = N (GELU) or N/2 (SwiGLU) quantized columns */
+    void *qout;               /* (>= M, NQ/2) uint8, row stride ld_qout bytes                                   */
+    void *oscales;            /* (NQ/64, >= M) T, group stride ld_oscales                                       */
+    const void *smooth_next;  /* (NQ,) T or NULL                                                                */
+    const void *lora_down_t;  /* (R2, NQ) T, the next layer's (NQ, R2) LoRA-down transposed; NULL iff R2 = 0    */
+    float *lora_act_out;      /* (>= M, R2) fp32, row stride ld_lora_act_out                                    */
+    float *scratch;           /* svdq_gemm_w4a4_scratch_bytes() bytes of fp32 LoRA-down partial sums, or NULL    */
+    int32_t R2, ld_qout, ld_oscales, ld_lora_act_out;
+    float shift;              /* 0.171875 for GELU (ops/triton/gemm_w4a4.py:918), 0 for SwiGLU                  */
+} svdq_gemm_args;
+
+int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream);
+
+/* Bytes of `scratch` needed by a requantizing epilogue with LoRA-down (0 when R2 == 0). */
+size_t svdq_gemm_w4a4_scratch_bytes(int32_t M, int32_t N, int32_t R2, int32_t epilogue);
+
+/*
+ * Debug: exact int32 accumulators of one scale group, p[m, n] = sum_{k in group g} a[m, k] * w[n, k], computed by
+ * the same nibble unpack + v_mfma_i32_32x32x32_i8 sequence the GEMM uses.  out (M, N) int32 row-major.
+ */
+int svdq_group_acc_i32(const void *act, const void *wgt, int32_t *out, int32_t M, int32_t N, int32_t K,
+                       int32_t ld_act, int32_t ld_wgt, int32_t group, int32_t act_unsigned, void *stream);
+
+/*
+ * AWQ W4A16 GEMV, group 64, TinyChat packing (models/text_encoders/tinychat_utils.py:76-106):
+ * out[m, n] = sum_c s[c, n] * sum_{k in c} x[m, k] q[n, k] + z[c, n] * sum_{k in c} x[m, k]   (ops/triton/awq.py:160-182)
+ */
+typedef struct {
+    const void *x;       /* (M, K) T, row stride ld_x                               */
+    const void *qweight; /* (N/4, K) int16 (= (N/4, K/2) int32), row stride K int16 */
+    const void *scales;  /* (K/64, N) T, group stride ld_scales                     */
+    const void *zeros;   /* (K/64, N) T, same stride                                */
+    void *out;           /* (M, N) T, row stride ld_out                             */
+    int32_t M, N, K;     /* M <= 32, N % 32 == 0, K % 64 == 0                       */
+    int32_t ld_x, ld_scales, ld_out;
+    int32_t dtype;
+} svdq_awq_gemv_args;
+
+int svdq_awq_gemv_w4a16(const svdq_awq_gemv_args *args, void *stream);
+
+/* Message for the last non-zero return on the calling thread ("" if none). */
+const char *svdq_last_error(void);
+
+/* SVDQ_ABI_VERSION the library was built with. */
+int svdq_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SVDQ_MI355X_H */

@@ -1,0 +1,189 @@
+// AWQ W4A16 GEMV (group 64, TinyChat-packed weights) for gfx950, small M (<= 32 rows).
+//
+// Arithmetic (reference: nunchaku/ops/triton/awq.py:160-182):
+//   out[m, n] = sum_c  s[c, n] * sum_{k in c} x[m, k] q[n, k]  +  z[c, n] * sum_{k in c} x[m, k]      (fp32)
+//
+// The kernel is HBM-bound: N*K/2 bytes of weights are read exactly once, for all M rows together (the reference
+// launches one pass over the weights per row).
+//
+// Storage order is the access order.  Packed row a = n / 4 holds, for scale group c, 128 contiguous bytes =
+// 4 channels (b = n % 4) x 2 halves (h) x 16 bytes; the 16 bytes of (n, c, h) are eight int16 whose nibble j' holds
+// k = 64 c + 32 h + 8 j' + j (j = position of the int16).  Lane (n = lane % 32, h = lane / 32) of a wavefront loads
+// exactly that 16-byte piece, so one load instruction reads 8 packed rows x 128 contiguous bytes.  Nibble plane j' of
+// the loaded dwords, OR-ed with the bit pattern of 128.0 (bf16) / 1024.0 (fp16), is directly the B operand of one
+// 32x32x16 MFMA (exact: 128 + q and 1024 + q are representable); the A operand is the matching 16 bytes of x.  Four
+// MFMAs cover the group; the constant offset is folded into the zero-point term:
+//   s * (D - OFF * xs) + z * xs = s * D + (z - OFF * s) * xs,   xs = sum_{k in c} x[m, k]  (precomputed in LDS).
+// Only accumulator registers whose rows are < M are post-processed (rows m = 8 (i / 4) + 4 h + i % 4).
+//
+// One workgroup = 32 channels x all of K; its four wavefronts take groups round-robin with the weight loads running
+// four groups ahead, and add their partial sums through LDS in a fixed order.
+#include "svdq_common.h"
+
+namespace svdq {
+
+constexpr int AWQ_WAVES = 4;
+constexpr int AWQ_NB = 32;  // channels per workgroup
+constexpr int AWQ_PF = 4;   // weight loads in flight per lane
+
+template <typename T>
+struct AwqMagic;
+template <>
+struct AwqMagic<BF16> {
+    static constexpr uint32_t bits = 0x43004300u;  // two bf16 128.0
+    static constexpr float off = 128.0f;
+};
+template <>
+struct AwqMagic<FP16> {
+    static constexpr uint32_t bits = 0x64006400u;  // two fp16 1024.0
+    static constexpr float off = 1024.0f;
+};
+
+template <typename T, int MQ>  // MQ = ceil(M / 8): accumulator register quads that hold real rows
+__global__ __launch_bounds__(AWQ_WAVES * 64) void awq_gemv_kernel(svdq_awq_gemv_args a) {
+    extern __shared__ __align__(16) float lds[];  // xs[K/64][8*MQ], then red[AWQ_WAVES][8*MQ][32]
+    const int MR = 8 * MQ;
+    const int ngroups = a.K / GROUP;
+    float *xs = lds;
+    float *red = lds + (size_t)ngroups * MR;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int l32 = lane & 31, half = lane >> 5;
+    const int n = blockIdx.x * AWQ_NB + l32;
+    const uint16_t *x = (const uint16_t *)a.x;
+
+    // weight stream of this lane: packed row n / 4, int16 column 64 c + 16 (n % 4) + 8 h
+    const uint16_t *wq = (const uint16_t *)a.qweight + (size_t)(n >> 2) * a.K + 16 * (n & 3) + 8 * half;
+    const int nmy = (ngroups - wave + AWQ_WAVES - 1) / AWQ_WAVES;  // groups c = wave + 4 i
+    v4i wreg[AWQ_PF];
+#pragma unroll
+    for (int u = 0; u < AWQ_PF; u++)
+        if (u < nmy) wreg[u] = *(const v4i *)(wq + (size_t)(wave + AWQ_WAVES * u) * GROUP);
+
+    // xs[c][m] = sum of the group's 64 activations (fp32), while the first weight loads are in flight
+    for (int p = tid; p < ngroups * MR; p += AWQ_WAVES * 64) {
+        const int c = p / MR, m = p % MR;
+        float s = 0.0f;
+        if (m < a.M) {
+            const v4i *xp = (const v4i *)(x + (size_t)m * a.ld_x + c * GROUP);
+#pragma unroll
+            for (int q = 0; q < 8; q++) {
+                const v4i v = xp[q];
+#pragma unroll
+                for (int e = 0; e < 4; e++) s += T::lo_f32((uint32_t)v[e]) + T::hi_f32((uint32_t)v[e]);
+            }
+        }
+        xs[p] = s;
+    }
+    __syncthreads();
+
+    float acc[4 * MQ];
+#pragma unroll
+    for (int i = 0; i < 4 * MQ; i++) acc[i] = 0.0f;
+
+    const bool row_ok = l32 < a.M;  // A operand row of this lane
+    const uint16_t *xrow = x + (size_t)(row_ok ? l32 : 0) * a.ld_x + 32 * half;
+    const uint16_t *sc = (const uint16_t *)a.scales + n;
+    const uint16_t *zr = (const uint16_t *)a.zeros + n;
+
+    for (int base = 0; base < nmy; base += AWQ_PF) {
+#pragma unroll
+        for (int u = 0; u < AWQ_PF; u++) {
+            const int idx = base + u;
+            if (idx >= nmy) break;
+            const int c = wave + AWQ_WAVES * idx;
+            const v4i w = wreg[u];
+            if (idx + AWQ_PF < nmy) wreg[u] = *(const v4i *)(wq + (size_t)(c + AWQ_WAVES * AWQ_PF) * GROUP);
+            const float s = T::to_f32(sc[(size_t)c * a.ld_scales]);
+            const float zz = T::to_f32(zr[(size_t)c * a.ld_scales]) - AwqMagic<T>::off * s;
+
+            v16f d;
+#pragma unroll
+            for (int i = 0; i < 16; i++) d[i] = 0.0f;
+#pragma unroll
+            for (int pl = 0; pl < 4; pl++) {
+                typedef unsigned v4u __attribute__((ext_vector_type(4)));
+                const v4u wu = __builtin_bit_cast(v4u, w);
+                const v4i wb = __builtin_bit_cast(v4i, ((wu >> (4 * pl)) & 0x000F000Fu) | AwqMagic<T>::bits);
+                v4i xa = (v4i){0, 0, 0, 0};
+                if (row_ok) xa = *(const v4i *)(xrow + c * GROUP + 8 * pl);
+                d = mfma32_16bit<T>(xa, wb, d);
+            }
+#pragma unroll
+            for (int q = 0; q < MQ; q++) {
+                const v4f xv = *(const v4f *)(xs + c * MR + 8 * q + 4 * half);
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    acc[4 * q + e] = __builtin_fmaf(s, d[4 * q + e], acc[4 * q + e]);
+                    acc[4 * q + e] = __builtin_fmaf(zz, xv[e], acc[4 * q + e]);
+                }
+            }
+        }
+    }
+
+    // fixed-order sum over the four wavefronts, then store T
+#pragma unroll
+    for (int q = 0; q < MQ; q++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) red[(wave * MR + 8 * q + 4 * half + e) * AWQ_NB + l32] = acc[4 * q + e];
+    __syncthreads();
+    for (int o = tid; o < a.M * AWQ_NB; o += AWQ_WAVES * 64) {
+        const int m = o / AWQ_NB, nn = o % AWQ_NB;
+        float s = red[(0 * MR + m) * AWQ_NB + nn];
+#pragma unroll
+        for (int w = 1; w < AWQ_WAVES; w++) s += red[(w * MR + m) * AWQ_NB + nn];
+        ((uint16_t *)a.out)[(size_t)m * a.ld_out + blockIdx.x * AWQ_NB + nn] = T::from_f32(s);
+    }
+}
+
+template <typename T>
+static void launch_awq(const svdq_awq_gemv_args &a, hipStream_t s) {
+    const int MQ = (a.M + 7) / 8;
+    const dim3 grid(a.N / AWQ_NB), block(AWQ_WAVES * 64);
+    const size_t sh = ((size_t)(a.K / GROUP) * 8 * MQ + (size_t)AWQ_WAVES * 8 * MQ * AWQ_NB) * sizeof(float);
+    switch (MQ) {
+        case 1: hipLaunchKernelGGL((awq_gemv_kernel<T, 1>), grid, block, sh, s, a); break;
+        case 2: hipLaunchKernelGGL((awq_gemv_kernel<T, 2>), grid, block, sh, s, a); break;
+        case 3: hipLaunchKernelGGL((awq_gemv_kernel<T, 3>), grid, block, sh, s, a); break;
+        default: hipLaunchKernelGGL((awq_gemv_kernel<T, 4>), grid, block, sh, s, a); break;
+    }
+}
+
+}  // namespace svdq
+
+using namespace svdq;
+
+extern "C" int svdq_awq_gemv_w4a16(const svdq_awq_gemv_args *args, void *stream) {
+    if (!args) {
+        set_error("svdq_awq_gemv_w4a16: null args");
+        return SVDQ_E_INVALID;
+    }
+    const svdq_awq_gemv_args &a = *args;
+    if (a.dtype != SVDQ_BF16 && a.dtype != SVDQ_FP16) {
+        set_error("svdq_awq_gemv_w4a16: dtype %d", a.dtype);
+        return SVDQ_E_INVALID;
+    }
+    if (a.M < 0 || a.M > 32 || a.N <= 0 || a.N % AWQ_NB || a.K <= 0 || a.K % GROUP) {
+        set_error("svdq_awq_gemv_w4a16: M=%d N=%d K=%d needs M <= 32, N %% 32 == 0, K %% 64 == 0", a.M, a.N, a.K);
+        return SVDQ_E_INVALID;
+    }
+    if (!a.x || !a.qweight || !a.scales || !a.zeros || !a.out) {
+        set_error("svdq_awq_gemv_w4a16: null tensor");
+        return SVDQ_E_INVALID;
+    }
+    if (((uintptr_t)a.x & 15) || a.ld_x % 8 || a.ld_x < a.K || ((uintptr_t)a.qweight & 15) || a.ld_scales < a.N ||
+        a.ld_out < a.N) {
+        set_error("svdq_awq_gemv_w4a16: x rows and qweight must be 16-byte aligned; leading dimensions >= row length");
+        return SVDQ_E_INVALID;
+    }
+    if ((size_t)(a.K / GROUP) * 32 * 4 + 16384 > 65536) {
+        set_error("svdq_awq_gemv_w4a16: K=%d too large for the LDS group-sum table", a.K);
+        return SVDQ_E_UNSUPPORTED;
+    }
+    if (a.M == 0) return SVDQ_OK;
+    if (a.dtype == SVDQ_BF16)
+        launch_awq<BF16>(a, (hipStream_t)stream);
+    else
+        launch_awq<FP16>(a, (hipStream_t)stream);
+    return check_launch("svdq_awq_gemv_w4a16");
+}

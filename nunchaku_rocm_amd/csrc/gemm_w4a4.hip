@@ -1,0 +1,627 @@
+// W4A4 GEMM for gfx950 with per-group-64 scales on both operands, LoRA-up, bias and fused epilogues.
+//
+// Arithmetic contract (reference: nunchaku/ops/triton/gemm_w4a4.py:447-488, 156-209, 499-521, 730-778):
+//   out[m, n] = sum_g as[g, m] * ws[g, n] * p_g[m, n]  +  T(lora_act[m, :]) . lora_up[n, :]  +  bias[n]
+// with p_g the exact int32 dot product of the group's 64 int4 pairs.
+//
+// How it maps to CDNA4:
+//  * p_g comes from two v_mfma_i32_32x32x32_i8 per 32x32 block.  A 16-byte LDS read holds 32 nibbles; the even and
+//    the odd nibbles are split into two int8 planes with shift/mask only (signed values land in the high nibble of
+//    each byte, i.e. times 16; unsigned activations in the low nibble, times 1).  Both operands use the same split,
+//    so the K order inside a group is a shared permutation and the dot product is unchanged.  The power-of-two
+//    factor (256 signed, 16 unsigned) is folded exactly into the fp32 activation scale.
+//  * The MFMA accumulator starts at the bit pattern of 1.5*2^23, so the int32 result read as fp32 is (2^23*1.5 + p)
+//    exactly and  fma(bits, as', -1.5*2^23*as')  gives p*as' with one rounding and no int->float convert; a second
+//    fma applies ws[g, n] and accumulates.  Two VALU ops per accumulator element per group.
+//  * The MFMA's A operand is the weight tile and its B operand the activation tile, so a lane owns one activation
+//    row m and its registers walk n in runs of four.  Row-wise epilogue work (RMSNorm sum of squares, RoPE pairs,
+//    group absmax, nibble packing, the next layer's LoRA-down B operand) is therefore in-lane plus one exchange with
+//    lane ^ 32.
+//  * 256 threads = 2x2 wavefronts of 64x64 on a 128x128 tile; K is staged through LDS 128 at a time (two scale
+//    groups) with register prefetch of the next stage and two LDS buffers (one barrier per stage).  LDS rows are
+//    padded to 80 bytes so the 16-byte operand reads are bank-conflict free.
+//  * Workgroup ids are first regrouped so that each XCD (ids are dealt round-robin over 8 XCDs) works on a
+//    contiguous range of tiles, then swizzled in bands of m-tiles for L2 reuse of the weight tile.
+#include "svdq_common.h"
+
+namespace svdq {
+
+constexpr int BM = 128, BN = 128;     // workgroup tile (activation rows x weight rows)
+constexpr int KSTAGE = 128;           // K per LDS stage = two scale groups
+constexpr int LDS_ROW = 80;           // bytes per staged row: 64 data + 16 pad
+constexpr int A_OFF = 0;
+constexpr int W_OFF = BM * LDS_ROW;                       // 10240
+constexpr int AS_OFF = W_OFF + BN * LDS_ROW;              // 20480: float as'[2][BM]
+constexpr int NM_OFF = AS_OFF + 2 * BM * 4;               // float -magic*as'[2][BM]
+constexpr int WS_OFF = NM_OFF + 2 * BM * 4;               // float ws[2][BN]
+constexpr int BUF_BYTES = WS_OFF + 2 * BN * 4;            // 23552
+constexpr int SMEM_BYTES = 2 * BUF_BYTES;                 // 47104
+constexpr int GROUP_M_TILES = 8;      // m-tiles per raster band
+constexpr int NUM_XCD = 8;
+
+__device__ inline void unpack_signed(v4i p, v4i &even, v4i &odd) {
+    even = (p << 4) & (int)0xF0F0F0F0;  // 16 * value in each byte
+    odd = p & (int)0xF0F0F0F0;
+}
+__device__ inline void unpack_unsigned(v4i p, v4i &even, v4i &odd) {
+    typedef unsigned v4u __attribute__((ext_vector_type(4)));
+    v4u u = __builtin_bit_cast(v4u, p);
+    even = __builtin_bit_cast(v4i, u & 0x0F0F0F0Fu);
+    odd = __builtin_bit_cast(v4i, (u >> 4) & 0x0F0F0F0Fu);
+}
+
+__device__ inline v16i magic_acc() {
+    v16i c;
+#pragma unroll
+    for (int i = 0; i < 16; i++) c[i] = RNE_MAGIC_BITS;
+    return c;
+}
+
+// (pid_m, pid_n) of this workgroup: XCD-contiguous renumbering, then m-banded raster.
+__device__ inline void tile_ids(int tiles_m, int tiles_n, int &pid_m, int &pid_n) {
+    const int nb = gridDim.x;
+    const int bid = blockIdx.x;
+    const int xcd = bid % NUM_XCD, loc = bid / NUM_XCD;
+    const int per = (nb + NUM_XCD - 1) / NUM_XCD, rem = nb % NUM_XCD;
+    const int start = (rem == 0 || xcd < rem) ? xcd * per : rem * per + (xcd - rem) * (per - 1);
+    const int id = start + loc;
+    const int band = GROUP_M_TILES * tiles_n;
+    const int first_m = (id / band) * GROUP_M_TILES;
+    const int gm = min(tiles_m - first_m, GROUP_M_TILES);
+    pid_m = first_m + (id % band) % gm;
+    pid_n = (id % band) / gm;
+}
+
+template <typename T, bool ACT_UNSIGNED, int EPI>
+__global__ __launch_bounds__(256, 2) void gemm_w4a4_kernel(svdq_gemm_args a) {
+    __shared__ __align__(16) uint8_t smem[SMEM_BYTES];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wn = wave & 1, wm = wave >> 1;  // wavefront position in the 2x2 arrangement
+    const int l32 = lane & 31, half = lane >> 5;
+
+    int pid_m, pid_n;
+    tile_ids((a.M + BM - 1) / BM, (a.N + BN - 1) / BN, pid_m, pid_n);
+    const int m0 = pid_m * BM, n0 = pid_n * BN;
+
+    // ---- global -> register staging roles -------------------------------------------------------
+    // 512 16-byte chunks per operand tile and stage: chunk c -> row c / 4, 16-byte column c % 4
+    const uint8_t *gA[2], *gW[2];
+    int sA[2];
+#pragma unroll
+    for (int p = 0; p < 2; p++) {
+        const int c = tid + 256 * p, row = c >> 2, col = c & 3;
+        gA[p] = (const uint8_t *)a.act + (size_t)min(m0 + row, a.M - 1) * a.ld_act + col * 16;
+        gW[p] = (const uint8_t *)a.wgt + (size_t)min(n0 + row, a.N - 1) * a.ld_wgt + col * 16;
+        sA[p] = row * LDS_ROW + col * 16;
+    }
+    const int sg = tid >> 7, sr = tid & 127;  // scale loader: group within stage, row within tile
+    const uint16_t *gAS = (const uint16_t *)a.ascales + (size_t)sg * a.ld_ascales + min(m0 + sr, a.M - 1);
+    const uint16_t *gWS = (const uint16_t *)a.wscales + (size_t)sg * a.ld_wscales + min(n0 + sr, a.N - 1);
+    const float fold = ACT_UNSIGNED ? (1.0f / 16.0f) : (1.0f / 256.0f);
+
+    v4i ra[2], rw[2];
+    uint16_t ras, rws;
+    auto load_stage = [&](int s) {
+#pragma unroll
+        for (int p = 0; p < 2; p++) {
+            ra[p] = *(const v4i *)(gA[p] + (size_t)s * (KSTAGE / 2));
+            rw[p] = *(const v4i *)(gW[p] + (size_t)s * (KSTAGE / 2));
+        }
+        ras = gAS[(size_t)s * 2 * a.ld_ascales];
+        rws = gWS[(size_t)s * 2 * a.ld_wscales];
+    };
+    auto store_stage = [&](int b) {
+        uint8_t *base = smem + b * BUF_BYTES;
+#pragma unroll
+        for (int p = 0; p < 2; p++) {
+            *(v4i *)(base + A_OFF + sA[p]) = ra[p];
+            *(v4i *)(base + W_OFF + sA[p]) = rw[p];
+        }
+        const float as = T::to_f32(ras) * fold;
+        ((float *)(base + AS_OFF))[sg * BM + sr] = as;
+        ((float *)(base + NM_OFF))[sg * BM + sr] = -RNE_MAGIC * as;
+        ((float *)(base + WS_OFF))[sg * BN + sr] = T::to_f32(rws);
+    };
+
+    v16f acc[2][2];
+#pragma unroll
+    for (int bn = 0; bn < 2; bn++)
+#pragma unroll
+        for (int bm = 0; bm < 2; bm++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[bn][bm][i] = 0.0f;
+
+    const v16i cmagic = magic_acc();
+    const int nstages = a.K / KSTAGE;
+    const int rowW = (wn * 64 + l32) * LDS_ROW + half * 16;
+    const int rowA = (wm * 64 + l32) * LDS_ROW + half * 16;
+
+    load_stage(0);
+    for (int s = 0; s < nstages; s++) {
+        const int b = s & 1;
+        store_stage(b);
+        __syncthreads();
+        if (s + 1 < nstages) load_stage(s + 1);
+        const uint8_t *base = smem + b * BUF_BYTES;
+#pragma unroll
+        for (int gg = 0; gg < 2; gg++) {
+            v4i we[2], wo[2], ae[2], ao[2];
+#pragma unroll
+            for (int blk = 0; blk < 2; blk++) {
+                v4i wp = *(const v4i *)(base + W_OFF + rowW + blk * 32 * LDS_ROW + gg * 32);
+                v4i ap = *(const v4i *)(base + A_OFF + rowA + blk * 32 * LDS_ROW + gg * 32);
+                unpack_signed(wp, we[blk], wo[blk]);
+                if (ACT_UNSIGNED)
+                    unpack_unsigned(ap, ae[blk], ao[blk]);
+                else
+                    unpack_signed(ap, ae[blk], ao[blk]);
+            }
+            float asl[2], nml[2];
+#pragma unroll
+            for (int bm = 0; bm < 2; bm++) {
+                asl[bm] = ((const float *)(base + AS_OFF))[gg * BM + wm * 64 + bm * 32 + l32];
+                nml[bm] = ((const float *)(base + NM_OFF))[gg * BM + wm * 64 + bm * 32 + l32];
+            }
+#pragma unroll
+            for (int bn = 0; bn < 2; bn++) {
+                v4f wsr[4];
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+                    wsr[j] = *(const v4f *)((const float *)(base + WS_OFF) + gg * BN + wn * 64 + bn * 32 + 8 * j + 4 * half);
+#pragma unroll
+                for (int bm = 0; bm < 2; bm++) {
+                    v16i t = __builtin_amdgcn_mfma_i32_32x32x32_i8(we[bn], ae[bm], cmagic, 0, 0, 0);
+                    t = __builtin_amdgcn_mfma_i32_32x32x32_i8(wo[bn], ao[bm], t, 0, 0, 0);
+#pragma unroll
+                    for (int i = 0; i < 16; i++) {
+                        const float u = __builtin_fmaf(__int_as_float(t[i]), asl[bm], nml[bm]);
+                        acc[bn][bm][i] = __builtin_fmaf(u, wsr[i >> 2][i & 3], acc[bn][bm][i]);
+                    }
+                }
+            }
+        }
+    }
+
+    // ---- epilogue: LoRA-up and bias ----------------------------------------------------------------
+    const int nw0 = n0 + wn * 64, mw0 = m0 + wm * 64;
+    if (a.R > 0) {
+        const uint16_t *lu = (const uint16_t *)a.lora_up;
+        for (int r0 = 0; r0 < a.R; r0 += 16) {
+            v4i ua[2], ub[2];
+#pragma unroll
+            for (int blk = 0; blk < 2; blk++) {
+                const int n = nw0 + blk * 32 + l32, m = mw0 + blk * 32 + l32;
+                ua[blk] = (v4i){0, 0, 0, 0};
+                ub[blk] = (v4i){0, 0, 0, 0};
+                if (n < a.N) ua[blk] = *(const v4i *)(lu + (size_t)n * a.ld_lora_up + r0 + half * 8);
+                if (m < a.M) {
+                    const float *lp = a.lora_act + (size_t)m * a.ld_lora_act + r0 + half * 8;
+                    const v4f f0 = *(const v4f *)lp, f1 = *(const v4f *)(lp + 4);
+                    ub[blk][0] = (int)pack2<T>(f0[0], f0[1]);
+                    ub[blk][1] = (int)pack2<T>(f0[2], f0[3]);
+                    ub[blk][2] = (int)pack2<T>(f1[0], f1[1]);
+                    ub[blk][3] = (int)pack2<T>(f1[2], f1[3]);
+                }
+            }
+#pragma unroll
+            for (int bn = 0; bn < 2; bn++)
+#pragma unroll
+                for (int bm = 0; bm < 2; bm++) acc[bn][bm] = mfma32_16bit<T>(ua[bn], ub[bm], acc[bn][bm]);
+        }
+    }
+    if (a.bias != nullptr) {
+        const uint16_t *bias = (const uint16_t *)a.bias;
+#pragma unroll
+        for (int bn = 0; bn < 2; bn++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int n = nw0 + bn * 32 + 8 * j + 4 * half;
+                if (n < a.N) {
+                    const uint2 bb = *(const uint2 *)(bias + n);
+                    const float b0 = T::lo_f32(bb.x), b1 = T::hi_f32(bb.x), b2 = T::lo_f32(bb.y), b3 = T::hi_f32(bb.y);
+#pragma unroll
+                    for (int bm = 0; bm < 2; bm++) {
+                        acc[bn][bm][4 * j + 0] += b0;
+                        acc[bn][bm][4 * j + 1] += b1;
+                        acc[bn][bm][4 * j + 2] += b2;
+                        acc[bn][bm][4 * j + 3] += b3;
+                    }
+                }
+            }
+    }
+
+    auto store_out = [&]() {
+        uint16_t *out = (uint16_t *)a.out;
+#pragma unroll
+        for (int bm = 0; bm < 2; bm++) {
+            const int m = mw0 + bm * 32 + l32;
+            if (m >= a.actual_m) continue;
+#pragma unroll
+            for (int bn = 0; bn < 2; bn++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const int n = nw0 + bn * 32 + 8 * j + 4 * half;
+                    if (n < a.N) {
+                        uint2 v;
+                        v.x = pack2<T>(acc[bn][bm][4 * j], acc[bn][bm][4 * j + 1]);
+                        v.y = pack2<T>(acc[bn][bm][4 * j + 2], acc[bn][bm][4 * j + 3]);
+                        *(uint2 *)(out + (size_t)m * a.ld_out + n) = v;
+                    }
+                }
+        }
+    };
+
+    if (EPI == SVDQ_EPI_PLAIN) {
+        store_out();
+        return;
+    }
+
+    if (EPI == SVDQ_EPI_QK_NORM_ROPE) {
+        // the 128-wide tile is one head; part 0 = Q, 1 = K, 2 = V (untouched)
+        const int part = n0 / (a.N / 3);
+        if (part < 2) {
+            float *red = (float *)smem;  // [2 (wn)][BM]
+            __syncthreads();             // main-loop LDS reads are done
+#pragma unroll
+            for (int bm = 0; bm < 2; bm++) {
+                float ss = 0.0f;
+#pragma unroll
+                for (int bn = 0; bn < 2; bn++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++) ss += acc[bn][bm][i] * acc[bn][bm][i];
+                ss += __shfl_xor(ss, 32);
+                if (half == 0) red[wn * BM + wm * 64 + bm * 32 + l32] = ss;
+            }
+            __syncthreads();
+            const uint16_t *nw = (const uint16_t *)(part == 0 ? a.norm_q : a.norm_k);
+#pragma unroll
+            for (int bm = 0; bm < 2; bm++) {
+                const int ml = wm * 64 + bm * 32 + l32;
+                const int m = m0 + ml;
+                const float tot = red[ml] + red[BM + ml];
+                const float rstd = 1.0f / sqrtf(tot / 128.0f + a.eps);
+                const bool rok = m < a.actual_m;
+                const float *rot = a.rotary + (size_t)(rok ? m : 0) * a.ld_rotary;
+#pragma unroll
+                for (int bn = 0; bn < 2; bn++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        const int d = wn * 64 + bn * 32 + 8 * j + 4 * half;  // channel within the head
+                        const uint2 wb = *(const uint2 *)(nw + d);
+                        const v4f sc = *(const v4f *)(rot + d);  // (sin, cos, sin, cos)
+                        const float x0 = acc[bn][bm][4 * j + 0] * rstd * T::lo_f32(wb.x);
+                        const float x1 = acc[bn][bm][4 * j + 1] * rstd * T::hi_f32(wb.x);
+                        const float x2 = acc[bn][bm][4 * j + 2] * rstd * T::lo_f32(wb.y);
+                        const float x3 = acc[bn][bm][4 * j + 3] * rstd * T::hi_f32(wb.y);
+                        acc[bn][bm][4 * j + 0] = x0 * sc[1] - x1 * sc[0];
+                        acc[bn][bm][4 * j + 1] = x0 * sc[0] + x1 * sc[1];
+                        acc[bn][bm][4 * j + 2] = x2 * sc[3] - x3 * sc[2];
+                        acc[bn][bm][4 * j + 3] = x2 * sc[2] + x3 * sc[3];
+                    }
+            }
+        }
+        store_out();
+        return;
+    }
+
+    if (EPI == SVDQ_EPI_GELU_QUANT) {
+        if (a.out != nullptr) store_out();  // pre-GELU output, when asked for
+        const uint16_t *ldt = (const uint16_t *)a.lora_down_t;
+        float *lds_part = (float *)smem;  // [2 (wm)][2 (bm)][16 regs][64 lanes] floats = 16 KB
+        __syncthreads();
+#pragma unroll
+        for (int bn = 0; bn < 2; bn++)
+#pragma unroll
+            for (int bm = 0; bm < 2; bm++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) acc[bn][bm][i] = gelu_tanh(acc[bn][bm][i]);
+
+        // next layer's LoRA-down on the un-shifted, un-smoothed GELU output rounded to T:
+        // D[r][m] = sum_n ldT[r][n] * x[n][m]; registers [8 s, 8 s + 8) of a block are one MFMA's B operand
+        for (int rc = 0; rc < a.R2; rc += 32) {
+            v16f d[2];
+#pragma unroll
+            for (int bm = 0; bm < 2; bm++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) d[bm][i] = 0.0f;
+            const int r = rc + l32;
+#pragma unroll
+            for (int bn = 0; bn < 2; bn++)
+#pragma unroll
+                for (int s = 0; s < 2; s++) {
+                    v4i la = (v4i){0, 0, 0, 0};
+                    if (r < a.R2) {
+                        const uint16_t *lp = ldt + (size_t)r * a.N + nw0 + bn * 32 + 16 * s + 4 * half;
+                        const uint2 q0 = *(const uint2 *)lp, q1 = *(const uint2 *)(lp + 8);
+                        la = (v4i){(int)q0.x, (int)q0.y, (int)q1.x, (int)q1.y};
+                    }
+#pragma unroll
+                    for (int bm = 0; bm < 2; bm++) {
+                        v4i xb;
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            xb[e] = (int)pack2<T>(acc[bn][bm][8 * s + 2 * e], acc[bn][bm][8 * s + 2 * e + 1]);
+                        d[bm] = mfma32_16bit<T>(la, xb, d[bm]);
+                    }
+                }
+            // add the two n-wavefronts in a fixed order (wn = 0 first), then one partial per n-tile
+            if (wn == 1) {
+#pragma unroll
+                for (int bm = 0; bm < 2; bm++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++) lds_part[((wm * 2 + bm) * 16 + i) * 64 + lane] = d[bm][i];
+            }
+            __syncthreads();
+            if (wn == 0) {
+#pragma unroll
+                for (int bm = 0; bm < 2; bm++) {
+                    const int m = mw0 + bm * 32 + l32;
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        v4f o;
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            o[e] = d[bm][4 * j + e] + lds_part[((wm * 2 + bm) * 16 + 4 * j + e) * 64 + lane];
+                        const int rr = rc + 8 * j + 4 * half;
+                        if (m < a.M && rr < a.R2)
+                            *(v4f *)(a.scratch + ((size_t)pid_n * a.M + m) * a.R2 + rr) = o;
+                    }
+                }
+            }
+            __syncthreads();
+        }
+
+        // +shift, * 1/smooth, unsigned per-64 quantization: the wavefront's 64 columns are one group
+        float *lds_rs = (float *)smem;  // [BN]
+        if (tid < BN) {
+            float rs = 1.0f;
+            if (a.smooth_next != nullptr && n0 + tid < a.N)
+                rs = 1.0f / T::to_f32(((const uint16_t *)a.smooth_next)[n0 + tid]);
+            lds_rs[tid] = rs;
+        }
+        __syncthreads();
+        const int g = nw0 / GROUP;
+#pragma unroll
+        for (int bm = 0; bm < 2; bm++) {
+            const int m = mw0 + bm * 32 + l32;
+            float gmax = 0.0f;
+#pragma unroll
+            for (int bn = 0; bn < 2; bn++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const v4f rs = *(const v4f *)(lds_rs + wn * 64 + bn * 32 + 8 * j + 4 * half);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const float v = (acc[bn][bm][4 * j + e] + a.shift) * rs[e];
+                        acc[bn][bm][4 * j + e] = v;
+                        gmax = fmaxf(gmax, v);
+                    }
+                }
+            gmax = fmaxf(gmax, __shfl_xor(gmax, 32));
+            const float scale = gmax / 15.0f;
+            const float safe = (scale == 0.0f) ? 1.0f : scale;
+            const float rq = 1.0f / safe;
+            if (half == 0 && m < a.M && nw0 < a.N) ((uint16_t *)a.oscales)[(size_t)g * a.ld_oscales + m] = T::from_f32(scale);
+#pragma unroll
+            for (int bn = 0; bn < 2; bn++) {
+                uint32_t mine[4];
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    uint32_t w = 0;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const float q = __builtin_amdgcn_fmed3f(acc[bn][bm][4 * j + e] * rq, 0.0f, 15.0f) + RNE_MAGIC;
+                        w |= (__float_as_uint(q) & 0xFu) << (4 * e);
+                    }
+                    mine[j] = w;  // 16 bits: columns 8 j + 4 half + 0..3
+                }
+                // lane and lane ^ 32 hold alternating 16-bit pieces of one 16-byte run (dword j = piece of half 0 in
+                // the low 16 bits, piece of half 1 in the high 16 bits); trade so half 0 stores dwords 0-1 and half 1
+                // stores dwords 2-3
+                uint32_t dw[2];
+#pragma unroll
+                for (int t = 0; t < 2; t++) {
+                    const uint32_t keep = half ? mine[2 + t] : mine[t];
+                    const uint32_t send = half ? mine[t] : mine[2 + t];
+                    const uint32_t theirs = __shfl_xor(send, 32);
+                    dw[t] = half ? (theirs | (keep << 16)) : (keep | (theirs << 16));
+                }
+                if (m < a.M)
+                    *(uint2 *)((uint8_t *)a.qout + (size_t)m * a.ld_qout + (nw0 + bn * 32) / 2 + 8 * half) =
+                        make_uint2(dw[0], dw[1]);
+            }
+        }
+        return;
+    }
+}
+
+// lora_act_out[m, r] = sum over n-tiles of the partial LoRA-down products, in tile order (deterministic)
+__global__ void lora_part_reduce_kernel(const float *part, float *out, int tiles, int M, int R2, int ld_out) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= M * R2) return;
+    float s = 0.0f;
+    for (int t = 0; t < tiles; t++) s += part[(size_t)t * M * R2 + idx];
+    out[(size_t)(idx / R2) * ld_out + idx % R2] = s;
+}
+
+// Debug read-out of one group's exact int32 accumulators: one wavefront per 32x32 block, operands straight from
+// global memory, same unpack + MFMA sequence as the GEMM main loop.
+template <bool ACT_UNSIGNED>
+__global__ __launch_bounds__(64) void group_acc_kernel(const uint8_t *act, const uint8_t *wgt, int32_t *out, int M,
+                                                       int N, int ld_act, int ld_wgt, int group) {
+    const int lane = threadIdx.x, l32 = lane & 31, half = lane >> 5;
+    const int nb = blockIdx.x * 32, mb = blockIdx.y * 32;
+    const v4i wp = *(const v4i *)(wgt + (size_t)min(nb + l32, N - 1) * ld_wgt + group * 32 + half * 16);
+    const v4i ap = *(const v4i *)(act + (size_t)min(mb + l32, M - 1) * ld_act + group * 32 + half * 16);
+    v4i we, wo, ae, ao;
+    unpack_signed(wp, we, wo);
+    if (ACT_UNSIGNED)
+        unpack_unsigned(ap, ae, ao);
+    else
+        unpack_signed(ap, ae, ao);
+    v16i t = __builtin_amdgcn_mfma_i32_32x32x32_i8(we, ae, magic_acc(), 0, 0, 0);
+    t = __builtin_amdgcn_mfma_i32_32x32x32_i8(wo, ao, t, 0, 0, 0);
+    const int m = mb + l32;
+    if (m >= M) return;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        const int n = nb + 8 * (i >> 2) + 4 * half + (i & 3);
+        if (n < N) out[(size_t)m * N + n] = (t[i] - RNE_MAGIC_BITS) >> (ACT_UNSIGNED ? 4 : 8);
+    }
+}
+
+template <typename T, bool U>
+static void launch_gemm_epi(const svdq_gemm_args &a, hipStream_t s) {
+    const dim3 grid(((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN)), block(256);
+    switch (a.epilogue) {
+        case SVDQ_EPI_PLAIN:
+            hipLaunchKernelGGL((gemm_w4a4_kernel<T, U, SVDQ_EPI_PLAIN>), grid, block, 0, s, a);
+            break;
+        case SVDQ_EPI_QK_NORM_ROPE:
+            hipLaunchKernelGGL((gemm_w4a4_kernel<T, U, SVDQ_EPI_QK_NORM_ROPE>), grid, block, 0, s, a);
+            break;
+        case SVDQ_EPI_GELU_QUANT:
+            hipLaunchKernelGGL((gemm_w4a4_kernel<T, U, SVDQ_EPI_GELU_QUANT>), grid, block, 0, s, a);
+            break;
+    }
+}
+
+}  // namespace svdq
+
+using namespace svdq;
+
+static bool al16(const void *p) { return ((uintptr_t)p & 15) == 0; }
+
+extern "C" size_t svdq_gemm_w4a4_scratch_bytes(int32_t M, int32_t N, int32_t R2, int32_t epilogue) {
+    if (R2 <= 0 || (epilogue != SVDQ_EPI_GELU_QUANT && epilogue != SVDQ_EPI_SWIGLU_QUANT)) return 0;
+    return (size_t)((N + BN - 1) / BN) * (size_t)M * (size_t)R2 * sizeof(float);
+}
+
+extern "C" int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream) {
+    if (!args) {
+        set_error("svdq_gemm_w4a4: null args");
+        return SVDQ_E_INVALID;
+    }
+    const svdq_gemm_args &a = *args;
+    if (a.dtype != SVDQ_BF16 && a.dtype != SVDQ_FP16) {
+        set_error("svdq_gemm_w4a4: dtype %d", a.dtype);
+        return SVDQ_E_INVALID;
+    }
+    if (a.M < 0 || a.N <= 0 || a.K <= 0 || a.K % KSTAGE || a.N % 8) {
+        set_error("svdq_gemm_w4a4: M=%d N=%d K=%d needs K %% 128 == 0 and N %% 8 == 0", a.M, a.N, a.K);
+        return SVDQ_E_INVALID;
+    }
+    if (!a.act || !a.wgt || !a.ascales || !a.wscales) {
+        set_error("svdq_gemm_w4a4: act, wgt, ascales and wscales are required");
+        return SVDQ_E_INVALID;
+    }
+    if (!al16(a.act) || !al16(a.wgt) || a.ld_act % 16 || a.ld_wgt % 16 || a.ld_act < a.K / 2 || a.ld_wgt < a.K / 2) {
+        set_error("svdq_gemm_w4a4: act/wgt rows must be 16-byte aligned and at least K/2 bytes (ld_act=%d ld_wgt=%d)",
+                  a.ld_act, a.ld_wgt);
+        return SVDQ_E_INVALID;
+    }
+    if (a.ld_ascales < a.M || a.ld_wscales < a.N) {
+        set_error("svdq_gemm_w4a4: scale rows shorter than M / N");
+        return SVDQ_E_INVALID;
+    }
+    if (a.R < 0 || a.R % 16 || (a.R > 0 && (!a.lora_act || !a.lora_up))) {
+        set_error("svdq_gemm_w4a4: R=%d must be a multiple of 16 with lora_act and lora_up given", a.R);
+        return SVDQ_E_INVALID;
+    }
+    if (a.R > 0 && (!al16(a.lora_act) || !al16(a.lora_up) || a.ld_lora_act % 4 || a.ld_lora_up % 8 ||
+                    a.ld_lora_act < a.R || a.ld_lora_up < a.R)) {
+        set_error("svdq_gemm_w4a4: LoRA rows must be 16-byte aligned");
+        return SVDQ_E_INVALID;
+    }
+    if (a.bias && ((uintptr_t)a.bias & 7)) {
+        set_error("svdq_gemm_w4a4: bias must be 8-byte aligned");
+        return SVDQ_E_INVALID;
+    }
+    if (a.actual_m < 0 || a.actual_m > a.M) {
+        set_error("svdq_gemm_w4a4: actual_m=%d outside [0, M=%d]", a.actual_m, a.M);
+        return SVDQ_E_INVALID;
+    }
+    const bool quant = a.epilogue == SVDQ_EPI_GELU_QUANT || a.epilogue == SVDQ_EPI_SWIGLU_QUANT;
+    if (!quant && !a.out) {
+        set_error("svdq_gemm_w4a4: out is required for this epilogue");
+        return SVDQ_E_INVALID;
+    }
+    if (a.out && (((uintptr_t)a.out & 7) || a.ld_out % 4 || a.ld_out < a.N)) {
+        set_error("svdq_gemm_w4a4: out rows must be 8-byte aligned and at least N long (ld_out=%d)", a.ld_out);
+        return SVDQ_E_INVALID;
+    }
+    if (a.epilogue == SVDQ_EPI_QK_NORM_ROPE) {
+        if (a.N % 3 || (a.N / 3) % 128) {
+            set_error("svdq_gemm_w4a4: N=%d is not three whole sets of 128-wide heads", a.N);
+            return SVDQ_E_INVALID;
+        }
+        if (!a.norm_q || !a.norm_k || !a.rotary || ((uintptr_t)a.norm_q & 7) || ((uintptr_t)a.norm_k & 7) ||
+            !al16(a.rotary) || a.ld_rotary % 4 || a.ld_rotary < 128) {
+            set_error("svdq_gemm_w4a4: norm_q, norm_k (128,) and rotary (actual_m, 128) fp32 16-byte aligned rows are required");
+            return SVDQ_E_INVALID;
+        }
+    } else if (a.epilogue == SVDQ_EPI_GELU_QUANT) {
+        if (a.N % 128 || a.M % 16) {
+            set_error("svdq_gemm_w4a4: the GELU requantizing epilogue needs N %% 128 == 0 and M %% 16 == 0 (M=%d N=%d)", a.M, a.N);
+            return SVDQ_E_INVALID;
+        }
+        if (!a.qout || !a.oscales || ((uintptr_t)a.qout & 7) || a.ld_qout % 8 || a.ld_qout < a.N / 2 || a.ld_oscales < a.M) {
+            set_error("svdq_gemm_w4a4: qout (8-byte aligned rows) and oscales are required");
+            return SVDQ_E_INVALID;
+        }
+        if (a.R2 < 0 || a.R2 % 16 ||
+            (a.R2 > 0 && (!a.lora_down_t || !a.lora_act_out || !a.scratch || ((uintptr_t)a.lora_down_t & 7) ||
+                          !al16(a.scratch) || a.ld_lora_act_out < a.R2))) {
+            set_error("svdq_gemm_w4a4: R2=%d must be a multiple of 16 with lora_down_t, lora_act_out and scratch given", a.R2);
+            return SVDQ_E_INVALID;
+        }
+    } else if (a.epilogue == SVDQ_EPI_SWIGLU_QUANT) {
+        set_error("svdq_gemm_w4a4: the SwiGLU requantizing epilogue is not implemented yet");
+        return SVDQ_E_UNSUPPORTED;
+    } else if (a.epilogue != SVDQ_EPI_PLAIN) {
+        set_error("svdq_gemm_w4a4: unknown epilogue %d", a.epilogue);
+        return SVDQ_E_INVALID;
+    }
+    if (a.M == 0) return SVDQ_OK;
+    hipStream_t s = (hipStream_t)stream;
+    if (a.dtype == SVDQ_BF16) {
+        if (a.act_unsigned)
+            launch_gemm_epi<BF16, true>(a, s);
+        else
+            launch_gemm_epi<BF16, false>(a, s);
+    } else {
+        if (a.act_unsigned)
+            launch_gemm_epi<FP16, true>(a, s);
+        else
+            launch_gemm_epi<FP16, false>(a, s);
+    }
+    int rc = check_launch("svdq_gemm_w4a4");
+    if (rc) return rc;
+    if (quant && a.R2 > 0) {
+        const int n = a.M * a.R2;
+        hipLaunchKernelGGL(lora_part_reduce_kernel, dim3((n + 255) / 256), dim3(256), 0, s, a.scratch, a.lora_act_out,
+                           (a.N + BN - 1) / BN, a.M, a.R2, a.ld_lora_act_out);
+        rc = check_launch("svdq_gemm_w4a4 (LoRA-down partial sum)");
+    }
+    return rc;
+}
+
+extern "C" int svdq_group_acc_i32(const void *act, const void *wgt, int32_t *out, int32_t M, int32_t N, int32_t K,
+                                  int32_t ld_act, int32_t ld_wgt, int32_t group, int32_t act_unsigned, void *stream) {
+    if (!act || !wgt || !out || M <= 0 || N <= 0 || K <= 0 || K % GROUP || group < 0 || group >= K / GROUP ||
+        !al16(act) || !al16(wgt) || ld_act % 16 || ld_wgt % 16) {
+        set_error("svdq_group_acc_i32: bad arguments (M=%d N=%d K=%d group=%d)", M, N, K, group);
+        return SVDQ_E_INVALID;
+    }
+    const dim3 grid((N + 31) / 32, (M + 31) / 32), block(64);
+    if (act_unsigned)
+        hipLaunchKernelGGL(group_acc_kernel<true>, grid, block, 0, (hipStream_t)stream, (const uint8_t *)act,
+                           (const uint8_t *)wgt, out, M, N, ld_act, ld_wgt, group);
+    else
+        hipLaunchKernelGGL(group_acc_kernel<false>, grid, block, 0, (hipStream_t)stream, (const uint8_t *)act,
+                           (const uint8_t *)wgt, out, M, N, ld_act, ld_wgt, group);
+    return check_launch("svdq_group_acc_i32");
+}

@@ -1,0 +1,95 @@
+// Shared device/host helpers for the gfx950 SVDQuant kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/svdq_mi355x.h"
+
+namespace svdq {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef short v8s __attribute__((ext_vector_type(8)));
+
+constexpr int GROUP = 64;            // int4 scale group along K
+constexpr float RNE_MAGIC = 12582912.0f;  // 1.5 * 2^23: adding it rounds an fp32 at the units place (RNE)
+constexpr int RNE_MAGIC_BITS = 0x4B400000;
+
+// ---- 16-bit float types -------------------------------------------------------------------------
+struct BF16 {
+    static constexpr int code = SVDQ_BF16;
+    __device__ static inline float to_f32(uint16_t h) { return __uint_as_float(((uint32_t)h) << 16); }
+    // two packed values: low half / high half of a dword
+    __device__ static inline float lo_f32(uint32_t w) { return __uint_as_float(w << 16); }
+    __device__ static inline float hi_f32(uint32_t w) { return __uint_as_float(w & 0xFFFF0000u); }
+    __device__ static inline uint16_t from_f32(float f) {  // round to nearest even
+        uint32_t u = __float_as_uint(f);
+        if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40);
+        u += 0x7FFFu + ((u >> 16) & 1u);
+        return (uint16_t)(u >> 16);
+    }
+};
+
+struct FP16 {
+    static constexpr int code = SVDQ_FP16;
+    __device__ static inline float to_f32(uint16_t h) {
+        _Float16 v;
+        __builtin_memcpy(&v, &h, 2);
+        return (float)v;
+    }
+    __device__ static inline float lo_f32(uint32_t w) { return to_f32((uint16_t)(w & 0xFFFFu)); }
+    __device__ static inline float hi_f32(uint32_t w) { return to_f32((uint16_t)(w >> 16)); }
+    __device__ static inline uint16_t from_f32(float f) {
+        _Float16 v = (_Float16)f;  // v_cvt_f16_f32: round to nearest even
+        uint16_t h;
+        __builtin_memcpy(&h, &v, 2);
+        return h;
+    }
+};
+
+template <typename T>
+__device__ inline uint32_t pack2(float a, float b) {
+    return (uint32_t)T::from_f32(a) | ((uint32_t)T::from_f32(b) << 16);
+}
+
+// MFMA on eight 16-bit values per lane (K = 16 for 32x32, K = 32 for 16x16); operands passed as raw bits.
+template <typename T>
+__device__ inline v16f mfma32_16bit(v4i a, v4i b, v16f c);
+template <>
+__device__ inline v16f mfma32_16bit<BF16>(v4i a, v4i b, v16f c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
+}
+template <>
+__device__ inline v16f mfma32_16bit<FP16>(v4i a, v4i b, v16f c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0, 0, 0);
+}
+template <typename T>
+__device__ inline v4f mfma16_16bit(v4i a, v4i b, v4f c);
+template <>
+__device__ inline v4f mfma16_16bit<BF16>(v4i a, v4i b, v4f c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, a), __builtin_bit_cast(v8bf, b), c, 0, 0, 0);
+}
+template <>
+__device__ inline v4f mfma16_16bit<FP16>(v4i a, v4i b, v4f c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0, 0, 0);
+}
+
+__device__ inline float gelu_tanh(float x) {
+    // 0.5 x (1 + tanh(0.79788456 (x + 0.044715 x^3))), tanh through exp as the reference spells it
+    float inner = 0.79788456f * (x + 0.044715f * x * x * x);
+    float t = 2.0f / (1.0f + __expf(-2.0f * inner)) - 1.0f;
+    return 0.5f * x * (1.0f + t);
+}
+
+__device__ inline float silu(float x) { return x / (1.0f + __expf(-x)); }
+
+// ---- host side ------------------------------------------------------------------------------------
+void set_error(const char *fmt, ...);
+int check_launch(const char *what);
+
+}  // namespace svdq

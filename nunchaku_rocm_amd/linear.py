@@ -1,0 +1,121 @@
+"""Quantized linear modules with the reference's parameter names and shapes
+(reference: nunchaku/models/linear.py:13-269 ``SVDQW4A4Linear``, :278-415 ``AWQW4A16Linear``), natural layout
+(``qweight (N, K/2)`` low nibble = even k, ``wscales (K/64, N)``), int4 only."""
+
+from __future__ import annotations
+
+import torch
+from torch import nn
+
+from .ops.gemm import svdq_gemm_w4a4_cuda
+from .ops.gemv import awq_gemv_w4a16_cuda
+from .ops.quantize import svdq_quantize_w4a4_act_fuse_lora_cuda
+
+
+class SVDQW4A4Linear(nn.Module):
+    """``y = (x / smooth) .q W4^T + (x @ proj_down) @ proj_up^T + bias`` with 4-bit activations and weights."""
+
+    def __init__(
+        self,
+        in_features: int,
+        out_features: int,
+        rank: int = 32,
+        bias: bool = True,
+        precision: str = "int4",
+        act_unsigned: bool = False,
+        torch_dtype: torch.dtype = torch.bfloat16,
+        device: str | torch.device | None = None,
+    ):
+        super().__init__()
+        if precision != "int4":
+            raise NotImplementedError(f"precision {precision!r}: only int4 is implemented")
+        if device is None:
+            device = torch.device("cpu")
+        self.in_features, self.out_features, self.rank = in_features, out_features, rank
+        self.precision, self.torch_dtype, self.group_size = precision, torch_dtype, 64
+        self.qweight = nn.Parameter(torch.empty(out_features, in_features // 2, dtype=torch.int8, device=device), requires_grad=False)
+        self.bias = nn.Parameter(torch.empty(out_features, dtype=torch_dtype, device=device)) if bias else None
+        self.wscales = nn.Parameter(torch.empty(in_features // 64, out_features, dtype=torch_dtype, device=device), requires_grad=False)
+        self.smooth_factor = nn.Parameter(torch.empty(in_features, dtype=torch_dtype, device=device), requires_grad=False)
+        self.smooth_factor_orig = nn.Parameter(torch.empty(in_features, dtype=torch_dtype, device=device), requires_grad=False)
+        self.proj_down = nn.Parameter(torch.empty(in_features, rank, dtype=torch_dtype, device=device))
+        self.proj_up = nn.Parameter(torch.empty(out_features, rank, dtype=torch_dtype, device=device))
+        self.wtscale = None
+        self.wcscales = None
+        self.act_unsigned = act_unsigned
+
+    @classmethod
+    def from_linear(cls, linear: nn.Linear, **kwargs):
+        in_features = kwargs.pop("in_features", linear.in_features)
+        torch_dtype = kwargs.pop("torch_dtype", linear.weight.dtype)
+        return cls(in_features=in_features, out_features=linear.out_features, bias=linear.bias is not None,
+                   torch_dtype=torch_dtype, device=linear.weight.device, **kwargs)  # fmt: skip
+
+    def forward(self, x: torch.Tensor, output: torch.Tensor | None = None) -> torch.Tensor:
+        batch_size, seq_len, channels = x.shape
+        x = x.reshape(batch_size * seq_len, channels)
+        if output is None:
+            output = torch.empty(batch_size * seq_len, self.out_features, dtype=x.dtype, device=x.device)
+        quantized_x, ascales, lora_act_out = self.quantize(x)
+        output = self.forward_quant(quantized_x, ascales, lora_act_out, output)
+        return output.reshape(batch_size, seq_len, -1)
+
+    def quantize(self, x: torch.Tensor, pad_size: int = 256):
+        return svdq_quantize_w4a4_act_fuse_lora_cuda(
+            x, lora_down=self.proj_down, smooth=self.smooth_factor, fp4=False, pad_size=pad_size
+        )
+
+    def forward_quant(self, quantized_x, ascales, lora_act, output: torch.Tensor | None = None) -> torch.Tensor:
+        if output is None:
+            output = torch.empty(quantized_x.shape[0], self.out_features, dtype=self.proj_up.dtype, device=quantized_x.device)
+        svdq_gemm_w4a4_cuda(
+            act=quantized_x,
+            wgt=self.qweight,
+            out=output,
+            ascales=ascales,
+            wscales=self.wscales,
+            lora_act_in=lora_act,
+            lora_up=self.proj_up,
+            bias=self.bias,
+            fp4=False,
+            alpha=self.wtscale,
+            wcscales=self.wcscales,
+            act_unsigned=self.act_unsigned,
+        )
+        return output
+
+    def __repr__(self):
+        return (f"SVDQW4A4Linear(in_features={self.in_features}, out_features={self.out_features}, rank={self.rank}, "
+                f"precision={self.precision}, act_unsigned={self.act_unsigned})")  # fmt: skip
+
+
+class AWQW4A16Linear(nn.Module):
+    """AWQ W4A16 linear, group 64, TinyChat-packed ``qweight (N/4, K/2) int32``; bias added after the GEMV."""
+
+    def __init__(self, in_features: int, out_features: int, bias: bool = True, group_size: int = 64,
+                 torch_dtype: torch.dtype = torch.bfloat16, device: str | torch.device | None = None):  # fmt: skip
+        super().__init__()
+        if device is None:
+            device = torch.device("cpu")
+        self.in_features, self.out_features, self.group_size = in_features, out_features, group_size
+        self.qweight = nn.Parameter(torch.empty(out_features // 4, in_features // 2, dtype=torch.int32, device=device), requires_grad=False)
+        self.bias = nn.Parameter(torch.empty(out_features, dtype=torch_dtype, device=device)) if bias else None
+        self.wscales = nn.Parameter(torch.empty(in_features // group_size, out_features, dtype=torch_dtype, device=device), requires_grad=False)
+        self.wzeros = nn.Parameter(torch.empty(in_features // group_size, out_features, dtype=torch_dtype, device=device), requires_grad=False)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        output = awq_gemv_w4a16_cuda(in_feats=x, kernel=self.qweight, scaling_factors=self.wscales, zeros=self.wzeros,
+                                     m=x.shape[0], n=self.out_features, k=self.in_features, group_size=self.group_size)  # fmt: skip
+        if self.bias is not None:
+            view_shape = [1] * (output.ndim - 1) + [-1]
+            output.add_(self.bias.view(view_shape))
+        return output
+
+    @classmethod
+    def from_linear(cls, linear: nn.Linear, group_size: int = 64, torch_dtype: torch.dtype = torch.bfloat16,
+                    device: str = "cpu", **kwargs):  # fmt: skip
+        return cls(in_features=linear.in_features, out_features=linear.out_features, bias=linear.bias is not None,
+                   group_size=group_size, torch_dtype=torch_dtype, device=device)  # fmt: skip
+
+    def __repr__(self):
+        return f"AWQW4A16Linear(in_features={self.in_features}, out_features={self.out_features}, group_size={self.group_size})"

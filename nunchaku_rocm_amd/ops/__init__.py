@@ -1,0 +1,16 @@
+"""Operator API of the SVDQuant path: same names and signatures as ``nunchaku.ops`` in the reference."""
+
+from .fused import fused_gelu_mlp, fused_qkv_norm_rottary, fused_swiglu_mlp, interleave_swiglu_linear_
+from .gemm import svdq_gemm_w4a4_cuda
+from .gemv import awq_gemv_w4a16_cuda
+from .quantize import svdq_quantize_w4a4_act_fuse_lora_cuda
+
+__all__ = [
+    "svdq_quantize_w4a4_act_fuse_lora_cuda",
+    "svdq_gemm_w4a4_cuda",
+    "awq_gemv_w4a16_cuda",
+    "fused_gelu_mlp",
+    "fused_qkv_norm_rottary",
+    "fused_swiglu_mlp",
+    "interleave_swiglu_linear_",
+]

@@ -1,0 +1,209 @@
+"""W4A4 GEMM operator (reference: nunchaku/ops/gemm.py:12-207 and the dispatcher nunchaku/ops/triton/gemm_w4a4.py:1003-1314)."""
+
+from __future__ import annotations
+
+import torch
+
+from .. import _lib
+from ._prep import lora_down_t as _lora_down_t
+
+HEAD_DIM = 128
+GELU_SHIFT = 0.171875
+
+
+def svdq_gemm_w4a4_cuda(
+    act: torch.Tensor,
+    wgt: torch.Tensor,
+    out: torch.Tensor | None = None,
+    qout: torch.Tensor | None = None,
+    ascales: torch.Tensor | None = None,
+    wscales: torch.Tensor | None = None,
+    oscales: torch.Tensor | None = None,
+    poolout: torch.Tensor | None = None,
+    lora_act_in: torch.Tensor | None = None,
+    lora_up: torch.Tensor | None = None,
+    lora_down: torch.Tensor | None = None,
+    lora_act_out: torch.Tensor | None = None,
+    norm_q: torch.Tensor | None = None,
+    norm_k: torch.Tensor | None = None,
+    rotary_emb: torch.Tensor | None = None,
+    bias: torch.Tensor | None = None,
+    smooth_factor: torch.Tensor | None = None,
+    out_vk: torch.Tensor | None = None,
+    out_linearattn: torch.Tensor | None = None,
+    act_unsigned: bool = False,
+    lora_scales: list[float] | None = None,
+    fuse_silu: bool = False,
+    fp4: bool = False,
+    alpha: float | None = 1.0,
+    wcscales: torch.Tensor | None = None,
+    out_q: torch.Tensor | None = None,
+    out_k: torch.Tensor | None = None,
+    out_v: torch.Tensor | None = None,
+    attn_tokens: int = 0,
+    fuse_swiglu: bool = False,
+):
+    """
+    ``out = deq(act) @ deq(wgt).T + lora_act_in @ lora_up.T + bias`` on packed int4 operands with per-group-64 scales,
+    written in place; positional order is the reference operator's (29 arguments; ``fuse_swiglu`` is keyword-only
+    in spirit and selects the SwiGLU requantizing epilogue of the reference's Triton-level ``gemm_w4a4``).
+
+    * ``norm_q``/``norm_k``/``rotary_emb``: fused per-head RMSNorm + RoPE on the Q and K thirds of ``out``.
+    * ``qout``/``oscales`` (+ ``smooth_factor``, ``lora_down``, ``lora_act_out``): fused GELU, next layer's LoRA-down
+      and unsigned int4 requantization; ``out`` may then be ``None``.
+    * ``act`` may have more (padded) rows than ``out``; only ``out.shape[0]`` rows are written.
+
+    Raises ``NotImplementedError`` for the arguments the reference's ROCm backend rejects as well (``poolout``,
+    ``out_vk``, ``out_linearattn``, ``out_q/k/v``) and for the NVFP4-only ones (``fp4``, ``wcscales``, ``alpha != 1``,
+    ``fuse_silu``).  ``lora_scales`` is accepted and ignored, as in the reference's ROCm backend.  Returns ``None``.
+    """
+    unsupported = {
+        "poolout": poolout,
+        "out_vk": out_vk,
+        "out_linearattn": out_linearattn,
+        "out_q": out_q,
+        "out_k": out_k,
+        "out_v": out_v,
+    }
+    active = sorted(name for name, value in unsupported.items() if value is not None)
+    if active:
+        raise NotImplementedError("these fused gemm_w4a4 epilogues are not implemented: " + ", ".join(active))
+    if fp4 or wcscales is not None or fuse_silu or not (alpha is None or alpha == 1.0):
+        raise NotImplementedError("NVFP4 options (fp4, wcscales, alpha != 1) and fuse_silu are not implemented (int4 only)")
+    assert ascales is not None and wscales is not None, "W4A4 GEMM requires both scale tensors"
+
+    act = act.reshape(-1, act.shape[-1])
+    M, K, N = act.shape[0], act.shape[1] * 2, wgt.shape[0]
+    assert wgt.shape[1] * 2 == K, f"weight K mismatch: {wgt.shape[1] * 2} vs {K}"
+    dev = _lib.require_cuda(act, wgt, out, qout, ascales, wscales, oscales, lora_act_in, lora_up, lora_down,
+                            lora_act_out, norm_q, norm_k, rotary_emb, bias, smooth_factor)  # fmt: skip
+
+    want_quant = qout is not None or oscales is not None
+    want_qk = norm_q is not None or norm_k is not None or rotary_emb is not None
+    if want_quant:
+        assert qout is not None and oscales is not None, "qout and oscales must be given together"
+        assert (lora_down is None) == (lora_act_out is None), "lora_down and lora_act_out must be given together"
+        if want_qk:
+            raise NotImplementedError("requantizing epilogue together with Q/K norm + RoPE")
+    if want_qk:
+        assert norm_q is not None and norm_k is not None and rotary_emb is not None, (
+            "norm_q, norm_k, and rotary_emb must all be given together"
+        )
+    if fuse_swiglu:
+        assert out is None and want_quant, "fuse_swiglu writes qout/oscales, not out"
+
+    T = out.dtype if out is not None else (oscales.dtype if oscales is not None else ascales.dtype)
+    if out is None and not want_quant:
+        out = torch.empty(M, N, dtype=T, device=dev)  # computed and dropped, as the reference does
+    out2d = out.reshape(-1, N) if out is not None else None
+    actual_m = out2d.shape[0] if out2d is not None else M
+    assert actual_m <= M, f"out has more rows ({actual_m}) than act ({M})"
+
+    has_lora = lora_act_in is not None and lora_up is not None
+    R = lora_up.shape[1] if has_lora else 0
+
+    for name, t in (("act", act), ("wgt", wgt)):
+        if t.element_size() != 1 or t.stride(-1) != 1:
+            raise ValueError(f"{name} must be a packed byte tensor with unit inner stride")
+    for name, s, rows in (("ascales", ascales, M), ("wscales", wscales, N)):
+        if s.dtype != T or s.dim() != 2 or s.shape[0] < K // 64 or s.shape[1] < rows or s.stride(1) != 1:
+            raise ValueError(f"{name} must be (K/64, >= {rows}) of dtype {T}, got {tuple(s.shape)} {s.dtype}")
+    if bias is not None and (bias.dtype != T or bias.dim() != 1 or bias.shape[0] < N or bias.stride(0) != 1):
+        raise ValueError("bias must be a contiguous (N,) tensor of the output dtype")
+    if has_lora:
+        if lora_act_in.dtype != torch.float32 or lora_up.dtype != T:
+            raise ValueError(f"LoRA dtypes {lora_act_in.dtype}/{lora_up.dtype}")
+        if lora_up.shape[0] < N or lora_act_in.shape[0] < M or lora_act_in.shape[1] < R:
+            raise ValueError("LoRA shapes")
+        if lora_act_in.stride(1) != 1 or lora_up.stride(1) != 1:
+            raise ValueError("LoRA tensors need unit inner stride")
+    if out2d is not None and out2d.stride(1) != 1:
+        raise ValueError("out not row-major")
+
+    args = _lib.GemmArgs(
+        act=act.data_ptr(),
+        wgt=wgt.data_ptr(),
+        ascales=ascales.data_ptr(),
+        wscales=wscales.data_ptr(),
+        bias=_lib.ptr(bias),
+        lora_act=lora_act_in.data_ptr() if R else None,
+        lora_up=lora_up.data_ptr() if R else None,
+        out=_lib.ptr(out2d),
+        M=M,
+        N=N,
+        K=K,
+        R=R,
+        actual_m=actual_m,
+        ld_act=act.stride(0),
+        ld_wgt=wgt.stride(0),
+        ld_ascales=ascales.stride(0),
+        ld_wscales=wscales.stride(0),
+        ld_lora_act=lora_act_in.stride(0) if R else 0,
+        ld_lora_up=lora_up.stride(0) if R else 0,
+        ld_out=out2d.stride(0) if out2d is not None else 0,
+        dtype=_lib.dtype_code(T),
+        act_unsigned=int(act_unsigned),
+        epilogue=_lib.EPI_PLAIN,
+        eps=1e-6,
+    )
+    keep = []  # tensors that must outlive the launch call
+    lib = _lib.load()
+    if want_qk:
+        if rotary_emb.dtype != torch.float32:
+            raise ValueError("rotary_emb must be float32")
+        rot = rotary_emb.reshape(actual_m, HEAD_DIM)
+        if rot.stride(1) != 1:
+            rot = rot.contiguous()
+        for name, w in (("norm_q", norm_q), ("norm_k", norm_k)):
+            if w.dtype != T or w.numel() != HEAD_DIM or not w.is_contiguous():
+                raise ValueError(f"{name} must be a contiguous ({HEAD_DIM},) tensor of the output dtype")
+        keep.append(rot)
+        args.epilogue = _lib.EPI_QK_NORM_ROPE
+        args.norm_q, args.norm_k, args.rotary = norm_q.data_ptr(), norm_k.data_ptr(), rot.data_ptr()
+        args.ld_rotary = rot.stride(0)
+    elif want_quant:
+        NQ = N // 2 if fuse_swiglu else N
+        qout2d = qout.reshape(-1, qout.shape[-1])
+        if qout2d.element_size() != 1 or qout2d.shape[0] < M or qout2d.shape[1] != NQ // 2 or qout2d.stride(1) != 1:
+            raise ValueError(f"qout shape/dtype {tuple(qout.shape)} {qout.dtype}")
+        if oscales.dtype != T or oscales.dim() != 2 or oscales.shape[0] != NQ // 64 or oscales.shape[1] < M or oscales.stride(1) != 1:
+            raise ValueError(f"oscales shape {tuple(oscales.shape)}")
+        if smooth_factor is not None and (smooth_factor.dtype != T or smooth_factor.numel() != NQ or not smooth_factor.is_contiguous()):
+            raise ValueError("smooth_factor must be a contiguous (N,) tensor of the output dtype")
+        R2 = lora_down.shape[1] if lora_down is not None else 0
+        if R2:
+            if lora_down.dtype != T or lora_down.dim() != 2 or lora_down.shape[0] != NQ:
+                raise ValueError(f"lora_down shape/dtype {tuple(lora_down.shape)} {lora_down.dtype}")
+            if lora_act_out.dtype != torch.float32 or lora_act_out.dim() != 2 or lora_act_out.shape[0] < M or lora_act_out.shape[1] != R2:
+                raise ValueError("lora_act_out must be (>= M, R2) fp32")
+            ldt = _lora_down_t(lora_down)
+            epi = _lib.EPI_SWIGLU_QUANT if fuse_swiglu else _lib.EPI_GELU_QUANT
+            nbytes = lib.svdq_gemm_w4a4_scratch_bytes(M, N, R2, epi)
+            scratch = torch.empty(nbytes // 4, dtype=torch.float32, device=dev)
+            keep += [ldt, scratch]
+            args.lora_down_t, args.lora_act_out, args.scratch = ldt.data_ptr(), lora_act_out.data_ptr(), scratch.data_ptr()
+            args.ld_lora_act_out = lora_act_out.stride(0)
+        args.epilogue = _lib.EPI_SWIGLU_QUANT if fuse_swiglu else _lib.EPI_GELU_QUANT
+        args.qout, args.oscales, args.smooth_next = qout2d.data_ptr(), oscales.data_ptr(), _lib.ptr(smooth_factor)
+        args.R2, args.ld_qout, args.ld_oscales = R2, qout2d.stride(0), oscales.stride(0)
+        args.shift = 0.0 if fuse_swiglu else GELU_SHIFT
+
+    with torch.cuda.device(dev):
+        _lib.check(lib.svdq_gemm_w4a4(args, _lib.stream_of(act)))
+    return None
+
+
+def group_acc_i32(act: torch.Tensor, wgt: torch.Tensor, group: int, act_unsigned: bool = False) -> torch.Tensor:
+    """Debug read-out: exact int32 accumulators ``sum_{k in group} a[m, k] * w[n, k]`` from the GEMM's MFMA path."""
+    act = act.reshape(-1, act.shape[-1])
+    dev = _lib.require_cuda(act, wgt)
+    M, K, N = act.shape[0], act.shape[1] * 2, wgt.shape[0]
+    out = torch.empty(M, N, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.check(
+            _lib.load().svdq_group_acc_i32(
+                act.data_ptr(), wgt.data_ptr(), out.data_ptr(), M, N, K, act.stride(0), wgt.stride(0), group,
+                int(act_unsigned), _lib.stream_of(act),
+            )  # fmt: skip
+        )
+    return out

@@ -1,0 +1,127 @@
+"""Activation quantizer operator (reference: nunchaku/ops/quantize.py:11-88)."""
+
+from __future__ import annotations
+
+import torch
+
+from .. import _lib
+from ._prep import lora_down_t as _lora_down_t
+
+
+def _ceil_divide(a: int, b: int) -> int:
+    return (a + b - 1) // b
+
+
+def quantize_w4a4_act_fuse_lora(
+    input: torch.Tensor,
+    output: torch.Tensor | None = None,
+    oscales: torch.Tensor | None = None,
+    lora_down: torch.Tensor | None = None,
+    lora_act_out: torch.Tensor | None = None,
+    smooth: torch.Tensor | None = None,
+    fuse_glu: bool = False,
+    fp4: bool = False,
+    fuse_gelu: bool = False,
+    shift_value: float = 0.0,
+    unsigned: bool = False,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """
+    Backend-level quantizer with the reference's full option set (reference:
+    nunchaku/ops/triton/gemm_w4a4.py:1521-1565): no row padding, outputs allocated when not given, ``unsigned`` /
+    ``shift_value`` for activations known to be non-negative after a shift.  ``fuse_gelu`` (the reference's unfused
+    fallback prologue) is not implemented: the GELU lives in the GEMM epilogue here.
+    """
+    if fp4:
+        raise NotImplementedError("NVFP4 quantization is not implemented (int4 only)")
+    if fuse_gelu:
+        raise NotImplementedError("fuse_gelu: GELU is fused into the producing GEMM's epilogue instead")
+    inp = input.reshape(-1, input.shape[-1])
+    _lib.require_cuda(inp, output, oscales, lora_down, lora_act_out, smooth)
+    M = inp.shape[0]
+    K = inp.shape[1] // 2 if fuse_glu else inp.shape[1]
+    if K % 64:
+        raise ValueError(f"K={K} must be a multiple of the group size 64")
+    rank = lora_down.shape[1] if lora_down is not None else 0
+    if output is None:
+        output = torch.empty(M, K // 2, dtype=torch.uint8, device=inp.device)
+    if oscales is None:
+        oscales = torch.empty(K // 64, M, dtype=inp.dtype, device=inp.device)
+    if lora_act_out is None and lora_down is not None:
+        lora_act_out = torch.empty(M, rank, dtype=torch.float32, device=inp.device)
+
+    if inp.stride(1) != 1 or inp.stride(0) % 8 or inp.data_ptr() % 16:
+        inp = inp.contiguous()
+    if output.element_size() != 1 or output.stride(1) != 1 or output.shape[0] < M:
+        raise ValueError("output must be a (>= M, K/2) byte tensor with unit inner stride")
+    if oscales.dtype != inp.dtype or oscales.stride(1) != 1 or oscales.shape[1] < M or oscales.shape[0] < K // 64:
+        raise ValueError("oscales must be (K/64, >= M) of the input dtype with unit inner stride")
+    if rank and (lora_act_out.dtype != torch.float32 or lora_act_out.stride(1) != 1 or lora_act_out.shape[0] < M):
+        raise ValueError("lora_act_out must be (>= M, R) float32 with unit inner stride")
+    if smooth is not None and (smooth.dtype != inp.dtype or not smooth.is_contiguous() or smooth.numel() != K):
+        raise ValueError("smooth must be a contiguous (K,) tensor of the input dtype")
+    if lora_down is not None and (lora_down.dtype != inp.dtype or lora_down.shape[0] != K):
+        raise ValueError("lora_down must be (K, R) of the input dtype")
+
+    args = _lib.QuantizeArgs(
+        x=inp.data_ptr(),
+        smooth=_lib.ptr(smooth),
+        lora_down_t=_lora_down_t(lora_down).data_ptr() if rank else None,
+        out=output.data_ptr(),
+        scales=oscales.data_ptr(),
+        lora_act=lora_act_out.data_ptr() if rank else None,
+        M=M,
+        K=K,
+        R=rank,
+        ld_x=inp.stride(0),
+        ld_out=output.stride(0),
+        ld_scales=oscales.stride(0),
+        ld_lora_act=lora_act_out.stride(0) if rank else 0,
+        dtype=_lib.dtype_code(inp.dtype),
+        is_unsigned=int(unsigned),
+        fuse_glu=int(fuse_glu),
+        shift=float(shift_value),
+    )
+    with torch.cuda.device(inp.device):
+        _lib.check(_lib.load().svdq_quantize_act(args, _lib.stream_of(inp)))
+    return output, oscales, lora_act_out
+
+
+def svdq_quantize_w4a4_act_fuse_lora_cuda(
+    input: torch.Tensor,
+    output: torch.Tensor | None = None,
+    oscales: torch.Tensor | None = None,
+    lora_down: torch.Tensor | None = None,
+    lora_act_out: torch.Tensor | None = None,
+    smooth: torch.Tensor | None = None,
+    fuse_glu: bool = False,
+    fp4: bool = False,
+    pad_size: int = 256,
+) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """
+    Quantize activations to int4 (per-group-64 absmax, after dividing by ``smooth``) and compute the LoRA
+    down-projection ``input @ lora_down`` in the same pass (reference: nunchaku/ops/quantize.py:11-88).
+
+    Same signature and return value as the reference operator: ``(output (M_pad, C/2) uint8,
+    oscales (C/64, M_pad) input.dtype, lora_act_out (M_pad, R) float32)`` with ``C = input.shape[1]`` and
+    ``M_pad = ceil(M / pad_size) * pad_size``.  Only rows ``< M`` are written; pad rows keep whatever the freshly
+    allocated buffers held.
+
+    Unlike the reference wrapper (which dereferences ``lora_down.shape`` unconditionally), ``lora_down=None`` is
+    accepted and returns ``lora_act_out`` with zero columns.
+    """
+    if fp4:
+        raise NotImplementedError("NVFP4 quantization is not implemented (int4 only)")
+    if input.dim() != 2:
+        raise ValueError(f"input must be 2-D (M, K), got {tuple(input.shape)}")
+    batch_size, channels = input.shape
+    rank = lora_down.shape[1] if lora_down is not None else 0
+    batch_size_pad = _ceil_divide(batch_size, pad_size) * pad_size
+    if output is None:
+        output = torch.empty(batch_size_pad, channels // 2, dtype=torch.uint8, device=input.device)
+    if oscales is None:
+        assert channels % 64 == 0
+        oscales = torch.empty(channels // 64, batch_size_pad, dtype=input.dtype, device=input.device)
+    if lora_act_out is None:
+        lora_act_out = torch.empty(batch_size_pad, rank, dtype=torch.float32, device=input.device)
+    quantize_w4a4_act_fuse_lora(input, output, oscales, lora_down, lora_act_out if rank else None, smooth, fuse_glu, fp4)
+    return output, oscales, lora_act_out

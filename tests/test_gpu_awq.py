@@ -1,0 +1,59 @@
+"""GPU parity of the AWQ W4A16 GEMV against the CPU oracle (fp32 result, then one rounding to the 16-bit type)."""
+
+import pytest
+import torch
+
+from oracle import svdq_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(dev, m, N, K, dtype, seed):
+    from nunchaku_rocm_amd import ops
+
+    lin = O.make_awq_linear(K, N, seed=seed, dtype=dtype)
+    g = torch.Generator().manual_seed(seed + 1)
+    x = torch.randn(m, K, generator=g).to(dtype)
+    out = ops.awq_gemv_w4a16_cuda(x.to(dev), lin["qweight"].to(dev), lin["wscales"].to(dev), lin["wzeros"].to(dev), m, N, K)
+    torch.cuda.synchronize()
+    ref = O.awq_gemv(x, lin["qweight"].view(torch.int16).reshape(N // 4, K), lin["wscales"], lin["wzeros"])
+    return out.cpu(), ref
+
+
+@pytest.mark.parametrize("m", [1, 2, 8, 5, 32, 40])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_small_shapes(dev, m, dtype):
+    print(f"case m={m} {dtype}", flush=True)
+    out, ref = _case(dev, m, 128, 256, dtype, seed=m)
+    assert out.shape == (m, 128) and out.dtype == dtype
+    # fp32 accumulation then one rounding: within one 16-bit ulp of the oracle's rounded value
+    tol = ref.abs() * (2**-7 if dtype == torch.bfloat16 else 2**-10) + 1e-3
+    assert ((out.float() - ref).abs() <= tol).all()
+    assert O.max_rel_err(out, ref) <= 1e-2
+
+
+@pytest.mark.parametrize("m", [1, 2, 8])
+def test_flux_adaln_shape(dev, m):
+    """K=3072, N=18432: the double-stream adaLN modulation linear."""
+    print(f"case m={m}", flush=True)
+    out, ref = _case(dev, m, 18432, 3072, torch.bfloat16, seed=20 + m)
+    assert O.max_rel_err(out, ref) <= 1e-2
+    assert ((out.float() - ref).abs() <= ref.abs() * 2**-7 + 2e-2).all()
+
+
+def test_linear_module_adds_bias_after_kernel(dev):
+    from nunchaku_rocm_amd.linear import AWQW4A16Linear
+
+    K, N = 256, 128
+    lin = O.make_awq_linear(K, N, seed=31)
+    mod = AWQW4A16Linear(K, N, bias=True, device=dev)
+    with torch.no_grad():
+        mod.qweight.copy_(lin["qweight"])
+        mod.wscales.copy_(lin["wscales"])
+        mod.wzeros.copy_(lin["wzeros"])
+        mod.bias.copy_(torch.arange(N).to(torch.bfloat16) * 0.01)
+    x = torch.randn(2, K, generator=torch.Generator().manual_seed(32)).to(torch.bfloat16)
+    y = mod(x.to(dev)).cpu()
+    ref = O.awq_gemv(x, lin["qweight"].view(torch.int16).reshape(N // 4, K), lin["wscales"], lin["wzeros"])
+    ref = ref.to(torch.bfloat16) + (torch.arange(N).to(torch.bfloat16) * 0.01)
+    assert O.max_rel_err(y, ref) <= 1e-2

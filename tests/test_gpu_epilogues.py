@@ -1,0 +1,149 @@
+"""GPU parity of the fused GEMM epilogues (Q/K RMSNorm + RoPE; GELU + next-layer requantization with LoRA-down) and of
+the composite operators built on them, against the CPU oracle."""
+
+import pytest
+import torch
+
+from oracle import svdq_oracle as O
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-2
+
+
+def _problem(M, N, K, R, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    return {
+        "act": torch.randint(0, 256, (M, K // 2), generator=g, dtype=torch.uint8),
+        "wgt": torch.randint(0, 256, (N, K // 2), generator=g, dtype=torch.uint8),
+        "asc": (torch.rand(K // 64, M, generator=g) * 0.02 + 0.01).to(dtype),
+        "wsc": (torch.rand(K // 64, N, generator=g) * 0.02 + 0.01).to(dtype),
+        "bias": torch.randn(N, generator=g).to(dtype),
+        "la": torch.randn(M, R, generator=g),
+        "lu": (torch.randn(N, R, generator=g) * 0.1).to(dtype),
+    }
+
+
+@pytest.mark.parametrize("unsigned", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,H,actual_m", [(136, 1, 130), (256, 2, 256)])
+def test_qk_norm_rope(dev, M, H, actual_m, unsigned, dtype):
+    from nunchaku_rocm_amd import ops
+
+    print(f"case M={M} H={H} actual_m={actual_m} unsigned={unsigned} {dtype}", flush=True)
+    N, K, R = 3 * H * 128, 256, 16
+    p = _problem(M, N, K, R, dtype, seed=M + H)
+    g = torch.Generator().manual_seed(99)
+    nq = (torch.rand(128, generator=g) + 0.5).to(dtype)
+    nk = (torch.rand(128, generator=g) + 0.5).to(dtype)
+    theta = torch.rand(actual_m, 64, generator=g) * 6.28
+    rot = torch.stack([torch.sin(theta), torch.cos(theta)], -1).reshape(actual_m, 64, 1, 2).float()
+    d = lambda t: t.to(dev)  # noqa: E731
+    buf = torch.full((actual_m + 8, N), float("nan"), dtype=dtype, device=dev)
+    kw = dict(act=d(p["act"]), wgt=d(p["wgt"]), ascales=d(p["asc"]), wscales=d(p["wsc"]), bias=d(p["bias"]),
+              lora_act_in=d(p["la"]), lora_up=d(p["lu"]), act_unsigned=unsigned)  # fmt: skip
+    ops.svdq_gemm_w4a4_cuda(out=buf[:actual_m], norm_q=d(nq), norm_k=d(nk), rotary_emb=d(rot), **kw)
+    plain = torch.empty(actual_m, N, dtype=dtype, device=dev)
+    ops.svdq_gemm_w4a4_cuda(out=plain, **kw)
+    torch.cuda.synchronize()
+    assert bool(buf[actual_m:].isnan().all())
+    out = buf[:actual_m].cpu()
+    lin = O.gemm_w4a4(p["act"], p["wgt"], p["asc"], p["wsc"], p["bias"], p["la"], p["lu"], unsigned)[:actual_m]
+    ref = O.qk_norm_rope(lin, nq, nk, rot.reshape(actual_m, 128))
+    assert O.max_rel_err(out[:, : 2 * N // 3], ref[:, : 2 * N // 3]) <= TOL
+    # the V third is exactly the plain GEMM's output
+    assert torch.equal(out[:, 2 * N // 3 :].view(torch.int16), plain[:, 2 * N // 3 :].cpu().view(torch.int16))
+
+
+@pytest.mark.parametrize("unsigned", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,N,R2,store_out", [(144, 256, 48, True), (64, 512, 32, False), (128, 128, 0, False)])
+def test_gelu_quant_epilogue(dev, M, N, R2, store_out, unsigned, dtype):
+    from nunchaku_rocm_amd import ops
+
+    print(f"case M={M} N={N} R2={R2} store_out={store_out} unsigned={unsigned} {dtype}", flush=True)
+    K, R = 256, 16
+    p = _problem(M, N, K, R, dtype, seed=N + R2)
+    g = torch.Generator().manual_seed(98)
+    smooth = (torch.rand(N, generator=g) + 0.5).to(dtype)
+    ld = (torch.randn(N, max(R2, 16), generator=g) * 0.1).to(dtype)[:, :R2].contiguous() if R2 else None
+    d = lambda t: None if t is None else t.to(dev)  # noqa: E731
+    qout = torch.zeros(M + 16, N // 2, dtype=torch.uint8, device=dev)
+    osc = torch.empty(N // 64, M, dtype=dtype, device=dev)
+    lao = torch.empty(M, R2, dtype=torch.float32, device=dev) if R2 else None
+    out = torch.empty(M, N, dtype=dtype, device=dev) if store_out else None
+    for _ in range(2):  # run twice: must be deterministic and must not depend on scratch contents
+        ops.svdq_gemm_w4a4_cuda(
+            act=d(p["act"]), wgt=d(p["wgt"]), out=out, qout=qout, ascales=d(p["asc"]), wscales=d(p["wsc"]), oscales=osc,
+            lora_act_in=d(p["la"]), lora_up=d(p["lu"]), lora_down=d(ld), lora_act_out=lao, bias=d(p["bias"]),
+            smooth_factor=d(smooth), act_unsigned=unsigned,
+        )  # fmt: skip
+        torch.cuda.synchronize()
+        first = (qout.clone(), osc.clone(), lao.clone() if R2 else None) if _ == 0 else first
+    assert torch.equal(first[0], qout) and torch.equal(first[1].view(torch.int16), osc.view(torch.int16))
+    assert R2 == 0 or torch.equal(first[2], lao)
+    assert (qout[M:] == 0).all()  # rows past M untouched
+
+    lin = O.gemm_w4a4(p["act"], p["wgt"], p["asc"], p["wsc"], p["bias"], p["la"], p["lu"], unsigned)
+    rp, rs, rl, rc = O.gelu_quant(lin, smooth, ld, dtype)
+    codes = O.unpack_int4(qout[:M].cpu(), False)
+    diff = (codes - rc).abs()
+    rate = (diff > 0).float().mean().item()
+    print(f"  code mismatch rate {rate:.2e}", flush=True)
+    assert diff.max() <= 1 and rate < 1e-3
+    ulp = 2**-7 if dtype == torch.bfloat16 else 2**-10
+    assert ((osc.cpu().float() - rs.float()).abs() <= rs.float().abs() * ulp + 1e-7).all()
+    if R2:
+        assert (lao.cpu() - rl).abs().max() <= TOL * rl.abs().max()
+    if store_out:
+        assert O.max_rel_err(out.cpu(), lin) <= TOL
+
+
+def test_fused_ops_on_flux_block_shapes(dev):
+    """fc1 (3072 -> 12288) + GELU + requantization -> fc2 (12288 -> 3072, unsigned activations), and the QKV projection
+    (3072 -> 9216) with Q/K RMSNorm + RoPE on the 64x64 image grid + 512 text tokens; oracle on a row sample."""
+    from nunchaku_rocm_amd import ops
+    from nunchaku_rocm_amd.linear import SVDQW4A4Linear
+
+    M, C, H4 = 4608, 3072, 12288
+
+    def module(K, N, seed, act_unsigned=False):
+        lin = O.make_svdq_linear(K, N, seed=seed)
+        mod = SVDQW4A4Linear(K, N, rank=32, act_unsigned=act_unsigned, device=dev)
+        with torch.no_grad():
+            for name in ("qweight", "wscales", "smooth_factor", "proj_down", "proj_up", "bias"):
+                getattr(mod, name).copy_(lin[name])
+        return mod, lin
+
+    x = O.make_activations(M, C, seed=41)
+    rows = torch.randperm(M, generator=torch.Generator().manual_seed(5))[:96].sort().values
+
+    # --- MLP
+    fc1, l1 = module(C, H4, 42)
+    fc2, l2 = module(H4, C, 43, act_unsigned=True)
+    y = ops.fused_gelu_mlp(x.to(dev).view(1, M, C), fc1, fc2).view(M, C)
+    torch.cuda.synchronize()
+    rp, rs, rl, _ = O.quantize_act(x[rows], l1["proj_down"], l1["smooth_factor"])
+    h = O.gemm_w4a4(rp, l1["qweight"], rs, l1["wscales"], l1["bias"], rl, l1["proj_up"])
+    hp, hs, hl, _ = O.gelu_quant(h, l2["smooth_factor"], l2["proj_down"], torch.bfloat16)
+    ref = O.gemm_w4a4(hp, l2["qweight"], hs, l2["wscales"], l2["bias"], hl, l2["proj_up"], act_unsigned=True)
+    err = O.max_rel_err(y[rows].cpu(), ref)
+    print(f"fused_gelu_mlp max rel err {err:.3e}", flush=True)
+    assert err <= TOL
+
+    # --- QKV with RMSNorm + RoPE
+    qkv, lq = module(C, 3 * C, 44)
+    nq = torch.nn.RMSNorm(128, eps=1e-6, device=dev, dtype=torch.bfloat16)
+    nk = torch.nn.RMSNorm(128, eps=1e-6, device=dev, dtype=torch.bfloat16)
+    g = torch.Generator().manual_seed(45)
+    with torch.no_grad():
+        nq.weight.copy_((torch.rand(128, generator=g) + 0.5).to(torch.bfloat16))
+        nk.weight.copy_((torch.rand(128, generator=g) + 0.5).to(torch.bfloat16))
+    rot = O.flux_rotary(O.flux_ids(512, 64, 64))
+    out = ops.fused_qkv_norm_rottary(x.to(dev).view(1, M, C), qkv, nq, nk, rot.to(dev)).view(M, 3 * C)
+    torch.cuda.synchronize()
+    rp, rs, rl, _ = O.quantize_act(x[rows], lq["proj_down"], lq["smooth_factor"])
+    lin = O.gemm_w4a4(rp, lq["qweight"], rs, lq["wscales"], lq["bias"], rl, lq["proj_up"])
+    ref = O.qk_norm_rope(lin, nq.weight.cpu(), nk.weight.cpu(), rot.reshape(M, 128)[rows])
+    err = O.max_rel_err(out[rows].cpu(), ref)
+    print(f"fused_qkv_norm_rottary max rel err {err:.3e}", flush=True)
+    assert err <= TOL

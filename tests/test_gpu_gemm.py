@@ -1,0 +1,157 @@
+"""GPU parity of the W4A4 GEMM against the CPU oracle.
+
+Bars: int32 group accumulators bit-exact; with unit scales the output is the exactly rounded integer GEMM
+(bit-exact); with real scales the 16-bit output is within max-rel-err 1e-2 of the oracle (relative to max |ref|, the
+reference self-test's measure) -- in practice within about one output ulp; rows past ``actual_m`` are never written;
+two runs give identical bits.
+"""
+
+import pytest
+import torch
+
+from oracle import svdq_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-2  # max |out - ref| / max |ref| per layer
+
+
+def _rand_problem(M, N, K, R, dtype, seed, scale=0.02):
+    g = torch.Generator().manual_seed(seed)
+    p = {
+        "act": torch.randint(0, 256, (M, K // 2), generator=g, dtype=torch.uint8),
+        "wgt": torch.randint(0, 256, (N, K // 2), generator=g, dtype=torch.uint8),
+        "asc": (torch.rand(K // 64, M, generator=g) * scale + scale / 2).to(dtype),
+        "wsc": (torch.rand(K // 64, N, generator=g) * scale + scale / 2).to(dtype),
+        "bias": torch.randn(N, generator=g).to(dtype),
+        "la": torch.randn(M, max(R, 16), generator=g)[:, :R].contiguous() if R else None,
+        "lu": (torch.randn(N, max(R, 16), generator=g) * 0.1).to(dtype)[:, :R].contiguous() if R else None,
+    }
+    return p
+
+
+def _gpu_gemm(p, dev, actual_m=None, unsigned=False, dtype=torch.bfloat16, canary=8, **extra):
+    from nunchaku_rocm_amd import ops
+
+    M, N = p["act"].shape[0], p["wgt"].shape[0]
+    am = M if actual_m is None else actual_m
+    buf = torch.full((am + canary, N), float("nan"), dtype=dtype, device=dev)
+    d = lambda t: None if t is None else t.to(dev)  # noqa: E731
+    ops.svdq_gemm_w4a4_cuda(
+        act=d(p["act"]), wgt=d(p["wgt"]), out=buf[:am], ascales=d(p["asc"]), wscales=d(p["wsc"]), bias=d(p.get("bias")),
+        lora_act_in=d(p.get("la")), lora_up=d(p.get("lu")), act_unsigned=unsigned, **{k: d(v) for k, v in extra.items()},
+    )  # fmt: skip
+    torch.cuda.synchronize()
+    assert bool(buf[am:].isnan().all()), "rows past actual_m were written"
+    return buf[:am].cpu()
+
+
+@pytest.mark.parametrize("unsigned", [False, True])
+@pytest.mark.parametrize("M,N,K", [(32, 32, 64), (136, 264, 256), (257, 96, 384)])
+def test_group_accumulators_bit_exact(dev, M, N, K, unsigned):
+    from nunchaku_rocm_amd.ops.gemm import group_acc_i32
+
+    print(f"case M={M} N={N} K={K} unsigned={unsigned}", flush=True)
+    p = _rand_problem(M, N, K, 0, torch.bfloat16, seed=M + N)
+    ref = O.group_acc_i32(p["act"], p["wgt"], unsigned)
+    for g in range(K // 64):
+        got = group_acc_i32(p["act"].to(dev), p["wgt"].to(dev), g, unsigned).cpu()
+        assert torch.equal(got, ref[g]), f"group {g}"
+
+
+@pytest.mark.parametrize("unsigned", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_unit_scales_exact_integer_gemm(dev, unsigned, dtype):
+    """With all scales 1 every fp32 partial sum is an exact integer, so the output must equal the oracle's bit for bit."""
+    M, N, K = 136, 264, 256
+    p = _rand_problem(M, N, K, 0, dtype, seed=1)
+    p["asc"] = torch.ones_like(p["asc"])
+    p["wsc"] = torch.ones_like(p["wsc"])
+    p["bias"] = None
+    out = _gpu_gemm(p, dev, unsigned=unsigned, dtype=dtype)
+    ref = O.gemm_w4a4(p["act"], p["wgt"], p["asc"], p["wsc"], act_unsigned=unsigned).to(dtype)
+    assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
+
+
+@pytest.mark.parametrize("unsigned", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,N,K,R,actual_m", [(136, 264, 256, 16, 130), (256, 256, 512, 32, 256), (64, 128, 1024, 48, 64), (128, 512, 256, 0, 100)])
+def test_scaled_gemm_bias_lora(dev, M, N, K, R, actual_m, unsigned, dtype):
+    print(f"case M={M} N={N} K={K} R={R} actual_m={actual_m} unsigned={unsigned} {dtype}", flush=True)
+    p = _rand_problem(M, N, K, R, dtype, seed=K + R)
+    out = _gpu_gemm(p, dev, actual_m=actual_m, unsigned=unsigned, dtype=dtype)
+    ref = O.gemm_w4a4(p["act"], p["wgt"], p["asc"], p["wsc"], p["bias"], p["la"], p["lu"], unsigned)[:actual_m]
+    assert O.max_rel_err(out, ref) <= TOL
+    ulp = 2**-7 if dtype == torch.bfloat16 else 2**-10
+    assert ((out.float() - ref).abs() <= ref.abs() * ulp * 1.01 + 1e-3 * ref.abs().max()).all()
+    out2 = _gpu_gemm(p, dev, actual_m=actual_m, unsigned=unsigned, dtype=dtype)
+    assert torch.equal(out.view(torch.int16), out2.view(torch.int16))
+
+
+def test_strided_row_views(dev):
+    """act/wgt/out may be row slices of wider buffers as long as rows stay 16-byte aligned."""
+    from nunchaku_rocm_amd import ops
+
+    M, N, K = 64, 128, 256
+    p = _rand_problem(M, N, K, 0, torch.bfloat16, seed=77)
+    wide_a = torch.zeros(M, K // 2 + 32, dtype=torch.uint8, device=dev)
+    wide_a[:, : K // 2] = p["act"].to(dev)
+    wide_o = torch.full((M, N + 8), float("nan"), dtype=torch.bfloat16, device=dev)
+    ops.svdq_gemm_w4a4_cuda(act=wide_a[:, : K // 2], wgt=p["wgt"].to(dev), out=wide_o[:, :N], ascales=p["asc"].to(dev),
+                            wscales=p["wsc"].to(dev), lora_scales=[1.0])  # fmt: skip
+    ref = O.gemm_w4a4(p["act"], p["wgt"], p["asc"], p["wsc"])
+    assert O.max_rel_err(wide_o[:, :N].cpu(), ref) <= TOL
+    assert bool(wide_o[:, N:].isnan().all())
+
+
+@pytest.mark.parametrize("M", [1024, 4608, 8192])
+def test_flux_qkv_shapes_quantizer_then_gemm(dev, M):
+    """The benchmark linear (K=3072, N=9216, R=32): quantizer -> GEMM on the GPU; oracle on the same seeded inputs.
+    The oracle runs on a row sample (rows are independent), all groups of which are also checked bit-exactly."""
+    from nunchaku_rocm_amd import ops
+    from nunchaku_rocm_amd.ops.gemm import group_acc_i32
+
+    print(f"case M={M}", flush=True)
+    K, N = 3072, 9216
+    lin = O.make_svdq_linear(K, N, seed=0)
+    x = O.make_activations(M, K, seed=1)
+    dl = {k: v.to(dev) for k, v in lin.items()}
+    qx, asc, la = ops.svdq_quantize_w4a4_act_fuse_lora_cuda(x.to(dev), lora_down=dl["proj_down"], smooth=dl["smooth_factor"])
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    ops.svdq_gemm_w4a4_cuda(act=qx, wgt=dl["qweight"], out=out, ascales=asc, wscales=dl["wscales"], lora_act_in=la,
+                            lora_up=dl["proj_up"], bias=dl["bias"])  # fmt: skip
+    torch.cuda.synchronize()
+    rows = torch.randperm(M, generator=torch.Generator().manual_seed(M))[:256].sort().values
+    rp, rs, rl, _ = O.quantize_act(x[rows], lin["proj_down"], lin["smooth_factor"])
+    assert torch.equal(qx[rows].cpu(), rp)
+    assert torch.equal(asc[:, rows].cpu().view(torch.int16), rs.view(torch.int16))
+    ref = O.gemm_w4a4(rp, lin["qweight"], rs, lin["wscales"], lin["bias"], rl, lin["proj_up"])
+    err = O.max_rel_err(out[rows].cpu(), ref)
+    print(f"M={M}: max rel err {err:.3e}", flush=True)
+    assert err <= TOL
+    for g in (0, 17, 47):
+        got = group_acc_i32(qx[rows].contiguous(), dl["qweight"], g).cpu()
+        assert torch.equal(got, O.group_acc_i32(rp, lin["qweight"], False, groups=[g])[0])
+
+
+def test_linear_module_matches_dequantised_reference(dev):
+    """SVDQW4A4Linear.forward against the SVDQuant formula y = (x / smooth) .q W^T + (x . down) . up^T + bias."""
+    from nunchaku_rocm_amd.linear import SVDQW4A4Linear
+
+    K, N, B, S = 512, 384, 2, 75
+    lin = O.make_svdq_linear(K, N, seed=5)
+    mod = SVDQW4A4Linear(K, N, rank=32, device=dev)
+    with torch.no_grad():
+        for name in ("qweight", "wscales", "smooth_factor", "proj_down", "proj_up", "bias"):
+            getattr(mod, name).copy_(lin[name])
+    x = O.make_activations(B * S, K, seed=6).view(B, S, K)
+    y = mod(x.to(dev)).cpu()
+    assert y.shape == (B, S, N)
+    rp, rs, rl, _ = O.quantize_act(x.view(-1, K), lin["proj_down"], lin["smooth_factor"])
+    ref = O.gemm_w4a4(rp, lin["qweight"], rs, lin["wscales"], lin["bias"], rl, lin["proj_up"])
+    assert O.max_rel_err(y.view(-1, N), ref) <= TOL
+    # and against the un-quantized-activation formula within 4-bit quantization noise
+    w = O.unpack_int4(lin["qweight"], True).double() * lin["wscales"].double().t().repeat_interleave(64, 1)
+    xd = x.view(-1, K).double()
+    truth = (xd / lin["smooth_factor"].double()) @ w.t() + (xd @ lin["proj_down"].double()) @ lin["proj_up"].double().t() + lin["bias"].double()
+    assert O.cosine(y.view(-1, N), truth) > 0.98

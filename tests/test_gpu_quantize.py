@@ -1,0 +1,104 @@
+"""GPU parity of the activation quantizer against the CPU oracle: int4 codes and 16-bit scales bit-exact, LoRA-down
+within fp32 accumulation-order noise, pad rows untouched, deterministic."""
+
+import pytest
+import torch
+
+from oracle import svdq_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(x, lin, dev, R, smooth=True, unsigned=False, shift=0.0, pad=0):
+    from nunchaku_rocm_amd.ops.quantize import quantize_w4a4_act_fuse_lora
+
+    M, K = x.shape
+    ld = lin["proj_down"][:, :R].contiguous() if R else None
+    sm = lin["smooth_factor"] if smooth else None
+    out = torch.full((M + pad, K // 2), 0xEE, dtype=torch.uint8, device=dev)
+    osc = torch.full((K // 64, M + pad), 7.0, dtype=x.dtype, device=dev)
+    la = torch.full((M + pad, max(R, 1)), 7.0, dtype=torch.float32, device=dev)[:, :R] if R else None
+    quantize_w4a4_act_fuse_lora(
+        x.to(dev), out, osc, ld.to(dev) if R else None, la, sm.to(dev) if smooth else None,
+        shift_value=shift, unsigned=unsigned,
+    )  # fmt: skip
+    torch.cuda.synchronize()
+    ref = O.quantize_act(x, ld, sm, unsigned=unsigned, shift=shift)
+    return (out.cpu(), osc.cpu(), la.cpu() if R else None), ref
+
+
+@pytest.mark.parametrize("M,K,R", [(1, 128, 16), (16, 256, 32), (130, 384, 48), (257, 3072, 32), (64, 512, 0), (33, 1024, 288)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_codes_and_scales_bit_exact(dev, M, K, R, dtype):
+    print(f"case M={M} K={K} R={R} {dtype}", flush=True)
+    x = O.make_activations(M, K, seed=M + K, dtype=dtype)
+    lin = O.make_svdq_linear(K, 64, R=max(R, 16), seed=K, dtype=dtype)
+    (out, osc, la), (rp, rs, rl, _) = _run(x, lin, dev, R, pad=5)
+    assert torch.equal(out[:M], rp)
+    assert torch.equal(osc[:, :M].view(torch.int16), rs.view(torch.int16))
+    assert (out[M:] == 0xEE).all() and (osc[:, M:] == 7.0).all()  # pad rows never written
+    if R:
+        ref64 = x.double() @ lin["proj_down"][:, :R].double()
+        assert (la[:M].double() - ref64).abs().max() <= 2e-5 * ref64.abs().max()
+        assert (la[M:] == 7.0).all()
+
+
+@pytest.mark.parametrize("smooth", [True, False])
+def test_unsigned_with_shift_bit_exact(dev, smooth):
+    M, K = 96, 512
+    g = torch.Generator().manual_seed(3)
+    x = (torch.nn.functional.gelu(torch.randn(M, K, generator=g) * 2, approximate="tanh")).to(torch.bfloat16)
+    lin = O.make_svdq_linear(K, 64, seed=4)
+    (out, osc, la), (rp, rs, rl, _) = _run(x, lin, dev, 32, smooth=smooth, unsigned=True, shift=0.171875)
+    assert torch.equal(out, rp)
+    assert torch.equal(osc.view(torch.int16), rs.view(torch.int16))
+
+
+def test_zero_groups_and_ties(dev):
+    x = torch.zeros(16, 128, dtype=torch.bfloat16)
+    x[1, :64] = torch.arange(64).float().sub(32).mul(0.5).clamp(-7, 7).to(torch.bfloat16)  # exact .5 ties at scale 1
+    x[2, 64:] = -3.0
+    lin = O.make_svdq_linear(128, 64, seed=5)
+    (out, osc, _), (rp, rs, _, _) = _run(x, lin, dev, 0, smooth=False)
+    assert torch.equal(out, rp) and torch.equal(osc.view(torch.int16), rs.view(torch.int16))
+    (out, osc, _), (rp, rs, _, _) = _run(x, lin, dev, 0, smooth=False, unsigned=True)
+    assert torch.equal(out, rp) and torch.equal(osc.view(torch.int16), rs.view(torch.int16))
+
+
+def test_full_size_qkv_input_bit_exact_and_deterministic(dev):
+    """The benchmark configuration: M=4608, K=3072, R=32, outlier channels, smooth U(0.5, 4)."""
+    M, K = 4608, 3072
+    x = O.make_activations(M, K, seed=1)
+    lin = O.make_svdq_linear(K, 64, seed=0)
+    (out, osc, la), (rp, rs, rl, _) = _run(x, lin, dev, 32)
+    assert torch.equal(out, rp)
+    assert torch.equal(osc.view(torch.int16), rs.view(torch.int16))
+    assert (la - rl).abs().max() <= 2e-5 * rl.abs().max()
+    (out2, osc2, la2), _ = _run(x, lin, dev, 32)
+    assert torch.equal(out, out2) and torch.equal(osc.view(torch.int16), osc2.view(torch.int16)) and torch.equal(la, la2)
+
+
+def test_operator_pads_rows_like_the_reference(dev):
+    from nunchaku_rocm_amd import ops
+
+    M, K = 300, 256
+    x = O.make_activations(M, K, seed=9).to(dev)
+    lin = O.make_svdq_linear(K, 64, seed=9)
+    out, osc, la = ops.svdq_quantize_w4a4_act_fuse_lora_cuda(x, lora_down=lin["proj_down"].to(dev), smooth=lin["smooth_factor"].to(dev))
+    assert out.shape == (512, K // 2) and osc.shape == (K // 64, 512) and la.shape == (512, 32) and la.dtype == torch.float32
+    rp, rs, rl, _ = O.quantize_act(x.cpu(), lin["proj_down"], lin["smooth_factor"])
+    assert torch.equal(out[:M].cpu(), rp) and torch.equal(osc[:, :M].cpu().view(torch.int16), rs.view(torch.int16))
+
+
+def test_fuse_glu_close_to_oracle(dev):
+    from nunchaku_rocm_amd.ops.quantize import quantize_w4a4_act_fuse_lora
+
+    M, K = 32, 512
+    g = torch.Generator().manual_seed(6)
+    x = torch.randn(M, 2 * K, generator=g).to(torch.bfloat16)
+    out, osc, _ = quantize_w4a4_act_fuse_lora(x.to(dev), fuse_glu=True)
+    rp, rs, _, rc = O.quantize_act(x, fuse_glu=True)
+    codes = O.unpack_int4(out.cpu(), True)
+    d = (codes - rc).abs()
+    assert d.max() <= 1 and (d > 0).float().mean() < 1e-3  # exp() differs between libraries
+    assert ((osc.cpu().float() - rs.float()).abs() <= rs.float().abs() * 2**-7 + 1e-9).all()
