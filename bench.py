@@ -1,0 +1,236 @@
+#!/usr/bin/env python3
+"""Benchmark of the SVDQuant kernel path on one MI355X.
+
+A step is one pass of the hot path over one batch of synthetic input: the FLUX.1 QKV linear
+(M=4608 tokens, K=3072, N=9216, group 64, LoRA rank 32) as activation quantizer + W4A4 GEMM, inputs resident in HBM.
+``value`` is 2*M*N*K / step time in TOP/s (the reference's GEMM convention, tests/triton/bench_kernels.py:61, charged
+with the quantizer's time as well).  The JSON line also carries the roofline of the dominant kernel (the GEMM, timed
+with HIP events inside the timed region), a per-kernel table (quantizer GB/s, AWQ GEMV GB/s, GEMM M-sweep and fused
+epilogue shapes), and the CPU baseline (the oracle's pure-PyTorch restatement of the reference's CPU path).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-extras]
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+INT8_MFMA_PEAK_TOPS = 5000.0  # MI355X dense int8 MFMA, published
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+
+
+def _events(n):
+    import torch
+
+    return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+
+
+def _time_kernel(fn, iters=50, warmup=10):
+    """Average launch duration in ms: HIP events on the launch stream around ``iters`` back-to-back launches."""
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    a, b = _events(2)
+    torch.cuda.synchronize()
+    a.record()
+    for _ in range(iters):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / iters
+
+
+def cpu_baseline(M, K, N):
+    """The oracle (a pure-PyTorch port of the reference's CPU-runnable path: quantizer restatement + per-group fp32
+    GEMM + LoRA-up + bias, nunchaku/ops/triton/native/w4a4.py:713-726) timed on this host's cores."""
+    import torch
+
+    from oracle import svdq_oracle as O
+
+    cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "0") or (os.cpu_count() or 1)))
+    torch.set_num_threads(cores)
+    lin = O.make_svdq_linear(K, N, seed=0)
+    x = O.make_activations(M, K, seed=1)
+
+    def run(rows):
+        rp, rs, rl, _ = O.quantize_act(x[:rows], lin["proj_down"], lin["smooth_factor"])
+        return O.gemm_w4a4(rp, lin["qweight"], rs, lin["wscales"], lin["bias"], rl, lin["proj_up"])
+
+    run(256)  # warm-up
+    times = []
+    for _ in range(2):
+        t0 = time.perf_counter()
+        run(M)
+        times.append(time.perf_counter() - t0)
+        if sum(times) > 25.0:
+            break
+    t = min(times)
+    return {
+        "value": round(2.0 * M * N * K / t / 1e12, 4),
+        "unit": "TOP/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"full config 0 (M={M}, K={K}, N={N}, R=32): quantizer + GEMM, best of {len(times)} runs, {t:.2f} s each, torch {torch.__version__} CPU fp32",
+        "seconds": round(t, 3),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs on one GPU only (the path shards over tokens with no exchange; "
+              "see DESIGN.md); run with --gpus 1", file=sys.stderr)  # fmt: skip
+        sys.exit(2)
+
+    import torch
+
+    from nunchaku_rocm_amd import _lib, ops
+    from oracle import svdq_oracle as O  # input generators only; nothing from the oracle is timed on the GPU side
+
+    _lib.load()
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    M, K, N, R = 4608, 3072, 9216, 32
+    lin = {k: v.to(dev) for k, v in O.make_svdq_linear(K, N, R, seed=0).items()}
+    x = O.make_activations(M, K, seed=1).to(dev)
+    qx = torch.empty(M, K // 2, dtype=torch.uint8, device=dev)
+    asc = torch.empty(K // 64, M, dtype=torch.bfloat16, device=dev)
+    la = torch.empty(M, R, dtype=torch.float32, device=dev)
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+
+    def quant():
+        ops.svdq_quantize_w4a4_act_fuse_lora_cuda(x, qx, asc, lin["proj_down"], la, lin["smooth_factor"])
+
+    def gemm():
+        ops.svdq_gemm_w4a4_cuda(act=qx, wgt=lin["qweight"], out=out, ascales=asc, wscales=lin["wscales"],
+                                lora_act_in=la, lora_up=lin["proj_up"], bias=lin["bias"])  # fmt: skip
+
+    for _ in range(args.warmup):
+        quant()
+        gemm()
+    ev = [_events(2) for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        quant()
+        ev[i][0].record()
+        gemm()
+        ev[i][1].record()
+    torch.cuda.synchronize()
+    step_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    gemm_ms = sum(a.elapsed_time(b) for a, b in ev) / args.steps
+    ops_per_gemm = 2.0 * M * N * K
+    achieved = ops_per_gemm / (gemm_ms * 1e-3) / 1e12
+
+    kernels = {}
+    if not args.no_extras:
+        q_ms = _time_kernel(quant)
+        q_bytes = 2 * M * K + M * K // 2 + 2 * (K // 64) * M + 4 * M * R + 2 * K * R + 2 * K
+        kernels["quantize_act M4608 K3072 R32"] = {
+            "ms": round(q_ms, 5), "GB/s": round(q_bytes / q_ms / 1e6, 1), "frac_hbm": round(q_bytes / q_ms / 1e6 / HBM_PEAK_GBS, 4),
+            "bytes": q_bytes, "GB/s_ref_convention": round((2 * M * K + M * K // 2) / q_ms / 1e6, 1),
+        }  # fmt: skip
+        g_ms = _time_kernel(gemm)
+        kernels["gemm_w4a4 M4608 K3072 N9216"] = {"ms": round(g_ms, 5), "TOP/s": round(ops_per_gemm / g_ms / 1e9, 1),
+                                                  "frac_int8_mfma": round(ops_per_gemm / g_ms / 1e9 / INT8_MFMA_PEAK_TOPS, 4)}  # fmt: skip
+        for Ms in (1024, 8192):
+            xs = O.make_activations(Ms, K, seed=1).to(dev)
+            q2, a2, l2 = ops.svdq_quantize_w4a4_act_fuse_lora_cuda(xs, lora_down=lin["proj_down"], smooth=lin["smooth_factor"])
+            o2 = torch.empty(Ms, N, dtype=torch.bfloat16, device=dev)
+            ms = _time_kernel(lambda: ops.svdq_gemm_w4a4_cuda(act=q2, wgt=lin["qweight"], out=o2, ascales=a2, wscales=lin["wscales"],
+                                                              lora_act_in=l2, lora_up=lin["proj_up"], bias=lin["bias"]))  # fmt: skip
+            kernels[f"gemm_w4a4 M{Ms} K3072 N9216"] = {"ms": round(ms, 5), "TOP/s": round(2.0 * Ms * N * K / ms / 1e9, 1),
+                                                       "frac_int8_mfma": round(2.0 * Ms * N * K / ms / 1e9 / INT8_MFMA_PEAK_TOPS, 4)}  # fmt: skip
+            del xs, q2, a2, l2, o2
+        # fused epilogues at the FLUX MLP / attention shapes
+        from nunchaku_rocm_amd.linear import SVDQW4A4Linear
+
+        def module(k, n, seed, act_unsigned=False):
+            p = O.make_svdq_linear(k, n, seed=seed)
+            m = SVDQW4A4Linear(k, n, rank=32, act_unsigned=act_unsigned, device=dev)
+            with torch.no_grad():
+                for name in ("qweight", "wscales", "smooth_factor", "proj_down", "proj_up", "bias"):
+                    getattr(m, name).copy_(p[name])
+            return m
+
+        fc1, fc2 = module(3072, 12288, 42), module(12288, 3072, 43, True)
+        q1, a1, l1 = fc1.quantize(x)
+        qo = torch.empty(M, 6144, dtype=torch.uint8, device=dev)
+        oo = torch.empty(192, M, dtype=torch.bfloat16, device=dev)
+        lo = torch.empty(M, 32, dtype=torch.float32, device=dev)
+        y2 = torch.empty(M, 3072, dtype=torch.bfloat16, device=dev)
+
+        def fc1_fused():
+            ops.svdq_gemm_w4a4_cuda(act=q1, wgt=fc1.qweight, qout=qo, ascales=a1, wscales=fc1.wscales, oscales=oo, lora_act_in=l1,
+                                    lora_up=fc1.proj_up, lora_down=fc2.proj_down, lora_act_out=lo, bias=fc1.bias,
+                                    smooth_factor=fc2.smooth_factor)  # fmt: skip
+
+        ms = _time_kernel(fc1_fused)
+        f = 2.0 * M * 12288 * 3072
+        kernels["gemm_w4a4+gelu+requant fc1 M4608 K3072 N12288"] = {"ms": round(ms, 5), "TOP/s": round(f / ms / 1e9, 1), "frac_int8_mfma": round(f / ms / 1e9 / INT8_MFMA_PEAK_TOPS, 4)}  # fmt: skip
+        ms = _time_kernel(lambda: fc2.forward_quant(qo, oo, lo, y2))
+        kernels["gemm_w4a4 fc2 (unsigned act) M4608 K12288 N3072"] = {"ms": round(ms, 5), "TOP/s": round(f / ms / 1e9, 1), "frac_int8_mfma": round(f / ms / 1e9 / INT8_MFMA_PEAK_TOPS, 4)}  # fmt: skip
+        nq = (torch.rand(128, device=dev) + 0.5).to(torch.bfloat16)
+        rot = O.flux_rotary(O.flux_ids(512, 64, 64)).to(dev)
+        ms = _time_kernel(lambda: ops.svdq_gemm_w4a4_cuda(act=qx, wgt=lin["qweight"], out=out, ascales=asc, wscales=lin["wscales"],
+                                                          lora_act_in=la, lora_up=lin["proj_up"], bias=lin["bias"], norm_q=nq, norm_k=nq, rotary_emb=rot))  # fmt: skip
+        kernels["gemm_w4a4+qknorm+rope M4608 K3072 N9216"] = {"ms": round(ms, 5), "TOP/s": round(ops_per_gemm / ms / 1e9, 1), "frac_int8_mfma": round(ops_per_gemm / ms / 1e9 / INT8_MFMA_PEAK_TOPS, 4)}  # fmt: skip
+        # AWQ GEMV, adaLN shape
+        aw = {k: v.to(dev) for k, v in O.make_awq_linear(3072, 18432, seed=2).items() if k != "codes"}
+        for m in (1, 2, 8):
+            xv = torch.randn(m, 3072, device=dev).to(torch.bfloat16)
+            ms = _time_kernel(lambda: ops.awq_gemv_w4a16_cuda(xv, aw["qweight"], aw["wscales"], aw["wzeros"], m, 18432, 3072), iters=200, warmup=20)
+            nbytes = 18432 * 3072 // 2 + 2 * 2 * 48 * 18432 + 2 * m * 3072 + 2 * m * 18432
+            kernels[f"awq_gemv_w4a16 M{m} K3072 N18432"] = {"ms": round(ms, 5), "GB/s": round(nbytes / ms / 1e6, 1),
+                                                           "frac_hbm": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4), "bytes": nbytes}  # fmt: skip
+
+    result = {
+        "metric": "W4A4 GEMM TOPS at the FLUX.1 QKV shape (quantizer + GEMM per step)",
+        "value": round(ops_per_gemm / (step_ms * 1e-3) / 1e12, 2),
+        "unit": "TOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(step_ms, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "i8",
+        "data": "synthetic",
+        "config": {"workload": "FLUX.1 QKV SVDQuant linear: activation quantizer + W4A4 GEMM, M=4608 K=3072 N=9216 group 64 LoRA rank 32 (BASELINE configs[1])",
+                   "M": M, "K": K, "N": N, "rank": R, "group": 64},  # fmt: skip
+        "roofline": {
+            "bound": "mfma",
+            "kernel": "gemm_w4a4_kernel<BF16, signed, plain>",
+            "achieved": round(achieved, 2),
+            "peak": INT8_MFMA_PEAK_TOPS,
+            "unit": "TFLOP/s",
+            "frac": round(achieved / INT8_MFMA_PEAK_TOPS, 4),
+            "traffic": None,
+            "ops_per_launch": ops_per_gemm,
+            "avg_launch_ms": round(gemm_ms, 5),
+            "note": "int8 MFMA ops (2*M*N*K), peak = published dense int8 5.0 POP/s",
+        },
+        "kernels": kernels,
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(M, K, N)
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()
