@@ -16,15 +16,17 @@
 //   s * (D - OFF * xs) + z * xs = s * D + (z - OFF * s) * xs,   xs = sum_{k in c} x[m, k]  (precomputed in LDS).
 // Only accumulator registers whose rows are < M are post-processed (rows m = 8 (i / 4) + 4 h + i % 4).
 //
-// One workgroup = 32 channels x all of K; its four wavefronts take groups round-robin with the weight loads running
-// four groups ahead, and add their partial sums through LDS in a fixed order.
+// One workgroup = 32 channels x all of K; its four wavefronts take groups round-robin with the weight, scale and
+// zero loads running six groups ahead (half of a wavefront's loads at K = 3072), the activations staged once in LDS
+// (up to 8 rows), and the partial sums added through LDS in a fixed order.
 #include "svdq_common.h"
 
 namespace svdq {
 
 constexpr int AWQ_WAVES = 4;
-constexpr int AWQ_NB = 32;  // channels per workgroup
-constexpr int AWQ_PF = 4;   // weight loads in flight per lane
+constexpr int AWQ_NB = 32;    // channels per workgroup
+constexpr int AWQ_PF = 6;     // weight loads in flight per lane
+constexpr int AWQ_XPAD = 8;   // 16-bit elements of padding per staged activation row
 
 template <typename T>
 struct AwqMagic;
@@ -39,33 +41,61 @@ struct AwqMagic<FP16> {
     static constexpr float off = 1024.0f;
 };
 
+// ((w >> sh) & mask) | magic with the mask held in a register so that the and/or pair is one v_and_or_b32
+__device__ inline int nibble_plane(int w, int sh, uint32_t mask, uint32_t magic) {
+    return (int)((((uint32_t)w >> sh) & mask) | magic);
+}
+
 template <typename T, int MQ>  // MQ = ceil(M / 8): accumulator register quads that hold real rows
-__global__ __launch_bounds__(AWQ_WAVES * 64) void awq_gemv_kernel(svdq_awq_gemv_args a) {
-    extern __shared__ __align__(16) float lds[];  // xs[K/64][8*MQ], then red[AWQ_WAVES][8*MQ][32]
-    const int MR = 8 * MQ;
+__global__ __launch_bounds__(AWQ_WAVES * 64, 4) void awq_gemv_kernel(svdq_awq_gemv_args a) {
+    // xs[K/64][8*MQ] fp32 | red[AWQ_WAVES][8*MQ][32] fp32 | (M <= 8 only) x[M][K + pad] 16-bit
+    extern __shared__ __align__(16) float lds[];
+    constexpr int MR = 8 * MQ;
+    constexpr bool X_IN_LDS = MQ == 1;
     const int ngroups = a.K / GROUP;
     float *xs = lds;
     float *red = lds + (size_t)ngroups * MR;
+    uint16_t *xl = (uint16_t *)(red + AWQ_WAVES * MR * AWQ_NB);
+    const int xld = a.K + AWQ_XPAD;
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keep it in an SGPR
     const int l32 = lane & 31, half = lane >> 5;
     const int n = blockIdx.x * AWQ_NB + l32;
-    const uint16_t *x = (const uint16_t *)a.x;
+    const uint16_t *__restrict__ x = (const uint16_t *)a.x;
 
-    // weight stream of this lane: packed row n / 4, int16 column 64 c + 16 (n % 4) + 8 h
-    const uint16_t *wq = (const uint16_t *)a.qweight + (size_t)(n >> 2) * a.K + 16 * (n & 3) + 8 * half;
-    const int nmy = (ngroups - wave + AWQ_WAVES - 1) / AWQ_WAVES;  // groups c = wave + 4 i
+    // weight / scale / zero streams of this lane: packed row n / 4, int16 column 64 c + 16 (n % 4) + 8 h
+    const uint16_t *__restrict__ wq =
+        (const uint16_t *)a.qweight + (size_t)(n >> 2) * a.K + 16 * (n & 3) + 8 * half + (size_t)wave * GROUP;
+    const uint16_t *__restrict__ sc = (const uint16_t *)a.scales + n + (size_t)wave * a.ld_scales;
+    const uint16_t *__restrict__ zr = (const uint16_t *)a.zeros + n + (size_t)wave * a.ld_scales;
+    const int wstep = AWQ_WAVES * GROUP, sstep = AWQ_WAVES * a.ld_scales;  // per group of this wavefront
+    const int nmy = (ngroups - wave + AWQ_WAVES - 1) / AWQ_WAVES;           // groups c = wave + AWQ_WAVES * i
     v4i wreg[AWQ_PF];
+    uint16_t sreg[AWQ_PF], zreg[AWQ_PF];
 #pragma unroll
     for (int u = 0; u < AWQ_PF; u++)
-        if (u < nmy) wreg[u] = *(const v4i *)(wq + (size_t)(wave + AWQ_WAVES * u) * GROUP);
+        if (u < nmy) {
+            wreg[u] = __builtin_nontemporal_load((const v4i *)(wq + (size_t)u * wstep));
+            sreg[u] = sc[(size_t)u * sstep];
+            zreg[u] = zr[(size_t)u * sstep];
+        }
 
-    // xs[c][m] = sum of the group's 64 activations (fp32), while the first weight loads are in flight
+    if (X_IN_LDS) {
+        // stage the activations once per workgroup (coalesced 16-byte pieces)
+        const int per_row = a.K / 8;
+        for (int p = tid; p < a.M * per_row; p += AWQ_WAVES * 64) {
+            const int m = p / per_row, q = p % per_row;
+            *(v4i *)(xl + m * xld + 8 * q) = *(const v4i *)(x + (size_t)m * a.ld_x + 8 * q);
+        }
+        __syncthreads();
+    }
+    // xs[c][m] = sum of the group's 64 activations (fp32)
     for (int p = tid; p < ngroups * MR; p += AWQ_WAVES * 64) {
         const int c = p / MR, m = p % MR;
         float s = 0.0f;
         if (m < a.M) {
-            const v4i *xp = (const v4i *)(x + (size_t)m * a.ld_x + c * GROUP);
+            const v4i *xp = X_IN_LDS ? (const v4i *)(xl + m * xld + c * GROUP) : (const v4i *)(x + (size_t)m * a.ld_x + c * GROUP);
 #pragma unroll
             for (int q = 0; q < 8; q++) {
                 const v4i v = xp[q];
@@ -81,37 +111,42 @@ __global__ __launch_bounds__(AWQ_WAVES * 64) void awq_gemv_kernel(svdq_awq_gemv_
 #pragma unroll
     for (int i = 0; i < 4 * MQ; i++) acc[i] = 0.0f;
 
-    const bool row_ok = l32 < a.M;  // A operand row of this lane
-    const uint16_t *xrow = x + (size_t)(row_ok ? l32 : 0) * a.ld_x + 32 * half;
-    const uint16_t *sc = (const uint16_t *)a.scales + n;
-    const uint16_t *zr = (const uint16_t *)a.zeros + n;
+    // A operand row of this lane; rows >= M repeat row M - 1 (their products land in accumulator rows nobody reads)
+    const int arow = min(l32, a.M - 1);
+    const uint16_t *xrow = (X_IN_LDS ? xl + arow * xld : x + (size_t)arow * a.ld_x) + 32 * half + wave * GROUP;
+    const float *xsp = xs + wave * MR + 4 * half;
+    uint32_t mask = 0x000F000Fu;
+    asm volatile("" : "+v"(mask));  // keep the mask in a VGPR: v_and_or_b32 takes only one literal
+    v16f zero16;
+#pragma unroll
+    for (int i = 0; i < 16; i++) zero16[i] = 0.0f;
 
     for (int base = 0; base < nmy; base += AWQ_PF) {
 #pragma unroll
         for (int u = 0; u < AWQ_PF; u++) {
             const int idx = base + u;
             if (idx >= nmy) break;
-            const int c = wave + AWQ_WAVES * idx;
             const v4i w = wreg[u];
-            if (idx + AWQ_PF < nmy) wreg[u] = *(const v4i *)(wq + (size_t)(c + AWQ_WAVES * AWQ_PF) * GROUP);
-            const float s = T::to_f32(sc[(size_t)c * a.ld_scales]);
-            const float zz = T::to_f32(zr[(size_t)c * a.ld_scales]) - AwqMagic<T>::off * s;
-
+            const float s = T::to_f32(sreg[u]);
+            const float zz = T::to_f32(zreg[u]) - AwqMagic<T>::off * s;
+            if (idx + AWQ_PF < nmy) {
+                wreg[u] = __builtin_nontemporal_load((const v4i *)(wq + (size_t)(idx + AWQ_PF) * wstep));
+                sreg[u] = sc[(size_t)(idx + AWQ_PF) * sstep];
+                zreg[u] = zr[(size_t)(idx + AWQ_PF) * sstep];
+            }
+            const uint16_t *xg = xrow + idx * wstep;
             v16f d;
 #pragma unroll
-            for (int i = 0; i < 16; i++) d[i] = 0.0f;
-#pragma unroll
             for (int pl = 0; pl < 4; pl++) {
-                typedef unsigned v4u __attribute__((ext_vector_type(4)));
-                const v4u wu = __builtin_bit_cast(v4u, w);
-                const v4i wb = __builtin_bit_cast(v4i, ((wu >> (4 * pl)) & 0x000F000Fu) | AwqMagic<T>::bits);
-                v4i xa = (v4i){0, 0, 0, 0};
-                if (row_ok) xa = *(const v4i *)(xrow + c * GROUP + 8 * pl);
-                d = mfma32_16bit<T>(xa, wb, d);
+                v4i wb;
+#pragma unroll
+                for (int e = 0; e < 4; e++) wb[e] = nibble_plane(w[e], 4 * pl, mask, AwqMagic<T>::bits);
+                const v4i xa = *(const v4i *)(xg + 8 * pl);
+                d = mfma32_16bit<T>(xa, wb, pl == 0 ? zero16 : d);
             }
 #pragma unroll
             for (int q = 0; q < MQ; q++) {
-                const v4f xv = *(const v4f *)(xs + c * MR + 8 * q + 4 * half);
+                const v4f xv = *(const v4f *)(xsp + idx * (AWQ_WAVES * MR) + 8 * q);
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     acc[4 * q + e] = __builtin_fmaf(s, d[4 * q + e], acc[4 * q + e]);
@@ -121,7 +156,7 @@ __global__ __launch_bounds__(AWQ_WAVES * 64) void awq_gemv_kernel(svdq_awq_gemv_
         }
     }
 
-    // fixed-order sum over the four wavefronts, then store T
+    // fixed-order sum over the wavefronts, then store T
 #pragma unroll
     for (int q = 0; q < MQ; q++)
 #pragma unroll
@@ -136,11 +171,18 @@ __global__ __launch_bounds__(AWQ_WAVES * 64) void awq_gemv_kernel(svdq_awq_gemv_
     }
 }
 
+static size_t awq_lds_bytes(int K, int M) {
+    const int MQ = (M + 7) / 8;
+    size_t b = ((size_t)(K / GROUP) * 8 * MQ + (size_t)AWQ_WAVES * 8 * MQ * AWQ_NB) * sizeof(float);
+    if (MQ == 1) b += (size_t)M * (K + AWQ_XPAD) * 2;
+    return b;
+}
+
 template <typename T>
 static void launch_awq(const svdq_awq_gemv_args &a, hipStream_t s) {
     const int MQ = (a.M + 7) / 8;
     const dim3 grid(a.N / AWQ_NB), block(AWQ_WAVES * 64);
-    const size_t sh = ((size_t)(a.K / GROUP) * 8 * MQ + (size_t)AWQ_WAVES * 8 * MQ * AWQ_NB) * sizeof(float);
+    const size_t sh = awq_lds_bytes(a.K, a.M);
     switch (MQ) {
         case 1: hipLaunchKernelGGL((awq_gemv_kernel<T, 1>), grid, block, sh, s, a); break;
         case 2: hipLaunchKernelGGL((awq_gemv_kernel<T, 2>), grid, block, sh, s, a); break;
@@ -176,8 +218,8 @@ extern "C" int svdq_awq_gemv_w4a16(const svdq_awq_gemv_args *args, void *stream)
         set_error("svdq_awq_gemv_w4a16: x rows and qweight must be 16-byte aligned; leading dimensions >= row length");
         return SVDQ_E_INVALID;
     }
-    if ((size_t)(a.K / GROUP) * 32 * 4 + 16384 > 65536) {
-        set_error("svdq_awq_gemv_w4a16: K=%d too large for the LDS group-sum table", a.K);
+    if (awq_lds_bytes(a.K, a.M) > 65536) {
+        set_error("svdq_awq_gemv_w4a16: K=%d too large for the LDS activation / group-sum tables", a.K);
         return SVDQ_E_UNSUPPORTED;
     }
     if (a.M == 0) return SVDQ_OK;

@@ -78,7 +78,7 @@ __global__ __launch_bounds__(256, 2) void gemm_w4a4_kernel(svdq_gemm_args a) {
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keep it in an SGPR
     const int wn = wave & 1, wm = wave >> 1;  // wavefront position in the 2x2 arrangement
     const int l32 = lane & 31, half = lane >> 5;
 

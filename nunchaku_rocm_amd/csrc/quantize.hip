@@ -7,7 +7,8 @@
 // add, clamp, low nibble first.  The LoRA-down product consumes the raw 16-bit activations (before shift and
 // smoothing) on the 16x16x32 MFMA with fp32 accumulation.
 //
-// Work split: one workgroup = 16 rows x all of K, four wavefronts taking scale groups round-robin.  Lane
+// Work split: one workgroup = 16 rows x all of K, eight wavefronts taking scale groups round-robin with two
+// groups of loads in flight each.  Lane
 // (m = lane % 16, q = lane / 16) owns 16 consecutive channels [64 g + 16 q, +16) of row m, so a wavefront reads
 // 16 rows x 128 contiguous bytes per group, a group's absmax needs two cross-lane steps, and the lane's two
 // 16-byte halves are exactly the B operands of two MFMAs whose A operands come from the transposed LoRA-down
@@ -20,63 +21,98 @@
 namespace svdq {
 
 constexpr int Q_ROWS = 16;
-constexpr int Q_WAVES = 4;
+constexpr int Q_WAVES = 8;
 constexpr int Q_RCHUNK = 32;  // LoRA ranks per pass over the row block
 
-template <typename T, bool UNSIGNED, bool GLU>
-__global__ __launch_bounds__(Q_WAVES * 64) void quantize_act_kernel(svdq_quantize_args a) {
+// sum_j (0x4B400000 << 4 j) mod 2^32: what eight magic-biased codes add up to besides their nibbles
+constexpr uint32_t pack_bias() {
+    uint32_t c = 0;
+    for (int j = 0; j < 8; j++) c += (uint32_t)RNE_MAGIC_BITS << (4 * j);
+    return c;
+}
+
+// One scale group's loads for one lane: 16 activations (+ 16 gate values), the matching LoRA-down operands
+template <bool GLU, bool HAS_LORA>
+struct QStage {
+    v4i xlo, xhi, glo, ghi, l0lo, l0hi, l1lo, l1hi;
+    uint16_t sm;
+};
+
+template <typename T, bool UNSIGNED, bool GLU, bool HAS_LORA, bool HAS_SMOOTH>
+__global__ __launch_bounds__(Q_WAVES * 64, 4) void quantize_act_kernel(svdq_quantize_args a) {
     __shared__ float lds_rs[Q_WAVES][64];
     __shared__ float lds_acc[Q_WAVES][Q_RCHUNK][Q_ROWS + 1];
 
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: keep it in an SGPR
     const int ml = lane & 15;
     const int kq = lane >> 4;
     const int m0 = blockIdx.x * Q_ROWS;
     const int m = m0 + ml;
     const bool row_ok = m < a.M;
     const int ngroups = a.K / GROUP;
-    const uint16_t *xrow = (const uint16_t *)a.x + (size_t)(row_ok ? m : 0) * a.ld_x;
-    const uint16_t *smooth = (const uint16_t *)a.smooth;
-    const uint16_t *ldt = (const uint16_t *)a.lora_down_t;
+    const int nmy = (ngroups - wave + Q_WAVES - 1) / Q_WAVES;  // groups g = wave + Q_WAVES * i
+    // uniform base pointers + 32-bit per-lane element offsets (rows >= M re-read row M - 1: valid memory, and
+    // nothing is stored for them)
+    const uint16_t *__restrict__ xbase = (const uint16_t *)a.x + (size_t)m0 * a.ld_x + wave * GROUP;
+    const uint32_t xoff = (uint32_t)(min(m, a.M - 1) - m0) * a.ld_x + kq * 16;
+    const uint16_t *__restrict__ smooth = (const uint16_t *)a.smooth + wave * GROUP;
+    uint8_t *__restrict__ outbase = (uint8_t *)a.out + (size_t)m0 * a.ld_out + wave * (GROUP / 2);
+    const uint32_t outoff = (uint32_t)ml * a.ld_out + kq * 8;
+    uint16_t *__restrict__ scales = (uint16_t *)a.scales + (size_t)wave * a.ld_scales + m0;
+    constexpr int GSTEP = Q_WAVES * GROUP;  // elements between consecutive groups of one wavefront
     const float qmax = UNSIGNED ? 15.0f : 7.0f;
-    const float qlo = UNSIGNED ? 0.0f : -8.0f;
-    const float qhi = UNSIGNED ? 15.0f : 7.0f;
+    const float rmagic = UNSIGNED ? RNE_MAGIC : RNE_MAGIC + 8.0f;  // signed codes are packed as c + 8, then ^ 8
+    const bool has_shift = a.shift != 0.0f;
 
-    const int nchunks = a.R > 0 ? (a.R + Q_RCHUNK - 1) / Q_RCHUNK : 1;
+    const int nchunks = HAS_LORA ? (a.R + Q_RCHUNK - 1) / Q_RCHUNK : 1;
     for (int rc = 0; rc < nchunks; rc++) {
-        v4f acc[2];
-        acc[0] = (v4f){0.f, 0.f, 0.f, 0.f};
-        acc[1] = (v4f){0.f, 0.f, 0.f, 0.f};
-        const int r0 = rc * Q_RCHUNK + ml;  // LoRA row of this lane's A operand (block 0), block 1 = +16
-        const bool r_ok0 = r0 < a.R, r_ok1 = r0 + 16 < a.R;
+        v4f acc0 = (v4f){0.f, 0.f, 0.f, 0.f}, acc1 = (v4f){0.f, 0.f, 0.f, 0.f};
+        // ranks >= R re-read rank R - 1; their accumulator rows are never stored
+        const int r0 = rc * Q_RCHUNK + ml;
+        const uint16_t *__restrict__ lbase = (const uint16_t *)a.lora_down_t + wave * GROUP;
+        uint32_t loff0 = 0, loff1 = 0;
+        if (HAS_LORA) {
+            loff0 = (uint32_t)min(r0, a.R - 1) * a.K + kq * 16;
+            loff1 = (uint32_t)min(r0 + 16, a.R - 1) * a.K + kq * 16;
+        }
+        const bool do_quant = rc == 0;
 
-        for (int g = wave; g < ngroups; g += Q_WAVES) {
-            const int k0 = g * GROUP + kq * 16;
-            v4i xlo = (v4i){0, 0, 0, 0}, xhi = (v4i){0, 0, 0, 0};
-            if (row_ok) {
-                xlo = *(const v4i *)(xrow + k0);
-                xhi = *(const v4i *)(xrow + k0 + 8);
+        auto issue = [&](QStage<GLU, HAS_LORA> &st, int i) {
+            const int k0 = min(i, nmy - 1) * GSTEP;  // past the end: re-read the last group, unused
+            const uint16_t *xg = xbase + k0;
+            st.xlo = *(const v4i *)(xg + xoff);
+            st.xhi = *(const v4i *)(xg + xoff + 8);
+            if (GLU) {
+                st.glo = *(const v4i *)(xg + a.K + xoff);
+                st.ghi = *(const v4i *)(xg + a.K + xoff + 8);
             }
+            if (HAS_LORA) {
+                const uint16_t *lg = lbase + k0;
+                st.l0lo = *(const v4i *)(lg + loff0);
+                st.l0hi = *(const v4i *)(lg + loff0 + 8);
+                st.l1lo = *(const v4i *)(lg + loff1);
+                st.l1hi = *(const v4i *)(lg + loff1 + 8);
+            }
+            if (HAS_SMOOTH) st.sm = (smooth + k0)[lane];
+        };
+
+        auto process = [&](const QStage<GLU, HAS_LORA> &st, int i) {
+            v4i cxlo = st.xlo, cxhi = st.xhi;
             float v[16];
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                v[2 * j] = T::lo_f32((uint32_t)xlo[j]);
-                v[2 * j + 1] = T::hi_f32((uint32_t)xlo[j]);
-                v[8 + 2 * j] = T::lo_f32((uint32_t)xhi[j]);
-                v[8 + 2 * j + 1] = T::hi_f32((uint32_t)xhi[j]);
+                v[2 * j] = T::lo_f32((uint32_t)cxlo[j]);
+                v[2 * j + 1] = T::hi_f32((uint32_t)cxlo[j]);
+                v[8 + 2 * j] = T::lo_f32((uint32_t)cxhi[j]);
+                v[8 + 2 * j + 1] = T::hi_f32((uint32_t)cxhi[j]);
             }
             if (GLU) {
                 // x[:, k] * silu(x[:, K + k]); the LoRA-down then sees the product rounded to T
-                v4i glo = (v4i){0, 0, 0, 0}, ghi = (v4i){0, 0, 0, 0};
-                if (row_ok) {
-                    glo = *(const v4i *)(xrow + a.K + k0);
-                    ghi = *(const v4i *)(xrow + a.K + k0 + 8);
-                }
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
-                    float g0 = T::lo_f32((uint32_t)glo[j]), g1 = T::hi_f32((uint32_t)glo[j]);
-                    float g2 = T::lo_f32((uint32_t)ghi[j]), g3 = T::hi_f32((uint32_t)ghi[j]);
+                    const float g0 = T::lo_f32((uint32_t)st.glo[j]), g1 = T::hi_f32((uint32_t)st.glo[j]);
+                    const float g2 = T::lo_f32((uint32_t)st.ghi[j]), g3 = T::hi_f32((uint32_t)st.ghi[j]);
                     v[2 * j] = v[2 * j] * (g0 / (1.0f + __expf(-g0)));
                     v[2 * j + 1] = v[2 * j + 1] * (g1 / (1.0f + __expf(-g1)));
                     v[8 + 2 * j] = v[8 + 2 * j] * (g2 / (1.0f + __expf(-g2)));
@@ -84,71 +120,90 @@ __global__ __launch_bounds__(Q_WAVES * 64) void quantize_act_kernel(svdq_quantiz
                 }
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
-                    xlo[j] = (int)pack2<T>(v[2 * j], v[2 * j + 1]);
-                    xhi[j] = (int)pack2<T>(v[8 + 2 * j], v[8 + 2 * j + 1]);
+                    cxlo[j] = (int)pack2<T>(v[2 * j], v[2 * j + 1]);
+                    cxhi[j] = (int)pack2<T>(v[8 + 2 * j], v[8 + 2 * j + 1]);
                 }
             }
-
-            if (a.R > 0) {
-                v4i z = (v4i){0, 0, 0, 0};
-                const uint16_t *lp = ldt + (size_t)r0 * a.K + k0;
-                v4i a0lo = r_ok0 ? *(const v4i *)(lp) : z;
-                v4i a0hi = r_ok0 ? *(const v4i *)(lp + 8) : z;
-                v4i a1lo = r_ok1 ? *(const v4i *)(lp + (size_t)16 * a.K) : z;
-                v4i a1hi = r_ok1 ? *(const v4i *)(lp + (size_t)16 * a.K + 8) : z;
-                acc[0] = mfma16_16bit<T>(a0lo, xlo, acc[0]);
-                acc[0] = mfma16_16bit<T>(a0hi, xhi, acc[0]);
-                acc[1] = mfma16_16bit<T>(a1lo, xlo, acc[1]);
-                acc[1] = mfma16_16bit<T>(a1hi, xhi, acc[1]);
+            if (HAS_LORA) {
+                acc0 = mfma16_16bit<T>(st.l0lo, cxlo, acc0);
+                acc0 = mfma16_16bit<T>(st.l0hi, cxhi, acc0);
+                acc1 = mfma16_16bit<T>(st.l1lo, cxlo, acc1);
+                acc1 = mfma16_16bit<T>(st.l1hi, cxhi, acc1);
             }
+            if (!do_quant) return;
+            if (has_shift) {
+#pragma unroll
+                for (int j = 0; j < 16; j++) v[j] = v[j] + a.shift;
+            }
+            if (HAS_SMOOTH) {
+                // 1/smooth for the group's 64 channels: one IEEE divide per lane, shared through LDS
+                lds_rs[wave][lane] = 1.0f / T::to_f32(st.sm);
+                __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const v4f rs = *(const v4f *)&lds_rs[wave][kq * 16 + 4 * j];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) v[4 * j + e] = v[4 * j + e] * rs[e];
+                }
+                __builtin_amdgcn_wave_barrier();
+            }
+            float gmax = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 16; j += 2)
+                gmax = UNSIGNED ? __builtin_fmaxf(__builtin_fmaxf(v[j], v[j + 1]), gmax)
+                                : __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(v[j]), __builtin_fabsf(v[j + 1])), gmax);
+            gmax = fmaxf(gmax, __shfl_xor(gmax, 16));
+            gmax = fmaxf(gmax, __shfl_xor(gmax, 32));
+            const float scale = gmax / qmax;
+            const float safe = (scale == 0.0f) ? 1.0f : scale;
+            const float rq = 1.0f / safe;
+            // The magic add rounds to nearest-even and leaves code (+ 8 when signed) in the low mantissa bits; shifted
+            // adds pack eight of them per dword (the constant upper bits add up to pack_bias()).  Signed codes need
+            // no clamp: |x| <= gmax gives |x * (1 / (gmax / 7))| <= 7 (1 + 3 * 2^-24), which rounds to <= 7; unsigned codes
+            // only need the lower clamp (negative values), the upper bound holds the same way.
+            uint32_t w0 = 0u - pack_bias(), w1 = 0u - pack_bias();
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                float q0 = v[j] * rq, q1 = v[8 + j] * rq;
+                if (UNSIGNED) {
+                    q0 = __builtin_fmaxf(q0, 0.0f);
+                    q1 = __builtin_fmaxf(q1, 0.0f);
+                }
+                const uint32_t b0 = __float_as_uint(q0 + rmagic), b1 = __float_as_uint(q1 + rmagic);
+                asm("v_lshl_add_u32 %0, %1, %2, %0" : "+v"(w0) : "v"(b0), "n"(4 * j));
+                asm("v_lshl_add_u32 %0, %1, %2, %0" : "+v"(w1) : "v"(b1), "n"(4 * j));
+            }
+            if (!UNSIGNED) {
+                w0 ^= 0x88888888u;
+                w1 ^= 0x88888888u;
+            }
+            if (row_ok) {
+                if (kq == 0) (scales + (size_t)i * Q_WAVES * a.ld_scales)[ml] = T::from_f32(scale);
+                *(uint2 *)(outbase + (size_t)i * (GSTEP / 2) + outoff) = make_uint2(w0, w1);
+            }
+        };
 
-            if (rc == 0) {
-                if (a.smooth != nullptr) {
-                    // 1/smooth for the group's 64 channels: one IEEE divide per lane, shared through LDS
-                    lds_rs[wave][lane] = 1.0f / T::to_f32(smooth[g * GROUP + lane]);
-                    __builtin_amdgcn_wave_barrier();
-#pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        v4f rs = *(const v4f *)&lds_rs[wave][kq * 16 + 4 * j];
-#pragma unroll
-                        for (int e = 0; e < 4; e++) v[4 * j + e] = (v[4 * j + e] + a.shift) * rs[e];
-                    }
-                    __builtin_amdgcn_wave_barrier();
-                } else {
-#pragma unroll
-                    for (int j = 0; j < 16; j++) v[j] = v[j] + a.shift;
-                }
-                float gmax = 0.0f;
-#pragma unroll
-                for (int j = 0; j < 16; j++) gmax = fmaxf(gmax, UNSIGNED ? v[j] : fabsf(v[j]));
-                gmax = fmaxf(gmax, __shfl_xor(gmax, 16));
-                gmax = fmaxf(gmax, __shfl_xor(gmax, 32));
-                const float scale = gmax / qmax;
-                const float safe = (scale == 0.0f) ? 1.0f : scale;
-                if (row_ok && kq == 0) ((uint16_t *)a.scales)[(size_t)g * a.ld_scales + m] = T::from_f32(scale);
-                const float rq = 1.0f / safe;
-                uint32_t w0 = 0, w1 = 0;
-#pragma unroll
-                for (int j = 0; j < 8; j++) {
-                    // clamp, then the magic add leaves the two's-complement nibble in the low mantissa bits
-                    float q0 = __builtin_amdgcn_fmed3f(v[j] * rq, qlo, qhi) + RNE_MAGIC;
-                    float q1 = __builtin_amdgcn_fmed3f(v[8 + j] * rq, qlo, qhi) + RNE_MAGIC;
-                    w0 |= (__float_as_uint(q0) & 0xFu) << (4 * j);
-                    w1 |= (__float_as_uint(q1) & 0xFu) << (4 * j);
-                }
-                if (row_ok) {
-                    uint2 pk = make_uint2(w0, w1);
-                    *(uint2 *)((uint8_t *)a.out + (size_t)m * a.ld_out + g * (GROUP / 2) + kq * 8) = pk;
-                }
+        // two groups in flight per wavefront
+        QStage<GLU, HAS_LORA> sa, sb;
+        issue(sa, 0);
+        issue(sb, 1);
+        for (int i = 0; i < nmy; i += 2) {
+            QStage<GLU, HAS_LORA> cur = sa;
+            issue(sa, i + 2);
+            process(cur, i);
+            if (i + 1 < nmy) {
+                cur = sb;
+                issue(sb, i + 3);
+                process(cur, i + 1);
             }
         }
 
-        if (a.R > 0) {
-            // fixed-order sum of the four wavefronts' partial products
+        if (HAS_LORA) {
+            // fixed-order sum of the wavefronts' partial products
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                lds_acc[wave][4 * kq + i][ml] = acc[0][i];
-                lds_acc[wave][16 + 4 * kq + i][ml] = acc[1][i];
+                lds_acc[wave][4 * kq + i][ml] = acc0[i];
+                lds_acc[wave][16 + 4 * kq + i][ml] = acc1[i];
             }
             __syncthreads();
             for (int o = threadIdx.x; o < Q_ROWS * Q_RCHUNK; o += Q_WAVES * 64) {
@@ -171,19 +226,32 @@ __global__ void transpose_kr_kernel(const uint16_t *in, uint16_t *out, int K, in
     out[idx] = in[(size_t)k * ld_in + r];
 }
 
+template <typename T, bool U, bool G>
+static void launch_quantize2(const svdq_quantize_args &a, hipStream_t s) {
+    dim3 grid((a.M + Q_ROWS - 1) / Q_ROWS), block(Q_WAVES * 64);
+    const bool lora = a.R > 0, sm = a.smooth != nullptr;
+    if (lora && sm)
+        hipLaunchKernelGGL((quantize_act_kernel<T, U, G, true, true>), grid, block, 0, s, a);
+    else if (lora)
+        hipLaunchKernelGGL((quantize_act_kernel<T, U, G, true, false>), grid, block, 0, s, a);
+    else if (sm)
+        hipLaunchKernelGGL((quantize_act_kernel<T, U, G, false, true>), grid, block, 0, s, a);
+    else
+        hipLaunchKernelGGL((quantize_act_kernel<T, U, G, false, false>), grid, block, 0, s, a);
+}
+
 template <typename T>
 static void launch_quantize(const svdq_quantize_args &a, hipStream_t s) {
-    dim3 grid((a.M + Q_ROWS - 1) / Q_ROWS), block(Q_WAVES * 64);
     if (a.fuse_glu) {
         if (a.is_unsigned)
-            hipLaunchKernelGGL((quantize_act_kernel<T, true, true>), grid, block, 0, s, a);
+            launch_quantize2<T, true, true>(a, s);
         else
-            hipLaunchKernelGGL((quantize_act_kernel<T, false, true>), grid, block, 0, s, a);
+            launch_quantize2<T, false, true>(a, s);
     } else {
         if (a.is_unsigned)
-            hipLaunchKernelGGL((quantize_act_kernel<T, true, false>), grid, block, 0, s, a);
+            launch_quantize2<T, true, false>(a, s);
         else
-            hipLaunchKernelGGL((quantize_act_kernel<T, false, false>), grid, block, 0, s, a);
+            launch_quantize2<T, false, false>(a, s);
     }
 }
 
