@@ -72,8 +72,12 @@ __device__ inline void tile_ids(int tiles_m, int tiles_n, int &pid_m, int &pid_n
     pid_n = (id % band) / gm;
 }
 
+#ifndef SVDQ_GEMM_MIN_WAVES
+#define SVDQ_GEMM_MIN_WAVES 2
+#endif
+
 template <typename T, bool ACT_UNSIGNED, int EPI>
-__global__ __launch_bounds__(256, 2) void gemm_w4a4_kernel(svdq_gemm_args a) {
+__global__ __launch_bounds__(256, SVDQ_GEMM_MIN_WAVES) void gemm_w4a4_kernel(svdq_gemm_args a) {
     __shared__ __align__(16) uint8_t smem[SMEM_BYTES];
 
     const int tid = threadIdx.x;
@@ -436,6 +440,139 @@ __global__ __launch_bounds__(256, 2) void gemm_w4a4_kernel(svdq_gemm_args a) {
         }
         return;
     }
+
+    if (EPI == SVDQ_EPI_SWIGLU_QUANT) {
+        // Output columns come in 16-blocks [gate | up]: registers j = 0, 1 of a 32-column block are gate values and
+        // j = 2, 3 the matching up values, so y = silu(gate) * up is formed in-lane.  The tile's 128 columns give 64
+        // y columns = one quantization group, shared by the two n-wavefronts (32 y columns each).
+        const int H = a.N / 2;
+        const uint16_t *ldt = (const uint16_t *)a.lora_down_t;
+        float y[2][2][8];  // [bm][bn][4 j + e]: y column 16 bn + 8 j + 4 half + e of the wavefront's 32
+#pragma unroll
+        for (int bm = 0; bm < 2; bm++)
+#pragma unroll
+            for (int bn = 0; bn < 2; bn++)
+#pragma unroll
+                for (int i = 0; i < 8; i++) y[bm][bn][i] = silu(acc[bn][bm][i]) * acc[bn][bm][8 + i];
+        const int yt0 = n0 / 2;          // first y column of the tile
+        const int yw0 = yt0 + 32 * wn;   // ... of this wavefront
+        float *lds_part = (float *)smem;  // [2 (wm)][2 (bm)][16 regs][64 lanes] floats = 16 KB
+        __syncthreads();
+        for (int rc = 0; rc < a.R2; rc += 32) {
+            v16f d[2];
+#pragma unroll
+            for (int bm = 0; bm < 2; bm++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) d[bm][i] = 0.0f;
+            const int r = rc + l32;
+#pragma unroll
+            for (int s = 0; s < 2; s++) {
+                v4i la = (v4i){0, 0, 0, 0};
+                if (r < a.R2) {
+                    const uint16_t *lp = ldt + (size_t)r * H + yw0 + 16 * s + 4 * half;
+                    const uint2 q0 = *(const uint2 *)lp, q1 = *(const uint2 *)(lp + 8);
+                    la = (v4i){(int)q0.x, (int)q0.y, (int)q1.x, (int)q1.y};
+                }
+#pragma unroll
+                for (int bm = 0; bm < 2; bm++) {
+                    v4i xb;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) xb[e] = (int)pack2<T>(y[bm][s][2 * e], y[bm][s][2 * e + 1]);
+                    d[bm] = mfma32_16bit<T>(la, xb, d[bm]);
+                }
+            }
+            if (wn == 1) {
+#pragma unroll
+                for (int bm = 0; bm < 2; bm++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++) lds_part[((wm * 2 + bm) * 16 + i) * 64 + lane] = d[bm][i];
+            }
+            __syncthreads();
+            if (wn == 0) {
+#pragma unroll
+                for (int bm = 0; bm < 2; bm++) {
+                    const int m = mw0 + bm * 32 + l32;
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        v4f o;
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            o[e] = d[bm][4 * j + e] + lds_part[((wm * 2 + bm) * 16 + 4 * j + e) * 64 + lane];
+                        const int rr = rc + 8 * j + 4 * half;
+                        if (m < a.M && rr < a.R2)
+                            *(v4f *)(a.scratch + ((size_t)pid_n * a.M + m) * a.R2 + rr) = o;
+                    }
+                }
+            }
+            __syncthreads();
+        }
+
+        // * 1/smooth, signed per-64 quantization over the tile's 64 y columns
+        float *lds_rs = (float *)smem;        // [64]
+        float *lds_max = (float *)smem + 64;  // [2 (wn)][BM]
+        if (tid < 64) {
+            float rs = 1.0f;
+            if (a.smooth_next != nullptr) rs = 1.0f / T::to_f32(((const uint16_t *)a.smooth_next)[yt0 + tid]);
+            lds_rs[tid] = rs;
+        }
+        __syncthreads();
+        float gm[2];
+#pragma unroll
+        for (int bm = 0; bm < 2; bm++) {
+            float gmax = 0.0f;
+#pragma unroll
+            for (int bn = 0; bn < 2; bn++)
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    const v4f rs = *(const v4f *)(lds_rs + 32 * wn + 16 * bn + 8 * j + 4 * half);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const float v = (y[bm][bn][4 * j + e] + a.shift) * rs[e];
+                        y[bm][bn][4 * j + e] = v;
+                        gmax = fmaxf(gmax, fabsf(v));
+                    }
+                }
+            gmax = fmaxf(gmax, __shfl_xor(gmax, 32));
+            if (half == 0) lds_max[wn * BM + wm * 64 + bm * 32 + l32] = gmax;
+            gm[bm] = gmax;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int bm = 0; bm < 2; bm++) {
+            const int ml = wm * 64 + bm * 32 + l32;
+            const int m = m0 + ml;
+            const float gmax = fmaxf(lds_max[ml], lds_max[BM + ml]);
+            const float scale = gmax / 7.0f;
+            const float safe = (scale == 0.0f) ? 1.0f : scale;
+            const float rq = 1.0f / safe;
+            if (wn == 0 && half == 0 && m < a.M)
+                ((uint16_t *)a.oscales)[(size_t)(yt0 / GROUP) * a.ld_oscales + m] = T::from_f32(scale);
+#pragma unroll
+            for (int bn = 0; bn < 2; bn++) {
+                uint32_t mine[2];
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    uint32_t w = 0;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const float q = __builtin_amdgcn_fmed3f(y[bm][bn][4 * j + e] * rq, -8.0f, 7.0f) + RNE_MAGIC;
+                        w |= (__float_as_uint(q) & 0xFu) << (4 * e);
+                    }
+                    mine[j] = w;  // 16 bits: y columns 16 bn + 8 j + 4 half + 0..3
+                }
+                // dword j of the block's 8-byte run = piece of half 0 (low 16 bits) | piece of half 1 (high 16 bits);
+                // half h keeps dword h
+                const uint32_t keep = half ? mine[1] : mine[0];
+                const uint32_t send = half ? mine[0] : mine[1];
+                const uint32_t theirs = __shfl_xor(send, 32);
+                const uint32_t dw = half ? (theirs | (keep << 16)) : (keep | (theirs << 16));
+                if (m < a.M)
+                    *(uint32_t *)((uint8_t *)a.qout + (size_t)m * a.ld_qout + (yw0 + 16 * bn) / 2 + 4 * half) = dw;
+            }
+        }
+        (void)gm;
+        return;
+    }
 }
 
 // lora_act_out[m, r] = sum over n-tiles of the partial LoRA-down products, in tile order (deterministic)
@@ -485,6 +622,9 @@ static void launch_gemm_epi(const svdq_gemm_args &a, hipStream_t s) {
             break;
         case SVDQ_EPI_GELU_QUANT:
             hipLaunchKernelGGL((gemm_w4a4_kernel<T, U, SVDQ_EPI_GELU_QUANT>), grid, block, 0, s, a);
+            break;
+        case SVDQ_EPI_SWIGLU_QUANT:
+            hipLaunchKernelGGL((gemm_w4a4_kernel<T, U, SVDQ_EPI_SWIGLU_QUANT>), grid, block, 0, s, a);
             break;
     }
 }
@@ -563,12 +703,17 @@ extern "C" int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream) {
             set_error("svdq_gemm_w4a4: norm_q, norm_k (128,) and rotary (actual_m, 128) fp32 16-byte aligned rows are required");
             return SVDQ_E_INVALID;
         }
-    } else if (a.epilogue == SVDQ_EPI_GELU_QUANT) {
+    } else if (quant) {
+        const int NQ = a.epilogue == SVDQ_EPI_SWIGLU_QUANT ? a.N / 2 : a.N;
         if (a.N % 128 || a.M % 16) {
-            set_error("svdq_gemm_w4a4: the GELU requantizing epilogue needs N %% 128 == 0 and M %% 16 == 0 (M=%d N=%d)", a.M, a.N);
+            set_error("svdq_gemm_w4a4: the requantizing epilogues need N %% 128 == 0 and M %% 16 == 0 (M=%d N=%d)", a.M, a.N);
             return SVDQ_E_INVALID;
         }
-        if (!a.qout || !a.oscales || ((uintptr_t)a.qout & 7) || a.ld_qout % 8 || a.ld_qout < a.N / 2 || a.ld_oscales < a.M) {
+        if (a.epilogue == SVDQ_EPI_SWIGLU_QUANT && a.out) {
+            set_error("svdq_gemm_w4a4: the SwiGLU epilogue writes qout/oscales only; out must be NULL");
+            return SVDQ_E_INVALID;
+        }
+        if (!a.qout || !a.oscales || ((uintptr_t)a.qout & 7) || a.ld_qout % 8 || a.ld_qout < NQ / 2 || a.ld_oscales < a.M) {
             set_error("svdq_gemm_w4a4: qout (8-byte aligned rows) and oscales are required");
             return SVDQ_E_INVALID;
         }
@@ -578,9 +723,6 @@ extern "C" int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream) {
             set_error("svdq_gemm_w4a4: R2=%d must be a multiple of 16 with lora_down_t, lora_act_out and scratch given", a.R2);
             return SVDQ_E_INVALID;
         }
-    } else if (a.epilogue == SVDQ_EPI_SWIGLU_QUANT) {
-        set_error("svdq_gemm_w4a4: the SwiGLU requantizing epilogue is not implemented yet");
-        return SVDQ_E_UNSUPPORTED;
     } else if (a.epilogue != SVDQ_EPI_PLAIN) {
         set_error("svdq_gemm_w4a4: unknown epilogue %d", a.epilogue);
         return SVDQ_E_INVALID;

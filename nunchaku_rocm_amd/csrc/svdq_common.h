@@ -27,11 +27,15 @@ struct BF16 {
     // two packed values: low half / high half of a dword
     __device__ static inline float lo_f32(uint32_t w) { return __uint_as_float(w << 16); }
     __device__ static inline float hi_f32(uint32_t w) { return __uint_as_float(w & 0xFFFF0000u); }
-    __device__ static inline uint16_t from_f32(float f) {  // round to nearest even
-        uint32_t u = __float_as_uint(f);
-        if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40);
-        u += 0x7FFFu + ((u >> 16) & 1u);
-        return (uint16_t)(u >> 16);
+    __device__ static inline uint16_t from_f32(float f) {  // round to nearest even (v_cvt_pk_bf16_f32)
+        const __bf16 b = (__bf16)f;
+        return __builtin_bit_cast(uint16_t, b);
+    }
+    __device__ static inline uint32_t pack(float lo, float hi) {
+        typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+        typedef float f2 __attribute__((ext_vector_type(2)));
+        const f2 v = {lo, hi};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf2));
     }
 };
 
@@ -50,11 +54,17 @@ struct FP16 {
         __builtin_memcpy(&h, &v, 2);
         return h;
     }
+    __device__ static inline uint32_t pack(float lo, float hi) {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        typedef float f2 __attribute__((ext_vector_type(2)));
+        const f2 v = {lo, hi};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, h2));
+    }
 };
 
 template <typename T>
 __device__ inline uint32_t pack2(float a, float b) {
-    return (uint32_t)T::from_f32(a) | ((uint32_t)T::from_f32(b) << 16);
+    return T::pack(a, b);
 }
 
 // MFMA on eight 16-bit values per lane (K = 16 for 32x32, K = 32 for 16x16); operands passed as raw bits.

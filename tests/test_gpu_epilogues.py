@@ -147,3 +147,73 @@ def test_fused_ops_on_flux_block_shapes(dev):
     err = O.max_rel_err(out[rows].cpu(), ref)
     print(f"fused_qkv_norm_rottary max rel err {err:.3e}", flush=True)
     assert err <= TOL
+
+
+@pytest.mark.parametrize("unsigned", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,N,R2", [(144, 256, 48), (64, 512, 32), (128, 128, 0)])
+def test_swiglu_quant_epilogue(dev, M, N, R2, unsigned, dtype):
+    """``wgt`` rows in the 16-interleaved [gate | up] order; the epilogue quantizes silu(gate) * up (signed int4)."""
+    from nunchaku_rocm_amd import ops
+
+    print(f"case M={M} N={N} R2={R2} unsigned={unsigned} {dtype}", flush=True)
+    K, R, H = 256, 16, N // 2
+    p = _problem(M, N, K, R, dtype, seed=N + R2 + 1)  # natural [gate | up] row order
+    g = torch.Generator().manual_seed(97)
+    smooth = (torch.rand(H, generator=g) + 0.5).to(dtype)
+    ld = (torch.randn(H, max(R2, 16), generator=g) * 0.1).to(dtype)[:, :R2].contiguous() if R2 else None
+    idx = O.interleave_swiglu(N)
+    d = lambda t: None if t is None else t.to(dev)  # noqa: E731
+    qout = torch.zeros(M + 16, H // 2, dtype=torch.uint8, device=dev)
+    osc = torch.empty(H // 64, M, dtype=dtype, device=dev)
+    lao = torch.empty(M, R2, dtype=torch.float32, device=dev) if R2 else None
+    ops.svdq_gemm_w4a4_cuda(
+        act=d(p["act"]), wgt=d(p["wgt"][idx].contiguous()), qout=qout, ascales=d(p["asc"]),
+        wscales=d(p["wsc"][:, idx].contiguous()), oscales=osc, lora_act_in=d(p["la"]), lora_up=d(p["lu"][idx].contiguous()),
+        lora_down=d(ld), lora_act_out=lao, bias=d(p["bias"][idx].contiguous()), smooth_factor=d(smooth),
+        act_unsigned=unsigned, fuse_swiglu=True,
+    )  # fmt: skip
+    torch.cuda.synchronize()
+    assert (qout[M:] == 0).all()
+    lin = O.gemm_w4a4(p["act"], p["wgt"], p["asc"], p["wsc"], p["bias"], p["la"], p["lu"], unsigned)
+    rp, rs, rl, rc = O.swiglu_quant(lin[:, idx], smooth, ld, dtype)
+    codes = O.unpack_int4(qout[:M].cpu(), True)
+    diff = (codes - rc).abs()
+    rate = (diff > 0).float().mean().item()
+    print(f"  code mismatch rate {rate:.2e}", flush=True)
+    assert diff.max() <= 1 and rate < 1e-3
+    ulp = 2**-7 if dtype == torch.bfloat16 else 2**-10
+    assert ((osc.cpu().float() - rs.float()).abs() <= rs.float().abs() * ulp + 1e-7).all()
+    if R2:
+        assert (lao.cpu() - rl).abs().max() <= TOL * rl.abs().max()
+
+
+def test_fused_swiglu_mlp(dev):
+    """FLUX.2-style SwiGLU MLP: fc1 (K -> 2H, rows interleaved in place), fused SwiGLU + requantization, fc2 (H -> C)."""
+    from nunchaku_rocm_amd import ops
+    from nunchaku_rocm_amd.linear import SVDQW4A4Linear
+
+    M, C, H = 320, 512, 1024
+
+    def module(K, N, seed):
+        lin = O.make_svdq_linear(K, N, seed=seed)
+        mod = SVDQW4A4Linear(K, N, rank=32, device=dev)
+        with torch.no_grad():
+            for name in ("qweight", "wscales", "smooth_factor", "proj_down", "proj_up", "bias"):
+                getattr(mod, name).copy_(lin[name])
+        return mod, lin
+
+    fc1, l1 = module(C, 2 * H, 51)
+    fc2, l2 = module(H, C, 52)
+    ops.interleave_swiglu_linear_(fc1)
+    x = O.make_activations(M, C, seed=53)
+    y = ops.fused_swiglu_mlp(x.to(dev), fc1, fc2)
+    torch.cuda.synchronize()
+    assert y.shape == (M, C)
+    rp, rs, rl, _ = O.quantize_act(x, l1["proj_down"], l1["smooth_factor"])
+    lin = O.gemm_w4a4(rp, l1["qweight"], rs, l1["wscales"], l1["bias"], rl, l1["proj_up"])  # [gate | up]
+    hp, hs, hl, _ = O.swiglu_quant(lin[:, O.interleave_swiglu(2 * H)], l2["smooth_factor"], l2["proj_down"], torch.bfloat16)
+    ref = O.gemm_w4a4(hp, l2["qweight"], hs, l2["wscales"], l2["bias"], hl, l2["proj_up"])
+    err = O.max_rel_err(y.cpu(), ref)
+    print(f"fused_swiglu_mlp max rel err {err:.3e}", flush=True)
+    assert err <= TOL
