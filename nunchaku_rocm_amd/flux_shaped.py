@@ -1,0 +1,260 @@
+"""FLUX.1-shaped transformer (diffusers-free) wired to the SVDQuant operators.
+
+Same dataflow as the reference's ``NunchakuFluxTransformer2DModelV2`` (nunchaku/models/transformers/
+transformer_flux_v2.py:144-343 blocks, :437-576 forward; nunchaku/models/normalization.py:85-98,155-165 adaLN with
+the interleaved 6-/3-way split and ``scale_shift = 0``; nunchaku/models/attention_processors/flux.py:62-109 attention;
+nunchaku/models/embeddings.py:11-97 rotary table): 19 double-stream + 38 single-stream blocks, hidden 3072, 24 heads
+x 128, MLP 12288, all block linears ``SVDQW4A4Linear`` (fused QKV + RMSNorm + RoPE, fused GELU MLP with unsigned fc2
+activations, plain out-projections) and all modulation linears ``AWQW4A16Linear``.  The sub-modules the reference
+inherits from diffusers (embedders, timestep/pooled-text MLPs, final AdaLayerNormContinuous + projection) are plain
+bf16 torch layers here.  Weights are random-init in the natural layout: there is no checkpoint to load offline.
+
+The quantized operators are reached through a small backend object (default: the HIP operators of this package), so a
+test can run the identical graph on another implementation of the same four operators.
+"""
+
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+
+import torch
+import torch.nn.functional as F
+from torch import nn
+
+from . import ops as _ops
+from .linear import AWQW4A16Linear, SVDQW4A4Linear
+
+
+@dataclass
+class FluxShapedConfig:
+    hidden: int = 3072
+    heads: int = 24
+    head_dim: int = 128
+    mlp: int = 12288
+    in_channels: int = 64
+    text_dim: int = 4096
+    pooled_dim: int = 768
+    n_double: int = 19
+    n_single: int = 38
+    axes_dim: tuple = (16, 56, 56)
+    theta: float = 10000.0
+    rank: int = 32
+
+
+class HipBackend:
+    """The product path: every call lands in ``libsvdq_mi355x.so``."""
+
+    @staticmethod
+    def linear(x, lin: SVDQW4A4Linear):
+        return lin(x)
+
+    @staticmethod
+    def gelu_mlp(x, fc1, fc2):
+        return _ops.fused_gelu_mlp(x, fc1, fc2)
+
+    @staticmethod
+    def qkv(x, proj, norm_q, norm_k, rot):
+        return _ops.fused_qkv_norm_rottary(x, proj, norm_q, norm_k, rot)
+
+    @staticmethod
+    def awq(x, lin: AWQW4A16Linear):
+        return lin(x)
+
+
+def rope_table(ids: torch.Tensor, axes_dim, theta: float) -> torch.Tensor:
+    """(T, n_axes) positions -> (T, sum(axes_dim) / 2, 1, 2) float32 rows of (sin, cos), computed in float64."""
+    out = []
+    for i, d in enumerate(axes_dim):
+        scale = torch.arange(0, d, 2, dtype=torch.float64, device=ids.device) / d
+        ang = ids[:, i].double()[:, None] * (1.0 / (theta**scale))[None, :]
+        out.append(torch.stack([torch.sin(ang), torch.cos(ang)], dim=-1))
+    return torch.cat(out, dim=1).float().unsqueeze(2)
+
+
+def flux_ids(txt_tokens: int, grid_h: int, grid_w: int, device=None) -> torch.Tensor:
+    img = torch.zeros(grid_h, grid_w, 3, device=device)
+    img[..., 1] = torch.arange(grid_h, device=device)[:, None]
+    img[..., 2] = torch.arange(grid_w, device=device)[None, :]
+    return torch.cat([torch.zeros(txt_tokens, 3, device=device), img.reshape(-1, 3)], dim=0)
+
+
+def _timestep_embedding(t: torch.Tensor, dim: int = 256) -> torch.Tensor:
+    half = dim // 2
+    freqs = torch.exp(-math.log(10000.0) * torch.arange(half, dtype=torch.float32, device=t.device) / half)
+    args = (t.float() * 1000.0)[:, None] * freqs[None, :]
+    return torch.cat([torch.cos(args), torch.sin(args)], dim=-1)
+
+
+def _init_svdq(lin: SVDQW4A4Linear, gen: torch.Generator) -> None:
+    """int4 codes uniform in [-8, 7] (uniform random bytes), scales U(0.005, 0.02), smooth U(0.5, 4), LoRA N(0, 0.02),
+    bias N(0, 0.01) -- drawn on the layer's device."""
+    dev, dt = lin.qweight.device, lin.wscales.dtype
+    r = lambda *s: torch.rand(*s, device=dev, generator=gen)  # noqa: E731
+    n = lambda *s: torch.randn(*s, device=dev, generator=gen)  # noqa: E731
+    with torch.no_grad():
+        lin.qweight.copy_(torch.randint(0, 256, lin.qweight.shape, device=dev, generator=gen, dtype=torch.uint8).view(torch.int8))
+        lin.wscales.copy_((r(*lin.wscales.shape) * 0.015 + 0.005).to(dt))
+        lin.smooth_factor.copy_((r(*lin.smooth_factor.shape) * 3.5 + 0.5).to(dt))
+        lin.smooth_factor_orig.copy_(lin.smooth_factor)
+        lin.proj_down.copy_((n(*lin.proj_down.shape) * 0.02).to(dt))
+        lin.proj_up.copy_((n(*lin.proj_up.shape) * 0.02).to(dt))
+        if lin.bias is not None:
+            lin.bias.copy_((n(*lin.bias.shape) * 0.01).to(dt))
+
+
+def _init_awq(lin: AWQW4A16Linear, gen: torch.Generator) -> None:
+    """uint4 codes uniform (uniform random int32 words), scales U(0.005, 0.02), zero-points uniform in [0, 15] stored
+    as ``-zp * s``, bias N(0, 0.01)."""
+    dev, dt = lin.qweight.device, lin.wscales.dtype
+    with torch.no_grad():
+        lin.qweight.copy_(torch.randint(-(2**31), 2**31 - 1, lin.qweight.shape, device=dev, generator=gen, dtype=torch.int64).to(torch.int32))
+        s = (torch.rand(*lin.wscales.shape, device=dev, generator=gen) * 0.015 + 0.005).to(dt)
+        zp = torch.randint(0, 16, lin.wzeros.shape, device=dev, generator=gen).float()
+        lin.wscales.copy_(s)
+        lin.wzeros.copy_((-(zp * s.float())).to(dt))
+        if lin.bias is not None:
+            lin.bias.copy_((torch.randn(*lin.bias.shape, device=dev, generator=gen) * 0.01).to(dt))
+
+
+class _Attention(nn.Module):
+    def __init__(self, cfg: FluxShapedConfig, joint: bool, single: bool, device, dtype):
+        super().__init__()
+        C, kw = cfg.hidden, dict(rank=cfg.rank, torch_dtype=dtype, device=device)
+        self.heads, self.head_dim = cfg.heads, cfg.head_dim
+        self.to_qkv = SVDQW4A4Linear(C, 3 * C, **kw)
+        self.norm_q = nn.RMSNorm(cfg.head_dim, eps=1e-6, device=device, dtype=dtype)
+        self.norm_k = nn.RMSNorm(cfg.head_dim, eps=1e-6, device=device, dtype=dtype)
+        self.to_out = SVDQW4A4Linear(C, C, **kw)
+        if joint:
+            self.add_qkv_proj = SVDQW4A4Linear(C, 3 * C, **kw)
+            self.norm_added_q = nn.RMSNorm(cfg.head_dim, eps=1e-6, device=device, dtype=dtype)
+            self.norm_added_k = nn.RMSNorm(cfg.head_dim, eps=1e-6, device=device, dtype=dtype)
+            self.to_add_out = SVDQW4A4Linear(C, C, **kw)
+        self.joint = joint
+
+    def forward(self, be, x, ctx, rot_img, rot_txt):
+        B = x.shape[0]
+        qkv = be.qkv(x, self.to_qkv, self.norm_q, self.norm_k, rot_img)
+        if self.joint:
+            qkv_ctx = be.qkv(ctx, self.add_qkv_proj, self.norm_added_q, self.norm_added_k, rot_txt)
+            qkv = torch.cat([qkv_ctx, qkv], dim=1)  # token order [txt, img]
+        q, k, v = (t.view(B, -1, self.heads, self.head_dim).transpose(1, 2) for t in qkv.chunk(3, dim=-1))
+        o = F.scaled_dot_product_attention(q, k, v)  # (B, H, T, D), scale D^-0.5, no mask
+        o = o.transpose(1, 2).reshape(B, -1, self.heads * self.head_dim).to(q.dtype)
+        if self.joint:
+            t_txt = ctx.shape[1]
+            return be.linear(o[:, t_txt:].contiguous(), self.to_out), be.linear(o[:, :t_txt].contiguous(), self.to_add_out)
+        return be.linear(o, self.to_out)
+
+
+class _DoubleBlock(nn.Module):
+    def __init__(self, cfg: FluxShapedConfig, device, dtype):
+        super().__init__()
+        C, kw = cfg.hidden, dict(rank=cfg.rank, torch_dtype=dtype, device=device)
+        self.norm1 = AWQW4A16Linear(C, 6 * C, torch_dtype=dtype, device=device)
+        self.norm1_context = AWQW4A16Linear(C, 6 * C, torch_dtype=dtype, device=device)
+        self.attn = _Attention(cfg, joint=True, single=False, device=device, dtype=dtype)
+        self.ff_fc1 = SVDQW4A4Linear(C, cfg.mlp, **kw)
+        self.ff_fc2 = SVDQW4A4Linear(cfg.mlp, C, act_unsigned=True, **kw)
+        self.ffc_fc1 = SVDQW4A4Linear(C, cfg.mlp, **kw)
+        self.ffc_fc2 = SVDQW4A4Linear(cfg.mlp, C, act_unsigned=True, **kw)
+        self.C = C
+
+    @staticmethod
+    def _mod6(be, lin, temb):
+        emb = be.awq(F.silu(temb), lin)
+        return emb.view(emb.shape[0], -1, 6).permute(2, 0, 1)  # interleaved split: channel c -> (c // 6, c % 6)
+
+    def forward(self, be, x, ctx, temb, rot_img, rot_txt):
+        ln = lambda t: F.layer_norm(t, (self.C,), eps=1e-6)  # noqa: E731
+        sh_a, sc_a, g_a, sh_m, sc_m, g_m = self._mod6(be, self.norm1, temb)
+        csh_a, csc_a, cg_a, csh_m, csc_m, cg_m = self._mod6(be, self.norm1_context, temb)
+        nx = ln(x) * sc_a[:, None] + sh_a[:, None]
+        nc = ln(ctx) * csc_a[:, None] + csh_a[:, None]
+        ax, ac = self.attn(be, nx, nc, rot_img, rot_txt)
+        x = x + g_a.unsqueeze(1) * ax
+        x = x + g_m.unsqueeze(1) * be.gelu_mlp(ln(x) * sc_m[:, None] + sh_m[:, None], self.ff_fc1, self.ff_fc2)
+        ctx = ctx + cg_a.unsqueeze(1) * ac
+        ctx = ctx + cg_m.unsqueeze(1) * be.gelu_mlp(ln(ctx) * csc_m[:, None] + csh_m[:, None], self.ffc_fc1, self.ffc_fc2)
+        return ctx, x
+
+
+class _SingleBlock(nn.Module):
+    def __init__(self, cfg: FluxShapedConfig, device, dtype):
+        super().__init__()
+        C, kw = cfg.hidden, dict(rank=cfg.rank, torch_dtype=dtype, device=device)
+        self.norm = AWQW4A16Linear(C, 3 * C, torch_dtype=dtype, device=device)
+        self.mlp_fc1 = SVDQW4A4Linear(C, cfg.mlp, **kw)
+        self.mlp_fc2 = SVDQW4A4Linear(cfg.mlp, C, act_unsigned=True, **kw)
+        self.attn = _Attention(cfg, joint=False, single=True, device=device, dtype=dtype)
+        self.C = C
+
+    def forward(self, be, x, temb, rot):
+        emb = be.awq(F.silu(temb), self.norm)
+        shift, scale, gate = emb.view(emb.shape[0], -1, 3).permute(2, 0, 1)
+        nx = F.layer_norm(x, (self.C,), eps=1e-6) * scale[:, None] + shift[:, None]
+        mlp = be.gelu_mlp(nx, self.mlp_fc1, self.mlp_fc2)
+        att = self.attn(be, nx, None, rot, None)
+        return x + gate.unsqueeze(1) * (att + mlp)
+
+
+class FluxShapedTransformer(nn.Module):
+    def __init__(self, cfg: FluxShapedConfig | None = None, device="cuda", dtype=torch.bfloat16, seed: int = 0, backend=None):
+        super().__init__()
+        self.cfg = cfg = cfg or FluxShapedConfig()
+        self.backend = backend or HipBackend()
+        C = cfg.hidden
+        kw = dict(device=device, dtype=dtype)
+        self.x_embedder = nn.Linear(cfg.in_channels, C, **kw)
+        self.context_embedder = nn.Linear(cfg.text_dim, C, **kw)
+        self.time_in = nn.Sequential(nn.Linear(256, C, **kw), nn.SiLU(), nn.Linear(C, C, **kw))
+        self.pooled_in = nn.Sequential(nn.Linear(cfg.pooled_dim, C, **kw), nn.SiLU(), nn.Linear(C, C, **kw))
+        self.double_blocks = nn.ModuleList([_DoubleBlock(cfg, device, dtype) for _ in range(cfg.n_double)])
+        self.single_blocks = nn.ModuleList([_SingleBlock(cfg, device, dtype) for _ in range(cfg.n_single)])
+        self.norm_out_linear = nn.Linear(C, 2 * C, **kw)
+        self.proj_out = nn.Linear(C, cfg.in_channels, **kw)
+        gen = torch.Generator(device=device).manual_seed(seed)
+        for m in self.modules():
+            if isinstance(m, SVDQW4A4Linear):
+                _init_svdq(m, gen)
+            elif isinstance(m, AWQW4A16Linear):
+                _init_awq(m, gen)
+            elif isinstance(m, nn.Linear):
+                with torch.no_grad():
+                    m.weight.copy_((torch.randn(m.weight.shape, device=device, generator=gen) / math.sqrt(m.in_features)).to(dtype))
+                    m.bias.zero_()
+            elif isinstance(m, nn.RMSNorm):
+                with torch.no_grad():
+                    m.weight.copy_((torch.rand(m.weight.shape, device=device, generator=gen) + 0.5).to(dtype))
+        self.requires_grad_(False)
+
+    @torch.no_grad()
+    def forward(self, latents, text, pooled, timestep, rot, backend=None):
+        """latents (B, T_img, 64), text (B, T_txt, 4096), pooled (B, 768), timestep (B,) in [0, 1], rot the
+        (T_txt + T_img, 64, 1, 2) rotary table (text rows first).  Returns the (B, T_img, 64) velocity."""
+        be = backend or self.backend
+        x = self.x_embedder(latents)
+        ctx = self.context_embedder(text)
+        temb = self.time_in(_timestep_embedding(timestep).to(x.dtype)) + self.pooled_in(pooled)
+        t_txt = ctx.shape[1]
+        rot_txt, rot_img = rot[:t_txt].contiguous(), rot[t_txt:].contiguous()
+        for blk in self.double_blocks:
+            ctx, x = blk(be, x, ctx, temb, rot_img, rot_txt)
+        x = torch.cat([ctx, x], dim=1)
+        for blk in self.single_blocks:
+            x = blk(be, x, temb, rot)
+        x = x[:, t_txt:]
+        scale, shift = self.norm_out_linear(F.silu(temb)).chunk(2, dim=1)
+        x = F.layer_norm(x, (self.cfg.hidden,), eps=1e-6) * (1 + scale)[:, None] + shift[:, None]
+        return self.proj_out(x)
+
+    @torch.no_grad()
+    def denoise(self, latents, text, pooled, rot, steps: int = 4, backend=None):
+        """Euler steps of the rectified flow from t = 1 to t = 0 (FLUX.1-schnell runs 4)."""
+        sig = torch.linspace(1.0, 0.0, steps + 1, device=latents.device)
+        for i in range(steps):
+            t = sig[i].expand(latents.shape[0])
+            v = self.forward(latents, text, pooled, t, rot, backend=backend)
+            latents = (latents.float() + (sig[i + 1] - sig[i]) * v.float()).to(latents.dtype)
+        return latents

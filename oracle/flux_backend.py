@@ -1,0 +1,45 @@
+"""Oracle implementation of the four quantized operators the FLUX.1-shaped harness calls (TEST INFRASTRUCTURE).
+
+Plain torch arithmetic from ``svdq_oracle`` on whatever device the tensors live on, so the same transformer graph can
+be evaluated without the HIP library: on the CPU for small configurations, and with ``dense=True`` (one fp32 matmul
+of dequantised operands per linear) on a GPU's plain torch kernels for the full-size model.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from . import svdq_oracle as O
+
+
+class OracleBackend:
+    def __init__(self, dense: bool = False):
+        self.gemm = O.gemm_w4a4_dense if dense else O.gemm_w4a4
+
+    def _lin32(self, x2d, lin, act_unsigned=False):
+        qx, sc, la, _ = O.quantize_act(x2d, lin.proj_down, lin.smooth_factor)
+        return self.gemm(qx, lin.qweight, sc, lin.wscales, lin.bias, la, lin.proj_up, act_unsigned)
+
+    def linear(self, x, lin):
+        B, S, C = x.shape
+        return self._lin32(x.reshape(B * S, C), lin).to(x.dtype).view(B, S, -1)
+
+    def gelu_mlp(self, x, fc1, fc2):
+        B, S, C = x.shape
+        h = self._lin32(x.reshape(B * S, C), fc1)
+        hp, hs, hl, _ = O.gelu_quant(h, fc2.smooth_factor, fc2.proj_down, x.dtype)
+        y = self.gemm(hp, fc2.qweight, hs, fc2.wscales, fc2.bias, hl, fc2.proj_up, True)
+        return y.to(x.dtype).view(B, S, -1)
+
+    def qkv(self, x, proj, norm_q, norm_k, rot):
+        B, S, C = x.shape
+        lin = self._lin32(x.reshape(B * S, C), proj)
+        out = O.qk_norm_rope(lin, norm_q.weight, norm_k.weight, rot.reshape(B * S, 128))
+        return out.to(x.dtype).view(B, S, -1)
+
+    def awq(self, x, lin):
+        N, K = lin.out_features, lin.in_features
+        y = O.awq_gemv(x, lin.qweight.view(torch.int16).reshape(N // 4, K), lin.wscales, lin.wzeros).to(x.dtype)
+        if lin.bias is not None:
+            y = y + lin.bias
+        return y

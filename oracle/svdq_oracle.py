@@ -123,22 +123,22 @@ def quantize_act(
     lora_act = None
     if lora_down is not None:
         # fp32 accumulation of 16-bit products, K walked in 64-blocks (:1411-1417)
-        lora_act = torch.zeros(M, lora_down.shape[1], dtype=torch.float32)
+        lora_act = torch.zeros(M, lora_down.shape[1], dtype=torch.float32, device=x.device)
         xt = xf.to(T).float()
         ld = lora_down.float()
         for k0 in range(0, K, GROUP):
             lora_act += xt[:, k0 : k0 + GROUP] @ ld[k0 : k0 + GROUP]
-    xf = xf + torch.tensor(shift, dtype=torch.float32)
+    xf = xf + torch.tensor(shift, dtype=torch.float32, device=x.device)
     if smooth is not None:
-        xf = xf * (torch.tensor(1.0, dtype=torch.float32) / smooth.float())[None, :]
+        xf = xf * (torch.tensor(1.0, dtype=torch.float32, device=x.device) / smooth.float())[None, :]
     qmax = 15.0 if unsigned else 7.0
     xg = xf.reshape(M, K // GROUP, GROUP)
     gmax = xg.amax(dim=2) if unsigned else xg.abs().amax(dim=2)
     gmax = torch.clamp_min(gmax, 0.0)
-    scale = gmax / torch.tensor(qmax, dtype=torch.float32)
+    scale = gmax / torch.tensor(qmax, dtype=torch.float32, device=x.device)
     scale_safe = torch.where(scale == 0.0, torch.ones_like(scale), scale)
-    q = xg * (torch.tensor(1.0, dtype=torch.float32) / scale_safe)[:, :, None]
-    magic = torch.tensor(RNE_MAGIC, dtype=torch.float32)
+    q = xg * (torch.tensor(1.0, dtype=torch.float32, device=x.device) / scale_safe)[:, :, None]
+    magic = torch.tensor(RNE_MAGIC, dtype=torch.float32, device=x.device)
     r = (q + magic) - magic
     lo, hi = (0.0, 15.0) if unsigned else (-8.0, 7.0)
     codes = torch.clamp(r, lo, hi).to(torch.int32).reshape(M, K)
@@ -181,13 +181,29 @@ def gemm_w4a4(
     a = unpack_int4(act, not act_unsigned).float()
     w = unpack_int4(wgt, True).float()
     M, N = a.shape[0], w.shape[0]
-    out = torch.zeros(M, N, dtype=torch.float32)
+    out = torch.zeros(M, N, dtype=torch.float32, device=a.device)
     for g in range(a.shape[1] // GROUP):
         sl = slice(g * GROUP, (g + 1) * GROUP)
         out += (a[:, sl] @ w[:, sl].t()) * ascales[g, :M].float()[:, None] * wscales[g, :N].float()[None, :]
     if lora_up is not None and lora_up.shape[1]:
         R = lora_up.shape[1]
         out += lora_act[:M, :R].to(lora_up.dtype).float() @ lora_up[:N].float().t()
+    if bias is not None:
+        out += bias[:N].float()
+    return out
+
+
+def gemm_w4a4_dense(act, wgt, ascales, wscales, bias=None, lora_act=None, lora_up=None, act_unsigned: bool = False):
+    """The same sum written as one fp32 matmul of element-wise dequantised operands (the form the reference's
+    parity tests use, tests/triton/test_w4a4.py:32-60); differs from :func:`gemm_w4a4` only by fp32 rounding order."""
+    K = act.shape[1] * 2
+    grp = torch.arange(K, device=act.device) // GROUP
+    M, N = act.shape[0], wgt.shape[0]
+    a = unpack_int4(act, not act_unsigned).float() * ascales.float()[grp, :M].t()
+    w = unpack_int4(wgt, True).float() * wscales.float()[grp, :N].t()
+    out = a @ w.t()
+    if lora_up is not None and lora_up.shape[1]:
+        out += lora_act[:M, : lora_up.shape[1]].to(lora_up.dtype).float() @ lora_up[:N].float().t()
     if bias is not None:
         out += bias[:N].float()
     return out
@@ -265,8 +281,8 @@ def awq_decode(packed_i16: torch.Tensor, n: int, k: int) -> torch.Tensor:
     nunchaku/ops/triton/awq.py:29-47: logical (n, k) lives in stored int16 column
     ``e = 64*c + 16*(n%4) + d`` of row ``n//4`` with ``t = (k//32)*8 + k%8``, ``c = t//16``,
     ``d = t%16``, at bit ``4*((k%32)//8)``."""
-    nn_ = torch.arange(n).view(-1, 1)
-    kk = torch.arange(k).view(1, -1)
+    nn_ = torch.arange(n, device=packed_i16.device).view(-1, 1)
+    kk = torch.arange(k, device=packed_i16.device).view(1, -1)
     a, b = nn_ // 4, nn_ % 4
     g, m, j = kk // 32, (kk % 32) // 8, kk % 8
     t = g * 8 + j
@@ -282,7 +298,7 @@ def awq_gemv(x: torch.Tensor, packed_i16: torch.Tensor, scales: torch.Tensor, ze
     n = scales.shape[1]
     q = awq_decode(packed_i16, n, k).float()
     xf = x.float()
-    out = torch.zeros(m, n, dtype=torch.float32)
+    out = torch.zeros(m, n, dtype=torch.float32, device=x.device)
     for c in range(k // GROUP):
         sl = slice(c * GROUP, (c + 1) * GROUP)
         dotq = xf[:, sl] @ q[:, sl].t()
