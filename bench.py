@@ -198,6 +198,30 @@ def main():
             kernels[f"awq_gemv_w4a16 M{m} K3072 N18432"] = {"ms": round(ms, 5), "GB/s": round(nbytes / ms / 1e6, 1),
                                                            "frac_hbm": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4), "bytes": nbytes}  # fmt: skip
 
+        # FLUX.1-schnell-shaped transformer, 4 denoising steps at 1024^2 (4096 image + 512 text tokens)
+        from nunchaku_rocm_amd.flux_shaped import FluxShapedConfig, FluxShapedTransformer, flux_ids, rope_table
+
+        del fc1, fc2, q1, a1, l1, qo, oo, lo, y2, aw
+        cfg = FluxShapedConfig()
+        model = FluxShapedTransformer(cfg, device=dev, seed=0)
+        lat = torch.randn(1, 4096, 64, device=dev).to(torch.bfloat16)
+        txt = torch.randn(1, 512, 4096, device=dev).to(torch.bfloat16)
+        pooled = torch.randn(1, 768, device=dev).to(torch.bfloat16)
+        rot = rope_table(flux_ids(512, 64, 64, device=dev), cfg.axes_dim, cfg.theta)
+        model.denoise(lat, txt, pooled, rot, steps=1)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        model.denoise(lat, txt, pooled, rot, steps=4)
+        torch.cuda.synchronize()
+        kernels["flux1_schnell_shaped 19+38 blocks 4608 tokens"] = {"s_per_step": round((time.perf_counter() - t1) / 4, 4), "steps": 4}
+        del model
+        # plain device copy of known size: the scale reference for the FETCH_SIZE / WRITE_SIZE counters
+        src = torch.zeros(64 << 20, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        torch.add(src, 1.0, out=dst)  # one elementwise kernel: reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
+
     result = {
         "metric": "W4A4 GEMM TOPS at the FLUX.1 QKV shape (quantizer + GEMM per step)",
         "value": round(ops_per_gemm / (step_ms * 1e-3) / 1e12, 2),
