@@ -82,6 +82,8 @@ int svdq_transpose_lora_down(const void *lora_down, void *lora_down_t, int32_t K
 typedef struct {
     const void *act;        /* (M, K/2) packed int4, row stride ld_act bytes (multiple of 16, base 16-B aligned) */
     const void *wgt;        /* (N, K/2) packed signed int4, row stride ld_wgt bytes (same alignment)            */
+    const void *wgt_planes; /* optional: the same weights re-laid-out by svdq_split_weight_planes (then `wgt` is  */
+                            /* not read); NULL = unpack `wgt` inside the GEMM                                    */
     const void *ascales;    /* (K/64, >= M) T, group stride ld_ascales elements                                 */
     const void *wscales;    /* (K/64, >= N) T, group stride ld_wscales elements                                 */
     const void *bias;       /* (N,) T or NULL                                                                   */
@@ -112,6 +114,15 @@ typedef struct {
 } svdq_gemm_args;
 
 int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream);
+
+/*
+ * One-time re-layout of a weight for the GEMM: every (32-row block, scale group) becomes two 1 KB int8 planes (even and
+ * odd nibbles, each value times 16) in the order the MFMA lanes read them, so the GEMM streams the weight tile into
+ * LDS without touching it.  `planes` needs svdq_weight_planes_bytes(N, K) bytes (= ceil(N/32)*32 * K).  No
+ * counterpart in the reference (its SwiGLU path re-orders weight rows at load in the same spirit, ops/fused.py:83-105).
+ */
+int svdq_split_weight_planes(const void *wgt, void *planes, int32_t N, int32_t K, int32_t ld_wgt, void *stream);
+size_t svdq_weight_planes_bytes(int32_t N, int32_t K);
 
 /* Bytes of `scratch` needed by a requantizing epilogue with LoRA-down (0 when R2 == 0). */
 size_t svdq_gemm_w4a4_scratch_bytes(int32_t M, int32_t N, int32_t R2, int32_t epilogue);

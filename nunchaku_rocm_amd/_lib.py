@@ -25,6 +25,8 @@ EXPORTS = (
     "svdq_transpose_lora_down",
     "svdq_gemm_w4a4",
     "svdq_gemm_w4a4_scratch_bytes",
+    "svdq_split_weight_planes",
+    "svdq_weight_planes_bytes",
     "svdq_group_acc_i32",
     "svdq_awq_gemv_w4a16",
     "svdq_last_error",
@@ -48,7 +50,7 @@ class GemmArgs(ctypes.Structure):
     """``svdq_gemm_args``"""
 
     _fields_ = (
-        [(n, _vp) for n in ("act", "wgt", "ascales", "wscales", "bias", "lora_act", "lora_up", "out")]
+        [(n, _vp) for n in ("act", "wgt", "wgt_planes", "ascales", "wscales", "bias", "lora_act", "lora_up", "out")]
         + [(n, _i32) for n in ("M", "N", "K", "R", "actual_m", "ld_act", "ld_wgt", "ld_ascales", "ld_wscales",
                                "ld_lora_act", "ld_lora_up", "ld_out", "dtype", "act_unsigned", "epilogue")]
         + [(n, _vp) for n in ("norm_q", "norm_k", "rotary")]
@@ -92,6 +94,9 @@ def load() -> ctypes.CDLL:
     lib.svdq_last_error.restype = ctypes.c_char_p
     lib.svdq_gemm_w4a4_scratch_bytes.restype = ctypes.c_size_t
     lib.svdq_gemm_w4a4_scratch_bytes.argtypes = [_i32, _i32, _i32, _i32]
+    lib.svdq_weight_planes_bytes.restype = ctypes.c_size_t
+    lib.svdq_weight_planes_bytes.argtypes = [_i32, _i32]
+    lib.svdq_split_weight_planes.argtypes = [_vp, _vp, _i32, _i32, _i32, _vp]
     lib.svdq_quantize_act.argtypes = [ctypes.POINTER(QuantizeArgs), _vp]
     lib.svdq_gemm_w4a4.argtypes = [ctypes.POINTER(GemmArgs), _vp]
     lib.svdq_awq_gemv_w4a16.argtypes = [ctypes.POINTER(AwqGemvArgs), _vp]

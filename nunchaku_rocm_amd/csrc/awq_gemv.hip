@@ -16,16 +16,25 @@
 //   s * (D - OFF * xs) + z * xs = s * D + (z - OFF * s) * xs,   xs = sum_{k in c} x[m, k]  (precomputed in LDS).
 // Only accumulator registers whose rows are < M are post-processed (rows m = 8 (i / 4) + 4 h + i % 4).
 //
-// One workgroup = 32 channels x all of K; its four wavefronts take groups round-robin with the weight, scale and
-// zero loads running six groups ahead (half of a wavefront's loads at K = 3072), the activations staged once in LDS
-// (up to 8 rows), and the partial sums added through LDS in a fixed order.
+// One workgroup = 32 channels x all of K; its eight wavefronts take groups round-robin.  The small loads (activations,
+// the channels' scales and zeros) are issued first and staged in LDS while up to six weight loads per lane (all of a
+// wavefront's groups at K = 3072) are in flight; partial sums are added through LDS in a fixed order.
 #include "svdq_common.h"
 
 namespace svdq {
 
-constexpr int AWQ_WAVES = 4;
+#ifndef SVDQ_AWQ_WAVES
+#define SVDQ_AWQ_WAVES 8
+#endif
+#ifndef SVDQ_AWQ_PF
+#define SVDQ_AWQ_PF 6
+#endif
+#ifndef SVDQ_AWQ_NT
+#define SVDQ_AWQ_NT 1
+#endif
+constexpr int AWQ_WAVES = SVDQ_AWQ_WAVES;
 constexpr int AWQ_NB = 32;    // channels per workgroup
-constexpr int AWQ_PF = 6;     // weight loads in flight per lane
+constexpr int AWQ_PF = SVDQ_AWQ_PF;    // weight loads in flight per lane (all of a wavefront's groups at K = 3072)
 constexpr int AWQ_XPAD = 8;   // 16-bit elements of padding per staged activation row
 
 template <typename T>
@@ -46,50 +55,90 @@ __device__ inline int nibble_plane(int w, int sh, uint32_t mask, uint32_t magic)
     return (int)((((uint32_t)w >> sh) & mask) | magic);
 }
 
+__device__ inline v4i awq_wload(const v4i *p) {
+#if SVDQ_AWQ_NT
+    return __builtin_nontemporal_load(p);  // streamed once: do not keep in cache
+#else
+    return *p;
+#endif
+}
+
 template <typename T, int MQ>  // MQ = ceil(M / 8): accumulator register quads that hold real rows
-__global__ __launch_bounds__(AWQ_WAVES * 64, 4) void awq_gemv_kernel(svdq_awq_gemv_args a) {
-    // xs[K/64][8*MQ] fp32 | red[AWQ_WAVES][8*MQ][32] fp32 | (M <= 8 only) x[M][K + pad] 16-bit
+__global__ __launch_bounds__(AWQ_WAVES * 64, AWQ_WAVES >= 16 ? 4 : (AWQ_WAVES >= 8 ? 6 : 4)) void awq_gemv_kernel(svdq_awq_gemv_args a) {
+    // xs[K/64][8*MQ] fp32 | red[AWQ_WAVES][8*MQ][32] fp32 | sz[K/64][2][32] 16-bit | (M <= 8 only) x[M][K + pad] 16-bit
     extern __shared__ __align__(16) float lds[];
     constexpr int MR = 8 * MQ;
     constexpr bool X_IN_LDS = MQ == 1;
     const int ngroups = a.K / GROUP;
     float *xs = lds;
     float *red = lds + (size_t)ngroups * MR;
-    uint16_t *xl = (uint16_t *)(red + AWQ_WAVES * MR * AWQ_NB);
+    uint16_t *sz = (uint16_t *)(red + AWQ_WAVES * MR * AWQ_NB);
+    uint16_t *xl = sz + (size_t)ngroups * 2 * AWQ_NB;
     const int xld = a.K + AWQ_XPAD;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keep it in an SGPR
     const int l32 = lane & 31, half = lane >> 5;
-    const int n = blockIdx.x * AWQ_NB + l32;
+    const int nb0 = blockIdx.x * AWQ_NB;
+    const int n = nb0 + l32;
     const uint16_t *__restrict__ x = (const uint16_t *)a.x;
 
-    // weight / scale / zero streams of this lane: packed row n / 4, int16 column 64 c + 16 (n % 4) + 8 h
+    // 1. the small loads first (activations, scales, zeros), so that waiting for them does not wait for the weights
+    v4i xst[3];  // up to 3 x 16-byte pieces of activations per thread (M * K / 8 <= 3 * 256 covers M = 2 at K = 3072)
+    const int per_row = a.K / 8, xpieces = X_IN_LDS ? a.M * per_row : 0;
+    if (X_IN_LDS) {
+#pragma unroll
+        for (int u = 0; u < 3; u++) {
+            const int p = tid + u * AWQ_WAVES * 64;
+            if (p < xpieces) xst[u] = *(const v4i *)(x + (size_t)(p / per_row) * a.ld_x + 8 * (p % per_row));
+        }
+    }
+    // scales / zeros of the 32 channels: group c, 64 bytes each -> thread (c = p / 4, piece = p % 4)
+    v4i sst[2], zst[2];
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        const int p = tid + u * AWQ_WAVES * 64;
+        if (p < ngroups * 4) {
+            sst[u] = *(const v4i *)((const uint16_t *)a.scales + (size_t)(p >> 2) * a.ld_scales + nb0 + 8 * (p & 3));
+            zst[u] = *(const v4i *)((const uint16_t *)a.zeros + (size_t)(p >> 2) * a.ld_scales + nb0 + 8 * (p & 3));
+        }
+    }
+
+    // 2. this lane's weight stream: packed row n / 4, int16 column 64 c + 16 (n % 4) + 8 h, groups c = wave + 4 i
     const uint16_t *__restrict__ wq =
         (const uint16_t *)a.qweight + (size_t)(n >> 2) * a.K + 16 * (n & 3) + 8 * half + (size_t)wave * GROUP;
-    const uint16_t *__restrict__ sc = (const uint16_t *)a.scales + n + (size_t)wave * a.ld_scales;
-    const uint16_t *__restrict__ zr = (const uint16_t *)a.zeros + n + (size_t)wave * a.ld_scales;
-    const int wstep = AWQ_WAVES * GROUP, sstep = AWQ_WAVES * a.ld_scales;  // per group of this wavefront
-    const int nmy = (ngroups - wave + AWQ_WAVES - 1) / AWQ_WAVES;           // groups c = wave + AWQ_WAVES * i
+    const int wstep = AWQ_WAVES * GROUP;
+    const int nmy = (ngroups - wave + AWQ_WAVES - 1) / AWQ_WAVES;
     v4i wreg[AWQ_PF];
-    uint16_t sreg[AWQ_PF], zreg[AWQ_PF];
 #pragma unroll
     for (int u = 0; u < AWQ_PF; u++)
-        if (u < nmy) {
-            wreg[u] = __builtin_nontemporal_load((const v4i *)(wq + (size_t)u * wstep));
-            sreg[u] = sc[(size_t)u * sstep];
-            zreg[u] = zr[(size_t)u * sstep];
-        }
+        if (u < nmy) wreg[u] = awq_wload((const v4i *)(wq + (size_t)u * wstep));
 
+    // 3. stage the small data in LDS
     if (X_IN_LDS) {
-        // stage the activations once per workgroup (coalesced 16-byte pieces)
-        const int per_row = a.K / 8;
-        for (int p = tid; p < a.M * per_row; p += AWQ_WAVES * 64) {
-            const int m = p / per_row, q = p % per_row;
-            *(v4i *)(xl + m * xld + 8 * q) = *(const v4i *)(x + (size_t)m * a.ld_x + 8 * q);
+#pragma unroll
+        for (int u = 0; u < 3; u++) {
+            const int p = tid + u * AWQ_WAVES * 64;
+            if (p < xpieces) *(v4i *)(xl + (p / per_row) * xld + 8 * (p % per_row)) = xst[u];
         }
-        __syncthreads();
+        for (int p = tid + 3 * AWQ_WAVES * 64; p < xpieces; p += AWQ_WAVES * 64)  // more rows: plain copy loop
+            *(v4i *)(xl + (p / per_row) * xld + 8 * (p % per_row)) = *(const v4i *)(x + (size_t)(p / per_row) * a.ld_x + 8 * (p % per_row));
     }
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        const int p = tid + u * AWQ_WAVES * 64;
+        if (p < ngroups * 4) {
+            *(v4i *)(sz + ((p >> 2) * 2 + 0) * AWQ_NB + 8 * (p & 3)) = sst[u];
+            *(v4i *)(sz + ((p >> 2) * 2 + 1) * AWQ_NB + 8 * (p & 3)) = zst[u];
+        }
+    }
+    for (int p = tid + 2 * AWQ_WAVES * 64; p < ngroups * 4; p += AWQ_WAVES * 64) {  // K > 8192
+        *(v4i *)(sz + ((p >> 2) * 2 + 0) * AWQ_NB + 8 * (p & 3)) =
+            *(const v4i *)((const uint16_t *)a.scales + (size_t)(p >> 2) * a.ld_scales + nb0 + 8 * (p & 3));
+        *(v4i *)(sz + ((p >> 2) * 2 + 1) * AWQ_NB + 8 * (p & 3)) =
+            *(const v4i *)((const uint16_t *)a.zeros + (size_t)(p >> 2) * a.ld_scales + nb0 + 8 * (p & 3));
+    }
+    __syncthreads();
     // xs[c][m] = sum of the group's 64 activations (fp32)
     for (int p = tid; p < ngroups * MR; p += AWQ_WAVES * 64) {
         const int c = p / MR, m = p % MR;
@@ -115,45 +164,47 @@ __global__ __launch_bounds__(AWQ_WAVES * 64, 4) void awq_gemv_kernel(svdq_awq_ge
     const int arow = min(l32, a.M - 1);
     const uint16_t *xrow = (X_IN_LDS ? xl + arow * xld : x + (size_t)arow * a.ld_x) + 32 * half + wave * GROUP;
     const float *xsp = xs + wave * MR + 4 * half;
+    const uint16_t *szp = sz + wave * 2 * AWQ_NB + l32;
     uint32_t mask = 0x000F000Fu;
     asm volatile("" : "+v"(mask));  // keep the mask in a VGPR: v_and_or_b32 takes only one literal
     v16f zero16;
 #pragma unroll
     for (int i = 0; i < 16; i++) zero16[i] = 0.0f;
 
-    for (int base = 0; base < nmy; base += AWQ_PF) {
+    for (int base = 0;;) {
 #pragma unroll
         for (int u = 0; u < AWQ_PF; u++) {
             const int idx = base + u;
-            if (idx >= nmy) break;
-            const v4i w = wreg[u];
-            const float s = T::to_f32(sreg[u]);
-            const float zz = T::to_f32(zreg[u]) - AwqMagic<T>::off * s;
-            if (idx + AWQ_PF < nmy) {
-                wreg[u] = __builtin_nontemporal_load((const v4i *)(wq + (size_t)(idx + AWQ_PF) * wstep));
-                sreg[u] = sc[(size_t)(idx + AWQ_PF) * sstep];
-                zreg[u] = zr[(size_t)(idx + AWQ_PF) * sstep];
-            }
-            const uint16_t *xg = xrow + idx * wstep;
-            v16f d;
+            if (idx < nmy) {
+                const v4i w = wreg[u];
+                const float s = T::to_f32(szp[idx * (AWQ_WAVES * 2 * AWQ_NB)]);
+                const float zz = T::to_f32(szp[idx * (AWQ_WAVES * 2 * AWQ_NB) + AWQ_NB]) - AwqMagic<T>::off * s;
+                const uint16_t *xg = xrow + idx * wstep;
+                v16f d;
 #pragma unroll
-            for (int pl = 0; pl < 4; pl++) {
-                v4i wb;
+                for (int pl = 0; pl < 4; pl++) {
+                    v4i wb;
 #pragma unroll
-                for (int e = 0; e < 4; e++) wb[e] = nibble_plane(w[e], 4 * pl, mask, AwqMagic<T>::bits);
-                const v4i xa = *(const v4i *)(xg + 8 * pl);
-                d = mfma32_16bit<T>(xa, wb, pl == 0 ? zero16 : d);
-            }
+                    for (int e = 0; e < 4; e++) wb[e] = nibble_plane(w[e], 4 * pl, mask, AwqMagic<T>::bits);
+                    const v4i xa = *(const v4i *)(xg + 8 * pl);
+                    d = mfma32_16bit<T>(xa, wb, pl == 0 ? zero16 : d);
+                }
 #pragma unroll
-            for (int q = 0; q < MQ; q++) {
-                const v4f xv = *(const v4f *)(xsp + idx * (AWQ_WAVES * MR) + 8 * q);
+                for (int q = 0; q < MQ; q++) {
+                    const v4f xv = *(const v4f *)(xsp + idx * (AWQ_WAVES * MR) + 8 * q);
 #pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    acc[4 * q + e] = __builtin_fmaf(s, d[4 * q + e], acc[4 * q + e]);
-                    acc[4 * q + e] = __builtin_fmaf(zz, xv[e], acc[4 * q + e]);
+                    for (int e = 0; e < 4; e++) {
+                        acc[4 * q + e] = __builtin_fmaf(s, d[4 * q + e], acc[4 * q + e]);
+                        acc[4 * q + e] = __builtin_fmaf(zz, xv[e], acc[4 * q + e]);
+                    }
                 }
             }
         }
+        base += AWQ_PF;
+        if (base >= nmy) break;
+#pragma unroll
+        for (int u = 0; u < AWQ_PF; u++)  // K > 3072: next batch of this wavefront's groups
+            if (base + u < nmy) wreg[u] = awq_wload((const v4i *)(wq + (size_t)(base + u) * wstep));
     }
 
     // fixed-order sum over the wavefronts, then store T
@@ -167,13 +218,14 @@ __global__ __launch_bounds__(AWQ_WAVES * 64, 4) void awq_gemv_kernel(svdq_awq_ge
         float s = red[(0 * MR + m) * AWQ_NB + nn];
 #pragma unroll
         for (int w = 1; w < AWQ_WAVES; w++) s += red[(w * MR + m) * AWQ_NB + nn];
-        ((uint16_t *)a.out)[(size_t)m * a.ld_out + blockIdx.x * AWQ_NB + nn] = T::from_f32(s);
+        ((uint16_t *)a.out)[(size_t)m * a.ld_out + nb0 + nn] = T::from_f32(s);
     }
 }
 
 static size_t awq_lds_bytes(int K, int M) {
     const int MQ = (M + 7) / 8;
     size_t b = ((size_t)(K / GROUP) * 8 * MQ + (size_t)AWQ_WAVES * 8 * MQ * AWQ_NB) * sizeof(float);
+    b += (size_t)(K / GROUP) * 2 * AWQ_NB * 2;
     if (MQ == 1) b += (size_t)M * (K + AWQ_XPAD) * 2;
     return b;
 }
@@ -214,8 +266,8 @@ extern "C" int svdq_awq_gemv_w4a16(const svdq_awq_gemv_args *args, void *stream)
         return SVDQ_E_INVALID;
     }
     if (((uintptr_t)a.x & 15) || a.ld_x % 8 || a.ld_x < a.K || ((uintptr_t)a.qweight & 15) || a.ld_scales < a.N ||
-        a.ld_out < a.N) {
-        set_error("svdq_awq_gemv_w4a16: x rows and qweight must be 16-byte aligned; leading dimensions >= row length");
+        a.ld_out < a.N || ((uintptr_t)a.scales & 15) || ((uintptr_t)a.zeros & 15) || a.ld_scales % 8) {
+        set_error("svdq_awq_gemv_w4a16: x rows, qweight and scale / zero rows must be 16-byte aligned; leading dimensions >= row length");
         return SVDQ_E_INVALID;
     }
     if (awq_lds_bytes(a.K, a.M) > 65536) {

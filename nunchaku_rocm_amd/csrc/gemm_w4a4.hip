@@ -18,8 +18,11 @@
 //    group absmax, nibble packing, the next layer's LoRA-down B operand) is therefore in-lane plus one exchange with
 //    lane ^ 32.
 //  * 256 threads = 2x2 wavefronts of 64x64 on a 128x128 tile; K is staged through LDS 128 at a time (two scale
-//    groups) with register prefetch of the next stage and two LDS buffers (one barrier per stage).  LDS rows are
-//    padded to 80 bytes so the 16-byte operand reads are bank-conflict free.
+//    groups), two stages.  Operands go global -> LDS directly (global_load_lds_dwordx4, no registers), one stage
+//    ahead, into a lane-linear layout (LDS slot l of a 1 KB block = the 16 bytes MFMA lane l needs), so the operand
+//    reads are bank-conflict free by construction; one raw s_barrier per stage with explicit s_waitcnt.
+//  * Weights can be given pre-split (svdq_split_weight_planes: int8 even / odd planes stored block by block in MFMA
+//    lane order); their half of the unpack then disappears from the inner loop.
 //  * Workgroup ids are first regrouped so that each XCD (ids are dealt round-robin over 8 XCDs) works on a
 //    contiguous range of tiles, then swizzled in bands of m-tiles for L2 reuse of the weight tile.
 #include "svdq_common.h"
@@ -28,16 +31,24 @@ namespace svdq {
 
 constexpr int BM = 128, BN = 128;     // workgroup tile (activation rows x weight rows)
 constexpr int KSTAGE = 128;           // K per LDS stage = two scale groups
-constexpr int LDS_ROW = 80;           // bytes per staged row: 64 data + 16 pad
-constexpr int A_OFF = 0;
-constexpr int W_OFF = BM * LDS_ROW;                       // 10240
-constexpr int AS_OFF = W_OFF + BN * LDS_ROW;              // 20480: float as'[2][BM]
+constexpr int NSTAGE = 2;             // LDS stages: one being computed on, one being filled
+constexpr int BLK_BYTES = 64 * 16;    // one MFMA operand block (32 rows x 16 bytes per lane) of one group, lane-linear
+// stage layout: activation blocks [4 blocks of 32 rows][2 groups] packed (1 KB each), weight blocks
+// [4 blocks][2 groups][2 planes] (pre-split weights) or [4 blocks][2 groups] (packed), then the scales
+constexpr int W_OFF = 4 * 2 * BLK_BYTES;                  // 8192
+constexpr int AS_OFF = W_OFF + 4 * 2 * 2 * BLK_BYTES;     // 24576: float as'[2][BM]
 constexpr int NM_OFF = AS_OFF + 2 * BM * 4;               // float -magic*as'[2][BM]
 constexpr int WS_OFF = NM_OFF + 2 * BM * 4;               // float ws[2][BN]
-constexpr int BUF_BYTES = WS_OFF + 2 * BN * 4;            // 23552
-constexpr int SMEM_BYTES = 2 * BUF_BYTES;                 // 47104
+constexpr int BUF_BYTES = WS_OFF + 2 * BN * 4;            // 27648
+constexpr int SMEM_BYTES = NSTAGE * BUF_BYTES;            // 55296
 constexpr int GROUP_M_TILES = 8;      // m-tiles per raster band
 constexpr int NUM_XCD = 8;
+
+#define SVDQ_AS1 __attribute__((address_space(1)))
+#define SVDQ_AS3 __attribute__((address_space(3)))
+
+// s_waitcnt immediate (gfx9 encoding): vmcnt in bits [3:0] and [15:14], expcnt [6:4] left at 7, lgkmcnt [11:8]
+constexpr int waitcnt_imm(int vm, int lgkm) { return (vm & 0xF) | ((vm >> 4) << 14) | 0x70 | ((lgkm & 0xF) << 8); }
 
 __device__ inline void unpack_signed(v4i p, v4i &even, v4i &odd) {
     even = (p << 4) & (int)0xF0F0F0F0;  // 16 * value in each byte
@@ -76,7 +87,7 @@ __device__ inline void tile_ids(int tiles_m, int tiles_n, int &pid_m, int &pid_n
 #define SVDQ_GEMM_MIN_WAVES 2
 #endif
 
-template <typename T, bool ACT_UNSIGNED, int EPI>
+template <typename T, bool ACT_UNSIGNED, int EPI, bool WPL>
 __global__ __launch_bounds__(256, SVDQ_GEMM_MIN_WAVES) void gemm_w4a4_kernel(svdq_gemm_args a) {
     __shared__ __align__(16) uint8_t smem[SMEM_BYTES];
 
@@ -90,44 +101,63 @@ __global__ __launch_bounds__(256, SVDQ_GEMM_MIN_WAVES) void gemm_w4a4_kernel(svd
     tile_ids((a.M + BM - 1) / BM, (a.N + BN - 1) / BN, pid_m, pid_n);
     const int m0 = pid_m * BM, n0 = pid_n * BN;
 
-    // ---- global -> register staging roles -------------------------------------------------------
-    // 512 16-byte chunks per operand tile and stage: chunk c -> row c / 4, 16-byte column c % 4
-    const uint8_t *gA[2], *gW[2];
-    int sA[2];
+    // ---- operand staging: global -> LDS directly (global_load_lds_dwordx4), one stage ahead ----------------------
+    // A stage holds 1 KB operand blocks (operand, 32-row block, group[, plane]).  Lane l of a block load fetches the
+    // 16 bytes MFMA lane l will read and the hardware writes them to LDS slot l of the block: the layout the operand
+    // read wants, free of bank conflicts by construction.  Packed operands: lane l = (row l % 32, half l / 32) of a
+    // row-major tile.  Pre-split weights are already stored block by block in that order (1 KB contiguous per load).
+    // The 8 activation + (WPL ? 16 : 8) weight block loads of a stage are dealt round-robin to the four wavefronts.
+    constexpr int NLOADS = WPL ? 24 : 16, PER_WAVE = NLOADS / 4;
+    const uint8_t *gsrc[PER_WAVE];
+    int ldst[PER_WAVE], gstep[PER_WAVE];
+    const int G = a.K / GROUP;
 #pragma unroll
-    for (int p = 0; p < 2; p++) {
-        const int c = tid + 256 * p, row = c >> 2, col = c & 3;
-        gA[p] = (const uint8_t *)a.act + (size_t)min(m0 + row, a.M - 1) * a.ld_act + col * 16;
-        gW[p] = (const uint8_t *)a.wgt + (size_t)min(n0 + row, a.N - 1) * a.ld_wgt + col * 16;
-        sA[p] = row * LDS_ROW + col * 16;
+    for (int i = 0; i < PER_WAVE; i++) {
+        const int q = wave * PER_WAVE + i;  // wave-uniform
+        if (q < 8) {                        // activation block q: (blk = q / 2, group q % 2)
+            const int blk = q >> 1, gg = q & 1;
+            gsrc[i] = (const uint8_t *)a.act + (size_t)min(m0 + blk * 32 + l32, a.M - 1) * a.ld_act + gg * 32 + half * 16;
+            ldst[i] = (blk * 2 + gg) * BLK_BYTES;
+            gstep[i] = KSTAGE / 2;
+        } else if (WPL) {                   // weight plane block j: (blk = j / 4, group (j / 2) % 2, plane j % 2)
+            const int j = q - 8, blk = j >> 2, gg = (j >> 1) & 1, pl = j & 1;
+            const int nblk = min(n0 / 32 + blk, (a.N + 31) / 32 - 1);
+            gsrc[i] = (const uint8_t *)a.wgt_planes + ((((size_t)nblk * G + gg) * 2 + pl) * 64 + lane) * 16;
+            ldst[i] = W_OFF + ((blk * 2 + gg) * 2 + pl) * BLK_BYTES;
+            gstep[i] = 2 * 2 * BLK_BYTES;   // two groups x two planes per stage
+        } else {                            // packed weight block j: (blk = j / 2, group j % 2)
+            const int j = q - 8, blk = j >> 1, gg = j & 1;
+            gsrc[i] = (const uint8_t *)a.wgt + (size_t)min(n0 + blk * 32 + l32, a.N - 1) * a.ld_wgt + gg * 32 + half * 16;
+            ldst[i] = W_OFF + (blk * 2 + gg) * BLK_BYTES;
+            gstep[i] = KSTAGE / 2;
+        }
     }
+    auto dma_stage = [&](int s) {
+        uint8_t *dst = smem + (s % NSTAGE) * BUF_BYTES;
+#pragma unroll
+        for (int i = 0; i < PER_WAVE; i++)
+            __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)(gsrc[i] + (size_t)s * gstep[i]),
+                                             (SVDQ_AS3 void *)(dst + ldst[i]), 16, 0, 0);
+    };
+    // scales go through registers (they are converted to fp32 and pre-multiplied on the way), one stage ahead
     const int sg = tid >> 7, sr = tid & 127;  // scale loader: group within stage, row within tile
     const uint16_t *gAS = (const uint16_t *)a.ascales + (size_t)sg * a.ld_ascales + min(m0 + sr, a.M - 1);
     const uint16_t *gWS = (const uint16_t *)a.wscales + (size_t)sg * a.ld_wscales + min(n0 + sr, a.N - 1);
     const float fold = ACT_UNSIGNED ? (1.0f / 16.0f) : (1.0f / 256.0f);
-
-    v4i ra[2], rw[2];
-    uint16_t ras, rws;
-    auto load_stage = [&](int s) {
-#pragma unroll
-        for (int p = 0; p < 2; p++) {
-            ra[p] = *(const v4i *)(gA[p] + (size_t)s * (KSTAGE / 2));
-            rw[p] = *(const v4i *)(gW[p] + (size_t)s * (KSTAGE / 2));
-        }
-        ras = gAS[(size_t)s * 2 * a.ld_ascales];
-        rws = gWS[(size_t)s * 2 * a.ld_wscales];
+    // issued as inline asm so that the compiler does not pair them with a conservative vmcnt(0): the explicit
+    // s_waitcnt at the top of each iteration covers them (they are older than the stage's operand loads)
+    uint32_t ras, rws;
+    auto load_scales = [&](int s) {
+        const uint16_t *pa = gAS + (size_t)s * 2 * a.ld_ascales, *pw = gWS + (size_t)s * 2 * a.ld_wscales;
+        asm volatile("global_load_ushort %0, %1, off" : "=v"(ras) : "v"(pa) : "memory");
+        asm volatile("global_load_ushort %0, %1, off" : "=v"(rws) : "v"(pw) : "memory");
     };
-    auto store_stage = [&](int b) {
-        uint8_t *base = smem + b * BUF_BYTES;
-#pragma unroll
-        for (int p = 0; p < 2; p++) {
-            *(v4i *)(base + A_OFF + sA[p]) = ra[p];
-            *(v4i *)(base + W_OFF + sA[p]) = rw[p];
-        }
-        const float as = T::to_f32(ras) * fold;
+    auto store_scales = [&](int s) {
+        uint8_t *base = smem + (s % NSTAGE) * BUF_BYTES;
+        const float as = T::to_f32((uint16_t)ras) * fold;
         ((float *)(base + AS_OFF))[sg * BM + sr] = as;
         ((float *)(base + NM_OFF))[sg * BM + sr] = -RNE_MAGIC * as;
-        ((float *)(base + WS_OFF))[sg * BN + sr] = T::to_f32(rws);
+        ((float *)(base + WS_OFF))[sg * BN + sr] = T::to_f32((uint16_t)rws);
     };
 
     v16f acc[2][2];
@@ -140,24 +170,36 @@ __global__ __launch_bounds__(256, SVDQ_GEMM_MIN_WAVES) void gemm_w4a4_kernel(svd
 
     const v16i cmagic = magic_acc();
     const int nstages = a.K / KSTAGE;
-    const int rowW = (wn * 64 + l32) * LDS_ROW + half * 16;
-    const int rowA = (wm * 64 + l32) * LDS_ROW + half * 16;
+    const int offW = W_OFF + (wn * 2) * 2 * (WPL ? 2 : 1) * BLK_BYTES + lane * 16;
+    const int offA = (wm * 2) * 2 * BLK_BYTES + lane * 16;
 
-    load_stage(0);
+    load_scales(0);
+    dma_stage(0);
     for (int s = 0; s < nstages; s++) {
-        const int b = s & 1;
-        store_stage(b);
-        __syncthreads();
-        if (s + 1 < nstages) load_stage(s + 1);
-        const uint8_t *base = smem + b * BUF_BYTES;
+        // everything issued for stage s (scale registers, then operand blocks) has landed
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
+        asm volatile("" : "+v"(ras), "+v"(rws));  // the registers are valid from here on
+        store_scales(s);
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));  // scale writes visible before the barrier
+        __builtin_amdgcn_s_barrier();
+        if (s + 1 < nstages) {  // the other buffer was last read in iteration s - 1, before the barrier
+            load_scales(s + 1);
+            dma_stage(s + 1);
+        }
+        const uint8_t *base = smem + (s % NSTAGE) * BUF_BYTES;
 #pragma unroll
         for (int gg = 0; gg < 2; gg++) {
             v4i we[2], wo[2], ae[2], ao[2];
 #pragma unroll
             for (int blk = 0; blk < 2; blk++) {
-                v4i wp = *(const v4i *)(base + W_OFF + rowW + blk * 32 * LDS_ROW + gg * 32);
-                v4i ap = *(const v4i *)(base + A_OFF + rowA + blk * 32 * LDS_ROW + gg * 32);
-                unpack_signed(wp, we[blk], wo[blk]);
+                if (WPL) {
+                    we[blk] = *(const v4i *)(base + offW + ((blk * 2 + gg) * 2 + 0) * BLK_BYTES);
+                    wo[blk] = *(const v4i *)(base + offW + ((blk * 2 + gg) * 2 + 1) * BLK_BYTES);
+                } else {
+                    const v4i wp = *(const v4i *)(base + offW + (blk * 2 + gg) * BLK_BYTES);
+                    unpack_signed(wp, we[blk], wo[blk]);
+                }
+                const v4i ap = *(const v4i *)(base + offA + (blk * 2 + gg) * BLK_BYTES);
                 if (ACT_UNSIGNED)
                     unpack_unsigned(ap, ae[blk], ao[blk]);
                 else
@@ -188,6 +230,7 @@ __global__ __launch_bounds__(256, SVDQ_GEMM_MIN_WAVES) void gemm_w4a4_kernel(svd
             }
         }
     }
+    __syncthreads();  // every wavefront is done with the staging buffers: the epilogues reuse them
 
     // ---- epilogue: LoRA-up and bias ----------------------------------------------------------------
     const int nw0 = n0 + wn * 64, mw0 = m0 + wm * 64;
@@ -610,23 +653,46 @@ __global__ __launch_bounds__(64) void group_acc_kernel(const uint8_t *act, const
     }
 }
 
-template <typename T, bool U>
-static void launch_gemm_epi(const svdq_gemm_args &a, hipStream_t s) {
+template <typename T, bool U, bool WPL>
+static void launch_gemm_epi2(const svdq_gemm_args &a, hipStream_t s) {
     const dim3 grid(((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN)), block(256);
     switch (a.epilogue) {
         case SVDQ_EPI_PLAIN:
-            hipLaunchKernelGGL((gemm_w4a4_kernel<T, U, SVDQ_EPI_PLAIN>), grid, block, 0, s, a);
+            hipLaunchKernelGGL((gemm_w4a4_kernel<T, U, SVDQ_EPI_PLAIN, WPL>), grid, block, 0, s, a);
             break;
         case SVDQ_EPI_QK_NORM_ROPE:
-            hipLaunchKernelGGL((gemm_w4a4_kernel<T, U, SVDQ_EPI_QK_NORM_ROPE>), grid, block, 0, s, a);
+            hipLaunchKernelGGL((gemm_w4a4_kernel<T, U, SVDQ_EPI_QK_NORM_ROPE, WPL>), grid, block, 0, s, a);
             break;
         case SVDQ_EPI_GELU_QUANT:
-            hipLaunchKernelGGL((gemm_w4a4_kernel<T, U, SVDQ_EPI_GELU_QUANT>), grid, block, 0, s, a);
+            hipLaunchKernelGGL((gemm_w4a4_kernel<T, U, SVDQ_EPI_GELU_QUANT, WPL>), grid, block, 0, s, a);
             break;
         case SVDQ_EPI_SWIGLU_QUANT:
-            hipLaunchKernelGGL((gemm_w4a4_kernel<T, U, SVDQ_EPI_SWIGLU_QUANT>), grid, block, 0, s, a);
+            hipLaunchKernelGGL((gemm_w4a4_kernel<T, U, SVDQ_EPI_SWIGLU_QUANT, WPL>), grid, block, 0, s, a);
             break;
     }
+}
+
+template <typename T, bool U>
+static void launch_gemm_epi(const svdq_gemm_args &a, hipStream_t s) {
+    if (a.wgt_planes != nullptr)
+        launch_gemm_epi2<T, U, true>(a, s);
+    else
+        launch_gemm_epi2<T, U, false>(a, s);
+}
+
+// weight re-layout: thread (block of 32 rows, group, lane) splits its 16 packed bytes into the even / odd planes
+__global__ void split_weight_planes_kernel(const uint8_t *wgt, uint8_t *planes, int N, int G, int ld_wgt) {
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int lane = idx & 63;
+    const size_t bg = idx >> 6;  // nblk * G + g
+    const int g = (int)(bg % G), nblk = (int)(bg / G);
+    if (nblk >= (N + 31) / 32) return;
+    const int row = min(nblk * 32 + (lane & 31), N - 1);
+    const v4i p = *(const v4i *)(wgt + (size_t)row * ld_wgt + g * 32 + (lane >> 5) * 16);
+    v4i even, odd;
+    unpack_signed(p, even, odd);
+    *(v4i *)(planes + ((bg * 2 + 0) * 64 + lane) * 16) = even;
+    *(v4i *)(planes + ((bg * 2 + 1) * 64 + lane) * 16) = odd;
 }
 
 }  // namespace svdq
@@ -634,6 +700,23 @@ static void launch_gemm_epi(const svdq_gemm_args &a, hipStream_t s) {
 using namespace svdq;
 
 static bool al16(const void *p) { return ((uintptr_t)p & 15) == 0; }
+
+extern "C" size_t svdq_weight_planes_bytes(int32_t N, int32_t K) {
+    if (N <= 0 || K <= 0) return 0;
+    return (size_t)((N + 31) / 32) * 32 * (size_t)K;
+}
+
+extern "C" int svdq_split_weight_planes(const void *wgt, void *planes, int32_t N, int32_t K, int32_t ld_wgt, void *stream) {
+    if (!wgt || !planes || N <= 0 || K <= 0 || K % GROUP || ld_wgt % 16 || ld_wgt < K / 2 || ((uintptr_t)wgt & 15) ||
+        ((uintptr_t)planes & 15)) {
+        set_error("svdq_split_weight_planes: bad arguments (N=%d K=%d ld_wgt=%d; rows must be 16-byte aligned)", N, K, ld_wgt);
+        return SVDQ_E_INVALID;
+    }
+    const size_t n = (size_t)((N + 31) / 32) * (K / GROUP) * 64;
+    hipLaunchKernelGGL(split_weight_planes_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       (const uint8_t *)wgt, (uint8_t *)planes, N, K / GROUP, ld_wgt);
+    return check_launch("svdq_split_weight_planes");
+}
 
 extern "C" size_t svdq_gemm_w4a4_scratch_bytes(int32_t M, int32_t N, int32_t R2, int32_t epilogue) {
     if (R2 <= 0 || (epilogue != SVDQ_EPI_GELU_QUANT && epilogue != SVDQ_EPI_SWIGLU_QUANT)) return 0;
@@ -656,6 +739,10 @@ extern "C" int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream) {
     }
     if (!a.act || !a.wgt || !a.ascales || !a.wscales) {
         set_error("svdq_gemm_w4a4: act, wgt, ascales and wscales are required");
+        return SVDQ_E_INVALID;
+    }
+    if (a.wgt_planes && !al16(a.wgt_planes)) {
+        set_error("svdq_gemm_w4a4: wgt_planes must be 16-byte aligned");
         return SVDQ_E_INVALID;
     }
     if (!al16(a.act) || !al16(a.wgt) || a.ld_act % 16 || a.ld_wgt % 16 || a.ld_act < a.K / 2 || a.ld_wgt < a.K / 2) {

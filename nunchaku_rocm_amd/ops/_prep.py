@@ -1,4 +1,4 @@
-"""One-time re-layout of LoRA-down weights.
+"""One-time re-layouts of weights.
 
 The kernels read a LoRA-down weight ``(K, R)`` transposed, ``(R, K)``, so that MFMA operands are K-contiguous.  The
 operator signatures take the natural layout (as the reference does), so the transposed copy is made on first use and
@@ -36,6 +36,31 @@ def lora_down_t(lora_down: torch.Tensor) -> torch.Tensor:
     try:
         ref = weakref.ref(lora_down, lambda _r, k=key: _cache.pop(k, None))
         _cache[key] = (ref, lora_down._version, lora_down.data_ptr(), t)
+    except TypeError:
+        pass
+    return t
+
+
+_planes_cache: dict[int, tuple] = {}
+
+
+def weight_planes(qweight: torch.Tensor) -> torch.Tensor:
+    """Even / odd int8 nibble planes of a packed ``(N, K/2)`` weight in MFMA lane order (``svdq_split_weight_planes``),
+    made on first use and kept while the weight tensor lives unmodified.  Costs ``N * K`` bytes (twice the packed
+    weight) and removes the weight half of the nibble unpacking from the GEMM's inner loop."""
+    key = id(qweight)
+    hit = _planes_cache.get(key)
+    if hit is not None:
+        ref, version, data_ptr, t = hit
+        if ref() is qweight and version == qweight._version and data_ptr == qweight.data_ptr():
+            return t
+    N, K = qweight.shape[0], qweight.shape[1] * 2
+    lib = _lib.load()
+    t = torch.empty(lib.svdq_weight_planes_bytes(N, K), dtype=torch.uint8, device=qweight.device)
+    _lib.check(lib.svdq_split_weight_planes(qweight.data_ptr(), t.data_ptr(), N, K, qweight.stride(0), _lib.stream_of(qweight)))
+    try:
+        ref = weakref.ref(qweight, lambda _r, k=key: _planes_cache.pop(k, None))
+        _planes_cache[key] = (ref, qweight._version, qweight.data_ptr(), t)
     except TypeError:
         pass
     return t

@@ -6,6 +6,7 @@ import torch
 
 from .. import _lib
 from ._prep import lora_down_t as _lora_down_t
+from ._prep import weight_planes as _weight_planes
 
 HEAD_DIM = 128
 GELU_SHIFT = 0.171875
@@ -120,9 +121,12 @@ def svdq_gemm_w4a4_cuda(
     if out2d is not None and out2d.stride(1) != 1:
         raise ValueError("out not row-major")
 
+    # module weights (nn.Parameter) get the cached MFMA-ordered plane re-layout; ad-hoc tensors are unpacked in-kernel
+    planes = _weight_planes(wgt) if isinstance(wgt, torch.nn.Parameter) and wgt.stride(0) % 16 == 0 else None
     args = _lib.GemmArgs(
         act=act.data_ptr(),
         wgt=wgt.data_ptr(),
+        wgt_planes=_lib.ptr(planes),
         ascales=ascales.data_ptr(),
         wscales=wscales.data_ptr(),
         bias=_lib.ptr(bias),
@@ -146,7 +150,7 @@ def svdq_gemm_w4a4_cuda(
         epilogue=_lib.EPI_PLAIN,
         eps=1e-6,
     )
-    keep = []  # tensors that must outlive the launch call
+    keep = [planes]  # tensors that must outlive the launch call
     lib = _lib.load()
     if want_qk:
         if rotary_emb.dtype != torch.float32:

@@ -155,3 +155,40 @@ def test_linear_module_matches_dequantised_reference(dev):
     xd = x.view(-1, K).double()
     truth = (xd / lin["smooth_factor"].double()) @ w.t() + (xd @ lin["proj_down"].double()) @ lin["proj_up"].double().t() + lin["bias"].double()
     assert O.cosine(y.view(-1, N), truth) > 0.98
+
+
+def _planes_expected(wgt, N, K):
+    """Host restatement of the pre-split weight layout: [(block of 32 rows, group), plane, lane, 16 bytes], values x16."""
+    nb, G = (N + 31) // 32, K // 64
+    q = O.unpack_int4(wgt, signed=True).to(torch.int16)  # (N, K) in [-8, 7]
+    rows = torch.arange(nb * 32).clamp(max=N - 1)
+    q = q[rows].view(nb, 32, G, 2, 16, 2)  # (nblk, row in block, g, half, byte, even/odd)
+    v = ((q * 16) & 0xFF).to(torch.uint8)
+    # lane = half * 32 + row
+    return v.permute(0, 2, 5, 3, 1, 4).reshape(nb, G, 2, 64, 16).contiguous()
+
+
+@pytest.mark.parametrize("N,K", [(32, 64), (264, 256), (100, 128)])
+def test_weight_planes_layout(dev, N, K):
+    from nunchaku_rocm_amd.ops._prep import weight_planes
+
+    wgt = torch.randint(0, 256, (N, K // 2), generator=torch.Generator().manual_seed(N), dtype=torch.uint8)
+    got = weight_planes(wgt.to(dev)).cpu()
+    exp = _planes_expected(wgt, N, K)
+    assert got.numel() == exp.numel()
+    assert torch.equal(got.view(-1), exp.view(-1))
+
+
+@pytest.mark.parametrize("unsigned", [False, True])
+@pytest.mark.parametrize("M,N,K,R", [(136, 264, 256, 16), (256, 512, 1024, 32), (64, 72, 128, 0), (300, 3072, 3072, 32)])
+def test_presplit_weights_same_bits_as_packed(dev, M, N, K, R, unsigned):
+    """The GEMM gives identical bits whether it unpacks the weights itself or reads the pre-split planes."""
+    print(f"case M={M} N={N} K={K} R={R} unsigned={unsigned}", flush=True)
+    p = _rand_problem(M, N, K, R, torch.bfloat16, seed=7 + M)
+    packed = _gpu_gemm(p, dev, unsigned=unsigned)
+    q = dict(p)
+    q["wgt"] = torch.nn.Parameter(p["wgt"].to(dev), requires_grad=False)  # parameters take the cached pre-split path
+    split = _gpu_gemm(q, dev, unsigned=unsigned)
+    assert torch.equal(packed.view(torch.int16), split.view(torch.int16))
+    ref = O.gemm_w4a4(p["act"], p["wgt"], p["asc"], p["wsc"], bias=p["bias"], lora_act=p["la"], lora_up=p["lu"], act_unsigned=unsigned)
+    assert O.max_rel_err(split.float(), ref) <= TOL
