@@ -17,7 +17,9 @@
 //    row m and its registers walk n in runs of four.  Row-wise epilogue work (RMSNorm sum of squares, RoPE pairs,
 //    group absmax, nibble packing, the next layer's LoRA-down B operand) is therefore in-lane plus one exchange with
 //    lane ^ 32.
-//  * 256 threads = 2x2 wavefronts of 64x64 on a 128x128 tile; K is staged through LDS 128 at a time (two scale
+//  * 512 threads = 2 (n) x 4 (m) wavefronts of 64 weight rows x 32 activation rows on a 128x128 tile, two workgroups
+//    per CU = four wavefronts per SIMD: at half that occupancy the loop runs at about half the speed, its waits
+//    (LDS, MFMA results, barrier) exposed. K is staged through LDS 128 at a time (two scale
 //    groups), two stages.  Operands go global -> LDS directly (global_load_lds_dwordx4, no registers), one stage
 //    ahead, into a lane-linear layout (LDS slot l of a 1 KB block = the 16 bytes MFMA lane l needs), so the operand
 //    reads are bank-conflict free by construction; one raw s_barrier per stage with explicit s_waitcnt.
@@ -25,6 +27,8 @@
 //    lane order); their half of the unpack then disappears from the inner loop.
 //  * Workgroup ids are first regrouped so that each XCD (ids are dealt round-robin over 8 XCDs) works on a
 //    contiguous range of tiles, then swizzled in bands of m-tiles for L2 reuse of the weight tile.
+#include <type_traits>
+
 #include "svdq_common.h"
 
 namespace svdq {
@@ -41,6 +45,8 @@ constexpr int NM_OFF = AS_OFF + 2 * BM * 4;               // float -magic*as'[2]
 constexpr int WS_OFF = NM_OFF + 2 * BM * 4;               // float ws[2][BN]
 constexpr int BUF_BYTES = WS_OFF + 2 * BN * 4;            // 27648
 constexpr int SMEM_BYTES = NSTAGE * BUF_BYTES;            // 55296
+constexpr int NWAVES = 8, NTHREADS = NWAVES * 64;  // 2 wavefronts along n x 4 along m
+constexpr int NBM = 1, WROWS = NBM * 32;            // activation rows per wavefront (its 64 weight rows are 2 blocks)
 constexpr int GROUP_M_TILES = 8;      // m-tiles per raster band
 constexpr int NUM_XCD = 8;
 
@@ -83,18 +89,14 @@ __device__ inline void tile_ids(int tiles_m, int tiles_n, int &pid_m, int &pid_n
     pid_n = (id % band) / gm;
 }
 
-#ifndef SVDQ_GEMM_MIN_WAVES
-#define SVDQ_GEMM_MIN_WAVES 2
-#endif
-
 template <typename T, bool ACT_UNSIGNED, int EPI, bool WPL>
-__global__ __launch_bounds__(256, SVDQ_GEMM_MIN_WAVES) void gemm_w4a4_kernel(svdq_gemm_args a) {
+__global__ __launch_bounds__(NTHREADS, 4) void gemm_w4a4_kernel(svdq_gemm_args a) {
     __shared__ __align__(16) uint8_t smem[SMEM_BYTES];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keep it in an SGPR
-    const int wn = wave & 1, wm = wave >> 1;  // wavefront position in the 2x2 arrangement
+    const int wn = wave & 1, wm = wave >> 1;  // wavefront position: 2 along n (64 columns each) x 4 along m (32 rows each)
     const int l32 = lane & 31, half = lane >> 5;
 
     int pid_m, pid_n;
@@ -106,9 +108,11 @@ __global__ __launch_bounds__(256, SVDQ_GEMM_MIN_WAVES) void gemm_w4a4_kernel(svd
     // 16 bytes MFMA lane l will read and the hardware writes them to LDS slot l of the block: the layout the operand
     // read wants, free of bank conflicts by construction.  Packed operands: lane l = (row l % 32, half l / 32) of a
     // row-major tile.  Pre-split weights are already stored block by block in that order (1 KB contiguous per load).
-    // The 8 activation + (WPL ? 16 : 8) weight block loads of a stage are dealt round-robin to the four wavefronts.
-    constexpr int NLOADS = WPL ? 24 : 16, PER_WAVE = NLOADS / 4;
-    const uint8_t *gsrc[PER_WAVE];
+    // The 8 activation + (WPL ? 16 : 8) weight block loads of a stage are dealt in runs to the eight wavefronts.
+    constexpr int NLOADS = WPL ? 24 : 16, PER_WAVE = NLOADS / NWAVES;
+    // each load's address = wave-uniform base (SGPRs) + a 32-bit offset (lane part + stage * step; operands < 4 GiB)
+    const uint8_t *gbase[PER_WAVE];
+    uint32_t goff[PER_WAVE];
     int ldst[PER_WAVE], gstep[PER_WAVE];
     const int G = a.K / GROUP;
 #pragma unroll
@@ -116,80 +120,96 @@ __global__ __launch_bounds__(256, SVDQ_GEMM_MIN_WAVES) void gemm_w4a4_kernel(svd
         const int q = wave * PER_WAVE + i;  // wave-uniform
         if (q < 8) {                        // activation block q: (blk = q / 2, group q % 2)
             const int blk = q >> 1, gg = q & 1;
-            gsrc[i] = (const uint8_t *)a.act + (size_t)min(m0 + blk * 32 + l32, a.M - 1) * a.ld_act + gg * 32 + half * 16;
+            gbase[i] = (const uint8_t *)a.act + (size_t)m0 * a.ld_act + gg * 32;
+            goff[i] = (uint32_t)(min(m0 + blk * 32 + l32, a.M - 1) - m0) * (uint32_t)a.ld_act + half * 16;
             ldst[i] = (blk * 2 + gg) * BLK_BYTES;
             gstep[i] = KSTAGE / 2;
         } else if (WPL) {                   // weight plane block j: (blk = j / 4, group (j / 2) % 2, plane j % 2)
             const int j = q - 8, blk = j >> 2, gg = (j >> 1) & 1, pl = j & 1;
             const int nblk = min(n0 / 32 + blk, (a.N + 31) / 32 - 1);
-            gsrc[i] = (const uint8_t *)a.wgt_planes + ((((size_t)nblk * G + gg) * 2 + pl) * 64 + lane) * 16;
+            gbase[i] = (const uint8_t *)a.wgt_planes + (((size_t)nblk * G + gg) * 2 + pl) * BLK_BYTES;
+            goff[i] = lane * 16;
             ldst[i] = W_OFF + ((blk * 2 + gg) * 2 + pl) * BLK_BYTES;
             gstep[i] = 2 * 2 * BLK_BYTES;   // two groups x two planes per stage
         } else {                            // packed weight block j: (blk = j / 2, group j % 2)
             const int j = q - 8, blk = j >> 1, gg = j & 1;
-            gsrc[i] = (const uint8_t *)a.wgt + (size_t)min(n0 + blk * 32 + l32, a.N - 1) * a.ld_wgt + gg * 32 + half * 16;
+            gbase[i] = (const uint8_t *)a.wgt + (size_t)n0 * a.ld_wgt + gg * 32;
+            goff[i] = (uint32_t)(min(n0 + blk * 32 + l32, a.N - 1) - n0) * (uint32_t)a.ld_wgt + half * 16;
             ldst[i] = W_OFF + (blk * 2 + gg) * BLK_BYTES;
             gstep[i] = KSTAGE / 2;
         }
     }
+    auto dma_one = [&](int s, int buf, int i) {  // block load i of stage s into staging buffer buf
+        // pre-split weights: SGPR base + 32-bit offset; the packed path has the registers for neither form to spare
+        // and fares better with a 64-bit address
+        const uint8_t *src = WPL ? gbase[i] + (goff[i] + (uint32_t)s * (uint32_t)gstep[i])
+                                 : gbase[i] + (size_t)s * gstep[i] + goff[i];
+        __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)src, (SVDQ_AS3 void *)(smem + buf * BUF_BYTES + ldst[i]),
+                                         16, 0, 0);
+    };
     auto dma_stage = [&](int s) {
-        uint8_t *dst = smem + (s % NSTAGE) * BUF_BYTES;
 #pragma unroll
-        for (int i = 0; i < PER_WAVE; i++)
-            __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)(gsrc[i] + (size_t)s * gstep[i]),
-                                             (SVDQ_AS3 void *)(dst + ldst[i]), 16, 0, 0);
+        for (int i = 0; i < PER_WAVE; i++) dma_one(s, s % NSTAGE, i);
     };
     // scales go through registers (they are converted to fp32 and pre-multiplied on the way), one stage ahead
-    const int sg = tid >> 7, sr = tid & 127;  // scale loader: group within stage, row within tile
-    const uint16_t *gAS = (const uint16_t *)a.ascales + (size_t)sg * a.ld_ascales + min(m0 + sr, a.M - 1);
-    const uint16_t *gWS = (const uint16_t *)a.wscales + (size_t)sg * a.ld_wscales + min(n0 + sr, a.N - 1);
+    // wavefronts 0-3 fetch the activation scales of the stage (2 groups x 128 rows), wavefronts 4-7 the weight scales
+    const int sg = (tid >> 7) & 1, sr = tid & 127;  // scale loader: group within stage, row within tile
+    const bool loads_as = wave < 4;                 // wave-uniform
+    const int sgu = __builtin_amdgcn_readfirstlane(sg);
+    const uint16_t *gSC = loads_as ? (const uint16_t *)a.ascales + (size_t)sgu * a.ld_ascales + m0
+                                   : (const uint16_t *)a.wscales + (size_t)sgu * a.ld_wscales + n0;  // wave-uniform
+    const uint32_t sc_off = 2 * (uint32_t)(loads_as ? min(m0 + sr, a.M - 1) - m0 : min(n0 + sr, a.N - 1) - n0);
+    const uint32_t sc_step = 4 * (uint32_t)(loads_as ? a.ld_ascales : a.ld_wscales);  // bytes per stage (two groups)
     const float fold = ACT_UNSIGNED ? (1.0f / 16.0f) : (1.0f / 256.0f);
-    // issued as inline asm so that the compiler does not pair them with a conservative vmcnt(0): the explicit
-    // s_waitcnt at the top of each iteration covers them (they are older than the stage's operand loads)
-    uint32_t ras, rws;
+    // a plain load: its first use is the conversion at the top of the next stage, behind that stage's vmcnt(0)
+    uint16_t rsc;
     auto load_scales = [&](int s) {
-        const uint16_t *pa = gAS + (size_t)s * 2 * a.ld_ascales, *pw = gWS + (size_t)s * 2 * a.ld_wscales;
-        asm volatile("global_load_ushort %0, %1, off" : "=v"(ras) : "v"(pa) : "memory");
-        asm volatile("global_load_ushort %0, %1, off" : "=v"(rws) : "v"(pw) : "memory");
+        rsc = *(const uint16_t *)((const uint8_t *)gSC + (sc_off + (uint32_t)s * (uint32_t)sc_step));
     };
     auto store_scales = [&](int s) {
         uint8_t *base = smem + (s % NSTAGE) * BUF_BYTES;
-        const float as = T::to_f32((uint16_t)ras) * fold;
-        ((float *)(base + AS_OFF))[sg * BM + sr] = as;
-        ((float *)(base + NM_OFF))[sg * BM + sr] = -RNE_MAGIC * as;
-        ((float *)(base + WS_OFF))[sg * BN + sr] = T::to_f32((uint16_t)rws);
+        const float v = T::to_f32(rsc);
+        if (loads_as) {
+            ((float *)(base + AS_OFF))[sg * BM + sr] = v * fold;
+            ((float *)(base + NM_OFF))[sg * BM + sr] = -RNE_MAGIC * (v * fold);
+        } else {
+            ((float *)(base + WS_OFF))[sg * BN + sr] = v;
+        }
     };
 
-    v16f acc[2][2];
+    v16f acc[2][NBM];
 #pragma unroll
     for (int bn = 0; bn < 2; bn++)
 #pragma unroll
-        for (int bm = 0; bm < 2; bm++)
+        for (int bm = 0; bm < NBM; bm++)
 #pragma unroll
             for (int i = 0; i < 16; i++) acc[bn][bm][i] = 0.0f;
 
     const v16i cmagic = magic_acc();
     const int nstages = a.K / KSTAGE;
     const int offW = W_OFF + (wn * 2) * 2 * (WPL ? 2 : 1) * BLK_BYTES + lane * 16;
-    const int offA = (wm * 2) * 2 * BLK_BYTES + lane * 16;
+    const int offA = (wm * NBM) * 2 * BLK_BYTES + lane * 16;
 
     load_scales(0);
     dma_stage(0);
+    // One copy of the loop per position (0..3) at which the wavefront issues its loads within a stage: the four
+    // wavefronts that share a SIMD take different positions, so that one of them at a time waits for room in the
+    // memory pipeline while the others compute.  (A run-time test of the position inside one loop costs registers.)
+    auto main_loop = [&](auto pos_tag) {
+    constexpr int POS = decltype(pos_tag)::value;
     for (int s = 0; s < nstages; s++) {
         // everything issued for stage s (scale registers, then operand blocks) has landed
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
-        asm volatile("" : "+v"(ras), "+v"(rws));  // the registers are valid from here on
         store_scales(s);
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));  // scale writes visible before the barrier
         __builtin_amdgcn_s_barrier();
-        if (s + 1 < nstages) {  // the other buffer was last read in iteration s - 1, before the barrier
-            load_scales(s + 1);
-            dma_stage(s + 1);
-        }
+        // The other buffer was last read in iteration s - 1, before the barrier: refill it during this stage.  The last
+        // stage re-fetches itself into the idle buffer (harmless, and keeps the stage one basic block).
+        const int sn = min(s + 1, nstages - 1);
         const uint8_t *base = smem + (s % NSTAGE) * BUF_BYTES;
 #pragma unroll
         for (int gg = 0; gg < 2; gg++) {
-            v4i we[2], wo[2], ae[2], ao[2];
+            v4i we[2], wo[2], ae[NBM], ao[NBM];
 #pragma unroll
             for (int blk = 0; blk < 2; blk++) {
                 if (WPL) {
@@ -199,26 +219,34 @@ __global__ __launch_bounds__(256, SVDQ_GEMM_MIN_WAVES) void gemm_w4a4_kernel(svd
                     const v4i wp = *(const v4i *)(base + offW + (blk * 2 + gg) * BLK_BYTES);
                     unpack_signed(wp, we[blk], wo[blk]);
                 }
+            }
+#pragma unroll
+            for (int blk = 0; blk < NBM; blk++) {
                 const v4i ap = *(const v4i *)(base + offA + (blk * 2 + gg) * BLK_BYTES);
                 if (ACT_UNSIGNED)
                     unpack_unsigned(ap, ae[blk], ao[blk]);
                 else
                     unpack_signed(ap, ae[blk], ao[blk]);
             }
-            float asl[2], nml[2];
+            float asl[NBM], nml[NBM];
 #pragma unroll
-            for (int bm = 0; bm < 2; bm++) {
-                asl[bm] = ((const float *)(base + AS_OFF))[gg * BM + wm * 64 + bm * 32 + l32];
-                nml[bm] = ((const float *)(base + NM_OFF))[gg * BM + wm * 64 + bm * 32 + l32];
+            for (int bm = 0; bm < NBM; bm++) {
+                asl[bm] = ((const float *)(base + AS_OFF))[gg * BM + wm * WROWS + bm * 32 + l32];
+                nml[bm] = ((const float *)(base + NM_OFF))[gg * BM + wm * WROWS + bm * 32 + l32];
             }
 #pragma unroll
             for (int bn = 0; bn < 2; bn++) {
+                if (POS == gg * 2 + bn) {
+                    load_scales(sn);
+#pragma unroll
+                    for (int i = 0; i < PER_WAVE; i++) dma_one(sn, (s + 1) % NSTAGE, i);
+                }
                 v4f wsr[4];
 #pragma unroll
                 for (int j = 0; j < 4; j++)
                     wsr[j] = *(const v4f *)((const float *)(base + WS_OFF) + gg * BN + wn * 64 + bn * 32 + 8 * j + 4 * half);
 #pragma unroll
-                for (int bm = 0; bm < 2; bm++) {
+                for (int bm = 0; bm < NBM; bm++) {
                     v16i t = __builtin_amdgcn_mfma_i32_32x32x32_i8(we[bn], ae[bm], cmagic, 0, 0, 0);
                     t = __builtin_amdgcn_mfma_i32_32x32x32_i8(wo[bn], ao[bm], t, 0, 0, 0);
 #pragma unroll
@@ -230,20 +258,32 @@ __global__ __launch_bounds__(256, SVDQ_GEMM_MIN_WAVES) void gemm_w4a4_kernel(svd
             }
         }
     }
+    };
+    switch (wm) {  // wave-uniform
+        case 0: main_loop(std::integral_constant<int, 0>{}); break;
+        case 1: main_loop(std::integral_constant<int, 1>{}); break;
+        case 2: main_loop(std::integral_constant<int, 2>{}); break;
+        default: main_loop(std::integral_constant<int, 3>{}); break;
+    }
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));  // the last stage's (redundant) block loads have landed
     __syncthreads();  // every wavefront is done with the staging buffers: the epilogues reuse them
 
     // ---- epilogue: LoRA-up and bias ----------------------------------------------------------------
-    const int nw0 = n0 + wn * 64, mw0 = m0 + wm * 64;
+    const int nw0 = n0 + wn * 64, mw0 = m0 + wm * WROWS;
     if (a.R > 0) {
         const uint16_t *lu = (const uint16_t *)a.lora_up;
         for (int r0 = 0; r0 < a.R; r0 += 16) {
-            v4i ua[2], ub[2];
+            v4i ua[2], ub[NBM];
 #pragma unroll
             for (int blk = 0; blk < 2; blk++) {
-                const int n = nw0 + blk * 32 + l32, m = mw0 + blk * 32 + l32;
+                const int n = nw0 + blk * 32 + l32;
                 ua[blk] = (v4i){0, 0, 0, 0};
-                ub[blk] = (v4i){0, 0, 0, 0};
                 if (n < a.N) ua[blk] = *(const v4i *)(lu + (size_t)n * a.ld_lora_up + r0 + half * 8);
+            }
+#pragma unroll
+            for (int blk = 0; blk < NBM; blk++) {
+                const int m = mw0 + blk * 32 + l32;
+                ub[blk] = (v4i){0, 0, 0, 0};
                 if (m < a.M) {
                     const float *lp = a.lora_act + (size_t)m * a.ld_lora_act + r0 + half * 8;
                     const v4f f0 = *(const v4f *)lp, f1 = *(const v4f *)(lp + 4);
@@ -256,7 +296,7 @@ __global__ __launch_bounds__(256, SVDQ_GEMM_MIN_WAVES) void gemm_w4a4_kernel(svd
 #pragma unroll
             for (int bn = 0; bn < 2; bn++)
 #pragma unroll
-                for (int bm = 0; bm < 2; bm++) acc[bn][bm] = mfma32_16bit<T>(ua[bn], ub[bm], acc[bn][bm]);
+                for (int bm = 0; bm < NBM; bm++) acc[bn][bm] = mfma32_16bit<T>(ua[bn], ub[bm], acc[bn][bm]);
         }
     }
     if (a.bias != nullptr) {
@@ -270,7 +310,7 @@ __global__ __launch_bounds__(256, SVDQ_GEMM_MIN_WAVES) void gemm_w4a4_kernel(svd
                     const uint2 bb = *(const uint2 *)(bias + n);
                     const float b0 = T::lo_f32(bb.x), b1 = T::hi_f32(bb.x), b2 = T::lo_f32(bb.y), b3 = T::hi_f32(bb.y);
 #pragma unroll
-                    for (int bm = 0; bm < 2; bm++) {
+                    for (int bm = 0; bm < NBM; bm++) {
                         acc[bn][bm][4 * j + 0] += b0;
                         acc[bn][bm][4 * j + 1] += b1;
                         acc[bn][bm][4 * j + 2] += b2;
@@ -283,7 +323,7 @@ __global__ __launch_bounds__(256, SVDQ_GEMM_MIN_WAVES) void gemm_w4a4_kernel(svd
     auto store_out = [&]() {
         uint16_t *out = (uint16_t *)a.out;
 #pragma unroll
-        for (int bm = 0; bm < 2; bm++) {
+        for (int bm = 0; bm < NBM; bm++) {
             const int m = mw0 + bm * 32 + l32;
             if (m >= a.actual_m) continue;
 #pragma unroll
@@ -313,20 +353,20 @@ __global__ __launch_bounds__(256, SVDQ_GEMM_MIN_WAVES) void gemm_w4a4_kernel(svd
             float *red = (float *)smem;  // [2 (wn)][BM]
             __syncthreads();             // main-loop LDS reads are done
 #pragma unroll
-            for (int bm = 0; bm < 2; bm++) {
+            for (int bm = 0; bm < NBM; bm++) {
                 float ss = 0.0f;
 #pragma unroll
                 for (int bn = 0; bn < 2; bn++)
 #pragma unroll
                     for (int i = 0; i < 16; i++) ss += acc[bn][bm][i] * acc[bn][bm][i];
                 ss += __shfl_xor(ss, 32);
-                if (half == 0) red[wn * BM + wm * 64 + bm * 32 + l32] = ss;
+                if (half == 0) red[wn * BM + wm * WROWS + bm * 32 + l32] = ss;
             }
             __syncthreads();
             const uint16_t *nw = (const uint16_t *)(part == 0 ? a.norm_q : a.norm_k);
 #pragma unroll
-            for (int bm = 0; bm < 2; bm++) {
-                const int ml = wm * 64 + bm * 32 + l32;
+            for (int bm = 0; bm < NBM; bm++) {
+                const int ml = wm * WROWS + bm * 32 + l32;
                 const int m = m0 + ml;
                 const float tot = red[ml] + red[BM + ml];
                 const float rstd = 1.0f / sqrtf(tot / 128.0f + a.eps);
@@ -357,21 +397,21 @@ __global__ __launch_bounds__(256, SVDQ_GEMM_MIN_WAVES) void gemm_w4a4_kernel(svd
     if (EPI == SVDQ_EPI_GELU_QUANT) {
         if (a.out != nullptr) store_out();  // pre-GELU output, when asked for
         const uint16_t *ldt = (const uint16_t *)a.lora_down_t;
-        float *lds_part = (float *)smem;  // [2 (wm)][2 (bm)][16 regs][64 lanes] floats = 16 KB
+        float *lds_part = (float *)smem;  // [4 (wm)][16 regs][64 lanes] floats = 16 KB
         __syncthreads();
 #pragma unroll
         for (int bn = 0; bn < 2; bn++)
 #pragma unroll
-            for (int bm = 0; bm < 2; bm++)
+            for (int bm = 0; bm < NBM; bm++)
 #pragma unroll
                 for (int i = 0; i < 16; i++) acc[bn][bm][i] = gelu_tanh(acc[bn][bm][i]);
 
         // next layer's LoRA-down on the un-shifted, un-smoothed GELU output rounded to T:
         // D[r][m] = sum_n ldT[r][n] * x[n][m]; registers [8 s, 8 s + 8) of a block are one MFMA's B operand
         for (int rc = 0; rc < a.R2; rc += 32) {
-            v16f d[2];
+            v16f d[NBM];
 #pragma unroll
-            for (int bm = 0; bm < 2; bm++)
+            for (int bm = 0; bm < NBM; bm++)
 #pragma unroll
                 for (int i = 0; i < 16; i++) d[bm][i] = 0.0f;
             const int r = rc + l32;
@@ -386,7 +426,7 @@ __global__ __launch_bounds__(256, SVDQ_GEMM_MIN_WAVES) void gemm_w4a4_kernel(svd
                         la = (v4i){(int)q0.x, (int)q0.y, (int)q1.x, (int)q1.y};
                     }
 #pragma unroll
-                    for (int bm = 0; bm < 2; bm++) {
+                    for (int bm = 0; bm < NBM; bm++) {
                         v4i xb;
 #pragma unroll
                         for (int e = 0; e < 4; e++)
@@ -397,21 +437,21 @@ __global__ __launch_bounds__(256, SVDQ_GEMM_MIN_WAVES) void gemm_w4a4_kernel(svd
             // add the two n-wavefronts in a fixed order (wn = 0 first), then one partial per n-tile
             if (wn == 1) {
 #pragma unroll
-                for (int bm = 0; bm < 2; bm++)
+                for (int bm = 0; bm < NBM; bm++)
 #pragma unroll
-                    for (int i = 0; i < 16; i++) lds_part[((wm * 2 + bm) * 16 + i) * 64 + lane] = d[bm][i];
+                    for (int i = 0; i < 16; i++) lds_part[((wm * NBM + bm) * 16 + i) * 64 + lane] = d[bm][i];
             }
             __syncthreads();
             if (wn == 0) {
 #pragma unroll
-                for (int bm = 0; bm < 2; bm++) {
+                for (int bm = 0; bm < NBM; bm++) {
                     const int m = mw0 + bm * 32 + l32;
 #pragma unroll
                     for (int j = 0; j < 4; j++) {
                         v4f o;
 #pragma unroll
                         for (int e = 0; e < 4; e++)
-                            o[e] = d[bm][4 * j + e] + lds_part[((wm * 2 + bm) * 16 + 4 * j + e) * 64 + lane];
+                            o[e] = d[bm][4 * j + e] + lds_part[((wm * NBM + bm) * 16 + 4 * j + e) * 64 + lane];
                         const int rr = rc + 8 * j + 4 * half;
                         if (m < a.M && rr < a.R2)
                             *(v4f *)(a.scratch + ((size_t)pid_n * a.M + m) * a.R2 + rr) = o;
@@ -432,7 +472,7 @@ __global__ __launch_bounds__(256, SVDQ_GEMM_MIN_WAVES) void gemm_w4a4_kernel(svd
         __syncthreads();
         const int g = nw0 / GROUP;
 #pragma unroll
-        for (int bm = 0; bm < 2; bm++) {
+        for (int bm = 0; bm < NBM; bm++) {
             const int m = mw0 + bm * 32 + l32;
             float gmax = 0.0f;
 #pragma unroll
@@ -490,21 +530,21 @@ __global__ __launch_bounds__(256, SVDQ_GEMM_MIN_WAVES) void gemm_w4a4_kernel(svd
         // y columns = one quantization group, shared by the two n-wavefronts (32 y columns each).
         const int H = a.N / 2;
         const uint16_t *ldt = (const uint16_t *)a.lora_down_t;
-        float y[2][2][8];  // [bm][bn][4 j + e]: y column 16 bn + 8 j + 4 half + e of the wavefront's 32
+        float y[NBM][2][8];  // [bm][bn][4 j + e]: y column 16 bn + 8 j + 4 half + e of the wavefront's 32
 #pragma unroll
-        for (int bm = 0; bm < 2; bm++)
+        for (int bm = 0; bm < NBM; bm++)
 #pragma unroll
             for (int bn = 0; bn < 2; bn++)
 #pragma unroll
                 for (int i = 0; i < 8; i++) y[bm][bn][i] = silu(acc[bn][bm][i]) * acc[bn][bm][8 + i];
         const int yt0 = n0 / 2;          // first y column of the tile
         const int yw0 = yt0 + 32 * wn;   // ... of this wavefront
-        float *lds_part = (float *)smem;  // [2 (wm)][2 (bm)][16 regs][64 lanes] floats = 16 KB
+        float *lds_part = (float *)smem;  // [4 (wm)][16 regs][64 lanes] floats = 16 KB
         __syncthreads();
         for (int rc = 0; rc < a.R2; rc += 32) {
-            v16f d[2];
+            v16f d[NBM];
 #pragma unroll
-            for (int bm = 0; bm < 2; bm++)
+            for (int bm = 0; bm < NBM; bm++)
 #pragma unroll
                 for (int i = 0; i < 16; i++) d[bm][i] = 0.0f;
             const int r = rc + l32;
@@ -517,7 +557,7 @@ __global__ __launch_bounds__(256, SVDQ_GEMM_MIN_WAVES) void gemm_w4a4_kernel(svd
                     la = (v4i){(int)q0.x, (int)q0.y, (int)q1.x, (int)q1.y};
                 }
 #pragma unroll
-                for (int bm = 0; bm < 2; bm++) {
+                for (int bm = 0; bm < NBM; bm++) {
                     v4i xb;
 #pragma unroll
                     for (int e = 0; e < 4; e++) xb[e] = (int)pack2<T>(y[bm][s][2 * e], y[bm][s][2 * e + 1]);
@@ -526,21 +566,21 @@ __global__ __launch_bounds__(256, SVDQ_GEMM_MIN_WAVES) void gemm_w4a4_kernel(svd
             }
             if (wn == 1) {
 #pragma unroll
-                for (int bm = 0; bm < 2; bm++)
+                for (int bm = 0; bm < NBM; bm++)
 #pragma unroll
-                    for (int i = 0; i < 16; i++) lds_part[((wm * 2 + bm) * 16 + i) * 64 + lane] = d[bm][i];
+                    for (int i = 0; i < 16; i++) lds_part[((wm * NBM + bm) * 16 + i) * 64 + lane] = d[bm][i];
             }
             __syncthreads();
             if (wn == 0) {
 #pragma unroll
-                for (int bm = 0; bm < 2; bm++) {
+                for (int bm = 0; bm < NBM; bm++) {
                     const int m = mw0 + bm * 32 + l32;
 #pragma unroll
                     for (int j = 0; j < 4; j++) {
                         v4f o;
 #pragma unroll
                         for (int e = 0; e < 4; e++)
-                            o[e] = d[bm][4 * j + e] + lds_part[((wm * 2 + bm) * 16 + 4 * j + e) * 64 + lane];
+                            o[e] = d[bm][4 * j + e] + lds_part[((wm * NBM + bm) * 16 + 4 * j + e) * 64 + lane];
                         const int rr = rc + 8 * j + 4 * half;
                         if (m < a.M && rr < a.R2)
                             *(v4f *)(a.scratch + ((size_t)pid_n * a.M + m) * a.R2 + rr) = o;
@@ -561,7 +601,7 @@ __global__ __launch_bounds__(256, SVDQ_GEMM_MIN_WAVES) void gemm_w4a4_kernel(svd
         __syncthreads();
         float gm[2];
 #pragma unroll
-        for (int bm = 0; bm < 2; bm++) {
+        for (int bm = 0; bm < NBM; bm++) {
             float gmax = 0.0f;
 #pragma unroll
             for (int bn = 0; bn < 2; bn++)
@@ -576,13 +616,13 @@ __global__ __launch_bounds__(256, SVDQ_GEMM_MIN_WAVES) void gemm_w4a4_kernel(svd
                     }
                 }
             gmax = fmaxf(gmax, __shfl_xor(gmax, 32));
-            if (half == 0) lds_max[wn * BM + wm * 64 + bm * 32 + l32] = gmax;
+            if (half == 0) lds_max[wn * BM + wm * WROWS + bm * 32 + l32] = gmax;
             gm[bm] = gmax;
         }
         __syncthreads();
 #pragma unroll
-        for (int bm = 0; bm < 2; bm++) {
-            const int ml = wm * 64 + bm * 32 + l32;
+        for (int bm = 0; bm < NBM; bm++) {
+            const int ml = wm * WROWS + bm * 32 + l32;
             const int m = m0 + ml;
             const float gmax = fmaxf(lds_max[ml], lds_max[BM + ml]);
             const float scale = gmax / 7.0f;
@@ -655,7 +695,7 @@ __global__ __launch_bounds__(64) void group_acc_kernel(const uint8_t *act, const
 
 template <typename T, bool U, bool WPL>
 static void launch_gemm_epi2(const svdq_gemm_args &a, hipStream_t s) {
-    const dim3 grid(((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN)), block(256);
+    const dim3 grid(((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN)), block(NTHREADS);
     switch (a.epilogue) {
         case SVDQ_EPI_PLAIN:
             hipLaunchKernelGGL((gemm_w4a4_kernel<T, U, SVDQ_EPI_PLAIN, WPL>), grid, block, 0, s, a);
