@@ -320,24 +320,32 @@ __global__ __launch_bounds__(NTHREADS, 4) void gemm_w4a4_kernel(svdq_gemm_args a
             }
     }
 
+    // Output rows go out through LDS: in registers a lane holds 4 consecutive columns of one row, which stored directly
+    // is an 8-byte piece per row and lane; staged as a [row][column] tile, each store instruction writes four
+    // contiguous 256-byte row segments instead.
     auto store_out = [&]() {
-        uint16_t *out = (uint16_t *)a.out;
+        constexpr int PITCH = BN * 2 + 16;  // bytes per staged row (16-byte aligned, off the power of two)
+        static_assert(BM * PITCH <= SMEM_BYTES, "output tile does not fit the staging memory");
+        __syncthreads();  // earlier users of the staging memory are done
 #pragma unroll
-        for (int bm = 0; bm < NBM; bm++) {
-            const int m = mw0 + bm * 32 + l32;
-            if (m >= a.actual_m) continue;
+        for (int bm = 0; bm < NBM; bm++)
 #pragma unroll
             for (int bn = 0; bn < 2; bn++)
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
-                    const int n = nw0 + bn * 32 + 8 * j + 4 * half;
-                    if (n < a.N) {
-                        uint2 v;
-                        v.x = pack2<T>(acc[bn][bm][4 * j], acc[bn][bm][4 * j + 1]);
-                        v.y = pack2<T>(acc[bn][bm][4 * j + 2], acc[bn][bm][4 * j + 3]);
-                        *(uint2 *)(out + (size_t)m * a.ld_out + n) = v;
-                    }
+                    uint2 v;
+                    v.x = pack2<T>(acc[bn][bm][4 * j], acc[bn][bm][4 * j + 1]);
+                    v.y = pack2<T>(acc[bn][bm][4 * j + 2], acc[bn][bm][4 * j + 3]);
+                    *(uint2 *)(smem + (wm * WROWS + bm * 32 + l32) * PITCH + (wn * 64 + bn * 32 + 8 * j + 4 * half) * 2) = v;
                 }
+        __syncthreads();
+        uint16_t *out = (uint16_t *)a.out;
+        const int c = tid & 15, n = n0 + c * 8;
+#pragma unroll
+        for (int pass = 0; pass < BM * 16 / NTHREADS; pass++) {
+            const int row = pass * (NTHREADS / 16) + (tid >> 4), m = m0 + row;
+            if (m < a.actual_m && n < a.N)
+                *(v4i *)(out + (size_t)m * a.ld_out + n) = *(const v4i *)(smem + row * PITCH + c * 16);
         }
     };
 
@@ -816,8 +824,8 @@ extern "C" int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream) {
         set_error("svdq_gemm_w4a4: out is required for this epilogue");
         return SVDQ_E_INVALID;
     }
-    if (a.out && (((uintptr_t)a.out & 7) || a.ld_out % 4 || a.ld_out < a.N)) {
-        set_error("svdq_gemm_w4a4: out rows must be 8-byte aligned and at least N long (ld_out=%d)", a.ld_out);
+    if (a.out && (!al16(a.out) || a.ld_out % 8 || a.ld_out < a.N)) {
+        set_error("svdq_gemm_w4a4: out rows must be 16-byte aligned and at least N long (ld_out=%d)", a.ld_out);
         return SVDQ_E_INVALID;
     }
     if (a.epilogue == SVDQ_EPI_QK_NORM_ROPE) {
