@@ -667,12 +667,15 @@ __global__ __launch_bounds__(NTHREADS, 4) void gemm_w4a4_kernel(svdq_gemm_args a
 }
 
 // lora_act_out[m, r] = sum over n-tiles of the partial LoRA-down products, in tile order (deterministic)
-__global__ void lora_part_reduce_kernel(const float *part, float *out, int tiles, int M, int R2, int ld_out) {
-    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+__global__ __launch_bounds__(64) void lora_part_reduce_kernel(const float *part, float *out, int tiles, int M, int R2,
+                                                              int ld_out) {
+    const int idx = (blockIdx.x * 64 + threadIdx.x) * 4;  // four consecutive r of one row (R2 % 16 == 0)
     if (idx >= M * R2) return;
-    float s = 0.0f;
-    for (int t = 0; t < tiles; t++) s += part[(size_t)t * M * R2 + idx];
-    out[(size_t)(idx / R2) * ld_out + idx % R2] = s;
+    const size_t stride = (size_t)M * R2;
+    v4f s = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll 8
+    for (int t = 0; t < tiles; t++) s += *(const v4f *)(part + t * stride + idx);
+    *(v4f *)(out + (size_t)(idx / R2) * ld_out + idx % R2) = s;
 }
 
 // Debug read-out of one group's exact int32 accumulators: one wavefront per 32x32 block, operands straight from
@@ -854,8 +857,8 @@ extern "C" int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream) {
         }
         if (a.R2 < 0 || a.R2 % 16 ||
             (a.R2 > 0 && (!a.lora_down_t || !a.lora_act_out || !a.scratch || ((uintptr_t)a.lora_down_t & 7) ||
-                          !al16(a.scratch) || a.ld_lora_act_out < a.R2))) {
-            set_error("svdq_gemm_w4a4: R2=%d must be a multiple of 16 with lora_down_t, lora_act_out and scratch given", a.R2);
+                          !al16(a.scratch) || !al16(a.lora_act_out) || a.ld_lora_act_out % 4 || a.ld_lora_act_out < a.R2))) {
+            set_error("svdq_gemm_w4a4: R2=%d must be a multiple of 16 with lora_down_t, lora_act_out (16-byte aligned rows) and scratch given", a.R2);
             return SVDQ_E_INVALID;
         }
     } else if (a.epilogue != SVDQ_EPI_PLAIN) {
@@ -879,7 +882,7 @@ extern "C" int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream) {
     if (rc) return rc;
     if (quant && a.R2 > 0) {
         const int n = a.M * a.R2;
-        hipLaunchKernelGGL(lora_part_reduce_kernel, dim3((n + 255) / 256), dim3(256), 0, s, a.scratch, a.lora_act_out,
+        hipLaunchKernelGGL(lora_part_reduce_kernel, dim3((n / 4 + 63) / 64), dim3(64), 0, s, a.scratch, a.lora_act_out,
                            (a.N + BN - 1) / BN, a.M, a.R2, a.ld_lora_act_out);
         rc = check_launch("svdq_gemm_w4a4 (LoRA-down partial sum)");
     }
