@@ -270,35 +270,9 @@ __global__ __launch_bounds__(NTHREADS, 4) void gemm_w4a4_kernel(svdq_gemm_args a
 
     // ---- epilogue: LoRA-up and bias ----------------------------------------------------------------
     const int nw0 = n0 + wn * 64, mw0 = m0 + wm * WROWS;
-    if (a.R > 0) {
-        const uint16_t *lu = (const uint16_t *)a.lora_up;
-        for (int r0 = 0; r0 < a.R; r0 += 16) {
-            v4i ua[2], ub[NBM];
-#pragma unroll
-            for (int blk = 0; blk < 2; blk++) {
-                const int n = nw0 + blk * 32 + l32;
-                ua[blk] = (v4i){0, 0, 0, 0};
-                if (n < a.N) ua[blk] = *(const v4i *)(lu + (size_t)n * a.ld_lora_up + r0 + half * 8);
-            }
-#pragma unroll
-            for (int blk = 0; blk < NBM; blk++) {
-                const int m = mw0 + blk * 32 + l32;
-                ub[blk] = (v4i){0, 0, 0, 0};
-                if (m < a.M) {
-                    const float *lp = a.lora_act + (size_t)m * a.ld_lora_act + r0 + half * 8;
-                    const v4f f0 = *(const v4f *)lp, f1 = *(const v4f *)(lp + 4);
-                    ub[blk][0] = (int)pack2<T>(f0[0], f0[1]);
-                    ub[blk][1] = (int)pack2<T>(f0[2], f0[3]);
-                    ub[blk][2] = (int)pack2<T>(f1[0], f1[1]);
-                    ub[blk][3] = (int)pack2<T>(f1[2], f1[3]);
-                }
-            }
-#pragma unroll
-            for (int bn = 0; bn < 2; bn++)
-#pragma unroll
-                for (int bm = 0; bm < NBM; bm++) acc[bn][bm] = mfma32_16bit<T>(ua[bn], ub[bm], acc[bn][bm]);
-        }
-    }
+    // All global loads of this section (bias, then 32 ranks of both LoRA operands at a time) are issued before their
+    // first use: the section costs one memory latency per 32 ranks rather than one per load group.
+    uint2 bb[2][4];
     if (a.bias != nullptr) {
         const uint16_t *bias = (const uint16_t *)a.bias;
 #pragma unroll
@@ -306,16 +280,68 @@ __global__ __launch_bounds__(NTHREADS, 4) void gemm_w4a4_kernel(svdq_gemm_args a
 #pragma unroll
             for (int j = 0; j < 4; j++) {
                 const int n = nw0 + bn * 32 + 8 * j + 4 * half;
-                if (n < a.N) {
-                    const uint2 bb = *(const uint2 *)(bias + n);
-                    const float b0 = T::lo_f32(bb.x), b1 = T::hi_f32(bb.x), b2 = T::lo_f32(bb.y), b3 = T::hi_f32(bb.y);
+                bb[bn][j] = make_uint2(0u, 0u);
+                if (n < a.N) bb[bn][j] = *(const uint2 *)(bias + n);
+            }
+    }
+    if (a.R > 0) {
+        const uint16_t *lu = (const uint16_t *)a.lora_up;
+        for (int r0 = 0; r0 < a.R; r0 += 32) {
+            const bool two = r0 + 16 < a.R;  // uniform: the second 16 ranks of this pass exist
+            v4i ua[2][2];
+            v4f uf[2][NBM][2];
 #pragma unroll
-                    for (int bm = 0; bm < NBM; bm++) {
-                        acc[bn][bm][4 * j + 0] += b0;
-                        acc[bn][bm][4 * j + 1] += b1;
-                        acc[bn][bm][4 * j + 2] += b2;
-                        acc[bn][bm][4 * j + 3] += b3;
+            for (int c = 0; c < 2; c++) {
+                if (c == 1 && !two) break;
+#pragma unroll
+                for (int blk = 0; blk < 2; blk++) {
+                    const int n = nw0 + blk * 32 + l32;
+                    ua[c][blk] = (v4i){0, 0, 0, 0};
+                    if (n < a.N) ua[c][blk] = *(const v4i *)(lu + (size_t)n * a.ld_lora_up + r0 + 16 * c + half * 8);
+                }
+#pragma unroll
+                for (int blk = 0; blk < NBM; blk++) {
+                    const int m = mw0 + blk * 32 + l32;
+                    uf[c][blk][0] = uf[c][blk][1] = (v4f){0.f, 0.f, 0.f, 0.f};
+                    if (m < a.M) {
+                        const float *lp = a.lora_act + (size_t)m * a.ld_lora_act + r0 + 16 * c + half * 8;
+                        uf[c][blk][0] = *(const v4f *)lp;
+                        uf[c][blk][1] = *(const v4f *)(lp + 4);
                     }
+                }
+            }
+#pragma unroll
+            for (int c = 0; c < 2; c++) {
+                if (c == 1 && !two) break;
+                v4i ub[NBM];
+#pragma unroll
+                for (int blk = 0; blk < NBM; blk++) {
+                    const v4f f0 = uf[c][blk][0], f1 = uf[c][blk][1];
+                    ub[blk][0] = (int)pack2<T>(f0[0], f0[1]);
+                    ub[blk][1] = (int)pack2<T>(f0[2], f0[3]);
+                    ub[blk][2] = (int)pack2<T>(f1[0], f1[1]);
+                    ub[blk][3] = (int)pack2<T>(f1[2], f1[3]);
+                }
+#pragma unroll
+                for (int bn = 0; bn < 2; bn++)
+#pragma unroll
+                    for (int bm = 0; bm < NBM; bm++) acc[bn][bm] = mfma32_16bit<T>(ua[c][bn], ub[bm], acc[bn][bm]);
+            }
+        }
+    }
+    if (a.bias != nullptr) {
+#pragma unroll
+        for (int bn = 0; bn < 2; bn++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float b0 = T::lo_f32(bb[bn][j].x), b1 = T::hi_f32(bb[bn][j].x);
+                const float b2 = T::lo_f32(bb[bn][j].y), b3 = T::hi_f32(bb[bn][j].y);
+#pragma unroll
+                for (int bm = 0; bm < NBM; bm++) {
+                    acc[bn][bm][4 * j + 0] += b0;
+                    acc[bn][bm][4 * j + 1] += b1;
+                    acc[bn][bm][4 * j + 2] += b2;
+                    acc[bn][bm][4 * j + 3] += b3;
                 }
             }
     }
