@@ -8,6 +8,10 @@ from .. import _lib
 from ._prep import lora_down_t as _lora_down_t
 from ._prep import weight_planes as _weight_planes
 
+# Weights are re-laid-out once into MFMA-ordered int8 planes (cached per tensor, see _prep.weight_planes) and the GEMM
+# streams those; False makes the GEMM unpack the packed weight itself (no extra memory, about 15% slower).
+USE_WEIGHT_PLANES = True
+
 HEAD_DIM = 128
 GELU_SHIFT = 0.171875
 
@@ -122,7 +126,7 @@ def svdq_gemm_w4a4_cuda(
         raise ValueError("out not row-major")
 
     # module weights (nn.Parameter) get the cached MFMA-ordered plane re-layout; ad-hoc tensors are unpacked in-kernel
-    planes = _weight_planes(wgt) if isinstance(wgt, torch.nn.Parameter) and wgt.stride(0) % 16 == 0 else None
+    planes = _weight_planes(wgt) if USE_WEIGHT_PLANES and wgt.stride(0) % 16 == 0 else None
     args = _lib.GemmArgs(
         act=act.data_ptr(),
         wgt=wgt.data_ptr(),

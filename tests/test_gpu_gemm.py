@@ -185,10 +185,14 @@ def test_presplit_weights_same_bits_as_packed(dev, M, N, K, R, unsigned):
     """The GEMM gives identical bits whether it unpacks the weights itself or reads the pre-split planes."""
     print(f"case M={M} N={N} K={K} R={R} unsigned={unsigned}", flush=True)
     p = _rand_problem(M, N, K, R, torch.bfloat16, seed=7 + M)
-    packed = _gpu_gemm(p, dev, unsigned=unsigned)
-    q = dict(p)
-    q["wgt"] = torch.nn.Parameter(p["wgt"].to(dev), requires_grad=False)  # parameters take the cached pre-split path
-    split = _gpu_gemm(q, dev, unsigned=unsigned)
+    from nunchaku_rocm_amd.ops import gemm as gemm_mod
+
+    gemm_mod.USE_WEIGHT_PLANES = False
+    try:
+        packed = _gpu_gemm(p, dev, unsigned=unsigned)
+    finally:
+        gemm_mod.USE_WEIGHT_PLANES = True
+    split = _gpu_gemm(p, dev, unsigned=unsigned)
     assert torch.equal(packed.view(torch.int16), split.view(torch.int16))
     ref = O.gemm_w4a4(p["act"], p["wgt"], p["asc"], p["wsc"], bias=p["bias"], lora_act=p["la"], lora_up=p["lu"], act_unsigned=unsigned)
     assert O.max_rel_err(split.float(), ref) <= TOL
