@@ -50,11 +50,6 @@ constexpr int NBM = 1, WROWS = NBM * 32;            // activation rows per wavef
 constexpr int GROUP_M_TILES = 8;      // m-tiles per raster band
 constexpr int NUM_XCD = 8;
 
-#define SVDQ_AS1 __attribute__((address_space(1)))
-#define SVDQ_AS3 __attribute__((address_space(3)))
-
-// s_waitcnt immediate (gfx9 encoding): vmcnt in bits [3:0] and [15:14], expcnt [6:4] left at 7, lgkmcnt [11:8]
-constexpr int waitcnt_imm(int vm, int lgkm) { return (vm & 0xF) | ((vm >> 4) << 14) | 0x70 | ((lgkm & 0xF) << 8); }
 
 __device__ inline void unpack_signed(v4i p, v4i &even, v4i &odd) {
     even = (p << 4) & (int)0xF0F0F0F0;  // 16 * value in each byte

@@ -7,12 +7,14 @@
 // add, clamp, low nibble first.  The LoRA-down product consumes the raw 16-bit activations (before shift and
 // smoothing) on the 16x16x32 MFMA with fp32 accumulation.
 //
-// Work split: one workgroup = 16 rows x all of K, eight wavefronts taking scale groups round-robin with two
-// groups of loads in flight each.  Lane
-// (m = lane % 16, q = lane / 16) owns 16 consecutive channels [64 g + 16 q, +16) of row m, so a wavefront reads
-// 16 rows x 128 contiguous bytes per group, a group's absmax needs two cross-lane steps, and the lane's two
-// 16-byte halves are exactly the B operands of two MFMAs whose A operands come from the transposed LoRA-down
-// weight (R, K).
+// Work split: one workgroup = 16 rows x all of K, four wavefronts taking scale groups round-robin with two groups
+// in flight each.  A group's operands (16 rows x 128 bytes of activations, 32 ranks x 128 bytes of the transposed
+// LoRA-down weight (R, K)) are fetched straight into LDS (global_load_lds_dwordx4) by loads whose 64 lanes cover eight
+// full 128-byte rows -- read lane-per-row from global memory, the same bytes cost the memory pipeline four times as
+// many cycles -- and land in a tile whose 16-byte chunks are XOR-swizzled by the row so that the transposed read-back
+// is conflict free.  Lane (m = lane % 16, q = lane / 16) then owns the 16 consecutive channels [64 g + 16 q, +16)
+// of row m: a group's absmax needs two cross-lane steps, and the lane's two 16-byte halves are exactly the B operands
+// of two 16x16x32 MFMAs whose A operands come from the LoRA-down tile.
 #include "svdq_common.h"
 
 // the codes and scales are a bit-exact contract: no multiply-add contraction anywhere in this file
@@ -22,6 +24,7 @@ namespace svdq {
 
 constexpr int Q_ROWS = 16;
 constexpr int Q_WAVES = 8;
+constexpr int Q_ROW_BYTES = 128;  // one scale group of one row (64 x 16 bit)
 constexpr int Q_RCHUNK = 32;  // LoRA ranks per pass over the row block
 
 // sum_j (0x4B400000 << 4 j) mod 2^32: what eight magic-biased codes add up to besides their nibbles
@@ -31,17 +34,18 @@ constexpr uint32_t pack_bias() {
     return c;
 }
 
-// One scale group's loads for one lane: 16 activations (+ 16 gate values), the matching LoRA-down operands
-template <bool GLU, bool HAS_LORA>
-struct QStage {
-    v4i xlo, xhi, glo, ghi, l0lo, l0hi, l1lo, l1hi;
-    uint16_t sm;
-};
-
 template <typename T, bool UNSIGNED, bool GLU, bool HAS_LORA, bool HAS_SMOOTH>
-__global__ __launch_bounds__(Q_WAVES * 64, 4) void quantize_act_kernel(svdq_quantize_args a) {
+__global__ __launch_bounds__(Q_WAVES * 64, 2) void quantize_act_kernel(svdq_quantize_args a) {
+    // per wavefront: two activation stages (16 rows, + the gate tile with GLU) and one LoRA-down tile (32 ranks), 128
+    // bytes a row.  The LoRA-down tile is an L2 hit and the first thing a group consumes: one group ahead is enough.
+    constexpr int XS_BYTES = (GLU ? 2 : 1) * Q_ROWS * Q_ROW_BYTES, G_OFF = Q_ROWS * Q_ROW_BYTES;
+    constexpr int L_OFF = 2 * XS_BYTES;
+    constexpr int WAVE_BYTES = L_OFF + (HAS_LORA ? Q_RCHUNK * Q_ROW_BYTES : 0);
+    constexpr int ACC_BYTES = HAS_LORA ? Q_WAVES * Q_RCHUNK * (Q_ROWS + 1) * 4 : 0;  // cross-wave sum, after the loop
+    constexpr int STG_BYTES = Q_WAVES * WAVE_BYTES;
+    __shared__ __align__(16) uint8_t smem[STG_BYTES > ACC_BYTES ? STG_BYTES : ACC_BYTES];
     __shared__ float lds_rs[Q_WAVES][64];
-    __shared__ float lds_acc[Q_WAVES][Q_RCHUNK][Q_ROWS + 1];
+    float (*lds_acc)[Q_RCHUNK][Q_ROWS + 1] = (float (*)[Q_RCHUNK][Q_ROWS + 1])smem;
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: keep it in an SGPR
@@ -52,11 +56,18 @@ __global__ __launch_bounds__(Q_WAVES * 64, 4) void quantize_act_kernel(svdq_quan
     const bool row_ok = m < a.M;
     const int ngroups = a.K / GROUP;
     const int nmy = (ngroups - wave + Q_WAVES - 1) / Q_WAVES;  // groups g = wave + Q_WAVES * i
-    // uniform base pointers + 32-bit per-lane element offsets (rows >= M re-read row M - 1: valid memory, and
-    // nothing is stored for them)
-    const uint16_t *__restrict__ xbase = (const uint16_t *)a.x + (size_t)m0 * a.ld_x + wave * GROUP;
-    const uint32_t xoff = (uint32_t)(min(m, a.M - 1) - m0) * a.ld_x + kq * 16;
-    const uint16_t *__restrict__ smooth = (const uint16_t *)a.smooth + wave * GROUP;
+    // Block loads: lane l of load i fetches chunk (l % 8) ^ (l / 8) of tile row 8 i + l / 8 into LDS slot l of that
+    // load's 1 KB, i.e. tile[row][chunk ^ (row & 7)].  Rows >= M re-read row M - 1 and ranks >= R rank R - 1 (valid
+    // memory; nothing is stored for them).  Addresses = uniform base + 32-bit lane offset (+ uniform group step).
+    const int drow = lane >> 3, dchunk = (lane & 7) ^ drow;
+    const uint8_t *__restrict__ xbase = (const uint8_t *)a.x + (size_t)m0 * a.ld_x * 2;
+    uint32_t xdma[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) xdma[i] = (uint32_t)(min(m0 + 8 * i + drow, a.M - 1) - m0) * a.ld_x * 2 + dchunk * 16;
+    // read-back: lane (m, q) takes chunks 2 q and 2 q + 1 of tile row m (and of row m + 16 of the LoRA-down tile)
+    const int rd_lo = ml * Q_ROW_BYTES + (((2 * kq) ^ (ml & 7)) * 16), rd_hi = ml * Q_ROW_BYTES + (((2 * kq + 1) ^ (ml & 7)) * 16);
+    uint8_t *const wbase = smem + wave * WAVE_BYTES;
+    const uint16_t *__restrict__ smooth = (const uint16_t *)a.smooth;
     uint8_t *__restrict__ outbase = (uint8_t *)a.out + (size_t)m0 * a.ld_out + wave * (GROUP / 2);
     const uint32_t outoff = (uint32_t)ml * a.ld_out + kq * 8;
     uint16_t *__restrict__ scales = (uint16_t *)a.scales + (size_t)wave * a.ld_scales + m0;
@@ -70,35 +81,66 @@ __global__ __launch_bounds__(Q_WAVES * 64, 4) void quantize_act_kernel(svdq_quan
         v4f acc0 = (v4f){0.f, 0.f, 0.f, 0.f}, acc1 = (v4f){0.f, 0.f, 0.f, 0.f};
         // ranks >= R re-read rank R - 1; their accumulator rows are never stored
         const int r0 = rc * Q_RCHUNK + ml;
-        const uint16_t *__restrict__ lbase = (const uint16_t *)a.lora_down_t + wave * GROUP;
-        uint32_t loff0 = 0, loff1 = 0;
+        const uint8_t *__restrict__ lbase = (const uint8_t *)a.lora_down_t;
+        uint32_t ldma[4] = {0, 0, 0, 0};
         if (HAS_LORA) {
-            loff0 = (uint32_t)min(r0, a.R - 1) * a.K + kq * 16;
-            loff1 = (uint32_t)min(r0 + 16, a.R - 1) * a.K + kq * 16;
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                ldma[i] = (uint32_t)min(rc * Q_RCHUNK + 8 * i + drow, a.R - 1) * a.K * 2 + dchunk * 16;
         }
         const bool do_quant = rc == 0;
 
-        auto issue = [&](QStage<GLU, HAS_LORA> &st, int i) {
-            const int k0 = min(i, nmy - 1) * GSTEP;  // past the end: re-read the last group, unused
-            const uint16_t *xg = xbase + k0;
-            st.xlo = *(const v4i *)(xg + xoff);
-            st.xhi = *(const v4i *)(xg + xoff + 8);
+        constexpr int NX = GLU ? 4 : 2;  // block loads of one activation stage
+        auto group_off = [&](int i) {  // byte offset of group wave + Q_WAVES * i in a row; past the end: the last group
+            return (uint32_t)min(wave + Q_WAVES * i, ngroups - 1) * (GROUP * 2);
+        };
+        auto issue_x = [&](int i, uint16_t &sm) {
+            const uint32_t k0 = group_off(i);
+            uint8_t *dst = wbase + (i & 1) * XS_BYTES;
+            // the smooth factor of the lane's channel first: older than the block loads, its wait does not cover them
+            if (HAS_SMOOTH && do_quant) sm = smooth[(k0 >> 1) + lane];
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+                __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)(xbase + (xdma[j] + k0)),
+                                                 (SVDQ_AS3 void *)(dst + j * 1024), 16, 0, 0);
             if (GLU) {
-                st.glo = *(const v4i *)(xg + a.K + xoff);
-                st.ghi = *(const v4i *)(xg + a.K + xoff + 8);
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+                    __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)(xbase + (size_t)a.K * 2 + (xdma[j] + k0)),
+                                                     (SVDQ_AS3 void *)(dst + G_OFF + j * 1024), 16, 0, 0);
             }
-            if (HAS_LORA) {
-                const uint16_t *lg = lbase + k0;
-                st.l0lo = *(const v4i *)(lg + loff0);
-                st.l0hi = *(const v4i *)(lg + loff0 + 8);
-                st.l1lo = *(const v4i *)(lg + loff1);
-                st.l1hi = *(const v4i *)(lg + loff1 + 8);
-            }
-            if (HAS_SMOOTH) st.sm = (smooth + k0)[lane];
+        };
+        auto issue_l = [&](int i) {
+            if (!HAS_LORA) return;
+            const uint32_t k0 = group_off(i);
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)(lbase + (ldma[j] + k0)),
+                                                 (SVDQ_AS3 void *)(wbase + L_OFF + j * 1024), 16, 0, 0);
         };
 
-        auto process = [&](const QStage<GLU, HAS_LORA> &st, int i) {
-            v4i cxlo = st.xlo, cxhi = st.xhi;
+        struct Ops {
+            v4i xlo, xhi, glo, ghi, l0lo, l0hi, l1lo, l1hi;
+        };
+        auto fetch = [&](int i, Ops &o) {  // LDS -> registers, in the MFMA operand layout
+            const uint8_t *src = wbase + (i & 1) * XS_BYTES;
+            o.xlo = *(const v4i *)(src + rd_lo);
+            o.xhi = *(const v4i *)(src + rd_hi);
+            if (GLU) {
+                o.glo = *(const v4i *)(src + G_OFF + rd_lo);
+                o.ghi = *(const v4i *)(src + G_OFF + rd_hi);
+            }
+            if (HAS_LORA) {
+                o.l0lo = *(const v4i *)(wbase + L_OFF + rd_lo);
+                o.l0hi = *(const v4i *)(wbase + L_OFF + rd_hi);
+                o.l1lo = *(const v4i *)(wbase + L_OFF + 16 * Q_ROW_BYTES + rd_lo);
+                o.l1hi = *(const v4i *)(wbase + L_OFF + 16 * Q_ROW_BYTES + rd_hi);
+            }
+        };
+
+        auto process = [&](int i, const Ops &o, uint16_t smv) {
+            v4i cxlo = o.xlo, cxhi = o.xhi;
+            const v4i glo = o.glo, ghi = o.ghi, l0lo = o.l0lo, l0hi = o.l0hi, l1lo = o.l1lo, l1hi = o.l1hi;
             float v[16];
 #pragma unroll
             for (int j = 0; j < 4; j++) {
@@ -111,8 +153,8 @@ __global__ __launch_bounds__(Q_WAVES * 64, 4) void quantize_act_kernel(svdq_quan
                 // x[:, k] * silu(x[:, K + k]); the LoRA-down then sees the product rounded to T
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
-                    const float g0 = T::lo_f32((uint32_t)st.glo[j]), g1 = T::hi_f32((uint32_t)st.glo[j]);
-                    const float g2 = T::lo_f32((uint32_t)st.ghi[j]), g3 = T::hi_f32((uint32_t)st.ghi[j]);
+                    const float g0 = T::lo_f32((uint32_t)glo[j]), g1 = T::hi_f32((uint32_t)glo[j]);
+                    const float g2 = T::lo_f32((uint32_t)ghi[j]), g3 = T::hi_f32((uint32_t)ghi[j]);
                     v[2 * j] = v[2 * j] * (g0 / (1.0f + __expf(-g0)));
                     v[2 * j + 1] = v[2 * j + 1] * (g1 / (1.0f + __expf(-g1)));
                     v[8 + 2 * j] = v[8 + 2 * j] * (g2 / (1.0f + __expf(-g2)));
@@ -125,10 +167,10 @@ __global__ __launch_bounds__(Q_WAVES * 64, 4) void quantize_act_kernel(svdq_quan
                 }
             }
             if (HAS_LORA) {
-                acc0 = mfma16_16bit<T>(st.l0lo, cxlo, acc0);
-                acc0 = mfma16_16bit<T>(st.l0hi, cxhi, acc0);
-                acc1 = mfma16_16bit<T>(st.l1lo, cxlo, acc1);
-                acc1 = mfma16_16bit<T>(st.l1hi, cxhi, acc1);
+                acc0 = mfma16_16bit<T>(l0lo, cxlo, acc0);
+                acc0 = mfma16_16bit<T>(l0hi, cxhi, acc0);
+                acc1 = mfma16_16bit<T>(l1lo, cxlo, acc1);
+                acc1 = mfma16_16bit<T>(l1hi, cxhi, acc1);
             }
             if (!do_quant) return;
             if (has_shift) {
@@ -137,7 +179,7 @@ __global__ __launch_bounds__(Q_WAVES * 64, 4) void quantize_act_kernel(svdq_quan
             }
             if (HAS_SMOOTH) {
                 // 1/smooth for the group's 64 channels: one IEEE divide per lane, shared through LDS
-                lds_rs[wave][lane] = 1.0f / T::to_f32(st.sm);
+                lds_rs[wave][lane] = 1.0f / T::to_f32(smv);
                 __builtin_amdgcn_wave_barrier();
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
@@ -183,23 +225,34 @@ __global__ __launch_bounds__(Q_WAVES * 64, 4) void quantize_act_kernel(svdq_quan
             }
         };
 
-        // two groups in flight per wavefront
-        QStage<GLU, HAS_LORA> sa, sb;
-        issue(sa, 0);
-        issue(sb, 1);
+        // Two groups of activations and one LoRA-down tile in flight per wavefront; each wavefront owns its LDS, so no
+        // barrier in the loop.  Per group: wait for its tiles, pull them into registers, refill the freed LDS (next
+        // group's LoRA-down tile, the activations two groups on), then compute from the registers.
+        uint16_t sm_a = 0, sm_b = 0;
+        Ops ops;
+        issue_x(0, sm_a);
+        issue_l(0);
+        issue_x(1, sm_b);
+        auto step = [&](int i, uint16_t &sm) {
+            // group i's activations and LoRA-down tile have landed: the loads issued after them are at least the NX
+            // block loads of group i + 1's activations
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(NX, 15));
+            fetch(i, ops);
+            const uint16_t smv = sm;
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));  // the LDS reads have returned
+            issue_l(i + 1);
+            issue_x(i + 2, sm);
+            process(i, ops, smv);
+        };
         for (int i = 0; i < nmy; i += 2) {
-            QStage<GLU, HAS_LORA> cur = sa;
-            issue(sa, i + 2);
-            process(cur, i);
-            if (i + 1 < nmy) {
-                cur = sb;
-                issue(sb, i + 3);
-                process(cur, i + 1);
-            }
+            step(i, sm_a);
+            if (i + 1 < nmy) step(i + 1, sm_b);
         }
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
 
         if (HAS_LORA) {
             // fixed-order sum of the wavefronts' partial products
+            __syncthreads();  // every wavefront is done with its stages: the sum reuses the memory
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 lds_acc[wave][4 * kq + i][ml] = acc0[i];

@@ -16,6 +16,12 @@ typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef short v8s __attribute__((ext_vector_type(8)));
 
+#define SVDQ_AS1 __attribute__((address_space(1)))
+#define SVDQ_AS3 __attribute__((address_space(3)))
+
+// s_waitcnt immediate (gfx9 encoding): vmcnt in bits [3:0] and [15:14], expcnt [6:4] left at 7, lgkmcnt [11:8]
+constexpr int waitcnt_imm(int vm, int lgkm) { return (vm & 0xF) | ((vm >> 4) << 14) | 0x70 | ((lgkm & 0xF) << 8); }
+
 constexpr int GROUP = 64;            // int4 scale group along K
 constexpr float RNE_MAGIC = 12582912.0f;  // 1.5 * 2^23: adding it rounds an fp32 at the units place (RNE)
 constexpr int RNE_MAGIC_BITS = 0x4B400000;
