@@ -8,7 +8,7 @@ with the quantizer's time as well).  The JSON line also carries the roofline of 
 with HIP events inside the timed region), a per-kernel table (quantizer GB/s, AWQ GEMV GB/s, GEMM M-sweep and fused
 epilogue shapes), and the CPU baseline (the oracle's pure-PyTorch restatement of the reference's CPU path).
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-extras]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-extras] [--eager]
 """
 
 from __future__ import annotations
@@ -104,6 +104,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
+    ap.add_argument("--eager", action="store_true", help="time the small kernels eagerly too (no HIP graph): for counter runs")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on one GPU only (the path shards over tokens with no exchange; "
@@ -152,7 +153,7 @@ def main():
 
     kernels = {}
     if not args.no_extras:
-        q_ms = _time_kernel(quant, graph=True)
+        q_ms = _time_kernel(quant, graph=not args.eager)
         q_bytes = 2 * M * K + M * K // 2 + 2 * (K // 64) * M + 4 * M * R + 2 * K * R + 2 * K
         kernels["quantize_act M4608 K3072 R32"] = {
             "ms": round(q_ms, 5), "GB/s": round(q_bytes / q_ms / 1e6, 1), "frac_hbm": round(q_bytes / q_ms / 1e6 / HBM_PEAK_GBS, 4),
@@ -207,7 +208,7 @@ def main():
         aw = {k: v.to(dev) for k, v in O.make_awq_linear(3072, 18432, seed=2).items() if k != "codes"}
         for m in (1, 2, 8):
             xv = torch.randn(m, 3072, device=dev).to(torch.bfloat16)
-            ms = _time_kernel(lambda: ops.awq_gemv_w4a16_cuda(xv, aw["qweight"], aw["wscales"], aw["wzeros"], m, 18432, 3072), iters=200, warmup=20, graph=True)
+            ms = _time_kernel(lambda: ops.awq_gemv_w4a16_cuda(xv, aw["qweight"], aw["wscales"], aw["wzeros"], m, 18432, 3072), iters=200, warmup=20, graph=not args.eager)
             nbytes = 18432 * 3072 // 2 + 2 * 2 * 48 * 18432 + 2 * m * 3072 + 2 * m * 18432
             kernels[f"awq_gemv_w4a16 M{m} K3072 N18432"] = {"ms": round(ms, 5), "GB/s": round(nbytes / ms / 1e6, 1),
                                                            "frac_hbm": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4), "bytes": nbytes}  # fmt: skip
@@ -229,11 +230,15 @@ def main():
         torch.cuda.synchronize()
         kernels["flux1_schnell_shaped 19+38 blocks 4608 tokens"] = {"s_per_step": round((time.perf_counter() - t1) / 4, 4), "steps": 4}
         del model
-        # plain device copy of known size: the scale reference for the FETCH_SIZE / WRITE_SIZE counters
-        src = torch.zeros(64 << 20, dtype=torch.float32, device=dev)
+        # plain elementwise kernel of known size: the scale reference for the FETCH_SIZE / WRITE_SIZE counters
+        # (random data, and a second buffer written in between so that the read comes from HBM, not from cache)
+        src = torch.randn(64 << 20, dtype=torch.float32, device=dev)
         dst = torch.empty_like(src)
+        flush = torch.randn(128 << 20, dtype=torch.float32, device=dev)
+        torch.cuda.synchronize()
         torch.add(src, 1.0, out=dst)  # one elementwise kernel: reads 256 MiB, writes 256 MiB
         torch.cuda.synchronize()
+        del flush
         del src, dst
 
     result = {
