@@ -24,6 +24,9 @@ sys.path.insert(0, ROOT)
 
 INT8_MFMA_PEAK_TOPS = 5000.0  # MI355X dense int8 MFMA, published
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+# HBM bytes of one QKV GEMM launch: FETCH_SIZE + WRITE_SIZE (KiB per dispatch, counter scale 1.000) of the grid-1327104
+# launches in profiles/bench_all_kernels_hbm_traffic.txt; counters cannot be read from inside this process
+GEMM_QKV_HBM_BYTES = (121271.8 + 82944.0) * 1024
 
 
 def _events(n):
@@ -263,7 +266,8 @@ def main():
             "peak": INT8_MFMA_PEAK_TOPS,
             "unit": "TFLOP/s",
             "frac": round(achieved / INT8_MFMA_PEAK_TOPS, 4),
-            "traffic": None,
+            "traffic": GEMM_QKV_HBM_BYTES,
+            "traffic_unit": "bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, see profiles/)",
             "ops_per_launch": ops_per_gemm,
             "avg_launch_ms": round(gemm_ms, 5),
             "note": "int8 MFMA ops (2*M*N*K), peak = published dense int8 5.0 POP/s",
