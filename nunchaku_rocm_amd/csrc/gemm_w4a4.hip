@@ -260,8 +260,9 @@ __global__ __launch_bounds__(NTHREADS, 4) void gemm_w4a4_kernel(svdq_gemm_args a
         case 2: main_loop(std::integral_constant<int, 2>{}); break;
         default: main_loop(std::integral_constant<int, 3>{}); break;
     }
-    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));  // the last stage's (redundant) block loads have landed
-    __syncthreads();  // every wavefront is done with the staging buffers: the epilogues reuse them
+    // The last stage's (redundant) block loads of this wavefront have landed.  No barrier here: the LoRA-up / bias section
+    // does not touch LDS, and every epilogue starts its first use of the staging memory with a barrier of its own.
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
 
     // ---- epilogue: LoRA-up and bias ----------------------------------------------------------------
     const int nw0 = n0 + wn * 64, mw0 = m0 + wm * WROWS;
