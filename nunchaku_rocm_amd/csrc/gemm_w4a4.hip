@@ -19,10 +19,14 @@
 //    lane ^ 32.
 //  * 512 threads = 2 (n) x 4 (m) wavefronts of 64 weight rows x 32 activation rows on a 128x128 tile, two workgroups
 //    per CU = four wavefronts per SIMD: at half that occupancy the loop runs at about half the speed, its waits
-//    (LDS, MFMA results, barrier) exposed. K is staged through LDS 128 at a time (two scale
-//    groups), two stages.  Operands go global -> LDS directly (global_load_lds_dwordx4, no registers), one stage
-//    ahead, into a lane-linear layout (LDS slot l of a 1 KB block = the 16 bytes MFMA lane l needs), so the operand
-//    reads are bank-conflict free by construction; one raw s_barrier per stage with explicit s_waitcnt.
+//    (LDS, MFMA results, barrier) exposed.  K is staged through LDS 128 at a time (two scale groups), two stages.
+//    Operands go global -> LDS directly (global_load_lds_dwordx4, no registers), one stage ahead, into a lane-linear
+//    layout (LDS slot l of a 1 KB block = the 16 bytes MFMA lane l needs), so the operand reads are bank-conflict
+//    free by construction; one raw s_barrier per stage with explicit s_waitcnt.  The four wavefronts of a SIMD issue
+//    their block loads at four different points of the stage (a wavefront blocks at issue while the memory pipe is
+//    full; the others keep computing).
+//  * The 16-bit output tile leaves through LDS as 256-byte row segments (a lane's own accumulators are 8-byte pieces
+//    of 32 different rows, which the memory pipe takes one lane per cycle).
 //  * Weights can be given pre-split (svdq_split_weight_planes: int8 even / odd planes stored block by block in MFMA
 //    lane order); their half of the unpack then disappears from the inner loop.
 //  * Workgroup ids are first regrouped so that each XCD (ids are dealt round-robin over 8 XCDs) works on a
