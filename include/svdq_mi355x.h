@@ -14,6 +14,7 @@
  *   svdq_gemm_w4a4           nunchaku/ops/gemm.py:151-207        (_C.ops.gemm_w4a4 / ops/triton/gemm_w4a4.py:1003 gemm_w4a4),
  *                            kernel-argument structs modelled on ops/triton/native/w4a4.py:80-124
  *   svdq_awq_gemv_w4a16      nunchaku/ops/dispatch.py:19-34      (_C.ops.gemv_awq / ops/triton/awq.py:186 awq_gemv_w4a16)
+ *   svdq_attention_fp16      nunchaku/ops/dispatch.py:67-99      (_C.ops.attention_fp16 / ops/triton/attention.py:111 attention_fp16)
  *   svdq_transpose_lora_down no counterpart: one-time re-layout of a LoRA-down weight, see below
  *   svdq_group_acc_i32       no counterpart: debug read-out of the exact int32 group accumulators
  */
@@ -151,6 +152,28 @@ typedef struct {
 } svdq_awq_gemv_args;
 
 int svdq_awq_gemv_w4a16(const svdq_awq_gemv_args *args, void *stream);
+
+/*
+ * Unmasked scaled-dot-product attention, head dimension 128 (nunchaku/ops/dispatch.py:67-99 attention_fp16 /
+ * ops/triton/attention.py:111-169): o[b, t, h*128 + d] = softmax_k(scale * q[b,h,t,:] . k[b,h,k,:]) . v[b,h,k,d], fp32
+ * softmax and accumulation, P rounded to T.  Strides are in elements; the last dimension of q, k, v, o is contiguous.
+ * `vt` is a caller-owned workspace of svdq_attention_workspace_bytes(B, H, Tkv, 128) bytes (a transposed copy of v made
+ * by the call itself).
+ */
+typedef struct {
+    const void *q;  /* (B, H, Tq, 128) T  */
+    const void *k;  /* (B, H, Tkv, 128) T */
+    const void *v;  /* (B, H, Tkv, 128) T */
+    void *o;        /* (B, Tq, H * 128) T */
+    void *vt;       /* workspace          */
+    int64_t sqb, sqh, sqm, skb, skh, skn, svb, svh, svn, sob, som;
+    int32_t B, H, Tq, Tkv, D;
+    int32_t dtype;
+    float scale;    /* normally 128 ** -0.5 */
+} svdq_attention_args;
+
+int svdq_attention_fp16(const svdq_attention_args *args, void *stream);
+size_t svdq_attention_workspace_bytes(int32_t B, int32_t H, int32_t Tkv, int32_t D);
 
 /* Message for the last non-zero return on the calling thread ("" if none). */
 const char *svdq_last_error(void);

@@ -29,11 +29,13 @@ EXPORTS = (
     "svdq_weight_planes_bytes",
     "svdq_group_acc_i32",
     "svdq_awq_gemv_w4a16",
+    "svdq_attention_fp16",
+    "svdq_attention_workspace_bytes",
     "svdq_last_error",
     "svdq_abi_version",
 )
 
-_vp, _i32, _f32 = ctypes.c_void_p, ctypes.c_int32, ctypes.c_float
+_vp, _i32, _i64, _f32 = ctypes.c_void_p, ctypes.c_int32, ctypes.c_int64, ctypes.c_float
 
 
 class QuantizeArgs(ctypes.Structure):
@@ -70,6 +72,17 @@ class AwqGemvArgs(ctypes.Structure):
     )  # fmt: skip
 
 
+class AttentionArgs(ctypes.Structure):
+    """``svdq_attention_args``"""
+
+    _fields_ = (
+        [(n, _vp) for n in ("q", "k", "v", "o", "vt")]
+        + [(n, _i64) for n in ("sqb", "sqh", "sqm", "skb", "skh", "skn", "svb", "svh", "svn", "sob", "som")]
+        + [(n, _i32) for n in ("B", "H", "Tq", "Tkv", "D", "dtype")]
+        + [("scale", _f32)]
+    )  # fmt: skip
+
+
 _lib = None
 
 
@@ -100,6 +113,9 @@ def load() -> ctypes.CDLL:
     lib.svdq_quantize_act.argtypes = [ctypes.POINTER(QuantizeArgs), _vp]
     lib.svdq_gemm_w4a4.argtypes = [ctypes.POINTER(GemmArgs), _vp]
     lib.svdq_awq_gemv_w4a16.argtypes = [ctypes.POINTER(AwqGemvArgs), _vp]
+    lib.svdq_attention_fp16.argtypes = [ctypes.POINTER(AttentionArgs), _vp]
+    lib.svdq_attention_workspace_bytes.restype = ctypes.c_size_t
+    lib.svdq_attention_workspace_bytes.argtypes = [_i32, _i32, _i32, _i32]
     lib.svdq_transpose_lora_down.argtypes = [_vp, _vp, _i32, _i32, _i32, _vp]
     lib.svdq_group_acc_i32.argtypes = [_vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp]
     if lib.svdq_abi_version() != ABI_VERSION:

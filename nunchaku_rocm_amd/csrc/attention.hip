@@ -1,0 +1,286 @@
+// Unmasked scaled-dot-product attention (flash-attention forward) for gfx950, head dimension 128.
+//
+// Arithmetic (reference: nunchaku/ops/triton/attention.py:37-169): q is multiplied by scale * log2(e) and rounded to
+// the 16-bit type; per block of keys S = q k^T in fp32, online softmax with exp2 (running row maximum m and row sum
+// l), P rounded to the 16-bit type, O = O * 2^(m_old - m_new) + P v in fp32; at the end O / l, stored as
+// (B, Tq, H * 128).
+//
+// How it maps to CDNA4:
+//  * Everything is computed transposed.  S^T = K Q^T puts the keys in the MFMA's A operand and the queries in its B
+//    operand, so in the 32x32 accumulator a lane owns ONE query (column) and its registers walk the keys: the row
+//    maximum and row sum of the softmax are in-lane reductions plus one exchange with lane ^ 32, and the rescaling of
+//    the output accumulator is a per-lane scalar.  O^T = V^T P^T then takes P^T as its B operand straight from those
+//    accumulator registers (eight values of a lane are the eight k-slots the operand wants; the k order inside a
+//    16-key chunk is the permutation 0-3, 8-11 | 4-7, 12-15, which V^T simply shares), with no trip through LDS.
+//  * V^T is made once per call by a small transposing kernel (keys permuted as above, key count padded to 64); the
+//    main kernel then streams K tiles (64 keys x 256 bytes) and V^T tiles (128 rows x 128 bytes) global -> LDS
+//    directly (global_load_lds_dwordx4, whole rows per load, 16-byte chunks XOR-swizzled by the row so the operand
+//    reads are conflict free), one tile pair ahead, one barrier per 64 keys.
+//  * 256 threads = 4 wavefronts of 32 queries; Q stays in registers (pre-scaled), the output accumulator is 64
+//    registers; the accumulator is only rescaled when some lane's maximum moved.
+#include "svdq_common.h"
+
+namespace svdq {
+
+constexpr int AT_D = 128;                  // head dimension
+constexpr int AT_BQ = 128, AT_BK = 64;     // queries per workgroup, keys per tile
+constexpr int AT_KT_BYTES = AT_BK * AT_D * 2;  // 16 KB K tile: [key][16 chunks of 16 bytes]
+constexpr int AT_VT_BYTES = AT_D * AT_BK * 2;  // 16 KB V^T tile: [d][8 chunks of 16 bytes]
+constexpr int AT_STAGE = AT_KT_BYTES + AT_VT_BYTES;
+constexpr int AT_OPITCH = AT_D * 2 + 16;   // staged output row
+
+// position p of a 16-key chunk holds key sigma(p)
+__device__ __host__ inline int at_sigma(int p) { return (p & 3) | ((p & 4) << 1) | ((p & 8) >> 1); }
+
+// V (B, H, Tkv, 128) with arbitrary strides -> vt[(b * H + h) * 128 + d][Tpad], keys permuted inside 16-key chunks,
+// keys >= Tkv zero
+__global__ __launch_bounds__(256) void transpose_v_kernel(const uint16_t *v, uint16_t *vt, int H, int Tkv, int Tpad,
+                                                          long svb, long svh, long svn) {
+    __shared__ uint16_t tile[AT_BK][AT_D + 2];
+    const int k0 = blockIdx.x * AT_BK, h = blockIdx.y, b = blockIdx.z;
+    const uint16_t *vb = v + b * svb + h * svh;
+    for (int i = threadIdx.x; i < AT_BK * (AT_D / 8); i += 256) {
+        const int key = i / (AT_D / 8), c = i % (AT_D / 8);
+        v4i x = {0, 0, 0, 0};
+        if (k0 + key < Tkv) x = *(const v4i *)(vb + (long)(k0 + key) * svn + 8 * c);
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            tile[key][8 * c + 2 * e] = (uint16_t)((uint32_t)x[e] & 0xFFFFu);
+            tile[key][8 * c + 2 * e + 1] = (uint16_t)((uint32_t)x[e] >> 16);
+        }
+    }
+    __syncthreads();
+    uint16_t *ob = vt + ((size_t)(b * H + h) * AT_D) * Tpad + k0;
+    for (int i = threadIdx.x; i < AT_D * (AT_BK / 8); i += 256) {
+        const int d = i / (AT_BK / 8), c = i % (AT_BK / 8);  // 8 consecutive positions of row d
+        uint32_t w[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int p0 = 8 * c + 2 * e, p1 = p0 + 1;
+            const int key0 = (p0 & ~15) | at_sigma(p0 & 15), key1 = (p1 & ~15) | at_sigma(p1 & 15);
+            w[e] = (uint32_t)tile[key0][d] | ((uint32_t)tile[key1][d] << 16);
+        }
+        *(v4i *)(ob + (size_t)d * Tpad + 8 * c) = (v4i){(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a, int Tpad) {
+    __shared__ __align__(16) uint8_t smem[2 * AT_STAGE];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, half = lane >> 5;
+    const int h = blockIdx.y, b = blockIdx.z;
+    const int q0 = blockIdx.x * AT_BQ;
+
+    // ---- Q^T operand: lane (q, half) holds q[16 c + 8 half, +8) for c = 0..7, scaled and rounded to T ------------
+    const int qrow = min(q0 + wave * 32 + l32, a.Tq - 1);
+    const uint16_t *qp = (const uint16_t *)a.q + (long)b * a.sqb + (long)h * a.sqh + (long)qrow * a.sqm + 8 * half;
+    const float qscale = a.scale * 1.4426950408889634f;
+    v4i qop[8];
+#pragma unroll
+    for (int c = 0; c < 8; c++) {
+        const v4i raw = *(const v4i *)(qp + 16 * c);
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+            qop[c][e] = (int)pack2<T>(T::lo_f32((uint32_t)raw[e]) * qscale, T::hi_f32((uint32_t)raw[e]) * qscale);
+    }
+
+    // ---- tile loads: lane l of K load i fetches chunk (l % 16) ^ (row & 15) of key row 4 i + l / 16; of V^T load i,
+    // chunk (l % 8) ^ (row & 7) of d row 8 i + l / 8.  Four K loads and four V^T loads per wavefront and tile.
+    const uint8_t *kbase = (const uint8_t *)a.k + ((long)b * a.skb + (long)h * a.skh) * 2;
+    const uint8_t *vbase = (const uint8_t *)a.vt + ((size_t)(b * a.H + h) * AT_D) * Tpad * 2;
+    int krow[4];
+    uint32_t kch[4], voff[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int i = wave * 4 + j;
+        krow[j] = 4 * i + (lane >> 4);
+        kch[j] = (uint32_t)(((lane & 15) ^ (krow[j] & 15)) * 16);
+        const int vrow = 8 * i + (lane >> 3);
+        voff[j] = (uint32_t)vrow * (uint32_t)Tpad * 2 + (uint32_t)(((lane & 7) ^ (vrow & 7)) * 16);
+    }
+    auto issue = [&](int blk, int stage) {
+        const int k0 = blk * AT_BK;
+        uint8_t *dst = smem + stage * AT_STAGE;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint8_t *src = kbase + (long)min(k0 + krow[j], a.Tkv - 1) * a.skn * 2 + kch[j];
+            __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)src, (SVDQ_AS3 void *)(dst + (wave * 4 + j) * 1024), 16, 0, 0);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint8_t *src = vbase + (voff[j] + (uint32_t)k0 * 2);
+            __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)src,
+                                             (SVDQ_AS3 void *)(dst + AT_KT_BYTES + (wave * 4 + j) * 1024), 16, 0, 0);
+        }
+    };
+
+    // operand read offsets: K rows 32 t + l32 (chunk 2 c + half), V^T rows 32 dt + l32 (chunk 2 c + half)
+    int koff[8], vtoff[4];
+#pragma unroll
+    for (int c = 0; c < 8; c++) koff[c] = l32 * 256 + (((2 * c + half) ^ (l32 & 15)) * 16);
+#pragma unroll
+    for (int c = 0; c < 4; c++) vtoff[c] = AT_KT_BYTES + l32 * 128 + (((2 * c + half) ^ (l32 & 7)) * 16);
+
+    v16f acc_o[4];
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) acc_o[dt][i] = 0.0f;
+    float m_run = -INFINITY, l_run = 0.0f;
+    v16f zero16;
+#pragma unroll
+    for (int i = 0; i < 16; i++) zero16[i] = 0.0f;
+
+    const int nblk = (a.Tkv + AT_BK - 1) / AT_BK;
+    issue(0, 0);
+    for (int blk = 0; blk < nblk; blk++) {
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));  // this wavefront's share of tile blk has landed
+        __builtin_amdgcn_s_barrier();                    // everybody's has, and everybody is done with tile blk - 1
+        issue(min(blk + 1, nblk - 1), (blk + 1) & 1);    // past the end: the last tile again, into the idle stage
+        const uint8_t *st = smem + (blk & 1) * AT_STAGE;
+
+        // ---- S^T = K Q^T: two 32-key halves --------------------------------------------------------------------
+        v16f s[2];
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+#pragma unroll
+            for (int c = 0; c < 8; c++) {
+                const v4i kop = *(const v4i *)(st + t * (32 * 256) + koff[c]);
+                s[t] = mfma32_16bit<T>(kop, qop[c], c == 0 ? zero16 : s[t]);
+            }
+        }
+        if (blk == nblk - 1 && (a.Tkv & (AT_BK - 1))) {  // keys past the end count as -inf
+            const int k0 = blk * AT_BK;
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+#pragma unroll
+                for (int i = 0; i < 16; i++)
+                    if (k0 + 32 * t + 8 * (i >> 2) + 4 * half + (i & 3) >= a.Tkv) s[t][i] = -INFINITY;
+        }
+
+        // ---- online softmax: this lane's query, its 32 keys, then the other half's through lane ^ 32 ------------
+        float mx = s[0][0];
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) mx = fmaxf(mx, s[t][i]);
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m_run, mx);
+        if (__builtin_amdgcn_ballot_w64(m_new != m_run) != 0) {  // some maximum moved: rescale sum and accumulator
+            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+            l_run *= alpha;
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) acc_o[dt][i] *= alpha;
+            m_run = m_new;
+        }
+        // P^T operand: chunk cc of half t = accumulator quads j = 2 cc, 2 cc + 1
+        v4i pop[4];
+        float rs = 0.0f;
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+#pragma unroll
+            for (int cc = 0; cc < 2; cc++) {
+                float p[8];
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    p[e] = __builtin_amdgcn_exp2f(s[t][8 * cc + e] - m_run);
+                    rs += p[e];
+                }
+#pragma unroll
+                for (int e = 0; e < 4; e++) pop[2 * t + cc][e] = (int)pack2<T>(p[2 * e], p[2 * e + 1]);
+            }
+        l_run += rs;
+
+        // ---- O^T += V^T P^T --------------------------------------------------------------------------------------
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const v4i vop = *(const v4i *)(st + dt * (32 * 128) + vtoff[c]);
+                acc_o[dt] = mfma32_16bit<T>(vop, pop[c], acc_o[dt]);
+            }
+    }
+
+    // ---- O = O^T / l, staged through LDS so that rows leave as 256-byte segments -------------------------------------
+    l_run += __shfl_xor(l_run, 32);
+    const float inv = 1.0f / (l_run == 0.0f ? 1.0f : l_run);
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));  // the redundant last tile load has landed
+    __syncthreads();
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            uint2 w;
+            w.x = pack2<T>(acc_o[dt][4 * j] * inv, acc_o[dt][4 * j + 1] * inv);
+            w.y = pack2<T>(acc_o[dt][4 * j + 2] * inv, acc_o[dt][4 * j + 3] * inv);
+            *(uint2 *)(smem + (wave * 32 + l32) * AT_OPITCH + (32 * dt + 8 * j + 4 * half) * 2) = w;
+        }
+    __syncthreads();
+    uint16_t *op = (uint16_t *)a.o + (long)b * a.sob + (long)h * AT_D;
+    const int c = tid & 15;
+#pragma unroll
+    for (int pass = 0; pass < AT_BQ * 16 / 256; pass++) {
+        const int row = pass * 16 + (tid >> 4), q = q0 + row;
+        if (q < a.Tq) *(v4i *)(op + (long)q * a.som + 8 * c) = *(const v4i *)(smem + row * AT_OPITCH + c * 16);
+    }
+}
+
+}  // namespace svdq
+
+using namespace svdq;
+
+extern "C" size_t svdq_attention_workspace_bytes(int32_t B, int32_t H, int32_t Tkv, int32_t D) {
+    if (B <= 0 || H <= 0 || Tkv <= 0 || D != AT_D) return 0;
+    const size_t Tpad = (size_t)((Tkv + AT_BK - 1) / AT_BK) * AT_BK;
+    return (size_t)B * H * AT_D * Tpad * 2;
+}
+
+extern "C" int svdq_attention_fp16(const svdq_attention_args *args, void *stream) {
+    if (!args) {
+        set_error("svdq_attention_fp16: null args");
+        return SVDQ_E_INVALID;
+    }
+    const svdq_attention_args &a = *args;
+    if (a.dtype != SVDQ_BF16 && a.dtype != SVDQ_FP16) {
+        set_error("svdq_attention_fp16: dtype %d", a.dtype);
+        return SVDQ_E_INVALID;
+    }
+    if (a.D != AT_D) {
+        set_error("svdq_attention_fp16: head dimension %d is not supported (128 only)", a.D);
+        return SVDQ_E_UNSUPPORTED;
+    }
+    if (a.B <= 0 || a.H <= 0 || a.Tq < 0 || a.Tkv <= 0 || a.B > 65535 || a.H > 65535) {
+        set_error("svdq_attention_fp16: bad shape B=%d H=%d Tq=%d Tkv=%d", a.B, a.H, a.Tq, a.Tkv);
+        return SVDQ_E_INVALID;
+    }
+    if (!a.q || !a.k || !a.v || !a.o || !a.vt) {
+        set_error("svdq_attention_fp16: null tensor (q, k, v, o and the V^T workspace are required)");
+        return SVDQ_E_INVALID;
+    }
+    auto al = [](const void *p) { return ((uintptr_t)p & 15) == 0; };
+    if (!al(a.q) || !al(a.k) || !al(a.v) || !al(a.o) || !al(a.vt) || a.sqm % 8 || a.sqh % 8 || a.sqb % 8 || a.skn % 8 ||
+        a.skh % 8 || a.skb % 8 || a.svn % 8 || a.svh % 8 || a.svb % 8 || a.som % 8 || a.sob % 8) {
+        set_error("svdq_attention_fp16: tensors and their row / head / batch strides must be 16-byte aligned");
+        return SVDQ_E_INVALID;
+    }
+    if (a.Tq == 0) return SVDQ_OK;
+    const int Tpad = (a.Tkv + AT_BK - 1) / AT_BK * AT_BK;
+    if ((size_t)AT_D * Tpad * 2 >= ((size_t)1 << 32)) {
+        set_error("svdq_attention_fp16: Tkv=%d too long for 32-bit tile offsets", a.Tkv);
+        return SVDQ_E_UNSUPPORTED;
+    }
+    hipStream_t s = (hipStream_t)stream;
+    hipLaunchKernelGGL(transpose_v_kernel, dim3(Tpad / AT_BK, a.H, a.B), dim3(256), 0, s, (const uint16_t *)a.v,
+                       (uint16_t *)a.vt, a.H, a.Tkv, Tpad, (long)a.svb, (long)a.svh, (long)a.svn);
+    const dim3 grid((a.Tq + AT_BQ - 1) / AT_BQ, a.H, a.B);
+    if (a.dtype == SVDQ_BF16)
+        hipLaunchKernelGGL((attention_kernel<BF16>), grid, dim3(256), 0, s, a, Tpad);
+    else
+        hipLaunchKernelGGL((attention_kernel<FP16>), grid, dim3(256), 0, s, a, Tpad);
+    return check_launch("svdq_attention_fp16");
+}

@@ -1,5 +1,6 @@
 """Operator API of the SVDQuant path: same names and signatures as ``nunchaku.ops`` in the reference."""
 
+from .attention import attention_fp16, scaled_dot_product_attention
 from .fused import fused_gelu_mlp, fused_qkv_norm_rottary, fused_swiglu_mlp, interleave_swiglu_linear_
 from .gemm import svdq_gemm_w4a4_cuda
 from .gemv import awq_gemv_w4a16_cuda
@@ -13,4 +14,6 @@ __all__ = [
     "fused_qkv_norm_rottary",
     "fused_swiglu_mlp",
     "interleave_swiglu_linear_",
+    "attention_fp16",
+    "scaled_dot_product_attention",
 ]

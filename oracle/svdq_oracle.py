@@ -30,6 +30,9 @@ awq_pack / awq_decode  mutual inverse, written from two different statements
                        of the layout (view/permute vs. index formula)
 awq_gemv               fp64 dense dequantised matmul
 flux_rope              closed form cos/sin of pos * theta**(-2i/d) in fp64
+attention_fp16         fp64 softmax(q k^T * scale) v, independence of the key
+                       block size, uniform-weights / constant-v / dominant-key
+                       special cases
 =====================  =======================================================
 
 Floating point: every elementwise op below is an IEEE fp32 primitive on CPU
@@ -305,6 +308,34 @@ def awq_gemv(x: torch.Tensor, packed_i16: torch.Tensor, scales: torch.Tensor, ze
         xsum = xf[:, sl].sum(dim=1, keepdim=True)
         out += scales[c].float()[None, :] * dotq + zeros[c].float()[None, :] * xsum
     return out
+
+
+# --------------------------------------------------------------------------------------
+# Unmasked 16-bit attention
+# --------------------------------------------------------------------------------------
+def attention_fp16(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float, block_n: int = 64) -> torch.Tensor:
+    """nunchaku/ops/triton/attention.py:62-119, :139-141: q (B, H, Tq, D), k / v (B, H, Tkv, D) in fp16 or bf16 ->
+    (B, Tq, H * D) of the same type.  q * (scale * log2 e) is rounded to the 16-bit type; per block of ``block_n``
+    keys the scores are fp32, the running maximum m and sum l are fp32, p = exp2(s - m) is rounded to the 16-bit type
+    for the p @ v product (fp32 accumulation) but enters l unrounded; the result is acc / l."""
+    dt = q.dtype
+    B, H, Tq, D = q.shape
+    Tkv = k.shape[2]
+    qs = (q.float() * (scale * 1.4426950408889634)).to(dt).float()
+    kf, vf = k.float(), v.float()
+    m = torch.full((B, H, Tq), float("-inf"))
+    l = torch.zeros(B, H, Tq)
+    acc = torch.zeros(B, H, Tq, D)
+    for n0 in range(0, Tkv, block_n):
+        s = qs @ kf[:, :, n0 : n0 + block_n].transpose(-1, -2)
+        m_new = torch.maximum(m, s.amax(dim=-1))
+        p = torch.exp2(s - m_new[..., None])
+        alpha = torch.exp2(m - m_new)  # exp2(-inf) = 0 on the first block
+        l = l * alpha + p.sum(dim=-1)
+        acc = acc * alpha[..., None] + p.to(dt).float() @ vf[:, :, n0 : n0 + block_n]
+        m = m_new
+    out = acc / torch.where(l == 0, torch.ones_like(l), l)[..., None]
+    return out.to(dt).transpose(1, 2).reshape(B, Tq, H * D)
 
 
 # --------------------------------------------------------------------------------------

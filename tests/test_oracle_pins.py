@@ -296,3 +296,61 @@ def test_flux_rotary_closed_form():
         ang = axis_pos * 10000.0 ** (-(2 * i) / d)
         assert abs(rot[t, pair, 0, 0].item() - math.sin(ang)) < 1e-6
         assert abs(rot[t, pair, 0, 1].item() - math.cos(ang)) < 1e-6
+
+
+# ---- attention ------------------------------------------------------------------------------------------------------
+def _attn_inputs(B, H, Tq, Tkv, dtype, seed, spread=1.0):
+    g = torch.Generator().manual_seed(seed)
+    q = (torch.randn(B, H, Tq, 128, generator=g) * spread).to(dtype)
+    k = (torch.randn(B, H, Tkv, 128, generator=g) * spread).to(dtype)
+    v = torch.randn(B, H, Tkv, 128, generator=g).to(dtype)
+    return q, k, v
+
+
+def _attn_fp64(q, k, v, scale):
+    w = torch.softmax(q.double() @ k.double().transpose(-1, -2) * scale, dim=-1)
+    o = w @ v.double()
+    return o.transpose(1, 2).reshape(q.shape[0], q.shape[2], -1)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("Tq,Tkv,block", [(70, 200, 64), (33, 64, 64), (5, 131, 32), (40, 77, 128)])
+def test_attention_against_fp64_softmax(dtype, Tq, Tkv, block):
+    q, k, v = _attn_inputs(2, 3, Tq, Tkv, dtype, seed=Tq + Tkv, spread=1.5)
+    scale = 128**-0.5
+    got = O.attention_fp16(q, k, v, scale, block_n=block).double()
+    ref = _attn_fp64(q, k, v, scale)
+    # the only roundings are q * scale, p and the output, each to the 16-bit type: 2^-8 relative for bf16
+    tol = 2e-2 if dtype == torch.bfloat16 else 3e-3
+    assert (got - ref).abs().max() <= tol * ref.abs().max()
+    assert got.shape == (2, Tq, 3 * 128)
+
+
+def test_attention_special_cases():
+    scale = 128**-0.5
+    q, k, v = _attn_inputs(1, 2, 16, 96, torch.float16, seed=5)
+    # q = 0: uniform weights, the output is the mean of v over the keys (heads side by side in the last dimension)
+    o = O.attention_fp16(torch.zeros_like(q), k, v, scale, block_n=32).double()
+    mean = v.double().mean(dim=2)  # (1, 2, 128)
+    assert (o - mean.reshape(1, 1, 256)).abs().max() < 2e-3
+    # constant v rows: any weights return that row
+    vc = v[:, :, :1].expand_as(v).contiguous()
+    o = O.attention_fp16(q, k, vc, scale).double()
+    assert (o - vc[:, :, 0].double().reshape(1, 1, 256)).abs().max() < 2e-3
+    # one key dominates query t: the output row is that key's v (key index differs per query: a transposed or
+    # mis-indexed product cannot pass)
+    kk = torch.zeros(1, 2, 96, 128)
+    qq = torch.zeros(1, 2, 16, 128)
+    for t in range(16):
+        qq[0, :, t, t] = 60.0
+        kk[0, 0, 3 * t + 1, t] = 60.0
+        kk[0, 1, 95 - 2 * t, t] = 60.0
+    o = O.attention_fp16(qq.half(), kk.half(), v, scale, block_n=32).float()
+    for t in range(16):
+        assert torch.allclose(o[0, t, :128], v[0, 0, 3 * t + 1].float(), atol=1e-3)
+        assert torch.allclose(o[0, t, 128:], v[0, 1, 95 - 2 * t].float(), atol=1e-3)
+    # the key block size is an implementation choice: results agree to the rounding of p
+    q, k, v = _attn_inputs(1, 1, 48, 300, torch.bfloat16, seed=9, spread=2.0)
+    a = O.attention_fp16(q, k, v, scale, block_n=16).float()
+    b = O.attention_fp16(q, k, v, scale, block_n=300).float()
+    assert (a - b).abs().max() <= 2e-2 * b.abs().max()
