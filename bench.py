@@ -23,6 +23,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 INT8_MFMA_PEAK_TOPS = 5000.0  # MI355X dense int8 MFMA, published
+BF16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 / fp16 MFMA, published
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # HBM bytes of one QKV GEMM launch: FETCH_SIZE + WRITE_SIZE (KiB per dispatch, counter scale 1.000) of the grid-1327104
 # launches in profiles/bench_all_kernels_hbm_traffic.txt; counters cannot be read from inside this process
@@ -215,6 +216,16 @@ def main():
             nbytes = 18432 * 3072 // 2 + 2 * 2 * 48 * 18432 + 2 * m * 3072 + 2 * m * 18432
             kernels[f"awq_gemv_w4a16 M{m} K3072 N18432"] = {"ms": round(ms, 5), "GB/s": round(nbytes / ms / 1e6, 1),
                                                            "frac_hbm": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4), "bytes": nbytes}  # fmt: skip
+
+        # joint attention of one FLUX.1 block: 24 heads, 512 + 4096 tokens, q / k / v strided views of the fused projection
+        qkv_t = torch.randn(1, M, 3 * 3072, device=dev).to(torch.bfloat16)
+        aq, ak, av = (qkv_t[..., i * 3072 : (i + 1) * 3072].view(1, M, 24, 128).transpose(1, 2) for i in range(3))
+        ao = torch.empty(1, M, 3072, dtype=torch.bfloat16, device=dev)
+        ms = _time_kernel(lambda: ops.attention_fp16(aq, ak, av, ao, 128**-0.5))
+        fl = 4.0 * M * M * 128 * 24
+        kernels["attention bf16 H24 T4608 D128"] = {"ms": round(ms, 5), "TFLOP/s": round(fl / ms / 1e9, 1),
+                                                     "frac_bf16_mfma": round(fl / ms / 1e9 / BF16_MFMA_PEAK_TFLOPS, 4)}  # fmt: skip
+        del qkv_t, aq, ak, av, ao
 
         # FLUX.1-schnell-shaped transformer, 4 denoising steps at 1024^2 (4096 image + 512 text tokens)
         from nunchaku_rocm_amd.flux_shaped import FluxShapedConfig, FluxShapedTransformer, flux_ids, rope_table

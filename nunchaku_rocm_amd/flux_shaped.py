@@ -61,6 +61,10 @@ class HipBackend:
     def awq(x, lin: AWQW4A16Linear):
         return lin(x)
 
+    @staticmethod
+    def attention(q, k, v):
+        return _ops.scaled_dot_product_attention(q, k, v)
+
 
 def rope_table(ids: torch.Tensor, axes_dim, theta: float) -> torch.Tensor:
     """(T, n_axes) positions -> (T, sum(axes_dim) / 2, 1, 2) float32 rows of (sin, cos), computed in float64."""
@@ -140,7 +144,7 @@ class _Attention(nn.Module):
             qkv_ctx = be.qkv(ctx, self.add_qkv_proj, self.norm_added_q, self.norm_added_k, rot_txt)
             qkv = torch.cat([qkv_ctx, qkv], dim=1)  # token order [txt, img]
         q, k, v = (t.view(B, -1, self.heads, self.head_dim).transpose(1, 2) for t in qkv.chunk(3, dim=-1))
-        o = F.scaled_dot_product_attention(q, k, v)  # (B, H, T, D), scale D^-0.5, no mask
+        o = be.attention(q, k, v)  # (B, H, T, D), scale D^-0.5, no mask
         o = o.transpose(1, 2).reshape(B, -1, self.heads * self.head_dim).to(q.dtype)
         if self.joint:
             t_txt = ctx.shape[1]

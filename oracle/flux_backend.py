@@ -1,4 +1,4 @@
-"""Oracle implementation of the four quantized operators the FLUX.1-shaped harness calls (TEST INFRASTRUCTURE).
+"""Oracle implementation of the four quantized operators and the attention the FLUX.1-shaped harness calls (TEST INFRASTRUCTURE).
 
 Plain torch arithmetic from ``svdq_oracle`` on whatever device the tensors live on, so the same transformer graph can
 be evaluated without the HIP library: on the CPU for small configurations, and with ``dense=True`` (one fp32 matmul
@@ -43,3 +43,7 @@ class OracleBackend:
         if lin.bias is not None:
             y = y + lin.bias
         return y
+
+    def attention(self, q, k, v):
+        """fp32 softmax(q k^T / sqrt(D)) v on the tensors' device, rounded once to the input type."""
+        return torch.nn.functional.scaled_dot_product_attention(q.float(), k.float(), v.float()).to(q.dtype)
