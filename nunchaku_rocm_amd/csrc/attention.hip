@@ -64,15 +64,29 @@ __global__ __launch_bounds__(256) void transpose_v_kernel(const uint16_t *v, uin
     }
 }
 
+constexpr uint32_t AT_RSRC_FLAGS = 0x00020000;  // raw buffer, 32-bit data format (gfx9 family)
+constexpr float AT_LAZY = 8.0f;                 // the accumulator is rescaled when a row maximum grew by more than this
+
 template <typename T>
-__global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a, int Tpad) {
+__global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a, int Tpad, int ntile, int xcd_heads) {
     __shared__ __align__(16) uint8_t smem[2 * AT_STAGE];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31, half = lane >> 5;
-    const int h = blockIdx.y, b = blockIdx.z;
-    const int q0 = blockIdx.x * AT_BQ;
+    // workgroup -> (batch * head, query tile).  Workgroups are dealt to the eight XCDs round-robin; when the head count
+    // allows it, a head's query tiles all land on one XCD so that its K and V^T stay in that XCD's L2.
+    int bh, qt;
+    if (xcd_heads) {
+        const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
+        bh = (j / ntile) * 8 + xcd;
+        qt = j % ntile;
+    } else {
+        bh = blockIdx.x / ntile;
+        qt = blockIdx.x % ntile;
+    }
+    const int b = bh / a.H, h = bh % a.H;
+    const int q0 = qt * AT_BQ;
 
     // ---- Q^T operand: lane (q, half) holds q[16 c + 8 half, +8) for c = 0..7, scaled and rounded to T ------------
     const int qrow = min(q0 + wave * 32 + l32, a.Tq - 1);
@@ -87,34 +101,33 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a
             qop[c][e] = (int)pack2<T>(T::lo_f32((uint32_t)raw[e]) * qscale, T::hi_f32((uint32_t)raw[e]) * qscale);
     }
 
-    // ---- tile loads: lane l of K load i fetches chunk (l % 16) ^ (row & 15) of key row 4 i + l / 16; of V^T load i,
-    // chunk (l % 8) ^ (row & 7) of d row 8 i + l / 8.  Four K loads and four V^T loads per wavefront and tile.
+    // ---- tile loads (buffer -> LDS, 16 bytes per lane): lane l of K load i fetches chunk (l % 16) ^ (row & 15) of key
+    // row 4 i + l / 16; of V^T load i, chunk (l % 8) ^ (row / 2 & 7) of d row 8 i + l / 8 (rows are 128 bytes: two rows span the 64 banks).  Four K and four V^T loads per
+    // wavefront and tile.  The per-lane offsets never change; the tile is selected by the (scalar) buffer base, and
+    // key rows past the end lie outside the K buffer's range and arrive as zeros.
     const uint8_t *kbase = (const uint8_t *)a.k + ((long)b * a.skb + (long)h * a.skh) * 2;
-    const uint8_t *vbase = (const uint8_t *)a.vt + ((size_t)(b * a.H + h) * AT_D) * Tpad * 2;
-    int krow[4];
-    uint32_t kch[4], voff[4];
+    const uint8_t *vbase = (const uint8_t *)a.vt + ((size_t)bh * AT_D) * Tpad * 2;
+    const uint32_t kbytes = (uint32_t)(((long)(a.Tkv - 1) * a.skn + AT_D) * 2);
+    const uint32_t ktile = (uint32_t)(AT_BK * a.skn * 2);
+    uint32_t kvo[4], vvo[4];
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         const int i = wave * 4 + j;
-        krow[j] = 4 * i + (lane >> 4);
-        kch[j] = (uint32_t)(((lane & 15) ^ (krow[j] & 15)) * 16);
+        const int krow = 4 * i + (lane >> 4);
+        kvo[j] = (uint32_t)krow * (uint32_t)(a.skn * 2) + (uint32_t)(((lane & 15) ^ (krow & 15)) * 16);
         const int vrow = 8 * i + (lane >> 3);
-        voff[j] = (uint32_t)vrow * (uint32_t)Tpad * 2 + (uint32_t)(((lane & 7) ^ (vrow & 7)) * 16);
+        vvo[j] = (uint32_t)vrow * (uint32_t)Tpad * 2 + (uint32_t)(((lane & 7) ^ ((vrow >> 1) & 7)) * 16);
     }
-    auto issue = [&](int blk, int stage) {
-        const int k0 = blk * AT_BK;
-        uint8_t *dst = smem + stage * AT_STAGE;
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const uint8_t *src = kbase + (long)min(k0 + krow[j], a.Tkv - 1) * a.skn * 2 + kch[j];
-            __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)src, (SVDQ_AS3 void *)(dst + (wave * 4 + j) * 1024), 16, 0, 0);
-        }
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const uint8_t *src = vbase + (voff[j] + (uint32_t)k0 * 2);
-            __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)src,
-                                             (SVDQ_AS3 void *)(dst + AT_KT_BYTES + (wave * 4 + j) * 1024), 16, 0, 0);
-        }
+    const __amdgpu_buffer_rsrc_t vres = __builtin_amdgcn_make_buffer_rsrc((void *)vbase, 0, AT_D * Tpad * 2, AT_RSRC_FLAGS);
+    auto issue_k = [&](int blk, int stage, int j) {
+        const uint32_t off = (uint32_t)blk * ktile;
+        const __amdgpu_buffer_rsrc_t kres = __builtin_amdgcn_make_buffer_rsrc((void *)(kbase + off), 0, kbytes - off, AT_RSRC_FLAGS);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(kres, (SVDQ_AS3 void *)(smem + stage * AT_STAGE + (wave * 4 + j) * 1024), 16,
+                                                 kvo[j], 0, 0, 0);
+    };
+    auto issue_v = [&](int blk, int stage, int j) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(vres, (SVDQ_AS3 void *)(smem + stage * AT_STAGE + AT_KT_BYTES + (wave * 4 + j) * 1024),
+                                                 16, vvo[j], blk * (AT_BK * 2), 0, 0);
     };
 
     // operand read offsets: K rows 32 t + l32 (chunk 2 c + half), V^T rows 32 dt + l32 (chunk 2 c + half)
@@ -122,35 +135,51 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a
 #pragma unroll
     for (int c = 0; c < 8; c++) koff[c] = l32 * 256 + (((2 * c + half) ^ (l32 & 15)) * 16);
 #pragma unroll
-    for (int c = 0; c < 4; c++) vtoff[c] = AT_KT_BYTES + l32 * 128 + (((2 * c + half) ^ (l32 & 7)) * 16);
+    for (int c = 0; c < 4; c++) vtoff[c] = AT_KT_BYTES + l32 * 128 + (((2 * c + half) ^ ((l32 >> 1) & 7)) * 16);
 
     v16f acc_o[4];
 #pragma unroll
     for (int dt = 0; dt < 4; dt++)
 #pragma unroll
         for (int i = 0; i < 16; i++) acc_o[dt][i] = 0.0f;
-    float m_run = -INFINITY, l_run = 0.0f;
+    float m_ref = -INFINITY, l_run = 0.0f;  // p = 2^(s - m_ref); m_ref trails the true row maximum by at most AT_LAZY
     v16f zero16;
 #pragma unroll
     for (int i = 0; i < 16; i++) zero16[i] = 0.0f;
 
     const int nblk = (a.Tkv + AT_BK - 1) / AT_BK;
-    issue(0, 0);
+#pragma unroll
+    for (int j = 0; j < 4; j++) issue_k(0, 0, j);
+#pragma unroll
+    for (int j = 0; j < 4; j++) issue_v(0, 0, j);
     for (int blk = 0; blk < nblk; blk++) {
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));  // this wavefront's share of tile blk has landed
         __builtin_amdgcn_s_barrier();                    // everybody's has, and everybody is done with tile blk - 1
-        issue(min(blk + 1, nblk - 1), (blk + 1) & 1);    // past the end: the last tile again, into the idle stage
         const uint8_t *st = smem + (blk & 1) * AT_STAGE;
+        const int nxt = min(blk + 1, nblk - 1), nst = (blk + 1) & 1;  // past the end: the last tile again, idle stage
 
-        // ---- S^T = K Q^T: two 32-key halves --------------------------------------------------------------------
+        // ---- S^T = K Q^T: two 32-key halves (independent accumulators, alternating); all sixteen operand reads go out
+        // first, the next tile's loads are spread between the matrix instructions -----------------------------------
+        v4i ra[8], rb[8];
+#pragma unroll
+        for (int c = 0; c < 8; c++) {
+            ra[c] = *(const v4i *)(st + koff[c]);
+            rb[c] = *(const v4i *)(st + 32 * 256 + koff[c]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
         v16f s[2];
 #pragma unroll
-        for (int t = 0; t < 2; t++) {
+        for (int c = 0; c < 8; c++) {
+            s[0] = mfma32_16bit<T>(ra[c], qop[c], c == 0 ? zero16 : s[0]);
+            s[1] = mfma32_16bit<T>(rb[c], qop[c], c == 0 ? zero16 : s[1]);
+            if (c & 1) issue_k(nxt, nst, c >> 1); else issue_v(nxt, nst, c >> 1);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // V^T operands (d rows 0..63, 64..127) into the registers K has left; they arrive under the softmax
 #pragma unroll
-            for (int c = 0; c < 8; c++) {
-                const v4i kop = *(const v4i *)(st + t * (32 * 256) + koff[c]);
-                s[t] = mfma32_16bit<T>(kop, qop[c], c == 0 ? zero16 : s[t]);
-            }
+        for (int c = 0; c < 8; c++) {
+            ra[c] = *(const v4i *)(st + (c >> 2) * (32 * 128) + vtoff[c & 3]);
+            rb[c] = *(const v4i *)(st + (2 + (c >> 2)) * (32 * 128) + vtoff[c & 3]);
         }
         if (blk == nblk - 1 && (a.Tkv & (AT_BK - 1))) {  // keys past the end count as -inf
             const int k0 = blk * AT_BK;
@@ -168,15 +197,15 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a
 #pragma unroll
             for (int i = 0; i < 16; i++) mx = fmaxf(mx, s[t][i]);
         mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(m_run, mx);
-        if (__builtin_amdgcn_ballot_w64(m_new != m_run) != 0) {  // some maximum moved: rescale sum and accumulator
-            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+        if (__builtin_amdgcn_ballot_w64(mx > m_ref + AT_LAZY) != 0) {  // some maximum ran away: move every reference
+            const float m_new = fmaxf(m_ref, mx);
+            const float alpha = __builtin_amdgcn_exp2f(m_ref - m_new);  // 0 on the first tile (m_ref = -inf)
             l_run *= alpha;
 #pragma unroll
             for (int dt = 0; dt < 4; dt++)
 #pragma unroll
                 for (int i = 0; i < 16; i++) acc_o[dt][i] *= alpha;
-            m_run = m_new;
+            m_ref = m_new;
         }
         // P^T operand: chunk cc of half t = accumulator quads j = 2 cc, 2 cc + 1
         v4i pop[4];
@@ -188,22 +217,20 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a
                 float p[8];
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
-                    p[e] = __builtin_amdgcn_exp2f(s[t][8 * cc + e] - m_run);
+                    p[e] = __builtin_amdgcn_exp2f(s[t][8 * cc + e] - m_ref);
                     rs += p[e];
                 }
 #pragma unroll
                 for (int e = 0; e < 4; e++) pop[2 * t + cc][e] = (int)pack2<T>(p[2 * e], p[2 * e + 1]);
             }
         l_run += rs;
+        __builtin_amdgcn_sched_barrier(0);
 
         // ---- O^T += V^T P^T --------------------------------------------------------------------------------------
 #pragma unroll
-        for (int dt = 0; dt < 4; dt++)
+        for (int c = 0; c < 8; c++) acc_o[c >> 2] = mfma32_16bit<T>(ra[c], pop[c & 3], acc_o[c >> 2]);
 #pragma unroll
-            for (int c = 0; c < 4; c++) {
-                const v4i vop = *(const v4i *)(st + dt * (32 * 128) + vtoff[c]);
-                acc_o[dt] = mfma32_16bit<T>(vop, pop[c], acc_o[dt]);
-            }
+        for (int c = 0; c < 8; c++) acc_o[2 + (c >> 2)] = mfma32_16bit<T>(rb[c], pop[c & 3], acc_o[2 + (c >> 2)]);
     }
 
     // ---- O = O^T / l, staged through LDS so that rows leave as 256-byte segments -------------------------------------
@@ -270,17 +297,24 @@ extern "C" int svdq_attention_fp16(const svdq_attention_args *args, void *stream
     }
     if (a.Tq == 0) return SVDQ_OK;
     const int Tpad = (a.Tkv + AT_BK - 1) / AT_BK * AT_BK;
-    if ((size_t)AT_D * Tpad * 2 >= ((size_t)1 << 32)) {
-        set_error("svdq_attention_fp16: Tkv=%d too long for 32-bit tile offsets", a.Tkv);
+    if ((size_t)AT_D * Tpad * 2 >= ((size_t)1 << 31) || ((size_t)Tpad * a.skn + AT_D) * 2 >= ((size_t)1 << 31) ||
+        (size_t)a.B * a.H * ((a.Tq + AT_BQ - 1) / AT_BQ) >= ((size_t)1 << 31)) {
+        set_error("svdq_attention_fp16: Tq=%d Tkv=%d key stride %lld: too large for 32-bit tile offsets", a.Tq, a.Tkv, (long long)a.skn);
         return SVDQ_E_UNSUPPORTED;
+    }
+    if (a.skn < AT_D) {
+        set_error("svdq_attention_fp16: key rows overlap (stride %lld < 128)", (long long)a.skn);
+        return SVDQ_E_INVALID;
     }
     hipStream_t s = (hipStream_t)stream;
     hipLaunchKernelGGL(transpose_v_kernel, dim3(Tpad / AT_BK, a.H, a.B), dim3(256), 0, s, (const uint16_t *)a.v,
                        (uint16_t *)a.vt, a.H, a.Tkv, Tpad, (long)a.svb, (long)a.svh, (long)a.svn);
-    const dim3 grid((a.Tq + AT_BQ - 1) / AT_BQ, a.H, a.B);
+    const int ntile = (a.Tq + AT_BQ - 1) / AT_BQ;
+    const int xcd_heads = (a.B * a.H) % 8 == 0;
+    const dim3 grid((unsigned)(ntile * a.H * a.B));
     if (a.dtype == SVDQ_BF16)
-        hipLaunchKernelGGL((attention_kernel<BF16>), grid, dim3(256), 0, s, a, Tpad);
+        hipLaunchKernelGGL((attention_kernel<BF16>), grid, dim3(256), 0, s, a, Tpad, ntile, xcd_heads);
     else
-        hipLaunchKernelGGL((attention_kernel<FP16>), grid, dim3(256), 0, s, a, Tpad);
+        hipLaunchKernelGGL((attention_kernel<FP16>), grid, dim3(256), 0, s, a, Tpad, ntile, xcd_heads);
     return check_launch("svdq_attention_fp16");
 }
