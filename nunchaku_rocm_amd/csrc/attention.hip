@@ -148,89 +148,140 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a
     for (int i = 0; i < 16; i++) zero16[i] = 0.0f;
 
     const int nblk = (a.Tkv + AT_BK - 1) / AT_BK;
+    // Software pipeline.  Tile t lives in stage t & 1 and is handled as two halves of 32 keys, each a complete online-
+    // softmax step, so that the softmax arithmetic of one half is issued between the matrix instructions of the other:
+    //   (A) S0 = K[0:32] Q^T                            + V^T operand reads (keys 0..31)
+    //   (B) S1 = K[32:64] Q^T         ||  softmax(S0)   + V^T operand reads (keys 32..63)
+    //   (C) O^T += V^T[:, 0:32] P0^T  ||  softmax(S1)
+    //       barrier: tile t + 1 has landed for everybody, nobody reads tile t any more
+    //   (D) O^T += V^T[:, 32:64] P1^T                   + K operand reads of tile t + 1, loads of tile t + 2 into
+    //                                                     the stage tile t has left
+    // The compiler is kept from regrouping the slots (one matrix instruction plus its share of the rest).
 #pragma unroll
     for (int j = 0; j < 4; j++) issue_k(0, 0, j);
 #pragma unroll
     for (int j = 0; j < 4; j++) issue_v(0, 0, j);
+    {
+        const int t1 = min(1, nblk - 1);
+#pragma unroll
+        for (int j = 0; j < 4; j++) issue_k(t1, 1, j);
+#pragma unroll
+        for (int j = 0; j < 4; j++) issue_v(t1, 1, j);
+    }
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(8, 15));  // tile 0 (the older eight loads)
+    __builtin_amdgcn_s_barrier();
+    v4i rk[16], rv[16];  // rk[8 t + c]: K rows 32 t.., chunk c;  rv[4 dt + c]: V^T rows 32 dt.., 16-key chunk c
+#pragma unroll
+    for (int c = 0; c < 8; c++) {
+        rk[c] = *(const v4i *)(smem + koff[c]);
+        rk[8 + c] = *(const v4i *)(smem + 32 * 256 + koff[c]);
+    }
+
+    float m_new, alpha, rs;  // rs: this half's row sum, at the new reference
+    // row maximum of one half (16 scores of this lane, 16 of lane ^ 32), the lazily updated reference and the factor
+    // that moves the accumulator to it; returns whether any lane of the wavefront moved
+    auto row_max = [&](const v16f &sv) -> bool {
+        float mx = fmaxf(fmaxf(sv[0], sv[1]), sv[2]);
+#pragma unroll
+        for (int i = 3; i < 15; i += 2) mx = fmaxf(fmaxf(mx, sv[i]), sv[i + 1]);
+        mx = fmaxf(mx, sv[15]);
+        const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
+        mx = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+        const bool need = mx > m_ref + AT_LAZY;
+        m_new = need ? mx : m_ref;
+        alpha = __builtin_amdgcn_exp2f(m_ref - m_new);  // 1 when nothing moved, 0 on the first tile (m_ref = -inf)
+        m_ref = m_new;
+        return __builtin_amdgcn_ballot_w64(need) != 0;
+    };
+    // four scores -> two packed P values
+    auto exp4 = [&](const v16f &sv, int i0, v4i &pw, int e0) {
+        float p[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            p[e] = __builtin_amdgcn_exp2f(sv[i0 + e] - m_new);
+            rs += p[e];
+        }
+        pw[e0] = (int)pack2<T>(p[0], p[1]);
+        pw[e0 + 1] = (int)pack2<T>(p[2], p[3]);
+    };
+    auto rescale = [&]() {
+        l_run *= alpha;
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc_o[dt][i] *= alpha;
+    };
+
     for (int blk = 0; blk < nblk; blk++) {
-        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));  // this wavefront's share of tile blk has landed
-        __builtin_amdgcn_s_barrier();                    // everybody's has, and everybody is done with tile blk - 1
         const uint8_t *st = smem + (blk & 1) * AT_STAGE;
-        const int nxt = min(blk + 1, nblk - 1), nst = (blk + 1) & 1;  // past the end: the last tile again, idle stage
+        const uint8_t *sn = smem + ((blk + 1) & 1) * AT_STAGE;
+        const int nxt = min(blk + 2, nblk - 1);  // past the end: the last tile again, into a stage nobody reads
+        const bool ragged = blk == nblk - 1 && (a.Tkv & (AT_BK - 1));
+        v16f s0, s1;
+        v4i pop[4];  // P^T operand: chunk cc of half t = accumulator quads 2 cc, 2 cc + 1 of S_t
 
-        // ---- S^T = K Q^T: two 32-key halves (independent accumulators, alternating); all sixteen operand reads go out
-        // first, the next tile's loads are spread between the matrix instructions -----------------------------------
-        v4i ra[8], rb[8];
+        // ---- (A) ---------------------------------------------------------------------------------------------------------
 #pragma unroll
         for (int c = 0; c < 8; c++) {
-            ra[c] = *(const v4i *)(st + koff[c]);
-            rb[c] = *(const v4i *)(st + 32 * 256 + koff[c]);
+            s0 = mfma32_16bit<T>(rk[c], qop[c], c == 0 ? zero16 : s0);
+            rv[4 * (c & 3) + (c >> 2)] = *(const v4i *)(st + (c & 3) * (32 * 128) + vtoff[c >> 2]);  // chunks 0, 1: keys 0..31
+            __builtin_amdgcn_sched_barrier(0);
         }
-        __builtin_amdgcn_sched_barrier(0);
-        v16f s[2];
+        if (ragged) {  // keys past the end count as -inf
 #pragma unroll
-        for (int c = 0; c < 8; c++) {
-            s[0] = mfma32_16bit<T>(ra[c], qop[c], c == 0 ? zero16 : s[0]);
-            s[1] = mfma32_16bit<T>(rb[c], qop[c], c == 0 ? zero16 : s[1]);
-            if (c & 1) issue_k(nxt, nst, c >> 1); else issue_v(nxt, nst, c >> 1);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        // V^T operands (d rows 0..63, 64..127) into the registers K has left; they arrive under the softmax
-#pragma unroll
-        for (int c = 0; c < 8; c++) {
-            ra[c] = *(const v4i *)(st + (c >> 2) * (32 * 128) + vtoff[c & 3]);
-            rb[c] = *(const v4i *)(st + (2 + (c >> 2)) * (32 * 128) + vtoff[c & 3]);
-        }
-        if (blk == nblk - 1 && (a.Tkv & (AT_BK - 1))) {  // keys past the end count as -inf
-            const int k0 = blk * AT_BK;
-#pragma unroll
-            for (int t = 0; t < 2; t++)
-#pragma unroll
-                for (int i = 0; i < 16; i++)
-                    if (k0 + 32 * t + 8 * (i >> 2) + 4 * half + (i & 3) >= a.Tkv) s[t][i] = -INFINITY;
+            for (int i = 0; i < 16; i++)
+                if (blk * AT_BK + 8 * (i >> 2) + 4 * half + (i & 3) >= a.Tkv) s0[i] = -INFINITY;
         }
 
-        // ---- online softmax: this lane's query, its 32 keys, then the other half's through lane ^ 32 ------------
-        float mx = s[0][0];
+        // ---- (B) ---------------------------------------------------------------------------------------------------------
+        bool moved = false;
 #pragma unroll
-        for (int t = 0; t < 2; t++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) mx = fmaxf(mx, s[t][i]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        if (__builtin_amdgcn_ballot_w64(mx > m_ref + AT_LAZY) != 0) {  // some maximum ran away: move every reference
-            const float m_new = fmaxf(m_ref, mx);
-            const float alpha = __builtin_amdgcn_exp2f(m_ref - m_new);  // 0 on the first tile (m_ref = -inf)
-            l_run *= alpha;
-#pragma unroll
-            for (int dt = 0; dt < 4; dt++)
-#pragma unroll
-                for (int i = 0; i < 16; i++) acc_o[dt][i] *= alpha;
-            m_ref = m_new;
-        }
-        // P^T operand: chunk cc of half t = accumulator quads j = 2 cc, 2 cc + 1
-        v4i pop[4];
-        float rs = 0.0f;
-#pragma unroll
-        for (int t = 0; t < 2; t++)
-#pragma unroll
-            for (int cc = 0; cc < 2; cc++) {
-                float p[8];
-#pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    p[e] = __builtin_amdgcn_exp2f(s[t][8 * cc + e] - m_ref);
-                    rs += p[e];
-                }
-#pragma unroll
-                for (int e = 0; e < 4; e++) pop[2 * t + cc][e] = (int)pack2<T>(p[2 * e], p[2 * e + 1]);
+        for (int c = 0; c < 8; c++) {
+            s1 = mfma32_16bit<T>(rk[8 + c], qop[c], c == 0 ? zero16 : s1);
+            rv[4 * (c & 3) + 2 + (c >> 2)] = *(const v4i *)(st + (c & 3) * (32 * 128) + vtoff[2 + (c >> 2)]);  // keys 32..63
+            if (c == 0) {
+                moved = row_max(s0);
+                rs = 0.0f;
             }
+            if (c >= 1 && c <= 4) exp4(s0, 4 * (c - 1), pop[(c - 1) >> 1], 2 * ((c - 1) & 1));
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (moved) rescale();
+        l_run += rs;
+        if (ragged) {
+#pragma unroll
+            for (int i = 0; i < 16; i++)
+                if (blk * AT_BK + 32 + 8 * (i >> 2) + 4 * half + (i & 3) >= a.Tkv) s1[i] = -INFINITY;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+
+        // ---- (C) ---------------------------------------------------------------------------------------------------------
+#pragma unroll
+        for (int c = 0; c < 8; c++) {
+            acc_o[c & 3] = mfma32_16bit<T>(rv[4 * (c & 3) + (c >> 2)], pop[c >> 2], acc_o[c & 3]);
+            if (c == 0) {
+                moved = row_max(s1);
+                rs = 0.0f;
+            }
+            if (c >= 1 && c <= 4) exp4(s1, 4 * (c - 1), pop[2 + ((c - 1) >> 1)], 2 * ((c - 1) & 1));
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (moved) rescale();
         l_run += rs;
         __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));  // my loads of tile blk + 1 have landed, my reads of tile blk are done
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
 
-        // ---- O^T += V^T P^T --------------------------------------------------------------------------------------
+        // ---- (D) ---------------------------------------------------------------------------------------------------------
 #pragma unroll
-        for (int c = 0; c < 8; c++) acc_o[c >> 2] = mfma32_16bit<T>(ra[c], pop[c & 3], acc_o[c >> 2]);
-#pragma unroll
-        for (int c = 0; c < 8; c++) acc_o[2 + (c >> 2)] = mfma32_16bit<T>(rb[c], pop[c & 3], acc_o[2 + (c >> 2)]);
+        for (int c = 0; c < 8; c++) {
+            acc_o[c & 3] = mfma32_16bit<T>(rv[4 * (c & 3) + 2 + (c >> 2)], pop[2 + (c >> 2)], acc_o[c & 3]);
+            rk[2 * c] = *(const v4i *)(sn + (c >> 2) * (32 * 256) + koff[(2 * c) & 7]);
+            rk[2 * c + 1] = *(const v4i *)(sn + (c >> 2) * (32 * 256) + koff[(2 * c + 1) & 7]);
+            if (c & 1) issue_k(nxt, blk & 1, c >> 1); else issue_v(nxt, blk & 1, c >> 1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
     }
 
     // ---- O = O^T / l, staged through LDS so that rows leave as 256-byte segments -------------------------------------
