@@ -1,23 +1,32 @@
 // Unmasked scaled-dot-product attention (flash-attention forward) for gfx950, head dimension 128.
 //
 // Arithmetic (reference: nunchaku/ops/triton/attention.py:37-169): q is multiplied by scale * log2(e) and rounded to
-// the 16-bit type; per block of keys S = q k^T in fp32, online softmax with exp2 (running row maximum m and row sum
-// l), P rounded to the 16-bit type, O = O * 2^(m_old - m_new) + P v in fp32; at the end O / l, stored as
-// (B, Tq, H * 128).
+// the 16-bit type; per block of keys S = q k^T in fp32, online softmax with exp2 (a row reference m and row sum l),
+// P rounded to the 16-bit type, O = O * 2^(m_old - m_new) + P v in fp32; at the end O / l, stored as
+// (B, Tq, H * 128).  Two choices the mathematics leaves open differ from the reference: the reference m is only moved
+// when a row maximum exceeds it by more than 8 (P then lies in (0, 2^8] instead of (0, 1]: the same O / l, since P, O
+// and l all carry the same power of two), and l sums the rounded P the matrix instruction sees, not the unrounded one.
 //
 // How it maps to CDNA4:
 //  * Everything is computed transposed.  S^T = K Q^T puts the keys in the MFMA's A operand and the queries in its B
 //    operand, so in the 32x32 accumulator a lane owns ONE query (column) and its registers walk the keys: the row
-//    maximum and row sum of the softmax are in-lane reductions plus one exchange with lane ^ 32, and the rescaling of
-//    the output accumulator is a per-lane scalar.  O^T = V^T P^T then takes P^T as its B operand straight from those
-//    accumulator registers (eight values of a lane are the eight k-slots the operand wants; the k order inside a
-//    16-key chunk is the permutation 0-3, 8-11 | 4-7, 12-15, which V^T simply shares), with no trip through LDS.
+//    maximum and row sum of the softmax are in-lane reductions plus one exchange with lane ^ 32
+//    (v_permlane32_swap), and the rescaling of the output accumulator is a per-lane scalar.  O^T = V^T P^T then
+//    takes P^T as its B operand straight from those accumulator registers (eight values of a lane are the eight
+//    k-slots the operand wants; the k order inside a 16-key chunk is the permutation 0-3, 8-11 | 4-7, 12-15, which
+//    V^T simply shares), with no trip through LDS.
+//  * The S^T accumulator starts at minus the row reference, so the scores leave the matrix instruction ready for
+//    exp2: no subtraction per score.
 //  * V^T is made once per call by a small transposing kernel (keys permuted as above, key count padded to 64); the
-//    main kernel then streams K tiles (64 keys x 256 bytes) and V^T tiles (128 rows x 128 bytes) global -> LDS
-//    directly (global_load_lds_dwordx4, whole rows per load, 16-byte chunks XOR-swizzled by the row so the operand
-//    reads are conflict free), one tile pair ahead, one barrier per 64 keys.
-//  * 256 threads = 4 wavefronts of 32 queries; Q stays in registers (pre-scaled), the output accumulator is 64
-//    registers; the accumulator is only rescaled when some lane's maximum moved.
+//    main kernel then streams K tiles (64 keys x 256 bytes) and V^T tiles (128 rows x 128 bytes) buffer -> LDS
+//    directly (buffer_load_dwordx4 ... lds, whole rows per load, per-lane offsets fixed and the tile chosen by the
+//    scalar buffer base, 16-byte chunks XOR-swizzled so that the operand reads are conflict free), two tiles in
+//    flight, one barrier per 64 keys.
+//  * 256 threads = 4 wavefronts of 32 queries, two workgroups per CU; Q stays in registers (pre-scaled), the output
+//    accumulator is 64 registers.  A tile is processed as two 32-key halves so that the softmax instructions of one
+//    half sit between the matrix instructions of the other (see the pipeline comment in the kernel).
+//  * Workgroups of one head run on one XCD (when the head count is a multiple of 8), so K and V^T of a head are
+//    fetched into one L2 only.
 #include "svdq_common.h"
 
 namespace svdq {
@@ -142,10 +151,14 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a
     for (int dt = 0; dt < 4; dt++)
 #pragma unroll
         for (int i = 0; i < 16; i++) acc_o[dt][i] = 0.0f;
-    float m_ref = -INFINITY, l_run = 0.0f;  // p = 2^(s - m_ref); m_ref trails the true row maximum by at most AT_LAZY
-    v16f zero16;
+    // Scores come out of the matrix instructions already relative to the row's reference: the accumulator of S^T starts
+    // at -bias (cinit), so p = 2^s' with s' = s - bias needs no subtraction.  bias trails the true row maximum by at
+    // most AT_LAZY (it only moves when a maximum exceeds it by more than that), which keeps p <= 2^AT_LAZY.
+    // gap = reference - bias: 0 once a reference exists, -inf before the first keys.
+    float bias = 0.0f, gap = -INFINITY, l_run = 0.0f;
+    v16f cinit;
 #pragma unroll
-    for (int i = 0; i < 16; i++) zero16[i] = 0.0f;
+    for (int i = 0; i < 16; i++) cinit[i] = 0.0f;
 
     const int nblk = (a.Tkv + AT_BK - 1) / AT_BK;
     // Software pipeline.  Tile t lives in stage t & 1 and is handled as two halves of 32 keys, each a complete online-
@@ -177,39 +190,51 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a
         rk[8 + c] = *(const v4i *)(smem + 32 * 256 + koff[c]);
     }
 
-    float m_new, alpha, rs;  // rs: this half's row sum, at the new reference
-    // row maximum of one half (16 scores of this lane, 16 of lane ^ 32), the lazily updated reference and the factor
-    // that moves the accumulator to it; returns whether any lane of the wavefront moved
+    float shift, alpha, rs;  // rs: this half's row sum, at the new reference
+    auto max3 = [](float x, float y, float z) {
+        float r;
+        asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "v"(y), "v"(z));
+        return r;
+    };
+    // row maximum of one half (16 scores of this lane, 16 of lane ^ 32) relative to the bias; when it exceeds the
+    // allowance: shift = how far the reference moves, alpha = the factor that moves the accumulator there (0 before the
+    // first keys).  Returns whether any lane of the wavefront moved.
     auto row_max = [&](const v16f &sv) -> bool {
-        float mx = fmaxf(fmaxf(sv[0], sv[1]), sv[2]);
+        float mx = max3(sv[0], sv[1], sv[2]);
 #pragma unroll
-        for (int i = 3; i < 15; i += 2) mx = fmaxf(fmaxf(mx, sv[i]), sv[i + 1]);
-        mx = fmaxf(mx, sv[15]);
+        for (int i = 3; i < 15; i += 2) mx = max3(mx, sv[i], sv[i + 1]);
+        mx = max3(mx, sv[15], sv[15]);
         const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(mx), __float_as_uint(mx), false, false);
-        mx = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
-        const bool need = mx > m_ref + AT_LAZY;
-        m_new = need ? mx : m_ref;
-        alpha = __builtin_amdgcn_exp2f(m_ref - m_new);  // 1 when nothing moved, 0 on the first tile (m_ref = -inf)
-        m_ref = m_new;
+        mx = max3(__uint_as_float(sw[0]), __uint_as_float(sw[1]), __uint_as_float(sw[1]));
+        const bool need = mx > gap + AT_LAZY;
+        shift = need ? mx : 0.0f;
+        alpha = __builtin_amdgcn_exp2f(need ? gap - mx : 0.0f);
+        gap = need ? 0.0f : gap;
         return __builtin_amdgcn_ballot_w64(need) != 0;
     };
-    // four scores -> two packed P values
+    auto shift16 = [&](v16f &sv) {
+#pragma unroll
+        for (int i = 0; i < 16; i++) sv[i] -= shift;
+    };
+    // four scores -> two packed P values; the row sum adds what the matrix instruction will see (the rounded P)
     auto exp4 = [&](const v16f &sv, int i0, v4i &pw, int e0) {
         float p[4];
 #pragma unroll
-        for (int e = 0; e < 4; e++) {
-            p[e] = __builtin_amdgcn_exp2f(sv[i0 + e] - m_new);
-            rs += p[e];
-        }
+        for (int e = 0; e < 4; e++) p[e] = __builtin_amdgcn_exp2f(sv[i0 + e]);
         pw[e0] = (int)pack2<T>(p[0], p[1]);
         pw[e0 + 1] = (int)pack2<T>(p[2], p[3]);
+        rs = T::sum2((uint32_t)pw[e0], rs);
+        rs = T::sum2((uint32_t)pw[e0 + 1], rs);
     };
+    // the reference moved: accumulator and row sum to the new reference, later scores start from the new bias
     auto rescale = [&]() {
         l_run *= alpha;
 #pragma unroll
         for (int dt = 0; dt < 4; dt++)
 #pragma unroll
             for (int i = 0; i < 16; i++) acc_o[dt][i] *= alpha;
+        shift16(cinit);
+        bias += shift;
     };
 
     for (int blk = 0; blk < nblk; blk++) {
@@ -223,7 +248,7 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a
         // ---- (A) ---------------------------------------------------------------------------------------------------------
 #pragma unroll
         for (int c = 0; c < 8; c++) {
-            s0 = mfma32_16bit<T>(rk[c], qop[c], c == 0 ? zero16 : s0);
+            s0 = mfma32_16bit<T>(rk[c], qop[c], c == 0 ? cinit : s0);
             rv[4 * (c & 3) + (c >> 2)] = *(const v4i *)(st + (c & 3) * (32 * 128) + vtoff[c >> 2]);  // chunks 0, 1: keys 0..31
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -237,16 +262,20 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a
         bool moved = false;
 #pragma unroll
         for (int c = 0; c < 8; c++) {
-            s1 = mfma32_16bit<T>(rk[8 + c], qop[c], c == 0 ? zero16 : s1);
+            s1 = mfma32_16bit<T>(rk[8 + c], qop[c], c == 0 ? cinit : s1);
             rv[4 * (c & 3) + 2 + (c >> 2)] = *(const v4i *)(st + (c & 3) * (32 * 128) + vtoff[2 + (c >> 2)]);  // keys 32..63
             if (c == 0) {
                 moved = row_max(s0);
                 rs = 0.0f;
+                if (moved) shift16(s0);
             }
             if (c >= 1 && c <= 4) exp4(s0, 4 * (c - 1), pop[(c - 1) >> 1], 2 * ((c - 1) & 1));
             __builtin_amdgcn_sched_barrier(0);
         }
-        if (moved) rescale();
+        if (moved) {
+            shift16(s1);  // computed from the old bias
+            rescale();
+        }
         l_run += rs;
         if (ragged) {
 #pragma unroll
@@ -262,6 +291,7 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a
             if (c == 0) {
                 moved = row_max(s1);
                 rs = 0.0f;
+                if (moved) shift16(s1);
             }
             if (c >= 1 && c <= 4) exp4(s1, 4 * (c - 1), pop[2 + ((c - 1) >> 1)], 2 * ((c - 1) & 1));
             __builtin_amdgcn_sched_barrier(0);

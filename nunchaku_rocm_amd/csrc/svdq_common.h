@@ -43,6 +43,11 @@ struct BF16 {
         const f2 v = {lo, hi};
         return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf2));
     }
+    // acc + lo + hi of a packed pair (v_dot2c_f32_bf16 against (1, 1))
+    __device__ static inline float sum2(uint32_t w, float acc) {
+        typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf2, w), __builtin_bit_cast(bf2, 0x3F803F80u), acc, false);
+    }
 };
 
 struct FP16 {
@@ -65,6 +70,10 @@ struct FP16 {
         typedef float f2 __attribute__((ext_vector_type(2)));
         const f2 v = {lo, hi};
         return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, h2));
+    }
+    __device__ static inline float sum2(uint32_t w, float acc) {
+        typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(h2, w), __builtin_bit_cast(h2, 0x3C003C00u), acc, false);
     }
 };
 
