@@ -15,6 +15,7 @@
  *                            kernel-argument structs modelled on ops/triton/native/w4a4.py:80-124
  *   svdq_awq_gemv_w4a16      nunchaku/ops/dispatch.py:19-34      (_C.ops.gemv_awq / ops/triton/awq.py:186 awq_gemv_w4a16)
  *   svdq_attention_fp16      nunchaku/ops/dispatch.py:67-99      (_C.ops.attention_fp16 / ops/triton/attention.py:111 attention_fp16)
+ *   svdq_unpack_mma_*        nunchaku/ops/triton/layout.py:36-292 (checkpoint layout -> natural layout)
  *   svdq_transpose_lora_down no counterpart: one-time re-layout of a LoRA-down weight, see below
  *   svdq_group_acc_i32       no counterpart: debug read-out of the exact int32 group accumulators
  */
@@ -174,6 +175,25 @@ typedef struct {
 
 int svdq_attention_fp16(const svdq_attention_args *args, void *stream);
 size_t svdq_attention_workspace_bytes(int32_t B, int32_t H, int32_t Tkv, int32_t D);
+
+/*
+ * Checkpoint ingestion.  The published SVDQuant int4 checkpoints hold every tensor of a quantized linear pre-shuffled
+ * for the register fragments of the CUDA kernels (nunchaku/lora/flux/packer.py:173-226 pack_weight, :228-262
+ * pack_scale, :300-338 pack_lowrank_weight); these undo that in one pass on the device, as the reference does at load
+ * time (nunchaku/ops/triton/layout.py:36-120 unpack_weight[_packed_nibbles], :155-184 unpack_scale, :226-292
+ * convert_svdq_linear_to_natural_layout).  Source and destination must not overlap.
+ *
+ *   weight   packed (N, K / 2) bytes            -> natural (N, K / 2) bytes, low nibble = even k; N, K multiples of 128;
+ *                                                  ld_natural in bytes
+ *   scale    packed groups * N 16-bit values    -> natural (groups, N); N a multiple of 128.  groups = K / 64 for
+ *                                                  wscales, 1 for bias / smooth_factor / wcscales; ld_natural in elements
+ *   lowrank  packed (C, R) 16-bit values        -> natural (C, R): down = 0 for proj_up (C = out features), down = 1
+ *                                                  for proj_down (C = in features); C, R multiples of 16
+ */
+int svdq_unpack_mma_weight(const void *packed, void *natural, int32_t N, int32_t K, int32_t ld_natural, void *stream);
+int svdq_unpack_mma_scale(const void *packed, void *natural, int32_t N, int32_t groups, int32_t ld_natural, void *stream);
+int svdq_unpack_mma_lowrank(const void *packed, void *natural, int32_t C, int32_t R, int32_t down, int32_t ld_natural,
+                            void *stream);
 
 /* Message for the last non-zero return on the calling thread ("" if none). */
 const char *svdq_last_error(void);

@@ -31,6 +31,9 @@ EXPORTS = (
     "svdq_awq_gemv_w4a16",
     "svdq_attention_fp16",
     "svdq_attention_workspace_bytes",
+    "svdq_unpack_mma_weight",
+    "svdq_unpack_mma_scale",
+    "svdq_unpack_mma_lowrank",
     "svdq_last_error",
     "svdq_abi_version",
 )
@@ -116,6 +119,9 @@ def load() -> ctypes.CDLL:
     lib.svdq_attention_fp16.argtypes = [ctypes.POINTER(AttentionArgs), _vp]
     lib.svdq_attention_workspace_bytes.restype = ctypes.c_size_t
     lib.svdq_attention_workspace_bytes.argtypes = [_i32, _i32, _i32, _i32]
+    lib.svdq_unpack_mma_weight.argtypes = [_vp, _vp, _i32, _i32, _i32, _vp]
+    lib.svdq_unpack_mma_scale.argtypes = [_vp, _vp, _i32, _i32, _i32, _vp]
+    lib.svdq_unpack_mma_lowrank.argtypes = [_vp, _vp, _i32, _i32, _i32, _i32, _vp]
     lib.svdq_transpose_lora_down.argtypes = [_vp, _vp, _i32, _i32, _i32, _vp]
     lib.svdq_group_acc_i32.argtypes = [_vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp]
     if lib.svdq_abi_version() != ABI_VERSION:

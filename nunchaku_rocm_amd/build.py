@@ -14,7 +14,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libsvdq_mi355x.so")
-SOURCES = ["common.hip", "quantize.hip", "gemm_w4a4.hip", "awq_gemv.hip", "attention.hip"]
+SOURCES = ["common.hip", "quantize.hip", "gemm_w4a4.hip", "awq_gemv.hip", "attention.hip", "layout.hip"]
 FLAGS = [
     "--offload-arch=gfx950",
     "-O3",

@@ -1,0 +1,171 @@
+"""Checkpoint ingestion: tensors as the published SVDQuant int4 checkpoints hold them -> the natural layouts of
+``SVDQW4A4Linear`` (reference: nunchaku/ops/triton/layout.py:36-292; state-dict key names:
+nunchaku/models/transformers/transformer_flux_v2.py:579-649; file metadata: nunchaku/models/transformers/utils.py:32-60).
+
+The permutations run on the GPU through ``libsvdq_mi355x.so`` (``svdq_unpack_mma_*``): tensors must be CUDA tensors.
+Only the int4 format is handled; the NVFP4 micro-scale layout (group size 16) is not.
+"""
+
+from __future__ import annotations
+
+import json
+
+import torch
+
+from . import _lib
+
+__all__ = [
+    "unpack_weight",
+    "unpack_weight_packed_nibbles",
+    "unpack_scale",
+    "unpack_lowrank_weight",
+    "convert_svdq_linear_to_natural_layout",
+    "convert_flux_state_dict",
+    "load_checkpoint",
+]
+
+
+def _flat16(t: torch.Tensor) -> torch.Tensor:
+    if t.dtype not in (torch.float16, torch.bfloat16):
+        raise ValueError(f"expected a float16 / bfloat16 tensor, got {t.dtype}")
+    return t.contiguous()
+
+
+def unpack_weight_packed_nibbles(packed: torch.Tensor, n: int, k: int, bits: int = 4) -> torch.Tensor:
+    """Checkpoint ``qweight`` ``(n, k // 2)`` int8 -> natural ``(n, k // 2)`` uint8, column ``2 j`` in the low nibble
+    of byte ``j``.  ``n`` and ``k`` are the padded sizes (multiples of 128)."""
+    if bits != 4:
+        raise NotImplementedError("packed-nibble output is only defined for 4-bit codes")
+    _lib.require_cuda(packed)
+    if packed.numel() * packed.element_size() != n * k // 2:
+        raise ValueError(f"packed weight holds {packed.numel() * packed.element_size()} bytes, expected {n * k // 2}")
+    src = packed.contiguous()
+    out = torch.empty(n, k // 2, dtype=torch.uint8, device=packed.device)
+    with torch.cuda.device(packed.device):
+        _lib.check(_lib.load().svdq_unpack_mma_weight(src.data_ptr(), out.data_ptr(), n, k, k // 2, _lib.stream_of(src)))
+    return out
+
+
+def unpack_weight(packed: torch.Tensor, n: int, k: int, bits: int = 4) -> torch.Tensor:
+    """Checkpoint ``qweight`` -> logical ``(n, k)`` int32 codes in ``[0, 16)`` (not sign-interpreted)."""
+    b = unpack_weight_packed_nibbles(packed, n, k, bits=bits).to(torch.int32)
+    return torch.stack([b & 0xF, b >> 4], dim=-1).reshape(n, k)
+
+
+def unpack_scale(packed: torch.Tensor, n: int, group_size: int, bits: int = 4, warp_n: int = 128) -> torch.Tensor:
+    """Checkpoint scale tensor -> ``(k // group_size, n)`` (``wscales``), or ``(n,)`` for ``group_size=-1`` (``bias``,
+    ``smooth_factor``, ``wcscales``: the checkpoint keeps them in the same lane order)."""
+    if bits != 4 or warp_n != 128:
+        raise NotImplementedError("only the 4-bit packer with warp_n = 128 is implemented")
+    if group_size == 16:
+        raise NotImplementedError("NVFP4 micro-scales (group size 16) are not implemented: int4 checkpoints only")
+    _lib.require_cuda(packed)
+    src = _flat16(packed)
+    groups = 1 if group_size == -1 else src.numel() // n
+    if groups * n != src.numel():
+        raise ValueError(f"scale tensor of {src.numel()} elements does not divide into rows of {n}")
+    out = torch.empty(groups, n, dtype=src.dtype, device=src.device)
+    with torch.cuda.device(src.device):
+        _lib.check(_lib.load().svdq_unpack_mma_scale(src.data_ptr(), out.data_ptr(), n, groups, n, _lib.stream_of(src)))
+    return out.reshape(n) if group_size == -1 else out
+
+
+def unpack_lowrank_weight(weight: torch.Tensor, down: bool) -> torch.Tensor:
+    """Checkpoint low-rank factor -> natural: ``down=False``: ``proj_up`` ``(out_features, rank)``; ``down=True``:
+    the checkpoint's ``(in_features, rank)`` tensor -> ``proj_down`` ``(in_features, rank)``.  (The reference's packer
+    method of this name returns ``(rank, in_features)`` for ``down=True`` and its caller transposes; here the
+    transposed result comes out directly.)"""
+    _lib.require_cuda(weight)
+    src = _flat16(weight)
+    c, r = src.shape
+    out = torch.empty(c, r, dtype=src.dtype, device=src.device)
+    with torch.cuda.device(src.device):
+        _lib.check(_lib.load().svdq_unpack_mma_lowrank(src.data_ptr(), out.data_ptr(), c, r, int(bool(down)), r, _lib.stream_of(src)))
+    return out
+
+
+def convert_svdq_linear_to_natural_layout(linear) -> None:
+    """Convert one ``SVDQW4A4Linear`` in place from the checkpoint layout to the natural one.  Call exactly once per
+    loaded module: the conversion is not idempotent.  ``smooth_factor_orig`` is not read by any kernel and is left
+    as it is."""
+    n, half_k = linear.qweight.shape
+    k = 2 * half_k
+    with torch.no_grad():
+        linear.qweight.data = unpack_weight_packed_nibbles(linear.qweight.data, n, k).view(torch.int8)
+        linear.wscales.data = unpack_scale(linear.wscales.data, n, group_size=linear.group_size)
+        if linear.bias is not None:
+            linear.bias.data = unpack_scale(linear.bias.data, n, group_size=-1)
+        linear.smooth_factor.data = unpack_scale(linear.smooth_factor.data, k, group_size=-1)
+        if getattr(linear, "wcscales", None) is not None:
+            linear.wcscales.data = unpack_scale(linear.wcscales.data, n, group_size=-1)
+        if linear.proj_down.numel() > 0:
+            linear.proj_down.data = unpack_lowrank_weight(linear.proj_down.data, down=True)
+        if linear.proj_up.numel() > 0:
+            linear.proj_up.data = unpack_lowrank_weight(linear.proj_up.data, down=False)
+
+
+# legacy FLUX checkpoint module names -> names of the diffusers-style model, per block family; first match wins
+_DOUBLE_BLOCK_NAMES = (
+    (".mlp_context_fc1.", ".ff_context.net.0.proj."),
+    (".mlp_context_fc2.", ".ff_context.net.2."),
+    (".mlp_fc1.", ".ff.net.0.proj."),
+    (".mlp_fc2.", ".ff.net.2."),
+    (".qkv_proj_context.", ".attn.add_qkv_proj."),
+    (".qkv_proj.", ".attn.to_qkv."),
+    (".norm_added_q.", ".attn.norm_added_q."),
+    (".norm_added_k.", ".attn.norm_added_k."),
+    (".norm_q.", ".attn.norm_q."),
+    (".norm_k.", ".attn.norm_k."),
+    (".out_proj_context.", ".attn.to_add_out."),
+    (".out_proj.", ".attn.to_out.0."),
+)
+_SINGLE_BLOCK_NAMES = (
+    (".qkv_proj.", ".attn.to_qkv."),
+    (".out_proj.", ".attn.to_out."),
+    (".norm_q.", ".attn.norm_q."),
+    (".norm_k.", ".attn.norm_k."),
+)
+
+
+def _rename(key: str, table) -> str:
+    for old, new in table:
+        if old in key:
+            key = key.replace(old, new)
+            break
+    return key
+
+
+def convert_flux_state_dict(state_dict: dict[str, torch.Tensor]) -> dict[str, torch.Tensor]:
+    """Rename the keys of a legacy FLUX SVDQuant checkpoint to the names ``NunchakuFluxTransformer2DModelV2`` uses;
+    tensors are passed through untouched, keys outside the transformer blocks keep their names."""
+    out = {}
+    for key, value in state_dict.items():
+        if "single_transformer_blocks." in key:
+            table = _SINGLE_BLOCK_NAMES
+        elif "transformer_blocks." in key:
+            table = _DOUBLE_BLOCK_NAMES
+        else:
+            out[key] = value
+            continue
+        new_key = _rename(key, table)
+        new_key = new_key.replace(".lora_down", ".proj_down").replace(".lora_up", ".proj_up")
+        if ".smooth_orig" in key:
+            new_key = new_key.replace(".smooth_orig", ".smooth_factor_orig")
+        elif ".smooth" in key:
+            new_key = new_key.replace(".smooth", ".smooth_factor")
+        out[new_key] = value
+    return out
+
+
+def load_checkpoint(path, device: str | torch.device = "cpu") -> tuple[dict[str, torch.Tensor], dict[str, str], dict]:
+    """Read one ``.safetensors`` checkpoint: ``(state_dict, metadata, config)`` where ``config`` is the model config
+    the file carries as JSON under the ``config`` metadata key (``{}`` if absent)."""
+    from safetensors import safe_open
+
+    state_dict = {}
+    with safe_open(str(path), framework="pt", device=str(device)) as f:
+        metadata = dict(f.metadata() or {})
+        for key in f.keys():
+            state_dict[key] = f.get_tensor(key)
+    config = json.loads(metadata["config"]) if "config" in metadata else {}
+    return state_dict, metadata, config

@@ -56,7 +56,7 @@ def test_qk_norm_rope(dev, M, H, actual_m, unsigned, dtype):
 
 @pytest.mark.parametrize("unsigned", [False, True])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("M,N,R2,store_out", [(144, 256, 48, True), (64, 512, 32, False), (128, 128, 0, False)])
+@pytest.mark.parametrize("M,N,R2,store_out", [(144, 256, 48, True), (64, 512, 32, False), (128, 128, 0, False), (80, 256, 288, False)])
 def test_gelu_quant_epilogue(dev, M, N, R2, store_out, unsigned, dtype):
     from nunchaku_rocm_amd import ops
 
@@ -151,7 +151,7 @@ def test_fused_ops_on_flux_block_shapes(dev):
 
 @pytest.mark.parametrize("unsigned", [False, True])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("M,N,R2", [(144, 256, 48), (64, 512, 32), (128, 128, 0)])
+@pytest.mark.parametrize("M,N,R2", [(144, 256, 48), (64, 512, 32), (128, 128, 0), (80, 256, 160)])
 def test_swiglu_quant_epilogue(dev, M, N, R2, unsigned, dtype):
     """``wgt`` rows in the 16-interleaved [gate | up] order; the epilogue quantizes silu(gate) * up (signed int4)."""
     from nunchaku_rocm_amd import ops

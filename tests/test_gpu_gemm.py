@@ -75,7 +75,8 @@ def test_unit_scales_exact_integer_gemm(dev, unsigned, dtype):
 
 @pytest.mark.parametrize("unsigned", [False, True])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("M,N,K,R,actual_m", [(136, 264, 256, 16, 130), (256, 256, 512, 32, 256), (64, 128, 1024, 48, 64), (128, 512, 256, 0, 100)])
+@pytest.mark.parametrize("M,N,K,R,actual_m", [(136, 264, 256, 16, 130), (256, 256, 512, 32, 256), (64, 128, 1024, 48, 64), (128, 512, 256, 0, 100),
+                                                   (160, 256, 256, 160, 150), (72, 136, 512, 288, 72)])  # ranks grown at run time (32 + sum of LoRA ranks)
 def test_scaled_gemm_bias_lora(dev, M, N, K, R, actual_m, unsigned, dtype):
     print(f"case M={M} N={N} K={K} R={R} actual_m={actual_m} unsigned={unsigned} {dtype}", flush=True)
     p = _rand_problem(M, N, K, R, dtype, seed=K + R)

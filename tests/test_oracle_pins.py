@@ -354,3 +354,80 @@ def test_attention_special_cases():
     a = O.attention_fp16(q, k, v, scale, block_n=16).float()
     b = O.attention_fp16(q, k, v, scale, block_n=300).float()
     assert (a - b).abs().max() <= 2e-2 * b.abs().max()
+
+
+# ---- checkpoint packer ----------------------------------------------------------------------------------------------
+def test_pack_weight_fragment_rule_and_hand_positions():
+    """mma.m16n8k32 B fragment (PTX ISA, 'Matrix Fragments for mma.m16n8k32'): lane = 4 * groupID + threadID_in_group
+    owns column n = groupID and rows k = 8 * threadID_in_group .. + 7 of an 8 x 32 block, in one 32-bit register."""
+    from oracle import mma_packer as P
+
+    n, k = 256, 256
+    codes = np.zeros((n, k), dtype=np.int32)
+    tag = (np.arange(n)[:, None] * 7 + np.arange(k)[None, :] // 8) % 16  # constant over the 8 k of one word
+    codes[:] = tag
+    words = P.pack_weight(codes).view(np.uint32).reshape(-1)
+    assert (words % 0x11111111 == 0).all()  # every word holds eight equal nibbles: words never mix rows or k-octets
+    # word positions worked out by hand from the axis order [n_tile, k_tile, n_packs, n_lane, k_lane, n_pack, k_pack]
+    where = {0: (0, 0), 1: (0, 32), 2: (8, 0), 3: (8, 32), 4: (0, 8), 16: (1, 0), 17: (1, 32), 128: (16, 0), 1024: (0, 64), 1024 * 4: (128, 0)}
+    for w, (nn, kk) in where.items():
+        assert words[w] == int(tag[nn, kk]) * 0x11111111, (w, nn, kk)
+    # inside an 8 x 32 block: consecutive 4-word groups [n_pack, k_pack] of lane L = 4 * (n % 8) + (k / 8) % 4
+    for lane in range(32):
+        nn, kk = lane // 4, 8 * (lane % 4)
+        assert words[4 * lane] == int(tag[nn, kk]) * 0x11111111
+    # nibble order inside a word: k + j in bits 4 j
+    codes = np.arange(n * k, dtype=np.int64).reshape(n, k) % 16
+    b = P.pack_weight(codes.astype(np.int32))
+    assert [int(b[0, 0]) & 0xF, int(b[0, 0]) >> 4, int(b[0, 1]) & 0xF] == [0, 1, 2]
+    # a permutation of words: every (row, k-octet) appears exactly once
+    ids = (np.arange(n)[:, None] * (k // 8) + np.arange(k)[None, :] // 8).astype(np.int64)
+    seen = np.zeros(n * k // 8, dtype=np.int64)
+    for nib in range(4):  # 16 bits of id, 4 bits at a time
+        w = P.pack_weight(((ids >> (4 * nib)) & 0xF).astype(np.int32)).view(np.uint32).reshape(-1)
+        seen |= (w & 0xF).astype(np.int64) << (4 * nib)
+    assert sorted(seen.tolist()) == list(range(n * k // 8))
+
+
+def test_pack_scale_and_lowrank_hand_positions():
+    from oracle import mma_packer as P
+
+    n, g = 256, 3
+    s = (np.arange(n)[:, None] * 10 + np.arange(g)[None, :]).astype(np.float32)
+    flat = P.pack_scale(s)
+    # [n_group][g][a (8)][c (4)][b (2)][d (2)] with n = 16 a + 8 b + 2 c + d: positions 0..7 of a group hold
+    # n = 0, 1, 8, 9, 2, 3, 10, 11
+    assert (flat[:8] == s[[0, 1, 8, 9, 2, 3, 10, 11], 0]).all()
+    assert (flat[128 : 128 + 4] == s[[0, 1, 8, 9], 1]).all()  # next group of the same 128 rows
+    assert flat[3 * 128] == s[128, 0]  # next 128 rows
+    assert sorted(flat.tolist()) == sorted(s.reshape(-1).tolist())
+    v = np.arange(128, dtype=np.float32)
+    assert (P.pack_scale(v)[:8] == [0, 1, 8, 9, 2, 3, 10, 11]).all()
+
+    # low-rank, up factor (N, R): block (cp, rp) of 16 x 16, inside [n_lane 8][k_lane 4][n_pack 2][k_pack 2][2]
+    N, R = 32, 32
+    up = (np.arange(N)[:, None] * 100 + np.arange(R)[None, :]).astype(np.float32)
+    pu = P.pack_lowrank_weight(up, down=False).reshape(-1)
+    assert pu[:8].tolist() == [up[0, 0], up[0, 1], up[0, 8], up[0, 9], up[8, 0], up[8, 1], up[8, 8], up[8, 9]]
+    assert pu[8] == up[0, 2] and pu[32] == up[1, 0]
+    assert pu[256] == up[0, 16] and pu[512] == up[16, 0]  # blocks: rank blocks inside row blocks
+    # down factor: packed from (rank, in_features), viewed (in_features, rank); the reference's inverse
+    # (packer.py:340-373) restated as a loop gives the logical tensor back
+    K = 48
+    dn = (np.arange(R)[:, None] * 100 + np.arange(K)[None, :]).astype(np.float32)  # (rank, in_features)
+    pd = P.pack_lowrank_weight(dn, down=True)
+    assert pd.shape == (K, R)
+    flat = pd.reshape(-1)
+    assert flat[:4].tolist() == [dn[0, 0], dn[0, 1], dn[0, 8], dn[0, 9]] and flat[4] == dn[8, 0]
+    assert flat[256] == dn[16, 0] and flat[512] == dn[0, 16]  # blocks: rank blocks inside in-feature blocks
+    back = np.zeros_like(dn)
+    for cp in range(K // 16):
+        for rp in range(R // 16):
+            blk = flat[(cp * (R // 16) + rp) * 256 :][:256].reshape(8, 4, 2, 2, 2)  # [n_lane][k_lane][n_pack][k_pack][e]
+            for nl in range(8):
+                for kl in range(4):
+                    for ns in range(2):
+                        for ks in range(2):
+                            for e in range(2):
+                                back[rp * 16 + ns * 8 + nl, cp * 16 + ks * 8 + kl * 2 + e] = blk[nl, kl, ns, ks, e]
+    assert (back == dn).all()
