@@ -15,6 +15,7 @@
  *                            kernel-argument structs modelled on ops/triton/native/w4a4.py:80-124
  *   svdq_awq_gemv_w4a16      nunchaku/ops/dispatch.py:19-34      (_C.ops.gemv_awq / ops/triton/awq.py:186 awq_gemv_w4a16)
  *   svdq_attention_fp16      nunchaku/ops/dispatch.py:67-99      (_C.ops.attention_fp16 / ops/triton/attention.py:111 attention_fp16)
+ *   svdq_row_stats           nunchaku/models/normalization.py:97 (the LayerNorm statistics; applied inside svdq_quantize_act)
  *   svdq_unpack_mma_*        nunchaku/ops/triton/layout.py:36-292 (checkpoint layout -> natural layout)
  *   svdq_transpose_lora_down no counterpart: one-time re-layout of a LoRA-down weight, see below
  *   svdq_group_acc_i32       no counterpart: debug read-out of the exact int32 group accumulators
@@ -66,9 +67,23 @@ typedef struct {
     int32_t is_unsigned;     /* 0: codes in [-8, 7], absmax / 7;  1: codes in [0, 15], max / 15             */
     int32_t fuse_glu;        /* 1: x is (M, 2K) and the quantized value is x[:, :K] * silu(x[:, K:])        */
     float shift;             /* added before smoothing (0.171875 after GELU, else 0)                        */
+    /* Optional prologue (NULL norm_stats = off; not with fuse_glu): the quantized and LoRA-projected value is
+     * T(T(T((x - mean[m]) * rstd[m]) * norm_scale[k]) + norm_shift[k]), i.e. LayerNorm without affine followed by the
+     * adaLN modulate, each step rounded to T as separate elementwise kernels would
+     * (nunchaku/models/normalization.py:97-104, models/transformers/transformer_flux_v2.py:236-237). */
+    const float *norm_stats;       /* (M, 2) fp32 rows of (mean, rstd), from svdq_row_stats                  */
+    const void *norm_scale;        /* (batches, K) T: element (b, k) at b * norm_ld + k * norm_stride        */
+    const void *norm_shift;        /* (batches, K) T, same strides                                           */
+    int32_t norm_rows_per_batch;   /* rows m sharing one scale / shift vector (multiple of 16); 0 = all rows */
+    int32_t norm_ld, norm_stride;  /* in elements (the adaLN projection interleaves its six vectors: stride 6) */
 } svdq_quantize_args;
 
 int svdq_quantize_act(const svdq_quantize_args *args, void *stream);
+
+/* Per-row mean and 1 / sqrt(biased variance + eps) of x (M, K) T in fp32: stats[m] = (mean, rstd).  The statistics
+ * LayerNorm needs (nunchaku/models/normalization.py:97), for the quantizer's norm prologue. */
+int svdq_row_stats(const void *x, float *stats, int32_t M, int32_t K, int32_t ld_x, int32_t dtype, float eps,
+                   void *stream);
 
 /* (K, R) row-major T  ->  (R, K) row-major T.  Done once per weight; the quantizer and the fused
  * requantizing epilogues read the transposed form so their MFMA operands are K-contiguous. */

@@ -22,6 +22,7 @@ E_INVALID, E_UNSUPPORTED, E_LAUNCH = -1, -2, -3
 
 EXPORTS = (
     "svdq_quantize_act",
+    "svdq_row_stats",
     "svdq_transpose_lora_down",
     "svdq_gemm_w4a4",
     "svdq_gemm_w4a4_scratch_bytes",
@@ -48,6 +49,8 @@ class QuantizeArgs(ctypes.Structure):
         [(n, _vp) for n in ("x", "smooth", "lora_down_t", "out", "scales", "lora_act")]
         + [(n, _i32) for n in ("M", "K", "R", "ld_x", "ld_out", "ld_scales", "ld_lora_act", "dtype", "is_unsigned", "fuse_glu")]
         + [("shift", _f32)]
+        + [(n, _vp) for n in ("norm_stats", "norm_scale", "norm_shift")]
+        + [(n, _i32) for n in ("norm_rows_per_batch", "norm_ld", "norm_stride")]
     )  # fmt: skip
 
 
@@ -113,6 +116,7 @@ def load() -> ctypes.CDLL:
     lib.svdq_weight_planes_bytes.restype = ctypes.c_size_t
     lib.svdq_weight_planes_bytes.argtypes = [_i32, _i32]
     lib.svdq_split_weight_planes.argtypes = [_vp, _vp, _i32, _i32, _i32, _vp]
+    lib.svdq_row_stats.argtypes = [_vp, _vp, _i32, _i32, _i32, _i32, _f32, _vp]
     lib.svdq_quantize_act.argtypes = [ctypes.POINTER(QuantizeArgs), _vp]
     lib.svdq_gemm_w4a4.argtypes = [ctypes.POINTER(GemmArgs), _vp]
     lib.svdq_awq_gemv_w4a16.argtypes = [ctypes.POINTER(AwqGemvArgs), _vp]

@@ -34,8 +34,13 @@ constexpr uint32_t pack_bias() {
     return c;
 }
 
-template <typename T, bool UNSIGNED, bool GLU, bool HAS_LORA, bool HAS_SMOOTH>
-__global__ __launch_bounds__(Q_WAVES * 64, 2) void quantize_act_kernel(svdq_quantize_args a) {
+// per-group vectors a lane fetches for the group's 64 channels (one channel per lane), shared through LDS later
+struct QVecs {
+    uint16_t sm, ns, nh;  // smooth factor, norm scale, norm shift
+};
+
+template <typename T, bool UNSIGNED, bool GLU, bool HAS_LORA, bool HAS_SMOOTH, bool NORM>
+__global__ __launch_bounds__(Q_WAVES * 64, NORM ? 4 : 2) void quantize_act_kernel(svdq_quantize_args a) {
     // per wavefront: two activation stages (16 rows, + the gate tile with GLU) and one LoRA-down tile (32 ranks), 128
     // bytes a row.  The LoRA-down tile is an L2 hit and the first thing a group consumes: one group ahead is enough.
     constexpr int XS_BYTES = (GLU ? 2 : 1) * Q_ROWS * Q_ROW_BYTES, G_OFF = Q_ROWS * Q_ROW_BYTES;
@@ -45,6 +50,7 @@ __global__ __launch_bounds__(Q_WAVES * 64, 2) void quantize_act_kernel(svdq_quan
     constexpr int STG_BYTES = Q_WAVES * WAVE_BYTES;
     __shared__ __align__(16) uint8_t smem[STG_BYTES > ACC_BYTES ? STG_BYTES : ACC_BYTES];
     __shared__ float lds_rs[Q_WAVES][64];
+    __shared__ float lds_ns[NORM ? Q_WAVES : 1][64], lds_nh[NORM ? Q_WAVES : 1][64];
     float (*lds_acc)[Q_RCHUNK][Q_ROWS + 1] = (float (*)[Q_RCHUNK][Q_ROWS + 1])smem;
 
     const int lane = threadIdx.x & 63;
@@ -75,6 +81,17 @@ __global__ __launch_bounds__(Q_WAVES * 64, 2) void quantize_act_kernel(svdq_quan
     const float qmax = UNSIGNED ? 15.0f : 7.0f;
     const float rmagic = UNSIGNED ? RNE_MAGIC : RNE_MAGIC + 8.0f;  // signed codes are packed as c + 8, then ^ 8
     const bool has_shift = a.shift != 0.0f;
+    // norm prologue: this lane's row statistics, and the workgroup's scale / shift vectors (one batch per workgroup)
+    float n_mean = 0.0f, n_rstd = 1.0f;
+    const uint16_t *__restrict__ nscale = nullptr, *__restrict__ nshift = nullptr;
+    if (NORM) {
+        const int mr = min(m, a.M - 1);
+        n_mean = a.norm_stats[2 * mr];
+        n_rstd = a.norm_stats[2 * mr + 1];
+        const size_t voff = a.norm_rows_per_batch > 0 ? (size_t)(m0 / a.norm_rows_per_batch) * a.norm_ld : 0;
+        nscale = (const uint16_t *)a.norm_scale + voff;
+        nshift = (const uint16_t *)a.norm_shift + voff;
+    }
 
     const int nchunks = HAS_LORA ? (a.R + Q_RCHUNK - 1) / Q_RCHUNK : 1;
     for (int rc = 0; rc < nchunks; rc++) {
@@ -94,11 +111,16 @@ __global__ __launch_bounds__(Q_WAVES * 64, 2) void quantize_act_kernel(svdq_quan
         auto group_off = [&](int i) {  // byte offset of group wave + Q_WAVES * i in a row; past the end: the last group
             return (uint32_t)min(wave + Q_WAVES * i, ngroups - 1) * (GROUP * 2);
         };
-        auto issue_x = [&](int i, uint16_t &sm) {
+        auto issue_x = [&](int i, QVecs &qv) {
             const uint32_t k0 = group_off(i);
             uint8_t *dst = wbase + (i & 1) * XS_BYTES;
-            // the smooth factor of the lane's channel first: older than the block loads, its wait does not cover them
-            if (HAS_SMOOTH && do_quant) sm = smooth[(k0 >> 1) + lane];
+            // the per-channel vectors of the lane's channel first: older than the block loads, their wait does not
+            // cover them
+            if (HAS_SMOOTH && do_quant) qv.sm = smooth[(k0 >> 1) + lane];
+            if (NORM) {
+                qv.ns = nscale[((k0 >> 1) + lane) * a.norm_stride];
+                qv.nh = nshift[((k0 >> 1) + lane) * a.norm_stride];
+            }
 #pragma unroll
             for (int j = 0; j < 2; j++)
                 __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)(xbase + (xdma[j] + k0)),
@@ -138,7 +160,8 @@ __global__ __launch_bounds__(Q_WAVES * 64, 2) void quantize_act_kernel(svdq_quan
             }
         };
 
-        auto process = [&](int i, const Ops &o, uint16_t smv) {
+        auto process = [&](int i, const Ops &o, const QVecs qv) {
+            const uint16_t smv = qv.sm;
             v4i cxlo = o.xlo, cxhi = o.xhi;
             const v4i glo = o.glo, ghi = o.ghi, l0lo = o.l0lo, l0hi = o.l0hi, l1lo = o.l1lo, l1hi = o.l1hi;
             float v[16];
@@ -160,6 +183,29 @@ __global__ __launch_bounds__(Q_WAVES * 64, 2) void quantize_act_kernel(svdq_quan
                     v[8 + 2 * j] = v[8 + 2 * j] * (g2 / (1.0f + __expf(-g2)));
                     v[8 + 2 * j + 1] = v[8 + 2 * j + 1] * (g3 / (1.0f + __expf(-g3)));
                 }
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    cxlo[j] = (int)pack2<T>(v[2 * j], v[2 * j + 1]);
+                    cxhi[j] = (int)pack2<T>(v[8 + 2 * j], v[8 + 2 * j + 1]);
+                }
+            }
+            if (NORM) {
+                // LayerNorm, scale, shift, each rounded to T; the LoRA-down sees the result
+                lds_ns[wave][lane] = T::to_f32(qv.ns);
+                lds_nh[wave][lane] = T::to_f32(qv.nh);
+                __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const v4f sc = *(const v4f *)&lds_ns[wave][kq * 16 + 4 * j];
+                    const v4f sh = *(const v4f *)&lds_nh[wave][kq * 16 + 4 * j];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        float t = T::to_f32(T::from_f32((v[4 * j + e] - n_mean) * n_rstd));
+                        t = T::to_f32(T::from_f32(t * sc[e]));
+                        v[4 * j + e] = T::to_f32(T::from_f32(t + sh[e]));
+                    }
+                }
+                __builtin_amdgcn_wave_barrier();
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
                     cxlo[j] = (int)pack2<T>(v[2 * j], v[2 * j + 1]);
@@ -228,17 +274,17 @@ __global__ __launch_bounds__(Q_WAVES * 64, 2) void quantize_act_kernel(svdq_quan
         // Two groups of activations and one LoRA-down tile in flight per wavefront; each wavefront owns its LDS, so no
         // barrier in the loop.  Per group: wait for its tiles, pull them into registers, refill the freed LDS (next
         // group's LoRA-down tile, the activations two groups on), then compute from the registers.
-        uint16_t sm_a = 0, sm_b = 0;
+        QVecs sm_a = {0, 0, 0}, sm_b = {0, 0, 0};
         Ops ops;
         issue_x(0, sm_a);
         issue_l(0);
         issue_x(1, sm_b);
-        auto step = [&](int i, uint16_t &sm) {
+        auto step = [&](int i, QVecs &sm) {
             // group i's activations and LoRA-down tile have landed: the loads issued after them are at least the NX
             // block loads of group i + 1's activations
             __builtin_amdgcn_s_waitcnt(waitcnt_imm(NX, 15));
             fetch(i, ops);
-            const uint16_t smv = sm;
+            const QVecs smv = sm;
             __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));  // the LDS reads have returned
             issue_l(i + 1);
             issue_x(i + 2, sm);
@@ -272,6 +318,40 @@ __global__ __launch_bounds__(Q_WAVES * 64, 2) void quantize_act_kernel(svdq_quan
     }
 }
 
+// one wavefront per row: mean, then the centred sum of squares (second read from cache), fixed reduction order
+template <typename T>
+__global__ __launch_bounds__(256) void row_stats_kernel(const uint16_t *x, float *stats, int M, int K, long ld_x, float eps) {
+    const int lane = threadIdx.x & 63, m = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (m >= M) return;
+    const uint16_t *row = x + (long)m * ld_x;
+    auto wave_sum = [](float s) {
+#pragma unroll
+        for (int o = 32; o >= 1; o >>= 1) s += __shfl_xor(s, o);
+        return s;
+    };
+    float s = 0.0f;
+    for (int k = 8 * lane; k < K; k += 512) {
+        const v4i w = *(const v4i *)(row + k);
+#pragma unroll
+        for (int e = 0; e < 4; e++) s += T::lo_f32((uint32_t)w[e]) + T::hi_f32((uint32_t)w[e]);
+    }
+    const float mean = wave_sum(s) / (float)K;
+    float q = 0.0f;
+    for (int k = 8 * lane; k < K; k += 512) {
+        const v4i w = *(const v4i *)(row + k);
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const float d0 = T::lo_f32((uint32_t)w[e]) - mean, d1 = T::hi_f32((uint32_t)w[e]) - mean;
+            q += d0 * d0 + d1 * d1;
+        }
+    }
+    const float var = wave_sum(q) / (float)K;
+    if (lane == 0) {
+        stats[2 * m] = mean;
+        stats[2 * m + 1] = 1.0f / sqrtf(var + eps);
+    }
+}
+
 __global__ void transpose_kr_kernel(const uint16_t *in, uint16_t *out, int K, int R, int ld_in) {
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= K * R) return;
@@ -279,18 +359,29 @@ __global__ void transpose_kr_kernel(const uint16_t *in, uint16_t *out, int K, in
     out[idx] = in[(size_t)k * ld_in + r];
 }
 
-template <typename T, bool U, bool G>
-static void launch_quantize2(const svdq_quantize_args &a, hipStream_t s) {
+template <typename T, bool U, bool G, bool NORM>
+static void launch_quantize3(const svdq_quantize_args &a, hipStream_t s) {
     dim3 grid((a.M + Q_ROWS - 1) / Q_ROWS), block(Q_WAVES * 64);
     const bool lora = a.R > 0, sm = a.smooth != nullptr;
     if (lora && sm)
-        hipLaunchKernelGGL((quantize_act_kernel<T, U, G, true, true>), grid, block, 0, s, a);
+        hipLaunchKernelGGL((quantize_act_kernel<T, U, G, true, true, NORM>), grid, block, 0, s, a);
     else if (lora)
-        hipLaunchKernelGGL((quantize_act_kernel<T, U, G, true, false>), grid, block, 0, s, a);
+        hipLaunchKernelGGL((quantize_act_kernel<T, U, G, true, false, NORM>), grid, block, 0, s, a);
     else if (sm)
-        hipLaunchKernelGGL((quantize_act_kernel<T, U, G, false, true>), grid, block, 0, s, a);
+        hipLaunchKernelGGL((quantize_act_kernel<T, U, G, false, true, NORM>), grid, block, 0, s, a);
     else
-        hipLaunchKernelGGL((quantize_act_kernel<T, U, G, false, false>), grid, block, 0, s, a);
+        hipLaunchKernelGGL((quantize_act_kernel<T, U, G, false, false, NORM>), grid, block, 0, s, a);
+}
+
+template <typename T, bool U, bool G>
+static void launch_quantize2(const svdq_quantize_args &a, hipStream_t s) {
+    if constexpr (!G) {
+        if (a.norm_stats) {
+            launch_quantize3<T, U, false, true>(a, s);
+            return;
+        }
+    }
+    launch_quantize3<T, U, G, false>(a, s);
 }
 
 template <typename T>
@@ -347,12 +438,43 @@ extern "C" int svdq_quantize_act(const svdq_quantize_args *args, void *stream) {
         set_error("svdq_quantize_act: dtype %d", a.dtype);
         return SVDQ_E_INVALID;
     }
+    if (a.norm_stats) {
+        if (a.fuse_glu) {
+            set_error("svdq_quantize_act: the norm prologue cannot be combined with fuse_glu");
+            return SVDQ_E_UNSUPPORTED;
+        }
+        if (!a.norm_scale || !a.norm_shift || a.norm_rows_per_batch < 0 || a.norm_rows_per_batch % Q_ROWS ||
+            a.norm_stride < 1 || a.norm_ld < 0) {
+            set_error("svdq_quantize_act: the norm prologue needs norm_scale and norm_shift, norm_stride >= 1 and "
+                      "norm_rows_per_batch=%d a multiple of 16", a.norm_rows_per_batch);
+            return SVDQ_E_INVALID;
+        }
+    }
     if (a.M == 0) return SVDQ_OK;
     if (a.dtype == SVDQ_BF16)
         launch_quantize<BF16>(a, (hipStream_t)stream);
     else
         launch_quantize<FP16>(a, (hipStream_t)stream);
     return check_launch("svdq_quantize_act");
+}
+
+extern "C" int svdq_row_stats(const void *x, float *stats, int32_t M, int32_t K, int32_t ld_x, int32_t dtype, float eps,
+                              void *stream) {
+    if (!x || !stats || M < 0 || K <= 0 || K % 8 || ld_x < K || ld_x % 8 || ((uintptr_t)x & 15)) {
+        set_error("svdq_row_stats: bad arguments (M=%d K=%d ld_x=%d; K and ld_x multiples of 8, x 16-byte aligned)", M, K, ld_x);
+        return SVDQ_E_INVALID;
+    }
+    if (dtype != SVDQ_BF16 && dtype != SVDQ_FP16) {
+        set_error("svdq_row_stats: dtype %d", dtype);
+        return SVDQ_E_INVALID;
+    }
+    if (M == 0) return SVDQ_OK;
+    const dim3 grid((M + 3) / 4), block(256);
+    if (dtype == SVDQ_BF16)
+        hipLaunchKernelGGL(row_stats_kernel<BF16>, grid, block, 0, (hipStream_t)stream, (const uint16_t *)x, stats, M, K, (long)ld_x, eps);
+    else
+        hipLaunchKernelGGL(row_stats_kernel<FP16>, grid, block, 0, (hipStream_t)stream, (const uint16_t *)x, stats, M, K, (long)ld_x, eps);
+    return check_launch("svdq_row_stats");
 }
 
 extern "C" int svdq_transpose_lora_down(const void *lora_down, void *lora_down_t, int32_t K, int32_t R,

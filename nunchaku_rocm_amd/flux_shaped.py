@@ -49,13 +49,19 @@ class HipBackend:
     def linear(x, lin: SVDQW4A4Linear):
         return lin(x)
 
+    # mod = (scale, shift[, stats]): the block's LayerNorm + adaLN modulate of x, applied inside the quantizer
     @staticmethod
-    def gelu_mlp(x, fc1, fc2):
-        return _ops.fused_gelu_mlp(x, fc1, fc2)
+    def gelu_mlp(x, fc1, fc2, mod=None):
+        return _ops.fused_gelu_mlp(x, fc1, fc2, norm=mod)
 
     @staticmethod
-    def qkv(x, proj, norm_q, norm_k, rot):
-        return _ops.fused_qkv_norm_rottary(x, proj, norm_q, norm_k, rot)
+    def qkv(x, proj, norm_q, norm_k, rot, mod=None):
+        return _ops.fused_qkv_norm_rottary(x, proj, norm_q, norm_k, rot, norm=mod)
+
+    @staticmethod
+    def norm_stats(x):
+        """Row statistics of x, to share between several ``mod=`` consumers of the same rows."""
+        return _ops.layer_norm_stats(x)
 
     @staticmethod
     def awq(x, lin: AWQW4A16Linear):
@@ -137,11 +143,11 @@ class _Attention(nn.Module):
             self.to_add_out = SVDQW4A4Linear(C, C, **kw)
         self.joint = joint
 
-    def forward(self, be, x, ctx, rot_img, rot_txt):
+    def forward(self, be, x, ctx, rot_img, rot_txt, mod_x=None, mod_ctx=None):
         B = x.shape[0]
-        qkv = be.qkv(x, self.to_qkv, self.norm_q, self.norm_k, rot_img)
+        qkv = be.qkv(x, self.to_qkv, self.norm_q, self.norm_k, rot_img, mod=mod_x)
         if self.joint:
-            qkv_ctx = be.qkv(ctx, self.add_qkv_proj, self.norm_added_q, self.norm_added_k, rot_txt)
+            qkv_ctx = be.qkv(ctx, self.add_qkv_proj, self.norm_added_q, self.norm_added_k, rot_txt, mod=mod_ctx)
             qkv = torch.cat([qkv_ctx, qkv], dim=1)  # token order [txt, img]
         q, k, v = (t.view(B, -1, self.heads, self.head_dim).transpose(1, 2) for t in qkv.chunk(3, dim=-1))
         o = be.attention(q, k, v)  # (B, H, T, D), scale D^-0.5, no mask
@@ -171,16 +177,14 @@ class _DoubleBlock(nn.Module):
         return emb.view(emb.shape[0], -1, 6).permute(2, 0, 1)  # interleaved split: channel c -> (c // 6, c % 6)
 
     def forward(self, be, x, ctx, temb, rot_img, rot_txt):
-        ln = lambda t: F.layer_norm(t, (self.C,), eps=1e-6)  # noqa: E731
+        # layer_norm(x) * scale + shift in front of each quantized linear runs inside its quantizer (mod=)
         sh_a, sc_a, g_a, sh_m, sc_m, g_m = self._mod6(be, self.norm1, temb)
         csh_a, csc_a, cg_a, csh_m, csc_m, cg_m = self._mod6(be, self.norm1_context, temb)
-        nx = ln(x) * sc_a[:, None] + sh_a[:, None]
-        nc = ln(ctx) * csc_a[:, None] + csh_a[:, None]
-        ax, ac = self.attn(be, nx, nc, rot_img, rot_txt)
+        ax, ac = self.attn(be, x, ctx, rot_img, rot_txt, mod_x=(sc_a, sh_a), mod_ctx=(csc_a, csh_a))
         x = x + g_a.unsqueeze(1) * ax
-        x = x + g_m.unsqueeze(1) * be.gelu_mlp(ln(x) * sc_m[:, None] + sh_m[:, None], self.ff_fc1, self.ff_fc2)
+        x = x + g_m.unsqueeze(1) * be.gelu_mlp(x, self.ff_fc1, self.ff_fc2, mod=(sc_m, sh_m))
         ctx = ctx + cg_a.unsqueeze(1) * ac
-        ctx = ctx + cg_m.unsqueeze(1) * be.gelu_mlp(ln(ctx) * csc_m[:, None] + csh_m[:, None], self.ffc_fc1, self.ffc_fc2)
+        ctx = ctx + cg_m.unsqueeze(1) * be.gelu_mlp(ctx, self.ffc_fc1, self.ffc_fc2, mod=(csc_m, csh_m))
         return ctx, x
 
 
@@ -197,9 +201,9 @@ class _SingleBlock(nn.Module):
     def forward(self, be, x, temb, rot):
         emb = be.awq(F.silu(temb), self.norm)
         shift, scale, gate = emb.view(emb.shape[0], -1, 3).permute(2, 0, 1)
-        nx = F.layer_norm(x, (self.C,), eps=1e-6) * scale[:, None] + shift[:, None]
-        mlp = be.gelu_mlp(nx, self.mlp_fc1, self.mlp_fc2)
-        att = self.attn(be, nx, None, rot, None)
+        mod = (scale, shift, be.norm_stats(x))  # one set of row statistics for both consumers
+        mlp = be.gelu_mlp(x, self.mlp_fc1, self.mlp_fc2, mod=mod)
+        att = self.attn(be, x, None, rot, None, mod_x=mod)
         return x + gate.unsqueeze(1) * (att + mlp)
 
 

@@ -51,18 +51,20 @@ class SVDQW4A4Linear(nn.Module):
         return cls(in_features=in_features, out_features=linear.out_features, bias=linear.bias is not None,
                    torch_dtype=torch_dtype, device=linear.weight.device, **kwargs)  # fmt: skip
 
-    def forward(self, x: torch.Tensor, output: torch.Tensor | None = None) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, output: torch.Tensor | None = None, norm: tuple | None = None) -> torch.Tensor:
+        """``norm=(scale, shift[, stats])``: apply ``layer_norm(x) * scale + shift`` inside the quantizer (an addition
+        to the reference's signature; see ``ops.quantize``)."""
         batch_size, seq_len, channels = x.shape
         x = x.reshape(batch_size * seq_len, channels)
         if output is None:
             output = torch.empty(batch_size * seq_len, self.out_features, dtype=x.dtype, device=x.device)
-        quantized_x, ascales, lora_act_out = self.quantize(x)
+        quantized_x, ascales, lora_act_out = self.quantize(x, norm=norm)
         output = self.forward_quant(quantized_x, ascales, lora_act_out, output)
         return output.reshape(batch_size, seq_len, -1)
 
-    def quantize(self, x: torch.Tensor, pad_size: int = 256):
+    def quantize(self, x: torch.Tensor, pad_size: int = 256, norm: tuple | None = None):
         return svdq_quantize_w4a4_act_fuse_lora_cuda(
-            x, lora_down=self.proj_down, smooth=self.smooth_factor, fp4=False, pad_size=pad_size
+            x, lora_down=self.proj_down, smooth=self.smooth_factor, fp4=False, pad_size=pad_size, norm=norm
         )
 
     def forward_quant(self, quantized_x, ascales, lora_act, output: torch.Tensor | None = None) -> torch.Tensor:

@@ -4,7 +4,7 @@ from .attention import attention_fp16, scaled_dot_product_attention
 from .fused import fused_gelu_mlp, fused_qkv_norm_rottary, fused_swiglu_mlp, interleave_swiglu_linear_
 from .gemm import svdq_gemm_w4a4_cuda
 from .gemv import awq_gemv_w4a16_cuda
-from .quantize import svdq_quantize_w4a4_act_fuse_lora_cuda
+from .quantize import layer_norm_stats, svdq_quantize_w4a4_act_fuse_lora_cuda
 
 __all__ = [
     "svdq_quantize_w4a4_act_fuse_lora_cuda",
@@ -15,5 +15,6 @@ __all__ = [
     "fused_swiglu_mlp",
     "interleave_swiglu_linear_",
     "attention_fp16",
+    "layer_norm_stats",
     "scaled_dot_product_attention",
 ]

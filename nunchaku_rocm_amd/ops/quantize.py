@@ -12,6 +12,40 @@ def _ceil_divide(a: int, b: int) -> int:
     return (a + b - 1) // b
 
 
+def layer_norm_stats(input: torch.Tensor, eps: float = 1e-6) -> torch.Tensor:
+    """Per-row ``(mean, 1 / sqrt(var + eps))`` of a 16-bit ``(..., K)`` tensor as ``(M, 2)`` float32: the statistics of
+    ``LayerNorm(K, elementwise_affine=False, eps=eps)``, for the ``norm=`` prologue of the quantizer (one call can
+    serve several quantizations of the same rows)."""
+    inp = input.reshape(-1, input.shape[-1])
+    _lib.require_cuda(inp)
+    if inp.stride(1) != 1 or inp.stride(0) % 8 or inp.data_ptr() % 16:
+        inp = inp.contiguous()
+    stats = torch.empty(inp.shape[0], 2, dtype=torch.float32, device=inp.device)
+    with torch.cuda.device(inp.device):
+        _lib.check(_lib.load().svdq_row_stats(inp.data_ptr(), stats.data_ptr(), inp.shape[0], inp.shape[1], inp.stride(0),
+                                              _lib.dtype_code(inp.dtype), float(eps), _lib.stream_of(inp)))  # fmt: skip
+    return stats
+
+
+def _norm_args(norm, inp: torch.Tensor, M: int, K: int, eps: float):
+    """``norm = (scale, shift[, stats])`` -> (stats, scale, shift, rows_per_batch, ld, stride) for the C call.  scale
+    and shift are used where they lie when they share their strides (as the slices of one adaLN projection do)."""
+    scale, shift = norm[0], norm[1]
+    stats = norm[2] if len(norm) > 2 and norm[2] is not None else layer_norm_stats(inp, eps)
+    if scale.dim() == 1:
+        scale, shift = scale[None], shift[None]
+    batches = scale.shape[0]
+    if scale.shape != (batches, K) or shift.shape != scale.shape or scale.dtype != inp.dtype or shift.dtype != inp.dtype:
+        raise ValueError("norm scale and shift must both be (K,) or (batches, K) of the input dtype")
+    if M % batches or (batches > 1 and (M // batches) % 16):
+        raise ValueError(f"{M} rows do not split into {batches} batches of a multiple of 16 rows")
+    if stats.dtype != torch.float32 or stats.shape != (M, 2) or not stats.is_contiguous():
+        raise ValueError("norm stats must be a contiguous (M, 2) float32 tensor")
+    if scale.stride() != shift.stride() or scale.stride(1) < 1 or (batches > 1 and scale.stride(0) < 0):
+        scale, shift = scale.contiguous(), shift.contiguous()
+    return stats, scale, shift, (M // batches if batches > 1 else 0), scale.stride(0), scale.stride(1)
+
+
 def quantize_w4a4_act_fuse_lora(
     input: torch.Tensor,
     output: torch.Tensor | None = None,
@@ -24,12 +58,19 @@ def quantize_w4a4_act_fuse_lora(
     fuse_gelu: bool = False,
     shift_value: float = 0.0,
     unsigned: bool = False,
+    norm: tuple | None = None,
+    norm_eps: float = 1e-6,
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """
     Backend-level quantizer with the reference's full option set (reference:
     nunchaku/ops/triton/gemm_w4a4.py:1521-1565): no row padding, outputs allocated when not given, ``unsigned`` /
     ``shift_value`` for activations known to be non-negative after a shift.  ``fuse_gelu`` (the reference's unfused
     fallback prologue) is not implemented: the GELU lives in the GEMM epilogue here.
+
+    ``norm=(scale, shift)`` or ``(scale, shift, stats)`` (no counterpart in the reference, which runs these as separate
+    torch kernels): what is quantized and LoRA-projected is ``layer_norm(input) * scale + shift`` (no affine,
+    ``eps=norm_eps``, every step rounded to the input dtype), with ``scale`` / ``shift`` of shape ``(K,)`` or
+    ``(batches, K)`` (rows split evenly over the batches) and ``stats`` from :func:`layer_norm_stats`.
     """
     if fp4:
         raise NotImplementedError("NVFP4 quantization is not implemented (int4 only)")
@@ -62,7 +103,19 @@ def quantize_w4a4_act_fuse_lora(
     if lora_down is not None and (lora_down.dtype != inp.dtype or lora_down.shape[0] != K):
         raise ValueError("lora_down must be (K, R) of the input dtype")
 
+    nstats = nscale = nshift = None
+    nrows, nld, nstride = 0, 0, 1
+    if norm is not None:
+        if fuse_glu:
+            raise NotImplementedError("norm= cannot be combined with fuse_glu")
+        nstats, nscale, nshift, nrows, nld, nstride = _norm_args(norm, inp, M, K, norm_eps)
     args = _lib.QuantizeArgs(
+        norm_stats=_lib.ptr(nstats),
+        norm_scale=_lib.ptr(nscale),
+        norm_shift=_lib.ptr(nshift),
+        norm_rows_per_batch=nrows,
+        norm_ld=nld,
+        norm_stride=nstride,
         x=inp.data_ptr(),
         smooth=_lib.ptr(smooth),
         lora_down_t=_lora_down_t(lora_down).data_ptr() if rank else None,
@@ -96,6 +149,8 @@ def svdq_quantize_w4a4_act_fuse_lora_cuda(
     fuse_glu: bool = False,
     fp4: bool = False,
     pad_size: int = 256,
+    norm: tuple | None = None,
+    norm_eps: float = 1e-6,
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """
     Quantize activations to int4 (per-group-64 absmax, after dividing by ``smooth``) and compute the LoRA
@@ -107,7 +162,8 @@ def svdq_quantize_w4a4_act_fuse_lora_cuda(
     allocated buffers held.
 
     Unlike the reference wrapper (which dereferences ``lora_down.shape`` unconditionally), ``lora_down=None`` is
-    accepted and returns ``lora_act_out`` with zero columns.
+    accepted and returns ``lora_act_out`` with zero columns.  ``norm`` / ``norm_eps``: the LayerNorm + modulate
+    prologue described in :func:`quantize_w4a4_act_fuse_lora` (an addition; ``None`` = the reference's behaviour).
     """
     if fp4:
         raise NotImplementedError("NVFP4 quantization is not implemented (int4 only)")
@@ -123,5 +179,6 @@ def svdq_quantize_w4a4_act_fuse_lora_cuda(
         oscales = torch.empty(channels // 64, batch_size_pad, dtype=input.dtype, device=input.device)
     if lora_act_out is None:
         lora_act_out = torch.empty(batch_size_pad, rank, dtype=torch.float32, device=input.device)
-    quantize_w4a4_act_fuse_lora(input, output, oscales, lora_down, lora_act_out if rank else None, smooth, fuse_glu, fp4)
+    quantize_w4a4_act_fuse_lora(input, output, oscales, lora_down, lora_act_out if rank else None, smooth, fuse_glu, fp4,
+                                norm=norm, norm_eps=norm_eps)
     return output, oscales, lora_act_out

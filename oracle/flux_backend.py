@@ -24,16 +24,24 @@ class OracleBackend:
         B, S, C = x.shape
         return self._lin32(x.reshape(B * S, C), lin).to(x.dtype).view(B, S, -1)
 
-    def gelu_mlp(self, x, fc1, fc2):
+    @staticmethod
+    def _mod(x2d, mod):
+        return x2d if mod is None else O.layernorm_modulate(x2d, mod[0], mod[1])
+
+    @staticmethod
+    def norm_stats(x):
+        return None
+
+    def gelu_mlp(self, x, fc1, fc2, mod=None):
         B, S, C = x.shape
-        h = self._lin32(x.reshape(B * S, C), fc1)
+        h = self._lin32(self._mod(x.reshape(B * S, C), mod), fc1)
         hp, hs, hl, _ = O.gelu_quant(h, fc2.smooth_factor, fc2.proj_down, x.dtype)
         y = self.gemm(hp, fc2.qweight, hs, fc2.wscales, fc2.bias, hl, fc2.proj_up, True)
         return y.to(x.dtype).view(B, S, -1)
 
-    def qkv(self, x, proj, norm_q, norm_k, rot):
+    def qkv(self, x, proj, norm_q, norm_k, rot, mod=None):
         B, S, C = x.shape
-        lin = self._lin32(x.reshape(B * S, C), proj)
+        lin = self._lin32(self._mod(x.reshape(B * S, C), mod), proj)
         out = O.qk_norm_rope(lin, norm_q.weight, norm_k.weight, rot.reshape(B * S, 128))
         return out.to(x.dtype).view(B, S, -1)
 

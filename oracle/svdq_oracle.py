@@ -30,6 +30,8 @@ awq_pack / awq_decode  mutual inverse, written from two different statements
                        of the layout (view/permute vs. index formula)
 awq_gemv               fp64 dense dequantised matmul
 flux_rope              closed form cos/sin of pos * theta**(-2i/d) in fp64
+layernorm_modulate     torch.nn.functional.layer_norm in fp64 and torch's own
+                       bf16 elementwise kernels on the CPU
 attention_fp16         fp64 softmax(q k^T * scale) v, independence of the key
                        block size, uniform-weights / constant-v / dominant-key
                        special cases
@@ -308,6 +310,25 @@ def awq_gemv(x: torch.Tensor, packed_i16: torch.Tensor, scales: torch.Tensor, ze
         xsum = xf[:, sl].sum(dim=1, keepdim=True)
         out += scales[c].float()[None, :] * dotq + zeros[c].float()[None, :] * xsum
     return out
+
+
+# --------------------------------------------------------------------------------------
+# LayerNorm + adaLN modulate in front of a quantized linear
+# --------------------------------------------------------------------------------------
+def layernorm_modulate(x: torch.Tensor, scale: torch.Tensor, shift: torch.Tensor, eps: float = 1e-6) -> torch.Tensor:
+    """nunchaku/models/normalization.py:97-104 and models/transformers/transformer_flux_v2.py:236-237 as three 16-bit
+    elementwise steps: LayerNorm without affine (fp32 statistics, biased variance, ``(x - mean) * rstd`` rounded to the
+    16-bit type), ``* scale`` rounded, ``+ shift`` rounded.  x (M, K); scale, shift (K,) or (batches, K)."""
+    dt = x.dtype
+    M, K = x.shape
+    xf = x.float()
+    mean = xf.mean(dim=1, keepdim=True)
+    var = ((xf - mean) ** 2).mean(dim=1, keepdim=True)
+    n = ((xf - mean) * (1.0 / torch.sqrt(var + eps))).to(dt)
+    sc = scale.reshape(-1, K).repeat_interleave(M // scale.reshape(-1, K).shape[0], dim=0)
+    sh = shift.reshape(-1, K).repeat_interleave(M // shift.reshape(-1, K).shape[0], dim=0)
+    y = (n.float() * sc.float()).to(dt)
+    return (y.float() + sh.float()).to(dt)
 
 
 # --------------------------------------------------------------------------------------

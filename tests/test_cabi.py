@@ -37,7 +37,7 @@ def test_struct_layouts_match_c(tmp_path):
     src = tmp_path / "sz.c"
     fields = {
         "svdq_gemm_args": ("GemmArgs", ["act", "M", "actual_m", "epilogue", "norm_q", "eps", "qout", "R2", "shift"]),
-        "svdq_quantize_args": ("QuantizeArgs", ["x", "M", "ld_x", "dtype", "shift"]),
+        "svdq_quantize_args": ("QuantizeArgs", ["x", "M", "ld_x", "dtype", "shift", "norm_stats", "norm_shift", "norm_rows_per_batch", "norm_stride"]),
         "svdq_awq_gemv_args": ("AwqGemvArgs", ["x", "M", "ld_out", "dtype"]),
         "svdq_attention_args": ("AttentionArgs", ["q", "vt", "sqb", "som", "B", "D", "dtype", "scale"]),
     }

@@ -102,3 +102,51 @@ def test_fuse_glu_close_to_oracle(dev):
     d = (codes - rc).abs()
     assert d.max() <= 1 and (d > 0).float().mean() < 1e-3  # exp() differs between libraries
     assert ((osc.cpu().float() - rs.float()).abs() <= rs.float().abs() * 2**-7 + 1e-9).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,K,R,batches", [(48, 256, 32, 1), (130, 384, 48, 1), (64, 512, 16, 2), (4608, 3072, 32, 1), (96, 1024, 0, 3)])
+def test_norm_modulate_prologue(dev, M, K, R, batches, dtype):
+    """LayerNorm + scale + shift applied inside the quantizer: codes, scales and the LoRA-down product are those of
+    the oracle's quantizer fed with the oracle's layernorm_modulate output.  exp-free arithmetic, but the row
+    statistics are summed in another order than on the CPU: a 16-bit rounding may flip, so codes may differ by one
+    step on a small fraction of entries (the contract of the fused GELU epilogue,
+    tests/triton/test_native_epilogues.py:246-253)."""
+    from nunchaku_rocm_amd import ops
+
+    print(f"case M={M} K={K} R={R} batches={batches} {dtype}", flush=True)
+    g = torch.Generator().manual_seed(M + K)
+    x = (torch.randn(M, K, generator=g) * 1.7 + 0.3).to(dtype)
+    scale = (1 + 0.3 * torch.randn(batches, K, generator=g)).to(dtype)
+    shift = (0.2 * torch.randn(batches, K, generator=g)).to(dtype)
+    lin = O.make_svdq_linear(K, 64, R=max(R, 16), seed=K, dtype=dtype)
+    ld = lin["proj_down"][:, :R].contiguous() if R else None
+    q, s, la = ops.svdq_quantize_w4a4_act_fuse_lora_cuda(x.to(dev), lora_down=None if ld is None else ld.to(dev),
+                                                          smooth=lin["smooth_factor"].to(dev), norm=(scale.to(dev), shift.to(dev)))  # fmt: skip
+    torch.cuda.synchronize()
+    xm = O.layernorm_modulate(x, scale, shift)
+    rq, rs, rl, rc = O.quantize_act(xm, ld, lin["smooth_factor"])
+    codes = O.unpack_int4(q[:M].cpu(), True)
+    diff = (codes - rc).abs()
+    rate = (diff > 0).float().mean().item()
+    print(f"  code mismatch rate {rate:.2e}", flush=True)
+    assert diff.max() <= 1 and rate < 1e-3
+    # a group maximum that flipped by one 16-bit step moves the stored scale by up to two of its own steps
+    ulp = 2**-7 if dtype == torch.bfloat16 else 2**-10
+    sdiff = (s[:, :M].cpu().float() - rs.float()).abs()
+    assert (sdiff <= rs.float().abs() * 2.01 * ulp + 1e-7).all() and (sdiff > 0).float().mean() < 1e-3
+    if R:
+        assert (la[:M].cpu() - rl).abs().max() <= 1e-2 * rl.abs().max()
+    # statistics computed once and passed in give the same bits as computing them inside the call
+    st = ops.layer_norm_stats(x.to(dev))
+    ref_mean = x.float().mean(dim=1)
+    assert (st[:, 0].cpu() - ref_mean).abs().max() <= 1e-5 * (1 + ref_mean.abs().max())
+    q2, s2, _ = ops.svdq_quantize_w4a4_act_fuse_lora_cuda(x.to(dev), lora_down=None if ld is None else ld.to(dev),
+                                                          smooth=lin["smooth_factor"].to(dev), norm=(scale.to(dev), shift.to(dev), st))  # fmt: skip
+    assert torch.equal(q2[:M], q[:M]) and torch.equal(s2[:, :M].view(torch.int16), s[:, :M].view(torch.int16))
+    # scale / shift as interleaved slices of one projection output (element stride 6), used where they lie
+    emb = torch.zeros(batches, K, 6, dtype=dtype, device=dev)
+    emb[:, :, 1], emb[:, :, 0] = scale.to(dev), shift.to(dev)
+    q3, s3, _ = ops.svdq_quantize_w4a4_act_fuse_lora_cuda(x.to(dev), lora_down=None if ld is None else ld.to(dev),
+                                                          smooth=lin["smooth_factor"].to(dev), norm=(emb[:, :, 1], emb[:, :, 0], st))  # fmt: skip
+    assert torch.equal(q3[:M], q[:M]) and torch.equal(s3[:, :M].view(torch.int16), s[:, :M].view(torch.int16))

@@ -431,3 +431,27 @@ def test_pack_scale_and_lowrank_hand_positions():
                             for e in range(2):
                                 back[rp * 16 + ns * 8 + nl, cp * 16 + ks * 8 + kl * 2 + e] = blk[nl, kl, ns, ks, e]
     assert (back == dn).all()
+
+
+# ---- LayerNorm + modulate -------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_layernorm_modulate_against_library(dtype):
+    g = torch.Generator().manual_seed(3)
+    M, K = 48, 384
+    x = (torch.randn(M, K, generator=g) * 2 + 0.7).to(dtype)
+    scale = (1 + 0.3 * torch.randn(2, K, generator=g)).to(dtype)
+    shift = (0.2 * torch.randn(2, K, generator=g)).to(dtype)
+    got = O.layernorm_modulate(x, scale, shift)
+    # the mathematics, in fp64, with the batch split written out (rows 0..23 use vector 0)
+    n64 = torch.nn.functional.layer_norm(x.double(), (K,), eps=1e-6)
+    ref64 = torch.cat([n64[:24] * scale[0].double() + shift[0].double(), n64[24:] * scale[1].double() + shift[1].double()])
+    ulp = 2**-7 if dtype == torch.bfloat16 else 2**-10
+    assert ((got.double() - ref64).abs() <= 3 * ulp * ref64.abs() + 3 * ulp).all()
+    # the rounding sequence: torch's own 16-bit CPU kernels, one op at a time
+    lib = torch.nn.functional.layer_norm(x, (K,), eps=1e-6)
+    lib = torch.cat([lib[:24] * scale[0] + shift[0], lib[24:] * scale[1] + shift[1]])
+    mism = (got.view(torch.int16) != lib.view(torch.int16)).float().mean().item()
+    assert mism < 2e-3 and (got.float() - lib.float()).abs().max() <= 2 * ulp * lib.float().abs().max()
+    # a constant row has zero variance: the output is the shift
+    xc = torch.full((16, K), 1.5).to(dtype)
+    assert torch.equal(O.layernorm_modulate(xc, scale[0], shift[0]), shift[:1].expand(16, K).contiguous())
