@@ -27,7 +27,7 @@ BF16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 / fp16 MFMA, published
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # HBM bytes of one QKV GEMM launch: FETCH_SIZE + WRITE_SIZE (KiB per dispatch, counter scale 1.000) of the grid-1327104
 # launches in profiles/bench_all_kernels_hbm_traffic.txt; counters cannot be read from inside this process
-GEMM_QKV_HBM_BYTES = (121271.8 + 82944.0) * 1024
+GEMM_QKV_HBM_BYTES = (121391.7 + 82944.0) * 1024
 
 
 def _events(n):
@@ -163,6 +163,16 @@ def main():
             "ms": round(q_ms, 5), "GB/s": round(q_bytes / q_ms / 1e6, 1), "frac_hbm": round(q_bytes / q_ms / 1e6 / HBM_PEAK_GBS, 4),
             "bytes": q_bytes, "GB/s_ref_convention": round((2 * M * K + M * K // 2) / q_ms / 1e6, 1),
         }  # fmt: skip
+        # the same quantizer with LayerNorm + adaLN modulate applied on the way in, and the row statistics it needs
+        nsc = (1 + 0.3 * torch.randn(K, device=dev)).to(torch.bfloat16)
+        nsh = (0.2 * torch.randn(K, device=dev)).to(torch.bfloat16)
+        st = ops.layer_norm_stats(x)
+        ms = _time_kernel(lambda: ops.svdq_quantize_w4a4_act_fuse_lora_cuda(x, qx, asc, lin["proj_down"], la, lin["smooth_factor"], norm=(nsc, nsh, st)), graph=not args.eager)
+        nb = q_bytes + 8 * M + 4 * K
+        kernels["quantize_act + layernorm + modulate M4608 K3072 R32"] = {"ms": round(ms, 5), "GB/s": round(nb / ms / 1e6, 1), "frac_hbm": round(nb / ms / 1e6 / HBM_PEAK_GBS, 4), "bytes": nb}  # fmt: skip
+        ms = _time_kernel(lambda: ops.layer_norm_stats(x), graph=not args.eager)
+        nb = 2 * M * K + 8 * M
+        kernels["row_stats M4608 K3072"] = {"ms": round(ms, 5), "GB/s": round(nb / ms / 1e6, 1), "frac_hbm": round(nb / ms / 1e6 / HBM_PEAK_GBS, 4), "bytes": nb}  # fmt: skip
         g_ms = _time_kernel(gemm)
         kernels["gemm_w4a4 M4608 K3072 N9216"] = {"ms": round(g_ms, 5), "TOP/s": round(ops_per_gemm / g_ms / 1e9, 1),
                                                   "frac_int8_mfma": round(ops_per_gemm / g_ms / 1e9 / INT8_MFMA_PEAK_TOPS, 4)}  # fmt: skip
