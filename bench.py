@@ -173,6 +173,15 @@ def main():
         ms = _time_kernel(lambda: ops.layer_norm_stats(x), graph=not args.eager)
         nb = 2 * M * K + 8 * M
         kernels["row_stats M4608 K3072"] = {"ms": round(ms, 5), "GB/s": round(nb / ms / 1e6, 1), "frac_hbm": round(nb / ms / 1e6 / HBM_PEAK_GBS, 4), "bytes": nb}  # fmt: skip
+        # gated residual update (x + gate * y) with the row statistics of the result
+        xr = x.view(1, M, K)
+        yr = torch.randn(1, M, K, device=dev).to(torch.bfloat16)
+        gt = torch.randn(1, K, device=dev).to(torch.bfloat16)
+        orr = torch.empty_like(xr)
+        ms = _time_kernel(lambda: ops.gated_residual(xr, gt, yr, out=orr, want_stats=True), graph=not args.eager)
+        nb = 3 * 2 * M * K + 2 * K + 8 * M
+        kernels["gated_residual + row_stats M4608 K3072"] = {"ms": round(ms, 5), "GB/s": round(nb / ms / 1e6, 1), "frac_hbm": round(nb / ms / 1e6 / HBM_PEAK_GBS, 4), "bytes": nb}  # fmt: skip
+        del yr, orr
         g_ms = _time_kernel(gemm)
         kernels["gemm_w4a4 M4608 K3072 N9216"] = {"ms": round(g_ms, 5), "TOP/s": round(ops_per_gemm / g_ms / 1e9, 1),
                                                   "frac_int8_mfma": round(ops_per_gemm / g_ms / 1e9 / INT8_MFMA_PEAK_TOPS, 4)}  # fmt: skip

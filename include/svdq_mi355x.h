@@ -16,6 +16,7 @@
  *   svdq_awq_gemv_w4a16      nunchaku/ops/dispatch.py:19-34      (_C.ops.gemv_awq / ops/triton/awq.py:186 awq_gemv_w4a16)
  *   svdq_attention_fp16      nunchaku/ops/dispatch.py:67-99      (_C.ops.attention_fp16 / ops/triton/attention.py:111 attention_fp16)
  *   svdq_row_stats           nunchaku/models/normalization.py:97 (the LayerNorm statistics; applied inside svdq_quantize_act)
+ *   svdq_gated_residual      nunchaku/models/transformers/transformer_flux_v2.py:233-243, :326-330 (gate * y + residual)
  *   svdq_unpack_mma_*        nunchaku/ops/triton/layout.py:36-292 (checkpoint layout -> natural layout)
  *   svdq_transpose_lora_down no counterpart: one-time re-layout of a LoRA-down weight, see below
  *   svdq_group_acc_i32       no counterpart: debug read-out of the exact int32 group accumulators
@@ -84,6 +85,16 @@ int svdq_quantize_act(const svdq_quantize_args *args, void *stream);
  * LayerNorm needs (nunchaku/models/normalization.py:97), for the quantizer's norm prologue. */
 int svdq_row_stats(const void *x, float *stats, int32_t M, int32_t K, int32_t ld_x, int32_t dtype, float eps,
                    void *stream);
+
+/* Gated residual update of a transformer block, one pass: out[m, k] = T(x[m, k] + T(gate[b, k] * t[m, k])) with
+ * t = y, or T(y + y2) when y2 is given (the three elementwise torch kernels of
+ * nunchaku/models/transformers/transformer_flux_v2.py:233-234, :241-243 and :326-330, each step rounded to T), and,
+ * when stats is not NULL, the (mean, rstd) row statistics of out for the next layer's norm prologue.  gate element
+ * (b, k) is at b * gate_ld + k * gate_stride with b = m / rows_per_batch (rows_per_batch 0 = one vector).
+ * K % 8 == 0, K <= 8192; x, y, y2, out rows 16-byte aligned with the row strides ld_* in elements; out may be x. */
+int svdq_gated_residual(const void *x, const void *gate, const void *y, const void *y2, void *out, float *stats,
+                        int32_t M, int32_t K, int32_t ld_x, int32_t ld_y, int32_t ld_out, int32_t rows_per_batch,
+                        int32_t gate_ld, int32_t gate_stride, int32_t dtype, float eps, void *stream);
 
 /* (K, R) row-major T  ->  (R, K) row-major T.  Done once per weight; the quantizer and the fused
  * requantizing epilogues read the transposed form so their MFMA operands are K-contiguous. */

@@ -352,6 +352,80 @@ __global__ __launch_bounds__(256) void row_stats_kernel(const uint16_t *x, float
     }
 }
 
+// one wavefront per row; the rounded results stay in registers (packed) for the statistics, so the row is read once
+template <typename T, bool SUM2, bool STATS>
+__global__ __launch_bounds__(256) void gated_residual_kernel(const uint16_t *x, const uint16_t *gate, const uint16_t *y,
+                                                             const uint16_t *y2, uint16_t *out, float *stats, int M, int K,
+                                                             long ld_x, long ld_y, long ld_out, int rows_per_batch,
+                                                             long gate_ld, int gate_stride, float eps) {
+    constexpr int MAXC = 16;  // 16-byte chunks per lane: K <= 64 * 8 * 16
+    const int lane = threadIdx.x & 63, m = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (m >= M) return;
+    const uint16_t *xr = x + (long)m * ld_x, *yr = y + (long)m * ld_y, *y2r = SUM2 ? y2 + (long)m * ld_y : nullptr;
+    const uint16_t *gr = gate + (rows_per_batch > 0 ? (long)(m / rows_per_batch) * gate_ld : 0);
+    uint16_t *orow = out + (long)m * ld_out;
+    auto rnd = [](float f) { return T::to_f32(T::from_f32(f)); };
+    auto wave_sum = [](float s) {
+#pragma unroll
+        for (int o = 32; o >= 1; o >>= 1) s += __shfl_xor(s, o);
+        return s;
+    };
+    v4i res[MAXC];
+    float s = 0.0f;
+#pragma unroll
+    for (int c = 0; c < MAXC; c++) {
+        const int k = 8 * lane + 512 * c;
+        if (k < K) {
+            const v4i xv = *(const v4i *)(xr + k), yv = *(const v4i *)(yr + k);
+            v4i zv = {0, 0, 0, 0};
+            if (SUM2) zv = *(const v4i *)(y2r + k);
+            float g[8];
+            if (gate_stride == 1) {
+                const v4i gv = *(const v4i *)(gr + k);
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    g[2 * e] = T::lo_f32((uint32_t)gv[e]);
+                    g[2 * e + 1] = T::hi_f32((uint32_t)gv[e]);
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; e++) g[e] = T::to_f32(gr[(long)(k + e) * gate_stride]);
+            }
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                float t0 = T::lo_f32((uint32_t)yv[e]), t1 = T::hi_f32((uint32_t)yv[e]);
+                if (SUM2) {
+                    t0 = rnd(t0 + T::lo_f32((uint32_t)zv[e]));
+                    t1 = rnd(t1 + T::hi_f32((uint32_t)zv[e]));
+                }
+                const float o0 = rnd(T::lo_f32((uint32_t)xv[e]) + rnd(g[2 * e] * t0));
+                const float o1 = rnd(T::hi_f32((uint32_t)xv[e]) + rnd(g[2 * e + 1] * t1));
+                s += o0 + o1;
+                res[c][e] = (int)pack2<T>(o0, o1);
+            }
+            *(v4i *)(orow + k) = res[c];
+        }
+    }
+    if (!STATS) return;
+    const float mean = wave_sum(s) / (float)K;
+    float q = 0.0f;
+#pragma unroll
+    for (int c = 0; c < MAXC; c++) {
+        if (8 * lane + 512 * c < K) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const float d0 = T::lo_f32((uint32_t)res[c][e]) - mean, d1 = T::hi_f32((uint32_t)res[c][e]) - mean;
+                q += d0 * d0 + d1 * d1;
+            }
+        }
+    }
+    const float var = wave_sum(q) / (float)K;
+    if (lane == 0) {
+        stats[2 * m] = mean;
+        stats[2 * m + 1] = 1.0f / sqrtf(var + eps);
+    }
+}
+
 __global__ void transpose_kr_kernel(const uint16_t *in, uint16_t *out, int K, int R, int ld_in) {
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= K * R) return;
@@ -475,6 +549,55 @@ extern "C" int svdq_row_stats(const void *x, float *stats, int32_t M, int32_t K,
     else
         hipLaunchKernelGGL(row_stats_kernel<FP16>, grid, block, 0, (hipStream_t)stream, (const uint16_t *)x, stats, M, K, (long)ld_x, eps);
     return check_launch("svdq_row_stats");
+}
+
+template <typename T>
+static void launch_gated_residual(const void *x, const void *gate, const void *y, const void *y2, void *out, float *stats,
+                                  int M, int K, long ld_x, long ld_y, long ld_out, int rpb, long gate_ld, int gate_stride,
+                                  float eps, hipStream_t s) {
+    const dim3 grid((M + 3) / 4), block(256);
+#define SVDQ_GR(S2, ST)                                                                                                   \
+    hipLaunchKernelGGL((gated_residual_kernel<T, S2, ST>), grid, block, 0, s, (const uint16_t *)x, (const uint16_t *)gate, \
+                       (const uint16_t *)y, (const uint16_t *)y2, (uint16_t *)out, stats, M, K, ld_x, ld_y, ld_out, rpb,   \
+                       gate_ld, gate_stride, eps)
+    if (y2 && stats)
+        SVDQ_GR(true, true);
+    else if (y2)
+        SVDQ_GR(true, false);
+    else if (stats)
+        SVDQ_GR(false, true);
+    else
+        SVDQ_GR(false, false);
+#undef SVDQ_GR
+}
+
+extern "C" int svdq_gated_residual(const void *x, const void *gate, const void *y, const void *y2, void *out, float *stats,
+                                   int32_t M, int32_t K, int32_t ld_x, int32_t ld_y, int32_t ld_out, int32_t rows_per_batch,
+                                   int32_t gate_ld, int32_t gate_stride, int32_t dtype, float eps, void *stream) {
+    if (!x || !gate || !y || !out || M < 0 || K <= 0 || K % 8) {
+        set_error("svdq_gated_residual: x, gate, y and out are required and K=%d must be a positive multiple of 8 (M=%d)", K, M);
+        return SVDQ_E_INVALID;
+    }
+    if (K > 8192) {
+        set_error("svdq_gated_residual: K=%d exceeds 8192 (a row is held in one wavefront's registers)", K);
+        return SVDQ_E_UNSUPPORTED;
+    }
+    auto al = [](const void *p) { return ((uintptr_t)p & 15) == 0; };
+    if (ld_x < K || ld_y < K || ld_out < K || ld_x % 8 || ld_y % 8 || ld_out % 8 || !al(x) || !al(y) || !al(out) ||
+        (y2 && !al(y2)) || rows_per_batch < 0 || gate_stride < 1 || (gate_stride == 1 && (!al(gate) || gate_ld % 8))) {
+        set_error("svdq_gated_residual: rows of x, y, y2, out (and of a contiguous gate) must be 16-byte aligned and hold K elements");
+        return SVDQ_E_INVALID;
+    }
+    if (dtype != SVDQ_BF16 && dtype != SVDQ_FP16) {
+        set_error("svdq_gated_residual: dtype %d", dtype);
+        return SVDQ_E_INVALID;
+    }
+    if (M == 0) return SVDQ_OK;
+    if (dtype == SVDQ_BF16)
+        launch_gated_residual<BF16>(x, gate, y, y2, out, stats, M, K, ld_x, ld_y, ld_out, rows_per_batch, gate_ld, gate_stride, eps, (hipStream_t)stream);
+    else
+        launch_gated_residual<FP16>(x, gate, y, y2, out, stats, M, K, ld_x, ld_y, ld_out, rows_per_batch, gate_ld, gate_stride, eps, (hipStream_t)stream);
+    return check_launch("svdq_gated_residual");
 }
 
 extern "C" int svdq_transpose_lora_down(const void *lora_down, void *lora_down_t, int32_t K, int32_t R,

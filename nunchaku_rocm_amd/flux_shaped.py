@@ -59,6 +59,11 @@ class HipBackend:
         return _ops.fused_qkv_norm_rottary(x, proj, norm_q, norm_k, rot, norm=mod)
 
     @staticmethod
+    def gated_residual(x, gate, y, y2=None, want_stats=False):
+        """``(x + gate[:, None] * (y [+ y2]), row statistics of the result or None)``"""
+        return _ops.gated_residual(x, gate, y, y2, want_stats=want_stats)
+
+    @staticmethod
     def norm_stats(x):
         """Row statistics of x, to share between several ``mod=`` consumers of the same rows."""
         return _ops.layer_norm_stats(x)
@@ -181,10 +186,11 @@ class _DoubleBlock(nn.Module):
         sh_a, sc_a, g_a, sh_m, sc_m, g_m = self._mod6(be, self.norm1, temb)
         csh_a, csc_a, cg_a, csh_m, csc_m, cg_m = self._mod6(be, self.norm1_context, temb)
         ax, ac = self.attn(be, x, ctx, rot_img, rot_txt, mod_x=(sc_a, sh_a), mod_ctx=(csc_a, csh_a))
-        x = x + g_a.unsqueeze(1) * ax
-        x = x + g_m.unsqueeze(1) * be.gelu_mlp(x, self.ff_fc1, self.ff_fc2, mod=(sc_m, sh_m))
-        ctx = ctx + cg_a.unsqueeze(1) * ac
-        ctx = ctx + cg_m.unsqueeze(1) * be.gelu_mlp(ctx, self.ffc_fc1, self.ffc_fc2, mod=(csc_m, csh_m))
+        # x + gate * y in one kernel that also hands the next norm its row statistics
+        x, st = be.gated_residual(x, g_a, ax, want_stats=True)
+        x, _ = be.gated_residual(x, g_m, be.gelu_mlp(x, self.ff_fc1, self.ff_fc2, mod=(sc_m, sh_m, st)))
+        ctx, st = be.gated_residual(ctx, cg_a, ac, want_stats=True)
+        ctx, _ = be.gated_residual(ctx, cg_m, be.gelu_mlp(ctx, self.ffc_fc1, self.ffc_fc2, mod=(csc_m, csh_m, st)))
         return ctx, x
 
 
@@ -198,13 +204,14 @@ class _SingleBlock(nn.Module):
         self.attn = _Attention(cfg, joint=False, single=True, device=device, dtype=dtype)
         self.C = C
 
-    def forward(self, be, x, temb, rot):
+    def forward(self, be, x, temb, rot, stats=None):
+        """``stats``: row statistics of x if the producer of x already has them.  Returns (x, statistics of it)."""
         emb = be.awq(F.silu(temb), self.norm)
         shift, scale, gate = emb.view(emb.shape[0], -1, 3).permute(2, 0, 1)
-        mod = (scale, shift, be.norm_stats(x))  # one set of row statistics for both consumers
+        mod = (scale, shift, stats if stats is not None else be.norm_stats(x))  # one set for both consumers
         mlp = be.gelu_mlp(x, self.mlp_fc1, self.mlp_fc2, mod=mod)
         att = self.attn(be, x, None, rot, None, mod_x=mod)
-        return x + gate.unsqueeze(1) * (att + mlp)
+        return be.gated_residual(x, gate, att, mlp, want_stats=True)
 
 
 class FluxShapedTransformer(nn.Module):
@@ -250,8 +257,9 @@ class FluxShapedTransformer(nn.Module):
         for blk in self.double_blocks:
             ctx, x = blk(be, x, ctx, temb, rot_img, rot_txt)
         x = torch.cat([ctx, x], dim=1)
+        stats = None
         for blk in self.single_blocks:
-            x = blk(be, x, temb, rot)
+            x, stats = blk(be, x, temb, rot, stats)
         x = x[:, t_txt:]
         scale, shift = self.norm_out_linear(F.silu(temb)).chunk(2, dim=1)
         x = F.layer_norm(x, (self.cfg.hidden,), eps=1e-6) * (1 + scale)[:, None] + shift[:, None]

@@ -1,6 +1,7 @@
 """Operator API of the SVDQuant path: same names and signatures as ``nunchaku.ops`` in the reference."""
 
 from .attention import attention_fp16, scaled_dot_product_attention
+from .elementwise import gated_residual
 from .fused import fused_gelu_mlp, fused_qkv_norm_rottary, fused_swiglu_mlp, interleave_swiglu_linear_
 from .gemm import svdq_gemm_w4a4_cuda
 from .gemv import awq_gemv_w4a16_cuda
@@ -16,5 +17,6 @@ __all__ = [
     "interleave_swiglu_linear_",
     "attention_fp16",
     "layer_norm_stats",
+    "gated_residual",
     "scaled_dot_product_attention",
 ]

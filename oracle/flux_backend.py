@@ -32,6 +32,10 @@ class OracleBackend:
     def norm_stats(x):
         return None
 
+    @staticmethod
+    def gated_residual(x, gate, y, y2=None, want_stats=False):
+        return O.gated_residual(x, gate, y, y2), None
+
     def gelu_mlp(self, x, fc1, fc2, mod=None):
         B, S, C = x.shape
         h = self._lin32(self._mod(x.reshape(B * S, C), mod), fc1)

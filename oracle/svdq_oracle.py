@@ -30,6 +30,7 @@ awq_pack / awq_decode  mutual inverse, written from two different statements
                        of the layout (view/permute vs. index formula)
 awq_gemv               fp64 dense dequantised matmul
 flux_rope              closed form cos/sin of pos * theta**(-2i/d) in fp64
+gated_residual         torch's own 16-bit CPU kernels, op by op (bit-equal)
 layernorm_modulate     torch.nn.functional.layer_norm in fp64 and torch's own
                        bf16 elementwise kernels on the CPU
 attention_fp16         fp64 softmax(q k^T * scale) v, independence of the key
@@ -329,6 +330,16 @@ def layernorm_modulate(x: torch.Tensor, scale: torch.Tensor, shift: torch.Tensor
     sh = shift.reshape(-1, K).repeat_interleave(M // shift.reshape(-1, K).shape[0], dim=0)
     y = (n.float() * sc.float()).to(dt)
     return (y.float() + sh.float()).to(dt)
+
+
+def gated_residual(x: torch.Tensor, gate: torch.Tensor, y: torch.Tensor, y2: torch.Tensor | None = None) -> torch.Tensor:
+    """nunchaku/models/transformers/transformer_flux_v2.py:233-234, :241-243 (``x + gate.unsqueeze(1) * y``) and
+    :326-330 (``x + gate.unsqueeze(1) * (y + y2)``) as 16-bit elementwise steps: every +, * rounded to the dtype.
+    x, y (B, S, C); gate (B, C)."""
+    dt = x.dtype
+    t = y if y2 is None else (y.float() + y2.float()).to(dt)
+    g = (gate.float()[:, None, :] * t.float()).to(dt)
+    return (x.float() + g.float()).to(dt)
 
 
 # --------------------------------------------------------------------------------------

@@ -455,3 +455,12 @@ def test_layernorm_modulate_against_library(dtype):
     # a constant row has zero variance: the output is the shift
     xc = torch.full((16, K), 1.5).to(dtype)
     assert torch.equal(O.layernorm_modulate(xc, scale[0], shift[0]), shift[:1].expand(16, K).contiguous())
+
+
+def test_gated_residual_is_torchs_op_sequence():
+    g = torch.Generator().manual_seed(4)
+    for dtype in (torch.bfloat16, torch.float16):
+        x, y, y2 = (torch.randn(2, 5, 64, generator=g).to(dtype) for _ in range(3))
+        gate = torch.randn(2, 64, generator=g).to(dtype)
+        assert torch.equal(O.gated_residual(x, gate, y), x + gate.unsqueeze(1) * y)
+        assert torch.equal(O.gated_residual(x, gate, y, y2), x + gate.unsqueeze(1) * (y + y2))
