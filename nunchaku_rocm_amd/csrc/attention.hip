@@ -154,8 +154,8 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a
     // Scores come out of the matrix instructions already relative to the row's reference: the accumulator of S^T starts
     // at -bias (cinit), so p = 2^s' with s' = s - bias needs no subtraction.  bias trails the true row maximum by at
     // most AT_LAZY (it only moves when a maximum exceeds it by more than that), which keeps p <= 2^AT_LAZY.
-    // gap = reference - bias: 0 once a reference exists, -inf before the first keys.
-    float bias = 0.0f, gap = -INFINITY, l_run = 0.0f;
+    // The bias itself only lives in cinit; gap = reference - bias: 0 once a reference exists, -inf before the first keys.
+    float gap = -INFINITY, l_run = 0.0f;
     v16f cinit;
 #pragma unroll
     for (int i = 0; i < 16; i++) cinit[i] = 0.0f;
@@ -234,7 +234,6 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a
 #pragma unroll
             for (int i = 0; i < 16; i++) acc_o[dt][i] *= alpha;
         shift16(cinit);
-        bias += shift;
     };
 
     for (int blk = 0; blk < nblk; blk++) {

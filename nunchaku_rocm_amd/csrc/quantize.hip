@@ -97,7 +97,6 @@ __global__ __launch_bounds__(Q_WAVES * 64, NORM ? 4 : 2) void quantize_act_kerne
     for (int rc = 0; rc < nchunks; rc++) {
         v4f acc0 = (v4f){0.f, 0.f, 0.f, 0.f}, acc1 = (v4f){0.f, 0.f, 0.f, 0.f};
         // ranks >= R re-read rank R - 1; their accumulator rows are never stored
-        const int r0 = rc * Q_RCHUNK + ml;
         const uint8_t *__restrict__ lbase = (const uint8_t *)a.lora_down_t;
         uint32_t ldma[4] = {0, 0, 0, 0};
         if (HAS_LORA) {
