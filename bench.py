@@ -111,8 +111,8 @@ def main():
     ap.add_argument("--eager", action="store_true", help="time the small kernels eagerly too (no HIP graph): for counter runs")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py: this build runs on one GPU only (the path shards over tokens with no exchange; "
-              "see DESIGN.md); run with --gpus 1", file=sys.stderr)  # fmt: skip
+        print("bench.py: this build runs on one GPU only (the path would shard over tokens with no exchange between "
+              "GPUs, and no multi-GPU figure is produced); run with --gpus 1", file=sys.stderr)  # fmt: skip
         sys.exit(2)
 
     import torch
@@ -287,7 +287,7 @@ def main():
         "vs_baseline": None,
         "dtype": "i8",
         "data": "synthetic",
-        "config": {"workload": "FLUX.1 QKV SVDQuant linear: activation quantizer + W4A4 GEMM, M=4608 K=3072 N=9216 group 64 LoRA rank 32 (BASELINE configs[1])",
+        "config": {"workload": "FLUX.1 QKV SVDQuant linear: activation quantizer + W4A4 GEMM, M=4608 K=3072 N=9216 group 64 LoRA rank 32 (the reference's FLUX.1 QKV benchmark shape)",
                    "M": M, "K": K, "N": N, "rank": R, "group": 64},  # fmt: skip
         "roofline": {
             "bound": "mfma",
