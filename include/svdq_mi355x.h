@@ -181,22 +181,22 @@ typedef struct {
 int svdq_awq_gemv_w4a16(const svdq_awq_gemv_args *args, void *stream);
 
 /*
- * Unmasked scaled-dot-product attention, head dimension 128 (nunchaku/ops/dispatch.py:67-99 attention_fp16 /
- * ops/triton/attention.py:111-169): o[b, t, h*128 + d] = softmax_k(scale * q[b,h,t,:] . k[b,h,k,:]) . v[b,h,k,d], fp32
+ * Unmasked scaled-dot-product attention, head dimension D = 128 or 64 (nunchaku/ops/dispatch.py:67-99 attention_fp16 /
+ * ops/triton/attention.py:111-169): o[b, t, h*D + d] = softmax_k(scale * q[b,h,t,:] . k[b,h,k,:]) . v[b,h,k,d], fp32
  * softmax and accumulation, P rounded to T.  Strides are in elements; the last dimension of q, k, v, o is contiguous.
- * `vt` is a caller-owned workspace of svdq_attention_workspace_bytes(B, H, Tkv, 128) bytes (a transposed copy of v made
+ * `vt` is a caller-owned workspace of svdq_attention_workspace_bytes(B, H, Tkv, D) bytes (a transposed copy of v made
  * by the call itself).
  */
 typedef struct {
-    const void *q;  /* (B, H, Tq, 128) T  */
-    const void *k;  /* (B, H, Tkv, 128) T */
-    const void *v;  /* (B, H, Tkv, 128) T */
-    void *o;        /* (B, Tq, H * 128) T */
+    const void *q;  /* (B, H, Tq, D) T  */
+    const void *k;  /* (B, H, Tkv, D) T */
+    const void *v;  /* (B, H, Tkv, D) T */
+    void *o;        /* (B, Tq, H * D) T */
     void *vt;       /* workspace          */
     int64_t sqb, sqh, sqm, skb, skh, skn, svb, svh, svn, sob, som;
     int32_t B, H, Tq, Tkv, D;
     int32_t dtype;
-    float scale;    /* normally 128 ** -0.5 */
+    float scale;    /* normally D ** -0.5 */
 } svdq_attention_args;
 
 int svdq_attention_fp16(const svdq_attention_args *args, void *stream);

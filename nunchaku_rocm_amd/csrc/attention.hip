@@ -1,4 +1,4 @@
-// Unmasked scaled-dot-product attention (flash-attention forward) for gfx950, head dimension 128.
+// Unmasked scaled-dot-product attention (flash-attention forward) for gfx950, head dimension 128 or 64.
 //
 // Arithmetic (reference: nunchaku/ops/triton/attention.py:37-169): q is multiplied by scale * log2(e) and rounded to
 // the 16-bit type; per block of keys S = q k^T in fp32, online softmax with exp2 (a row reference m and row sum l),
@@ -18,12 +18,12 @@
 //  * The S^T accumulator starts at minus the row reference, so the scores leave the matrix instruction ready for
 //    exp2: no subtraction per score.
 //  * V^T is made once per call by a small transposing kernel (keys permuted as above, key count padded to 64); the
-//    main kernel then streams K tiles (64 keys x 256 bytes) and V^T tiles (128 rows x 128 bytes) buffer -> LDS
+//    main kernel then streams K tiles (64 keys x 2 D bytes) and V^T tiles (D rows x 128 bytes) buffer -> LDS
 //    directly (buffer_load_dwordx4 ... lds, whole rows per load, per-lane offsets fixed and the tile chosen by the
 //    scalar buffer base, 16-byte chunks XOR-swizzled so that the operand reads are conflict free), two tiles in
 //    flight, one barrier per 64 keys.
 //  * 256 threads = 4 wavefronts of 32 queries, two workgroups per CU; Q stays in registers (pre-scaled), the output
-//    accumulator is 64 registers.  A tile is processed as two 32-key halves so that the softmax instructions of one
+//    accumulator is D / 2 registers.  A tile is processed as two 32-key halves so that the softmax instructions of one
 //    half sit between the matrix instructions of the other (see the pipeline comment in the kernel).
 //  * Workgroups of one head run on one XCD (when the head count is a multiple of 8), so K and V^T of a head are
 //    fetched into one L2 only.
@@ -31,25 +31,39 @@
 
 namespace svdq {
 
-constexpr int AT_D = 128;                  // head dimension
 constexpr int AT_BQ = 128, AT_BK = 64;     // queries per workgroup, keys per tile
-constexpr int AT_KT_BYTES = AT_BK * AT_D * 2;  // 16 KB K tile: [key][16 chunks of 16 bytes]
-constexpr int AT_VT_BYTES = AT_D * AT_BK * 2;  // 16 KB V^T tile: [d][8 chunks of 16 bytes]
-constexpr int AT_STAGE = AT_KT_BYTES + AT_VT_BYTES;
-constexpr int AT_OPITCH = AT_D * 2 + 16;   // staged output row
+
+// Geometry for head dimension D (128 or 64).  A K tile is [key][2 D bytes], a V^T tile [d][128 bytes]; every block
+// load moves 1 KB (64 lanes x 16 bytes) = whole rows; 16-byte chunks are XOR-swizzled by the row so that the operand
+// reads (32 rows x one chunk per half-wave) touch every bank once: rows of 256 bytes by row & 15, rows of 128 bytes (two
+// rows span the 64 banks) by row / 2 & 7.
+template <int D>
+struct AtGeo {
+    static constexpr int NC = D / 16;               // 16-wide k chunks of q k^T = matrix instructions per 32-key half
+    static constexpr int NDT = D / 32;              // 32-row d tiles of O^T
+    static constexpr int KROW = 2 * D;              // bytes per key row
+    static constexpr int KCH = KROW / 16;           // chunks per key row (16 or 8)
+    static constexpr int KT_BYTES = AT_BK * KROW;   // K tile
+    static constexpr int VT_BYTES = D * AT_BK * 2;  // V^T tile
+    static constexpr int STAGE = KT_BYTES + VT_BYTES;
+    static constexpr int LOADS = KT_BYTES / 1024 / 4;  // block loads per wavefront and tile, of K and of V^T alike
+    static constexpr int OPITCH = 2 * D + 16;       // staged output row
+    __host__ __device__ static constexpr int kswz(int row) { return KROW == 256 ? (row & 15) : ((row >> 1) & 7); }
+};
 
 // position p of a 16-key chunk holds key sigma(p)
 __device__ __host__ inline int at_sigma(int p) { return (p & 3) | ((p & 4) << 1) | ((p & 8) >> 1); }
 
-// V (B, H, Tkv, 128) with arbitrary strides -> vt[(b * H + h) * 128 + d][Tpad], keys permuted inside 16-key chunks,
+// V (B, H, Tkv, D) with arbitrary strides -> vt[(b * H + h) * D + d][Tpad], keys permuted inside 16-key chunks,
 // keys >= Tkv zero
+template <int D>
 __global__ __launch_bounds__(256) void transpose_v_kernel(const uint16_t *v, uint16_t *vt, int H, int Tkv, int Tpad,
                                                           long svb, long svh, long svn) {
-    __shared__ uint16_t tile[AT_BK][AT_D + 2];
+    __shared__ uint16_t tile[AT_BK][D + 2];
     const int k0 = blockIdx.x * AT_BK, h = blockIdx.y, b = blockIdx.z;
     const uint16_t *vb = v + b * svb + h * svh;
-    for (int i = threadIdx.x; i < AT_BK * (AT_D / 8); i += 256) {
-        const int key = i / (AT_D / 8), c = i % (AT_D / 8);
+    for (int i = threadIdx.x; i < AT_BK * (D / 8); i += 256) {
+        const int key = i / (D / 8), c = i % (D / 8);
         v4i x = {0, 0, 0, 0};
         if (k0 + key < Tkv) x = *(const v4i *)(vb + (long)(k0 + key) * svn + 8 * c);
 #pragma unroll
@@ -59,8 +73,8 @@ __global__ __launch_bounds__(256) void transpose_v_kernel(const uint16_t *v, uin
         }
     }
     __syncthreads();
-    uint16_t *ob = vt + ((size_t)(b * H + h) * AT_D) * Tpad + k0;
-    for (int i = threadIdx.x; i < AT_D * (AT_BK / 8); i += 256) {
+    uint16_t *ob = vt + ((size_t)(b * H + h) * D) * Tpad + k0;
+    for (int i = threadIdx.x; i < D * (AT_BK / 8); i += 256) {
         const int d = i / (AT_BK / 8), c = i % (AT_BK / 8);  // 8 consecutive positions of row d
         uint32_t w[4];
 #pragma unroll
@@ -74,11 +88,22 @@ __global__ __launch_bounds__(256) void transpose_v_kernel(const uint16_t *v, uin
 }
 
 constexpr uint32_t AT_RSRC_FLAGS = 0x00020000;  // raw buffer, 32-bit data format (gfx9 family)
+
+// 16 bytes per lane from a raw buffer (`bytes` long from `base`; reads past it return zero) straight into LDS at
+// lds + 16 * lane.  Plain functions, so that the kernel template below calls no target builtin with dependent operands.
+__device__ inline __amdgpu_buffer_rsrc_t at_buffer(const void *base, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, (int)bytes, AT_RSRC_FLAGS);
+}
+__device__ inline void at_load16_lds(__amdgpu_buffer_rsrc_t r, uint8_t *lds, uint32_t lane_off, uint32_t wave_off) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (SVDQ_AS3 void *)lds, 16, lane_off, wave_off, 0, 0);
+}
 constexpr float AT_LAZY = 8.0f;                 // the accumulator is rescaled when a row maximum grew by more than this
 
-template <typename T>
+template <typename T, int D>
 __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a, int Tpad, int ntile, int xcd_heads) {
-    __shared__ __align__(16) uint8_t smem[2 * AT_STAGE];
+    using G = AtGeo<D>;
+    constexpr int NC = G::NC, NDT = G::NDT, LOADS = G::LOADS;
+    __shared__ __align__(16) uint8_t smem[2 * G::STAGE];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -97,58 +122,56 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a
     const int b = bh / a.H, h = bh % a.H;
     const int q0 = qt * AT_BQ;
 
-    // ---- Q^T operand: lane (q, half) holds q[16 c + 8 half, +8) for c = 0..7, scaled and rounded to T ------------
+    // ---- Q^T operand: lane (q, half) holds q[16 c + 8 half, +8) for c < NC, scaled and rounded to T ---------------
     const int qrow = min(q0 + wave * 32 + l32, a.Tq - 1);
     const uint16_t *qp = (const uint16_t *)a.q + (long)b * a.sqb + (long)h * a.sqh + (long)qrow * a.sqm + 8 * half;
     const float qscale = a.scale * 1.4426950408889634f;
-    v4i qop[8];
+    v4i qop[NC];
 #pragma unroll
-    for (int c = 0; c < 8; c++) {
+    for (int c = 0; c < NC; c++) {
         const v4i raw = *(const v4i *)(qp + 16 * c);
 #pragma unroll
         for (int e = 0; e < 4; e++)
             qop[c][e] = (int)pack2<T>(T::lo_f32((uint32_t)raw[e]) * qscale, T::hi_f32((uint32_t)raw[e]) * qscale);
     }
 
-    // ---- tile loads (buffer -> LDS, 16 bytes per lane): lane l of K load i fetches chunk (l % 16) ^ (row & 15) of key
-    // row 4 i + l / 16; of V^T load i, chunk (l % 8) ^ (row / 2 & 7) of d row 8 i + l / 8 (rows are 128 bytes: two rows span the 64 banks).  Four K and four V^T loads per
-    // wavefront and tile.  The per-lane offsets never change; the tile is selected by the (scalar) buffer base, and
-    // key rows past the end lie outside the K buffer's range and arrive as zeros.
+    // ---- tile loads (buffer -> LDS, 16 bytes per lane): lane l of K load i fetches one chunk of key row
+    // (64 / KCH) i + l / KCH; of V^T load i, one chunk of d row 8 i + l / 8.  LOADS K and LOADS V^T loads per wavefront
+    // and tile.  The per-lane offsets never change; the tile is selected by the (scalar) buffer base, and key rows
+    // past the end lie outside the K buffer's range and arrive as zeros.
     const uint8_t *kbase = (const uint8_t *)a.k + ((long)b * a.skb + (long)h * a.skh) * 2;
-    const uint8_t *vbase = (const uint8_t *)a.vt + ((size_t)bh * AT_D) * Tpad * 2;
-    const uint32_t kbytes = (uint32_t)(((long)(a.Tkv - 1) * a.skn + AT_D) * 2);
+    const uint8_t *vbase = (const uint8_t *)a.vt + ((size_t)bh * D) * Tpad * 2;
+    const uint32_t kbytes = (uint32_t)(((long)(a.Tkv - 1) * a.skn + D) * 2);
     const uint32_t ktile = (uint32_t)(AT_BK * a.skn * 2);
-    uint32_t kvo[4], vvo[4];
+    uint32_t kvo[LOADS], vvo[LOADS];
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-        const int i = wave * 4 + j;
-        const int krow = 4 * i + (lane >> 4);
-        kvo[j] = (uint32_t)krow * (uint32_t)(a.skn * 2) + (uint32_t)(((lane & 15) ^ (krow & 15)) * 16);
+    for (int j = 0; j < LOADS; j++) {
+        const int i = wave * LOADS + j;
+        const int krow = (64 / G::KCH) * i + lane / G::KCH;
+        kvo[j] = (uint32_t)krow * (uint32_t)(a.skn * 2) + (uint32_t)(((lane % G::KCH) ^ G::kswz(krow)) * 16);
         const int vrow = 8 * i + (lane >> 3);
         vvo[j] = (uint32_t)vrow * (uint32_t)Tpad * 2 + (uint32_t)(((lane & 7) ^ ((vrow >> 1) & 7)) * 16);
     }
-    const __amdgpu_buffer_rsrc_t vres = __builtin_amdgcn_make_buffer_rsrc((void *)vbase, 0, AT_D * Tpad * 2, AT_RSRC_FLAGS);
+    const __amdgpu_buffer_rsrc_t vres = at_buffer(vbase, (uint32_t)(D * Tpad * 2));
     auto issue_k = [&](int blk, int stage, int j) {
         const uint32_t off = (uint32_t)blk * ktile;
-        const __amdgpu_buffer_rsrc_t kres = __builtin_amdgcn_make_buffer_rsrc((void *)(kbase + off), 0, kbytes - off, AT_RSRC_FLAGS);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(kres, (SVDQ_AS3 void *)(smem + stage * AT_STAGE + (wave * 4 + j) * 1024), 16,
-                                                 kvo[j], 0, 0, 0);
+        at_load16_lds(at_buffer(kbase + off, kbytes - off), smem + stage * G::STAGE + (wave * G::LOADS + j) * 1024, kvo[j], 0);
     };
     auto issue_v = [&](int blk, int stage, int j) {
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(vres, (SVDQ_AS3 void *)(smem + stage * AT_STAGE + AT_KT_BYTES + (wave * 4 + j) * 1024),
-                                                 16, vvo[j], blk * (AT_BK * 2), 0, 0);
+        at_load16_lds(vres, smem + stage * G::STAGE + G::KT_BYTES + (wave * G::LOADS + j) * 1024, vvo[j],
+                      (uint32_t)blk * (AT_BK * 2));
     };
 
     // operand read offsets: K rows 32 t + l32 (chunk 2 c + half), V^T rows 32 dt + l32 (chunk 2 c + half)
-    int koff[8], vtoff[4];
+    int koff[NC], vtoff[4];
 #pragma unroll
-    for (int c = 0; c < 8; c++) koff[c] = l32 * 256 + (((2 * c + half) ^ (l32 & 15)) * 16);
+    for (int c = 0; c < NC; c++) koff[c] = l32 * G::KROW + (((2 * c + half) ^ G::kswz(l32)) * 16);
 #pragma unroll
-    for (int c = 0; c < 4; c++) vtoff[c] = AT_KT_BYTES + l32 * 128 + (((2 * c + half) ^ ((l32 >> 1) & 7)) * 16);
+    for (int c = 0; c < 4; c++) vtoff[c] = G::KT_BYTES + l32 * 128 + (((2 * c + half) ^ ((l32 >> 1) & 7)) * 16);
 
-    v16f acc_o[4];
+    v16f acc_o[NDT];
 #pragma unroll
-    for (int dt = 0; dt < 4; dt++)
+    for (int dt = 0; dt < NDT; dt++)
 #pragma unroll
         for (int i = 0; i < 16; i++) acc_o[dt][i] = 0.0f;
     // Scores come out of the matrix instructions already relative to the row's reference: the accumulator of S^T starts
@@ -171,23 +194,23 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a
     //                                                     the stage tile t has left
     // The compiler is kept from regrouping the slots (one matrix instruction plus its share of the rest).
 #pragma unroll
-    for (int j = 0; j < 4; j++) issue_k(0, 0, j);
+    for (int j = 0; j < LOADS; j++) issue_k(0, 0, j);
 #pragma unroll
-    for (int j = 0; j < 4; j++) issue_v(0, 0, j);
+    for (int j = 0; j < LOADS; j++) issue_v(0, 0, j);
     {
         const int t1 = min(1, nblk - 1);
 #pragma unroll
-        for (int j = 0; j < 4; j++) issue_k(t1, 1, j);
+        for (int j = 0; j < LOADS; j++) issue_k(t1, 1, j);
 #pragma unroll
-        for (int j = 0; j < 4; j++) issue_v(t1, 1, j);
+        for (int j = 0; j < LOADS; j++) issue_v(t1, 1, j);
     }
-    __builtin_amdgcn_s_waitcnt(waitcnt_imm(8, 15));  // tile 0 (the older eight loads)
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(2 * LOADS, 15));  // tile 0 (the older half of the loads)
     __builtin_amdgcn_s_barrier();
-    v4i rk[16], rv[16];  // rk[8 t + c]: K rows 32 t.., chunk c;  rv[4 dt + c]: V^T rows 32 dt.., 16-key chunk c
+    v4i rk[2 * NC], rv[4 * NDT];  // rk[NC t + c]: K rows 32 t.., chunk c;  rv[4 dt + c]: V^T rows 32 dt.., 16-key chunk c
 #pragma unroll
-    for (int c = 0; c < 8; c++) {
+    for (int c = 0; c < NC; c++) {
         rk[c] = *(const v4i *)(smem + koff[c]);
-        rk[8 + c] = *(const v4i *)(smem + 32 * 256 + koff[c]);
+        rk[NC + c] = *(const v4i *)(smem + 32 * G::KROW + koff[c]);
     }
 
     float shift, alpha, rs;  // rs: this half's row sum, at the new reference
@@ -230,15 +253,15 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a
     auto rescale = [&]() {
         l_run *= alpha;
 #pragma unroll
-        for (int dt = 0; dt < 4; dt++)
+        for (int dt = 0; dt < G::NDT; dt++)
 #pragma unroll
             for (int i = 0; i < 16; i++) acc_o[dt][i] *= alpha;
         shift16(cinit);
     };
 
     for (int blk = 0; blk < nblk; blk++) {
-        const uint8_t *st = smem + (blk & 1) * AT_STAGE;
-        const uint8_t *sn = smem + ((blk + 1) & 1) * AT_STAGE;
+        const uint8_t *st = smem + (blk & 1) * G::STAGE;
+        const uint8_t *sn = smem + ((blk + 1) & 1) * G::STAGE;
         const int nxt = min(blk + 2, nblk - 1);  // past the end: the last tile again, into a stage nobody reads
         const bool ragged = blk == nblk - 1 && (a.Tkv & (AT_BK - 1));
         v16f s0, s1;
@@ -246,9 +269,9 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a
 
         // ---- (A) ---------------------------------------------------------------------------------------------------------
 #pragma unroll
-        for (int c = 0; c < 8; c++) {
+        for (int c = 0; c < NC; c++) {
             s0 = mfma32_16bit<T>(rk[c], qop[c], c == 0 ? cinit : s0);
-            rv[4 * (c & 3) + (c >> 2)] = *(const v4i *)(st + (c & 3) * (32 * 128) + vtoff[c >> 2]);  // chunks 0, 1: keys 0..31
+            rv[4 * (c % NDT) + c / NDT] = *(const v4i *)(st + (c % NDT) * (32 * 128) + vtoff[c / NDT]);  // chunks 0, 1: keys 0..31
             __builtin_amdgcn_sched_barrier(0);
         }
         if (ragged) {  // keys past the end count as -inf
@@ -260,15 +283,17 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a
         // ---- (B) ---------------------------------------------------------------------------------------------------------
         bool moved = false;
 #pragma unroll
-        for (int c = 0; c < 8; c++) {
-            s1 = mfma32_16bit<T>(rk[8 + c], qop[c], c == 0 ? cinit : s1);
-            rv[4 * (c & 3) + 2 + (c >> 2)] = *(const v4i *)(st + (c & 3) * (32 * 128) + vtoff[2 + (c >> 2)]);  // keys 32..63
+        for (int c = 0; c < NC; c++) {
+            s1 = mfma32_16bit<T>(rk[NC + c], qop[c], c == 0 ? cinit : s1);
+            rv[4 * (c % NDT) + 2 + c / NDT] = *(const v4i *)(st + (c % NDT) * (32 * 128) + vtoff[2 + c / NDT]);  // keys 32..63
             if (c == 0) {
                 moved = row_max(s0);
                 rs = 0.0f;
                 if (moved) shift16(s0);
             }
-            if (c >= 1 && c <= 4) exp4(s0, 4 * (c - 1), pop[(c - 1) >> 1], 2 * ((c - 1) & 1));
+#pragma unroll
+            for (int j = 0; j < 4; j++)  // the four exp slices go with slots 1 .. 4 (the last slot takes what is left)
+                if (c == (1 + j < NC - 1 ? 1 + j : NC - 1)) exp4(s0, 4 * j, pop[j >> 1], 2 * (j & 1));
             __builtin_amdgcn_sched_barrier(0);
         }
         if (moved) {
@@ -285,14 +310,16 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a
 
         // ---- (C) ---------------------------------------------------------------------------------------------------------
 #pragma unroll
-        for (int c = 0; c < 8; c++) {
-            acc_o[c & 3] = mfma32_16bit<T>(rv[4 * (c & 3) + (c >> 2)], pop[c >> 2], acc_o[c & 3]);
+        for (int c = 0; c < NC; c++) {
+            acc_o[c % NDT] = mfma32_16bit<T>(rv[4 * (c % NDT) + c / NDT], pop[c / NDT], acc_o[c % NDT]);
             if (c == 0) {
                 moved = row_max(s1);
                 rs = 0.0f;
                 if (moved) shift16(s1);
             }
-            if (c >= 1 && c <= 4) exp4(s1, 4 * (c - 1), pop[2 + ((c - 1) >> 1)], 2 * ((c - 1) & 1));
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                if (c == (1 + j < NC - 1 ? 1 + j : NC - 1)) exp4(s1, 4 * j, pop[2 + (j >> 1)], 2 * (j & 1));
             __builtin_amdgcn_sched_barrier(0);
         }
         if (moved) rescale();
@@ -304,10 +331,10 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a
 
         // ---- (D) ---------------------------------------------------------------------------------------------------------
 #pragma unroll
-        for (int c = 0; c < 8; c++) {
-            acc_o[c & 3] = mfma32_16bit<T>(rv[4 * (c & 3) + 2 + (c >> 2)], pop[2 + (c >> 2)], acc_o[c & 3]);
-            rk[2 * c] = *(const v4i *)(sn + (c >> 2) * (32 * 256) + koff[(2 * c) & 7]);
-            rk[2 * c + 1] = *(const v4i *)(sn + (c >> 2) * (32 * 256) + koff[(2 * c + 1) & 7]);
+        for (int c = 0; c < NC; c++) {
+            acc_o[c % NDT] = mfma32_16bit<T>(rv[4 * (c % NDT) + 2 + c / NDT], pop[2 + c / NDT], acc_o[c % NDT]);
+            rk[2 * c] = *(const v4i *)(sn + ((2 * c) / NC) * (32 * G::KROW) + koff[(2 * c) % NC]);
+            rk[2 * c + 1] = *(const v4i *)(sn + ((2 * c + 1) / NC) * (32 * G::KROW) + koff[(2 * c + 1) % NC]);
             if (c & 1) issue_k(nxt, blk & 1, c >> 1); else issue_v(nxt, blk & 1, c >> 1);
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -319,22 +346,32 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));  // the redundant last tile load has landed
     __syncthreads();
 #pragma unroll
-    for (int dt = 0; dt < 4; dt++)
+    for (int dt = 0; dt < NDT; dt++)
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             uint2 w;
             w.x = pack2<T>(acc_o[dt][4 * j] * inv, acc_o[dt][4 * j + 1] * inv);
             w.y = pack2<T>(acc_o[dt][4 * j + 2] * inv, acc_o[dt][4 * j + 3] * inv);
-            *(uint2 *)(smem + (wave * 32 + l32) * AT_OPITCH + (32 * dt + 8 * j + 4 * half) * 2) = w;
+            *(uint2 *)(smem + (wave * 32 + l32) * G::OPITCH + (32 * dt + 8 * j + 4 * half) * 2) = w;
         }
     __syncthreads();
-    uint16_t *op = (uint16_t *)a.o + (long)b * a.sob + (long)h * AT_D;
-    const int c = tid & 15;
+    uint16_t *op = (uint16_t *)a.o + (long)b * a.sob + (long)h * D;
+    constexpr int OCH = D / 8, OROWS = 256 / OCH;  // 16-byte chunks per output row, rows per pass
+    const int c = tid % OCH;
 #pragma unroll
-    for (int pass = 0; pass < AT_BQ * 16 / 256; pass++) {
-        const int row = pass * 16 + (tid >> 4), q = q0 + row;
-        if (q < a.Tq) *(v4i *)(op + (long)q * a.som + 8 * c) = *(const v4i *)(smem + row * AT_OPITCH + c * 16);
+    for (int pass = 0; pass < AT_BQ / OROWS; pass++) {
+        const int row = pass * OROWS + tid / OCH, q = q0 + row;
+        if (q < a.Tq) *(v4i *)(op + (long)q * a.som + 8 * c) = *(const v4i *)(smem + row * G::OPITCH + c * 16);
     }
+}
+
+template <typename T, int D>
+static void launch_attention(const svdq_attention_args &a, int Tpad, hipStream_t s) {
+    hipLaunchKernelGGL(transpose_v_kernel<D>, dim3(Tpad / AT_BK, a.H, a.B), dim3(256), 0, s, (const uint16_t *)a.v,
+                       (uint16_t *)a.vt, a.H, a.Tkv, Tpad, (long)a.svb, (long)a.svh, (long)a.svn);
+    const int ntile = (a.Tq + AT_BQ - 1) / AT_BQ;
+    const int xcd_heads = (a.B * a.H) % 8 == 0;
+    hipLaunchKernelGGL((attention_kernel<T, D>), dim3((unsigned)(ntile * a.H * a.B)), dim3(256), 0, s, a, Tpad, ntile, xcd_heads);
 }
 
 }  // namespace svdq
@@ -342,9 +379,9 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a
 using namespace svdq;
 
 extern "C" size_t svdq_attention_workspace_bytes(int32_t B, int32_t H, int32_t Tkv, int32_t D) {
-    if (B <= 0 || H <= 0 || Tkv <= 0 || D != AT_D) return 0;
+    if (B <= 0 || H <= 0 || Tkv <= 0 || (D != 128 && D != 64)) return 0;
     const size_t Tpad = (size_t)((Tkv + AT_BK - 1) / AT_BK) * AT_BK;
-    return (size_t)B * H * AT_D * Tpad * 2;
+    return (size_t)B * H * D * Tpad * 2;
 }
 
 extern "C" int svdq_attention_fp16(const svdq_attention_args *args, void *stream) {
@@ -357,8 +394,8 @@ extern "C" int svdq_attention_fp16(const svdq_attention_args *args, void *stream
         set_error("svdq_attention_fp16: dtype %d", a.dtype);
         return SVDQ_E_INVALID;
     }
-    if (a.D != AT_D) {
-        set_error("svdq_attention_fp16: head dimension %d is not supported (128 only)", a.D);
+    if (a.D != 128 && a.D != 64) {
+        set_error("svdq_attention_fp16: head dimension %d is not supported (128 and 64 only)", a.D);
         return SVDQ_E_UNSUPPORTED;
     }
     if (a.B <= 0 || a.H <= 0 || a.Tq < 0 || a.Tkv <= 0 || a.B > 65535 || a.H > 65535) {
@@ -377,24 +414,26 @@ extern "C" int svdq_attention_fp16(const svdq_attention_args *args, void *stream
     }
     if (a.Tq == 0) return SVDQ_OK;
     const int Tpad = (a.Tkv + AT_BK - 1) / AT_BK * AT_BK;
-    if ((size_t)AT_D * Tpad * 2 >= ((size_t)1 << 31) || ((size_t)Tpad * a.skn + AT_D) * 2 >= ((size_t)1 << 31) ||
+    if ((size_t)a.D * Tpad * 2 >= ((size_t)1 << 31) || ((size_t)Tpad * a.skn + a.D) * 2 >= ((size_t)1 << 31) ||
         (size_t)a.B * a.H * ((a.Tq + AT_BQ - 1) / AT_BQ) >= ((size_t)1 << 31)) {
         set_error("svdq_attention_fp16: Tq=%d Tkv=%d key stride %lld: too large for 32-bit tile offsets", a.Tq, a.Tkv, (long long)a.skn);
         return SVDQ_E_UNSUPPORTED;
     }
-    if (a.skn < AT_D) {
-        set_error("svdq_attention_fp16: key rows overlap (stride %lld < 128)", (long long)a.skn);
+    if (a.skn < a.D) {
+        set_error("svdq_attention_fp16: key rows overlap (stride %lld < head dimension)", (long long)a.skn);
         return SVDQ_E_INVALID;
     }
     hipStream_t s = (hipStream_t)stream;
-    hipLaunchKernelGGL(transpose_v_kernel, dim3(Tpad / AT_BK, a.H, a.B), dim3(256), 0, s, (const uint16_t *)a.v,
-                       (uint16_t *)a.vt, a.H, a.Tkv, Tpad, (long)a.svb, (long)a.svh, (long)a.svn);
-    const int ntile = (a.Tq + AT_BQ - 1) / AT_BQ;
-    const int xcd_heads = (a.B * a.H) % 8 == 0;
-    const dim3 grid((unsigned)(ntile * a.H * a.B));
-    if (a.dtype == SVDQ_BF16)
-        hipLaunchKernelGGL((attention_kernel<BF16>), grid, dim3(256), 0, s, a, Tpad, ntile, xcd_heads);
-    else
-        hipLaunchKernelGGL((attention_kernel<FP16>), grid, dim3(256), 0, s, a, Tpad, ntile, xcd_heads);
+    if (a.D == 128) {
+        if (a.dtype == SVDQ_BF16)
+            launch_attention<BF16, 128>(a, Tpad, s);
+        else
+            launch_attention<FP16, 128>(a, Tpad, s);
+    } else {
+        if (a.dtype == SVDQ_BF16)
+            launch_attention<BF16, 64>(a, Tpad, s);
+        else
+            launch_attention<FP16, 64>(a, Tpad, s);
+    }
     return check_launch("svdq_attention_fp16");
 }

@@ -7,15 +7,15 @@ import torch.nn.functional as F
 
 from .. import _lib
 
-_HEAD_DIM = 128  # the head dimension the kernel is written for (FLUX, Qwen-Image)
+_HEAD_DIMS = (128, 64)  # the head dimensions the kernel is built for (FLUX / Qwen-Image, SDXL-class models)
 
 
 def attention_fp16(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: torch.Tensor, scale: float) -> None:
     """
     Fused scaled-dot-product attention without a mask, written into ``o``.
 
-    q : (B, H, TokensQ, 128);  k, v : (B, H, TokensKV, 128);  o : (B, TokensQ, H * 128);  fp16 or bf16, last
-    dimension contiguous.  ``scale`` is the softmax scale, normally ``128 ** -0.5``.
+    q : (B, H, TokensQ, D);  k, v : (B, H, TokensKV, D);  o : (B, TokensQ, H * D);  D = 128 or 64;  fp16 or bf16, last
+    dimension contiguous.  ``scale`` is the softmax scale, normally ``D ** -0.5``.
     """
     B, H, Tq, D = q.shape
     Tkv = k.shape[2]
@@ -29,7 +29,7 @@ def attention_fp16(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: torch.T
     lib = _lib.load()
     ws = lib.svdq_attention_workspace_bytes(B, H, Tkv, D)
     if ws == 0:
-        raise NotImplementedError(f"attention_fp16: head dimension {D} is not supported (128 only)")
+        raise NotImplementedError(f"attention_fp16: head dimension {D} is not supported (128 and 64 only)")
     vt = torch.empty(ws, dtype=torch.uint8, device=q.device)
     args = _lib.AttentionArgs(
         q=q.data_ptr(), k=k.data_ptr(), v=v.data_ptr(), o=o.data_ptr(), vt=vt.data_ptr(),
@@ -48,7 +48,7 @@ def _covered(query: torch.Tensor, key: torch.Tensor, value: torch.Tensor) -> boo
         query.is_cuda
         and query.dtype in (torch.float16, torch.bfloat16)
         and key.dtype == value.dtype == query.dtype
-        and query.shape[-1] == _HEAD_DIM
+        and query.shape[-1] in _HEAD_DIMS
         and key.shape[2] > 0
         and all(t.stride(-1) == 1 and t.data_ptr() % 16 == 0 and all(s % 8 == 0 for s in t.stride()[:-1]) for t in (query, key, value))
     )  # fmt: skip
@@ -59,7 +59,7 @@ def scaled_dot_product_attention(
 ) -> torch.Tensor:
     """
     Drop-in for ``F.scaled_dot_product_attention`` on ``(B, H, T, D)`` inputs (no dropout, not causal).  Unmasked
-    fp16 / bf16 attention with head dimension 128 runs on the HIP kernel; what the kernel does not cover (a mask,
+    fp16 / bf16 attention with head dimension 128 or 64 runs on the HIP kernel; what the kernel does not cover (a mask,
     fp32, another head dimension, a strided head dimension) goes to torch, as in the reference.
     """
     if attn_mask is not None or not _covered(query, key, value):

@@ -74,12 +74,13 @@ def test_invalid_arguments_are_rejected_without_launch(lib):
     a = _lib.AwqGemvArgs(x=16, qweight=16, scales=16, zeros=16, out=16, M=64, N=64, K=64, ld_x=64, ld_scales=64, ld_out=64)
     assert lib.svdq_awq_gemv_w4a16(a, None) == _lib.E_INVALID  # M > 32
     assert lib.svdq_gemm_w4a4(None, None) == _lib.E_INVALID
-    at = _lib.AttentionArgs(q=16, k=16, v=16, o=16, vt=16, B=1, H=1, Tq=8, Tkv=8, D=64)
+    at = _lib.AttentionArgs(q=16, k=16, v=16, o=16, vt=16, B=1, H=1, Tq=8, Tkv=8, D=32)
     assert lib.svdq_attention_fp16(at, None) == _lib.E_UNSUPPORTED  # head dimension
     at = _lib.AttentionArgs(q=16, k=16, v=16, o=16, vt=0, B=1, H=1, Tq=8, Tkv=8, D=128)
     assert lib.svdq_attention_fp16(at, None) == _lib.E_INVALID  # no workspace
     assert lib.svdq_attention_workspace_bytes(2, 3, 65, 128) == 2 * 3 * 128 * 128 * 2
-    assert lib.svdq_attention_workspace_bytes(1, 1, 64, 64) == 0
+    assert lib.svdq_attention_workspace_bytes(1, 1, 64, 64) == 64 * 64 * 2
+    assert lib.svdq_attention_workspace_bytes(1, 1, 64, 32) == 0
     assert lib.svdq_gemm_w4a4_scratch_bytes(256, 256, 32, _lib.EPI_GELU_QUANT) == 2 * 256 * 32 * 4
     assert lib.svdq_gemm_w4a4_scratch_bytes(256, 256, 32, _lib.EPI_PLAIN) == 0
 

@@ -12,11 +12,11 @@ pytestmark = pytest.mark.gpu
 TOL = 1e-2
 
 
-def _inputs(B, H, Tq, Tkv, dtype, seed, spread=1.0):
+def _inputs(B, H, Tq, Tkv, dtype, seed, spread=1.0, D=128):
     g = torch.Generator().manual_seed(seed)
-    q = (torch.randn(B, H, Tq, 128, generator=g) * spread).to(dtype)
-    k = (torch.randn(B, H, Tkv, 128, generator=g) * spread).to(dtype)
-    v = torch.randn(B, H, Tkv, 128, generator=g).to(dtype)
+    q = (torch.randn(B, H, Tq, D, generator=g) * spread).to(dtype)
+    k = (torch.randn(B, H, Tkv, D, generator=g) * spread).to(dtype)
+    v = torch.randn(B, H, Tkv, D, generator=g).to(dtype)
     return q, k, v
 
 
@@ -46,6 +46,24 @@ def test_against_oracle(dev, dtype, B, H, Tq, Tkv):
     assert O.max_rel_err(out, ref) <= TOL
     exact = torch.softmax(q.float() @ k.float().transpose(-1, -2) * scale, dim=-1) @ v.float()
     torch.testing.assert_close(out.float(), exact.transpose(1, 2).reshape(B, Tq, -1), rtol=3e-2, atol=3e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("B,H,Tq,Tkv", [(2, 8, 256, 256), (2, 2, 100, 77), (1, 3, 129, 65), (1, 1, 1, 1), (1, 16, 333, 1000)])
+def test_head_dimension_64(dev, dtype, B, H, Tq, Tkv):
+    """The reference's own test shapes with 64-dimensional heads (tests/triton/test_w4a4.py:242) and ragged ones."""
+    print(f"case D=64 {B}x{H}x{Tq}x{Tkv} {dtype}", flush=True)
+    q, k, v = _inputs(B, H, Tq, Tkv, dtype, seed=Tq + 3 * Tkv, D=64)
+    scale = 64**-0.5
+    out = _run(dev, q, k, v, scale)
+    ref = O.attention_fp16(q, k, v, scale)
+    assert out.shape == (B, Tq, H * 64) and torch.isfinite(out.float()).all()
+    assert O.max_rel_err(out, ref) <= TOL
+    exact = torch.softmax(q.float() @ k.float().transpose(-1, -2) * scale, dim=-1) @ v.float()
+    torch.testing.assert_close(out.float(), exact.transpose(1, 2).reshape(B, Tq, -1), rtol=3e-2, atol=3e-2)
+    # a sharp softmax moves the reference every tile
+    q2 = (q.float() * 6).to(dtype)
+    assert O.max_rel_err(_run(dev, q2, k, v, scale), O.attention_fp16(q2, k, v, scale)) <= TOL
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
@@ -99,13 +117,17 @@ def test_sdpa_wrapper(dev, dtype, layout):
     out = ops.scaled_dot_product_attention(q, k, v, attn_mask=mask)
     ref = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float(), v.float(), attn_mask=mask)
     torch.testing.assert_close(out.float(), ref, rtol=3e-2, atol=3e-2)
-    # head dimension 64 is outside the kernel: the wrapper goes to torch, the bare operator says so
-    q64, k64, v64 = (t[..., :64].contiguous() for t in (q, k, v))
-    out = ops.scaled_dot_product_attention(q64, k64, v64)
-    ref = torch.nn.functional.scaled_dot_product_attention(q64.float(), k64.float(), v64.float())
+    # head dimension 64 runs on the kernel too (here on strided slices of the 128-wide tensors)
+    out = ops.scaled_dot_product_attention(q[..., :64], k[..., :64], v[..., :64])
+    ref = torch.nn.functional.scaled_dot_product_attention(q[..., :64].float(), k[..., :64].float(), v[..., :64].float())
+    torch.testing.assert_close(out.float(), ref, rtol=3e-2, atol=3e-2)
+    # head dimension 32 is outside the kernel: the wrapper goes to torch, the bare operator says so
+    q32, k32, v32 = (t[..., :32].contiguous() for t in (q, k, v))
+    out = ops.scaled_dot_product_attention(q32, k32, v32)
+    ref = torch.nn.functional.scaled_dot_product_attention(q32.float(), k32.float(), v32.float())
     torch.testing.assert_close(out.float(), ref, rtol=3e-2, atol=3e-2)
     with pytest.raises(NotImplementedError):
-        ops.attention_fp16(q64, k64, v64, torch.empty(B, T, H * 64, dtype=dtype, device=dev), 0.125)
+        ops.attention_fp16(q32, k32, v32, torch.empty(B, T, H * 32, dtype=dtype, device=dev), 0.125)
 
 
 def test_flux_shape_sampled_queries(dev):
