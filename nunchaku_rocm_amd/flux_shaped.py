@@ -54,9 +54,11 @@ class HipBackend:
     def gelu_mlp(x, fc1, fc2, mod=None):
         return _ops.fused_gelu_mlp(x, fc1, fc2, norm=mod)
 
+    writes_in_place = True  # qkv(out=...) stores straight into a caller's (tokens, 3 C) buffer
+
     @staticmethod
-    def qkv(x, proj, norm_q, norm_k, rot, mod=None):
-        return _ops.fused_qkv_norm_rottary(x, proj, norm_q, norm_k, rot, norm=mod)
+    def qkv(x, proj, norm_q, norm_k, rot, mod=None, out=None):
+        return _ops.fused_qkv_norm_rottary(x, proj, norm_q, norm_k, rot, output=out, norm=mod)
 
     @staticmethod
     def gated_residual(x, gate, y, y2=None, want_stats=False):
@@ -150,10 +152,17 @@ class _Attention(nn.Module):
 
     def forward(self, be, x, ctx, rot_img, rot_txt, mod_x=None, mod_ctx=None):
         B = x.shape[0]
-        qkv = be.qkv(x, self.to_qkv, self.norm_q, self.norm_k, rot_img, mod=mod_x)
-        if self.joint:
-            qkv_ctx = be.qkv(ctx, self.add_qkv_proj, self.norm_added_q, self.norm_added_k, rot_txt, mod=mod_ctx)
-            qkv = torch.cat([qkv_ctx, qkv], dim=1)  # token order [txt, img]
+        if self.joint and B == 1 and getattr(be, "writes_in_place", False):
+            # both projections store into one (txt + img tokens, 3 C) buffer: no concatenation pass
+            t_txt, t_img = ctx.shape[1], x.shape[1]
+            qkv = torch.empty(1, t_txt + t_img, 3 * self.heads * self.head_dim, dtype=x.dtype, device=x.device)
+            be.qkv(ctx, self.add_qkv_proj, self.norm_added_q, self.norm_added_k, rot_txt, mod=mod_ctx, out=qkv[0, :t_txt])
+            be.qkv(x, self.to_qkv, self.norm_q, self.norm_k, rot_img, mod=mod_x, out=qkv[0, t_txt:])
+        else:
+            qkv = be.qkv(x, self.to_qkv, self.norm_q, self.norm_k, rot_img, mod=mod_x)
+            if self.joint:
+                qkv_ctx = be.qkv(ctx, self.add_qkv_proj, self.norm_added_q, self.norm_added_k, rot_txt, mod=mod_ctx)
+                qkv = torch.cat([qkv_ctx, qkv], dim=1)  # token order [txt, img]
         q, k, v = (t.view(B, -1, self.heads, self.head_dim).transpose(1, 2) for t in qkv.chunk(3, dim=-1))
         o = be.attention(q, k, v)  # (B, H, T, D), scale D^-0.5, no mask
         o = o.transpose(1, 2).reshape(B, -1, self.heads * self.head_dim).to(q.dtype)
