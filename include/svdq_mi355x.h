@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define SVDQ_ABI_VERSION 1
+#define SVDQ_ABI_VERSION 2
 
 enum { SVDQ_BF16 = 0, SVDQ_FP16 = 1 };
 
