@@ -56,6 +56,30 @@ class HipBackend:
 
     writes_in_place = True  # qkv(out=...) stores straight into a caller's (tokens, 3 C) buffer
 
+    def __init__(self, two_streams: bool = True):
+        # The text stream of a dual-stream block is 512 tokens: its GEMMs cover a fraction of the 256 CUs (96 to 288
+        # tiles for 512 workgroup slots).  Run on a second HIP stream (default priority) they fill the slots the image
+        # stream's launches leave empty instead of queueing behind them.
+        self.two_streams = two_streams
+        self._side = {}
+
+    def __deepcopy__(self, memo):
+        return HipBackend(self.two_streams)  # streams are per process, not part of a model copy
+
+    def side_stream(self, device):
+        if not self.two_streams:
+            return None
+        key = torch.device(device).index
+        if key not in self._side:
+            self._side[key] = torch.cuda.Stream(device)
+        return self._side[key]
+
+    def join(self, device):
+        """Make the current stream wait for everything queued on the side stream."""
+        side = self._side.get(torch.device(device).index)
+        if side is not None:
+            torch.cuda.current_stream(device).wait_stream(side)
+
     @staticmethod
     def qkv(x, proj, norm_q, norm_k, rot, mod=None, out=None):
         return _ops.fused_qkv_norm_rottary(x, proj, norm_q, norm_k, rot, output=out, norm=mod)
@@ -190,10 +214,42 @@ class _DoubleBlock(nn.Module):
         emb = be.awq(F.silu(temb), lin)
         return emb.view(emb.shape[0], -1, 6).permute(2, 0, 1)  # interleaved split: channel c -> (c // 6, c % 6)
 
+    def _forward_two_streams(self, be, side, x, ctx, mods_x, mods_ctx, rot_img, rot_txt):
+        """The text stream's kernels on ``side``, the image stream's and the joint attention on the current stream.
+        Tensors that cross from one stream to the other are registered with the allocator (record_stream)."""
+        sh_a, sc_a, g_a, sh_m, sc_m, g_m = mods_x
+        csh_a, csc_a, cg_a, csh_m, csc_m, cg_m = mods_ctx
+        at, dev = self.attn, x.device
+        main = torch.cuda.current_stream(dev)
+        t_txt = ctx.shape[1]
+        qkv = torch.empty(1, t_txt + x.shape[1], 3 * self.C, dtype=x.dtype, device=dev)
+        for t in (ctx, csh_a, qkv):  # made on this stream (the six text vectors share one storage), used on the side one
+            t.record_stream(side)
+        side.wait_stream(main)
+        with torch.cuda.stream(side):
+            be.qkv(ctx, at.add_qkv_proj, at.norm_added_q, at.norm_added_k, rot_txt, mod=(csc_a, csh_a), out=qkv[0, :t_txt])
+        be.qkv(x, at.to_qkv, at.norm_q, at.norm_k, rot_img, mod=(sc_a, sh_a), out=qkv[0, t_txt:])
+        main.wait_stream(side)
+        q, k, v = (t.view(1, -1, at.heads, at.head_dim).transpose(1, 2) for t in qkv.chunk(3, dim=-1))
+        o = be.attention(q, k, v).transpose(1, 2).reshape(1, -1, self.C)
+        o.record_stream(side)
+        side.wait_stream(main)
+        with torch.cuda.stream(side):
+            ctx, st = be.gated_residual(ctx, cg_a, be.linear(o[:, :t_txt], at.to_add_out), want_stats=True)
+            ctx, _ = be.gated_residual(ctx, cg_m, be.gelu_mlp(ctx, self.ffc_fc1, self.ffc_fc2, mod=(csc_m, csh_m, st)))
+        x, st = be.gated_residual(x, g_a, be.linear(o[:, t_txt:], at.to_out), want_stats=True)
+        x, _ = be.gated_residual(x, g_m, be.gelu_mlp(x, self.ff_fc1, self.ff_fc2, mod=(sc_m, sh_m, st)))
+        ctx.record_stream(main)  # read next on either stream
+        return ctx, x
+
     def forward(self, be, x, ctx, temb, rot_img, rot_txt):
         # layer_norm(x) * scale + shift in front of each quantized linear runs inside its quantizer (mod=)
         sh_a, sc_a, g_a, sh_m, sc_m, g_m = self._mod6(be, self.norm1, temb)
         csh_a, csc_a, cg_a, csh_m, csc_m, cg_m = self._mod6(be, self.norm1_context, temb)
+        side = be.side_stream(x.device) if x.shape[0] == 1 and hasattr(be, "side_stream") else None
+        if side is not None:
+            return self._forward_two_streams(be, side, x, ctx, (sh_a, sc_a, g_a, sh_m, sc_m, g_m),
+                                             (csh_a, csc_a, cg_a, csh_m, csc_m, cg_m), rot_img, rot_txt)
         ax, ac = self.attn(be, x, ctx, rot_img, rot_txt, mod_x=(sc_a, sh_a), mod_ctx=(csc_a, csh_a))
         # x + gate * y in one kernel that also hands the next norm its row statistics
         x, st = be.gated_residual(x, g_a, ax, want_stats=True)

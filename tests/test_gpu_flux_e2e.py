@@ -43,6 +43,23 @@ def test_small_config_against_cpu_oracle(dev):
     assert cos >= 0.999
 
 
+def test_two_streams_give_the_same_bits(dev):
+    """The text stream of the dual-stream blocks on a second HIP stream: every kernel is deterministic, so the result
+    must be bit-equal to the single-stream run, on repeated runs too (a missed dependency would show up here)."""
+    from nunchaku_rocm_amd.flux_shaped import FluxShapedConfig, FluxShapedTransformer, HipBackend
+
+    cfg = FluxShapedConfig(hidden=1024, heads=8, mlp=4096, text_dim=256, pooled_dim=64, n_double=4, n_single=2)
+    model = FluxShapedTransformer(cfg, device=dev, seed=5)
+    lat, txt, pooled, rot = _inputs(cfg, 512, 32, 32, dev)
+    one = model.denoise(lat, txt, pooled, rot, steps=2, backend=HipBackend(two_streams=False))
+    torch.cuda.synchronize()
+    two = HipBackend(two_streams=True)
+    for _ in range(3):
+        out = model.denoise(lat, txt, pooled, rot, steps=2, backend=two)
+        torch.cuda.synchronize()
+        assert torch.equal(out, one)
+
+
 def test_flux1_schnell_shape_four_steps(dev):
     """19 double + 38 single blocks, hidden 3072, 4096 image + 512 text tokens, 4 steps; the reference path is the
     oracle's dense-dequantised fp32 formulation evaluated with plain torch kernels on the same GPU."""
