@@ -274,8 +274,22 @@ class _SingleBlock(nn.Module):
         emb = be.awq(F.silu(temb), self.norm)
         shift, scale, gate = emb.view(emb.shape[0], -1, 3).permute(2, 0, 1)
         mod = (scale, shift, stats if stats is not None else be.norm_stats(x))  # one set for both consumers
-        mlp = be.gelu_mlp(x, self.mlp_fc1, self.mlp_fc2, mod=mod)
-        att = self.attn(be, x, None, rot, None, mod_x=mod)
+        side = be.side_stream(x.device) if hasattr(be, "side_stream") else None
+        if side is None:
+            mlp = be.gelu_mlp(x, self.mlp_fc1, self.mlp_fc2, mod=mod)
+            att = self.attn(be, x, None, rot, None, mod_x=mod)
+        else:
+            # the MLP branch on the second stream: its kernels fill the last, partly empty rounds of workgroups of the
+            # attention branch's kernels and the other way round
+            main = torch.cuda.current_stream(x.device)
+            for t in (x, scale, mod[2]):
+                t.record_stream(side)
+            side.wait_stream(main)
+            with torch.cuda.stream(side):
+                mlp = be.gelu_mlp(x, self.mlp_fc1, self.mlp_fc2, mod=mod)
+            att = self.attn(be, x, None, rot, None, mod_x=mod)
+            main.wait_stream(side)
+            mlp.record_stream(main)
         return be.gated_residual(x, gate, att, mlp, want_stats=True)
 
 
