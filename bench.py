@@ -27,7 +27,7 @@ BF16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 / fp16 MFMA, published
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # HBM bytes of one QKV GEMM launch: FETCH_SIZE + WRITE_SIZE (KiB per dispatch, counter scale 1.000) of the grid-1327104
 # launches in profiles/bench_all_kernels_hbm_traffic.txt; counters cannot be read from inside this process
-GEMM_QKV_HBM_BYTES = (121391.7 + 82944.0) * 1024
+GEMM_QKV_HBM_BYTES = (121379.2 + 82944.0) * 1024
 
 
 def _events(n):
