@@ -14,6 +14,7 @@
  *   svdq_gemm_w4a4           nunchaku/ops/gemm.py:151-207        (_C.ops.gemm_w4a4 / ops/triton/gemm_w4a4.py:1003 gemm_w4a4),
  *                            kernel-argument structs modelled on ops/triton/native/w4a4.py:80-124
  *   svdq_awq_gemv_w4a16      nunchaku/ops/dispatch.py:19-34      (_C.ops.gemv_awq / ops/triton/awq.py:186 awq_gemv_w4a16)
+ *   svdq_awq_dequantize      nunchaku/ops/dispatch.py:37-49      (_C.ops.gemm_awq / ops/triton/awq.py:83 awq_dequantize + torch.matmul)
  *   svdq_attention_fp16      nunchaku/ops/dispatch.py:67-99      (_C.ops.attention_fp16 / ops/triton/attention.py:111 attention_fp16)
  *   svdq_row_stats           nunchaku/models/normalization.py:97 (the LayerNorm statistics; applied inside svdq_quantize_act)
  *   svdq_gated_residual      nunchaku/models/transformers/transformer_flux_v2.py:233-243, :326-330 (gate * y + residual)
@@ -31,7 +32,7 @@
 extern "C" {
 #endif
 
-#define SVDQ_ABI_VERSION 2
+#define SVDQ_ABI_VERSION 3
 
 enum { SVDQ_BF16 = 0, SVDQ_FP16 = 1 };
 
@@ -179,6 +180,16 @@ typedef struct {
 } svdq_awq_gemv_args;
 
 int svdq_awq_gemv_w4a16(const svdq_awq_gemv_args *args, void *stream);
+
+/*
+ * Dense decode of a TinyChat-packed AWQ weight (nunchaku/ops/triton/awq.py:48-118 awq_dequantize, the first half of
+ * awq_gemm_w4a16 :232-251 and of the group_size != 64 branch of awq_gemv_w4a16 :226-228; the matmul that follows is
+ * the caller's): out[n, k] = T(q[n, k] * s[k / group_size, n] + z[k / group_size, n]) in fp32.
+ * qweight (N/4, K) int16 as above; scales / zeros (K / group_size, N) T with group stride ld_scales; out (N, K) T with
+ * row stride ld_out.  N % 4 == 0, K % 64 == 0, group_size a multiple of 32 that divides K.
+ */
+int svdq_awq_dequantize(const void *qweight, const void *scales, const void *zeros, void *out, int32_t N, int32_t K,
+                        int32_t group_size, int32_t ld_scales, int32_t ld_out, int32_t dtype, void *stream);
 
 /*
  * Unmasked scaled-dot-product attention, head dimension D = 128 or 64 (nunchaku/ops/dispatch.py:67-99 attention_fp16 /

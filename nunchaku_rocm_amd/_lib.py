@@ -14,7 +14,7 @@ import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libsvdq_mi355x.so")
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 BF16, FP16 = 0, 1
 EPI_PLAIN, EPI_QK_NORM_ROPE, EPI_GELU_QUANT, EPI_SWIGLU_QUANT = 0, 1, 2, 3
@@ -31,6 +31,7 @@ EXPORTS = (
     "svdq_weight_planes_bytes",
     "svdq_group_acc_i32",
     "svdq_awq_gemv_w4a16",
+    "svdq_awq_dequantize",
     "svdq_attention_fp16",
     "svdq_attention_workspace_bytes",
     "svdq_unpack_mma_weight",
@@ -122,6 +123,7 @@ def load() -> ctypes.CDLL:
     lib.svdq_quantize_act.argtypes = [ctypes.POINTER(QuantizeArgs), _vp]
     lib.svdq_gemm_w4a4.argtypes = [ctypes.POINTER(GemmArgs), _vp]
     lib.svdq_awq_gemv_w4a16.argtypes = [ctypes.POINTER(AwqGemvArgs), _vp]
+    lib.svdq_awq_dequantize.argtypes = [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _vp]
     lib.svdq_attention_fp16.argtypes = [ctypes.POINTER(AttentionArgs), _vp]
     lib.svdq_attention_workspace_bytes.restype = ctypes.c_size_t
     lib.svdq_attention_workspace_bytes.argtypes = [_i32, _i32, _i32, _i32]

@@ -222,6 +222,38 @@ __global__ __launch_bounds__(AWQ_WAVES * 64, AWQ_WAVES >= 16 ? 4 : (AWQ_WAVES >=
     }
 }
 
+// Dense decode of a TinyChat-packed weight: out[n, k] = T(q[n, k] * s[k / group, n] + z[k / group, n]), fp32 arithmetic
+// (reference: nunchaku/ops/triton/awq.py:48-79; q * s is exact in fp32, so there is one rounding before the one to T).
+// Thread idx walks the packed tensor in storage order, 16 bytes each: piece (a = n / 4, c = k / 64, b = n % 4,
+// h = (k / 32) % 2) holds eight int16 whose nibble j' is k = 64 c + 32 h + 8 j' + j (j = position of the int16), i.e.
+// the 32 consecutive outputs out[n, 64 c + 32 h ... + 32): reads are contiguous, stores are 64-byte row pieces.
+template <typename T>
+__global__ __launch_bounds__(256) void awq_dequant_kernel(const v4i *__restrict__ qweight, const uint16_t *__restrict__ scales,
+                                                          const uint16_t *__restrict__ zeros, uint16_t *__restrict__ out,
+                                                          int N, int K, int group, int ld_scales, int ld_out) {
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int g64 = K / GROUP;
+    if (idx >= (size_t)(N / 4) * g64 * 8) return;
+    const int h = idx & 1, b = (idx >> 1) & 3;
+    const int c = (int)((idx >> 3) % g64), a = (int)((idx >> 3) / g64);
+    const int n = 4 * a + b, k0 = GROUP * c + 32 * h;
+    const v4i w = awq_wload(qweight + idx);
+    const float s = T::to_f32(scales[(size_t)(k0 / group) * ld_scales + n]);
+    const float z = T::to_f32(zeros[(size_t)(k0 / group) * ld_scales + n]);
+    uint16_t *o = out + (size_t)n * ld_out + k0;
+#pragma unroll
+    for (int jp = 0; jp < 4; jp++) {  // nibble jp of the eight int16 = eight consecutive k
+        v4i r;
+#pragma unroll
+        for (int d = 0; d < 4; d++) {
+            const uint32_t word = (uint32_t)w[d];  // int16 2 d (low half) and 2 d + 1
+            const float lo = (float)((word >> (4 * jp)) & 15u), hi = (float)((word >> (16 + 4 * jp)) & 15u);
+            r[d] = (int)pack2<T>(__builtin_fmaf(lo, s, z), __builtin_fmaf(hi, s, z));
+        }
+        *(v4i *)(o + 8 * jp) = r;
+    }
+}
+
 static size_t awq_lds_bytes(int K, int M) {
     const int MQ = (M + 7) / 8;
     size_t b = ((size_t)(K / GROUP) * 8 * MQ + (size_t)AWQ_WAVES * 8 * MQ * AWQ_NB) * sizeof(float);
@@ -280,4 +312,32 @@ extern "C" int svdq_awq_gemv_w4a16(const svdq_awq_gemv_args *args, void *stream)
     else
         launch_awq<FP16>(a, (hipStream_t)stream);
     return check_launch("svdq_awq_gemv_w4a16");
+}
+
+extern "C" int svdq_awq_dequantize(const void *qweight, const void *scales, const void *zeros, void *out, int32_t N,
+                                   int32_t K, int32_t group_size, int32_t ld_scales, int32_t ld_out, int32_t dtype,
+                                   void *stream) {
+    if (dtype != SVDQ_BF16 && dtype != SVDQ_FP16) {
+        set_error("svdq_awq_dequantize: dtype %d", dtype);
+        return SVDQ_E_INVALID;
+    }
+    if (N <= 0 || N % 4 || K <= 0 || K % GROUP || group_size <= 0 || group_size % 32 || K % group_size) {
+        set_error("svdq_awq_dequantize: N=%d K=%d group_size=%d needs N %% 4 == 0, K %% 64 == 0, group_size %% 32 == 0 dividing K",
+                  N, K, group_size);
+        return SVDQ_E_INVALID;
+    }
+    if (!qweight || !scales || !zeros || !out || ((uintptr_t)qweight & 15) || ((uintptr_t)out & 15) || ld_out % 8 ||
+        ld_out < K || ld_scales < N) {
+        set_error("svdq_awq_dequantize: qweight and out rows must be 16-byte aligned; ld_out >= K, ld_scales >= N");
+        return SVDQ_E_INVALID;
+    }
+    const size_t pieces = (size_t)(N / 4) * (K / GROUP) * 8;
+    const dim3 grid((unsigned)((pieces + 255) / 256)), block(256);
+    if (dtype == SVDQ_BF16)
+        hipLaunchKernelGGL(awq_dequant_kernel<BF16>, grid, block, 0, (hipStream_t)stream, (const v4i *)qweight,
+                           (const uint16_t *)scales, (const uint16_t *)zeros, (uint16_t *)out, N, K, group_size, ld_scales, ld_out);
+    else
+        hipLaunchKernelGGL(awq_dequant_kernel<FP16>, grid, block, 0, (hipStream_t)stream, (const v4i *)qweight,
+                           (const uint16_t *)scales, (const uint16_t *)zeros, (uint16_t *)out, N, K, group_size, ld_scales, ld_out);
+    return check_launch("svdq_awq_dequantize");
 }

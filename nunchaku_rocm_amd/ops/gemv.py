@@ -1,4 +1,5 @@
-"""AWQ W4A16 GEMV operator (reference: nunchaku/ops/gemv.py:10-56, nunchaku/ops/triton/awq.py:186-229)."""
+"""AWQ W4A16 operators: the group-64 GEMV, the dense decode and the GEMM built on it (reference:
+nunchaku/ops/gemv.py:10-56, nunchaku/ops/dispatch.py:19-49, nunchaku/ops/triton/awq.py:83-118, 186-251)."""
 
 from __future__ import annotations
 
@@ -21,12 +22,16 @@ def awq_gemv_w4a16_cuda(
 ) -> torch.Tensor:
     """
     ``out = in_feats @ (q * scaling_factors + zeros).T`` with ``q`` the TinyChat-packed uint4 weight
-    (``kernel`` ``(n // 4, k // 2)`` int32), group size 64.  Returns ``in_feats.shape[:-1] + (n,)`` in the input dtype.
+    (``kernel`` ``(n // 4, k // 2)`` int32).  Group size 64 runs the fused GEMV kernel (weights read once for all ``m``
+    rows); other group sizes decode the weight and multiply, as the reference does.  Returns
+    ``in_feats.shape[:-1] + (n,)`` in the input dtype.
     """
-    if group_size != 64:
-        raise NotImplementedError(f"group_size={group_size}: only the group-64 GEMV of the FLUX adaLN layers is implemented")
     _lib.require_cuda(in_feats, kernel, scaling_factors, zeros)
     x = in_feats.reshape(m, k)
+    if group_size != 64 or n % 32:
+        # as the reference (ops/triton/awq.py:226-228): decode to a dense weight, then a library matmul
+        w = awq_dequantize(kernel, scaling_factors, zeros, n, k, group_size, x.dtype)
+        return torch.matmul(x, w.t()).reshape(*in_feats.shape[:-1], n)
     if x.stride(1) != 1 or x.stride(0) % 8 or x.data_ptr() % 16:
         x = x.contiguous()
     if kernel.element_size() * kernel.numel() != n * k // 2 or not kernel.is_contiguous():
@@ -56,3 +61,65 @@ def awq_gemv_w4a16_cuda(
             )
             _lib.check(lib.svdq_awq_gemv_w4a16(args, _lib.stream_of(x)))
     return out.reshape(*in_feats.shape[:-1], n)
+
+
+def awq_dequantize(
+    kernel: torch.Tensor,
+    scaling_factors: torch.Tensor,
+    zeros: torch.Tensor,
+    n: int,
+    k: int,
+    group_size: int,
+    dtype: torch.dtype,
+) -> torch.Tensor:
+    """
+    Unpack a TinyChat-packed AWQ W4 weight to a dense ``(n, k)`` tensor ``q * scaling_factors + zeros`` of ``dtype``
+    (reference: nunchaku/ops/triton/awq.py:83-118).
+    """
+    _lib.require_cuda(kernel, scaling_factors, zeros)
+    if kernel.element_size() * kernel.numel() != n * k // 2 or not kernel.is_contiguous():
+        raise ValueError(f"unexpected packed AWQ weight shape {tuple(kernel.shape)} for n={n}, k={k}")
+    if group_size <= 0 or k % group_size:
+        raise ValueError(f"group_size={group_size} does not divide k={k}")
+    groups = k // group_size
+    if scaling_factors.shape != (groups, n) or zeros.shape != (groups, n):
+        raise ValueError(f"scaling_factors / zeros must be ({groups}, {n})")
+    if scaling_factors.dtype != dtype or zeros.dtype != dtype:
+        raise ValueError("scaling_factors / zeros must have the output dtype")
+    if scaling_factors.stride(1) != 1 or zeros.stride() != scaling_factors.stride():
+        scaling_factors, zeros = scaling_factors.contiguous(), zeros.contiguous()
+    out = torch.empty(n, k, dtype=dtype, device=kernel.device)
+    with torch.cuda.device(kernel.device):
+        _lib.check(_lib.load().svdq_awq_dequantize(kernel.data_ptr(), scaling_factors.data_ptr(), zeros.data_ptr(),
+                                                   out.data_ptr(), n, k, group_size, scaling_factors.stride(0),
+                                                   out.stride(0), _lib.dtype_code(dtype), _lib.stream_of(kernel)))  # fmt: skip
+    return out
+
+
+def awq_gemm_w4a16(
+    in_feats: torch.Tensor,
+    kernel: torch.Tensor,
+    scaling_factors: torch.Tensor,
+    zeros: torch.Tensor,
+    group_size: int = 128,
+) -> torch.Tensor:
+    """
+    AWQ W4A16 GEMM for larger batches (reference: nunchaku/ops/triton/awq.py:232-251): the weight is decoded once by
+    :func:`awq_dequantize`, the product is a dense library matmul.
+    """
+    shape = in_feats.shape
+    k = shape[-1]
+    x = in_feats.reshape(-1, k)
+    n = scaling_factors.shape[-1]
+    w = awq_dequantize(kernel, scaling_factors, zeros, n, k, group_size, x.dtype)
+    return torch.matmul(x, w.t()).reshape(*shape[:-1], n)
+
+
+def gemv_awq(in_feats, kernel, scaling_factors, zeros, m: int, n: int, k: int, group_size: int) -> torch.Tensor:
+    """The reference's dispatcher name for :func:`awq_gemv_w4a16_cuda` (nunchaku/ops/dispatch.py:19-34)."""
+    return awq_gemv_w4a16_cuda(in_feats, kernel, scaling_factors, zeros, m, n, k, group_size)
+
+
+def gemm_awq(in_feats, kernel, scaling_factors, zeros) -> torch.Tensor:
+    """The reference's dispatcher name for :func:`awq_gemm_w4a16` (nunchaku/ops/dispatch.py:37-49)."""
+    return awq_gemm_w4a16(in_feats, kernel, scaling_factors, zeros)

@@ -29,6 +29,8 @@ swiglu                 torch.nn.functional.silu in fp64, interleave inverse
 awq_pack / awq_decode  mutual inverse, written from two different statements
                        of the layout (view/permute vs. index formula)
 awq_gemv               fp64 dense dequantised matmul
+awq_dequantize         fp64 q * s + z rounded once (q * s is exact), per-group
+                       constancy, zero-point identity q = zp -> 0
 flux_rope              closed form cos/sin of pos * theta**(-2i/d) in fp64
 gated_residual         torch's own 16-bit CPU kernels, op by op (bit-equal)
 layernorm_modulate     torch.nn.functional.layer_norm in fp64 and torch's own
@@ -311,6 +313,18 @@ def awq_gemv(x: torch.Tensor, packed_i16: torch.Tensor, scales: torch.Tensor, ze
         xsum = xf[:, sl].sum(dim=1, keepdim=True)
         out += scales[c].float()[None, :] * dotq + zeros[c].float()[None, :] * xsum
     return out
+
+
+def awq_dequantize(packed_i16: torch.Tensor, scales: torch.Tensor, zeros: torch.Tensor, group_size: int) -> torch.Tensor:
+    """Dense weight ``T(q * s + z)`` with fp32 arithmetic (nunchaku/ops/triton/awq.py:48-79): ``(n, k)`` in the dtype of
+    ``scales``, scale group ``k // group_size``."""
+    n = scales.shape[1]
+    k = packed_i16.shape[1]
+    q = awq_decode(packed_i16, n, k).float()
+    grp = torch.arange(k, device=scales.device) // group_size
+    s = scales.float().t()[:, grp]
+    z = zeros.float().t()[:, grp]
+    return (q * s + z).to(scales.dtype)
 
 
 # --------------------------------------------------------------------------------------

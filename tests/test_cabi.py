@@ -73,6 +73,9 @@ def test_invalid_arguments_are_rejected_without_launch(lib):
     assert rc in (_lib.E_UNSUPPORTED, _lib.E_INVALID)
     a = _lib.AwqGemvArgs(x=16, qweight=16, scales=16, zeros=16, out=16, M=64, N=64, K=64, ld_x=64, ld_scales=64, ld_out=64)
     assert lib.svdq_awq_gemv_w4a16(a, None) == _lib.E_INVALID  # M > 32
+    assert lib.svdq_awq_dequantize(16, 16, 16, 16, 8, 64, 48, 8, 64, 0, None) == _lib.E_INVALID  # group size
+    assert lib.svdq_awq_dequantize(16, 16, 16, 16, 6, 64, 64, 8, 64, 0, None) == _lib.E_INVALID  # N % 4
+    assert lib.svdq_awq_dequantize(16, 16, 16, 16, 8, 64, 64, 8, 32, 0, None) == _lib.E_INVALID  # ld_out < K
     assert lib.svdq_gemm_w4a4(None, None) == _lib.E_INVALID
     at = _lib.AttentionArgs(q=16, k=16, v=16, o=16, vt=16, B=1, H=1, Tq=8, Tkv=8, D=32)
     assert lib.svdq_attention_fp16(at, None) == _lib.E_UNSUPPORTED  # head dimension
@@ -95,8 +98,10 @@ def test_ops_refuse_cpu_tensors_loudly():
         ops.svdq_quantize_w4a4_act_fuse_lora_cuda(x, fp4=True)
     with pytest.raises(NotImplementedError):
         ops.svdq_gemm_w4a4_cuda(x, x, out_q=x, ascales=x, wscales=x)
-    with pytest.raises(NotImplementedError):
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
         ops.awq_gemv_w4a16_cuda(x, x, x, x, 4, 4, 64, group_size=128)
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        ops.awq_dequantize(torch.zeros(1, 32, dtype=torch.int32), x[:1, :4], x[:1, :4], 4, 64, 64, torch.bfloat16)
 
 
 def test_product_never_imports_the_oracle():

@@ -57,3 +57,59 @@ def test_linear_module_adds_bias_after_kernel(dev):
     ref = O.awq_gemv(x, lin["qweight"].view(torch.int16).reshape(N // 4, K), lin["wscales"], lin["wzeros"])
     ref = ref.to(torch.bfloat16) + (torch.arange(N).to(torch.bfloat16) * 0.01)
     assert O.max_rel_err(y, ref) <= 1e-2
+
+
+@pytest.mark.parametrize("group_size", [32, 64, 128])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_dequantize_bit_exact(dev, group_size, dtype):
+    """out = T(q * s + z): q * s is exact in fp32, so kernel and oracle perform the same single rounding."""
+    from nunchaku_rocm_amd import ops
+
+    print(f"case group_size={group_size} {dtype}", flush=True)
+    K, N = 384, 44
+    g = torch.Generator().manual_seed(40 + group_size)
+    q = torch.randint(0, 16, (N, K), generator=g, dtype=torch.int32)
+    s = (torch.rand(K // group_size, N, generator=g) * 0.015 + 0.005).to(dtype)
+    z = (-torch.randint(0, 16, (K // group_size, N), generator=g).float() * s.float()).to(dtype)
+    packed = O.awq_pack(q)
+    w = ops.awq_dequantize(packed.view(torch.int32).to(dev), s.to(dev), z.to(dev), N, K, group_size, dtype)
+    torch.cuda.synchronize()
+    assert w.shape == (N, K) and w.dtype == dtype
+    assert torch.equal(w.cpu(), O.awq_dequantize(packed, s, z, group_size))
+
+
+def test_dequantize_flux_adaln_weight(dev):
+    from nunchaku_rocm_amd import ops
+
+    K, N = 3072, 18432
+    lin = O.make_awq_linear(K, N, seed=41)
+    w = ops.awq_dequantize(lin["qweight"].to(dev), lin["wscales"].to(dev), lin["wzeros"].to(dev), N, K, 64, torch.bfloat16)
+    torch.cuda.synchronize()
+    ref = O.awq_dequantize(lin["qweight"].view(torch.int16).reshape(N // 4, K), lin["wscales"], lin["wzeros"], 64)
+    assert torch.equal(w.cpu(), ref)
+
+
+@pytest.mark.parametrize("m,group_size", [(48, 128), (3, 32), (300, 64)])
+def test_gemm_and_gemv_fallback_decode_then_matmul(dev, m, group_size):
+    """awq_gemm_w4a16 and the group_size != 64 branch of the GEMV: dense decode, then a library matmul."""
+    from nunchaku_rocm_amd import ops
+
+    print(f"case m={m} group_size={group_size}", flush=True)
+    K, N = 256, 96
+    g = torch.Generator().manual_seed(50 + m)
+    q = torch.randint(0, 16, (N, K), generator=g, dtype=torch.int32)
+    s = (torch.rand(K // group_size, N, generator=g) * 0.015 + 0.005).to(torch.bfloat16)
+    z = (-torch.randint(0, 16, (K // group_size, N), generator=g).float() * s.float()).to(torch.bfloat16)
+    x = torch.randn(2, m, K, generator=g).to(torch.bfloat16)
+    packed = O.awq_pack(q)
+    kern = packed.view(torch.int32).to(dev)
+    wref = O.awq_dequantize(packed, s, z, group_size)
+    ref = x.float() @ wref.float().t()
+    out = ops.awq_gemm_w4a16(x.to(dev), kern, s.to(dev), z.to(dev), group_size=group_size)
+    assert out.shape == (2, m, N) and out.dtype == torch.bfloat16
+    assert O.max_rel_err(out.cpu(), ref) <= 1e-2
+    out2 = ops.gemv_awq(x.to(dev), kern, s.to(dev), z.to(dev), 2 * m, N, K, group_size)
+    assert out2.shape == (2, m, N)
+    assert O.max_rel_err(out2.cpu(), ref) <= 1e-2
+    if group_size == 128:
+        assert torch.equal(ops.gemm_awq(x.to(dev), kern, s.to(dev), z.to(dev)), out)

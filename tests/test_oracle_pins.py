@@ -284,6 +284,30 @@ def test_awq_gemv_fp64_dense(m):
     assert (out_c - out).abs().max() <= 1e-5 * ref.abs().max()
 
 
+@pytest.mark.parametrize("group_size", [32, 64, 128])
+def test_awq_dequantize_fp64_and_zero_point(group_size):
+    K, N = 256, 32
+    g = torch.Generator().manual_seed(16)
+    q = torch.randint(0, 16, (N, K), generator=g, dtype=torch.int32)
+    s = (torch.rand(K // group_size, N, generator=g) * 0.015 + 0.005).to(torch.bfloat16)
+    zp = torch.randint(0, 16, (K // group_size, N), generator=g)
+    z = (-zp.float() * s.float()).to(torch.bfloat16)
+    w = O.awq_dequantize(O.awq_pack(q), s, z, group_size)
+    assert w.shape == (N, K) and w.dtype == torch.bfloat16
+    grp = torch.arange(K) // group_size
+    # q * s has at most 12 significant bits: the fp64 value of q * s + z is exact, so rounding it to fp32 and then to
+    # bf16 is what fp32 arithmetic gives
+    ref = (q.double() * s.double().t()[:, grp] + z.double().t()[:, grp]).float().to(torch.bfloat16)
+    assert torch.equal(w, ref)
+    # where the code equals the zero point the weight is the rounding error of -zp * s only
+    hit = q == zp.t()[:, grp]
+    assert hit.any() and (w[hit].float().abs() <= s.float().t()[:, grp][hit] * 16 * 2**-8).all()
+    # codes that differ by one within a group differ by the scale (up to output rounding)
+    w2 = O.awq_dequantize(O.awq_pack((q + 1).clamp(max=15)), s, z, group_size)
+    step = (w2.float() - w.float())[q < 15]
+    assert ((step - s.float().t()[:, grp][q < 15]).abs() <= 2**-7 * (w.float().abs()[q < 15] + s.float().max())).all()
+
+
 # ----------------------------------------------------------------------------- FLUX rotary table
 def test_flux_rotary_closed_form():
     ids = O.flux_ids(4, 3, 5)
