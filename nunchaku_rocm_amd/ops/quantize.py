@@ -139,6 +139,30 @@ def quantize_w4a4_act_fuse_lora(
     return output, oscales, lora_act_out
 
 
+def quantize_w4a4_act(
+    input: torch.Tensor,
+    output: torch.Tensor | None = None,
+    oscales: torch.Tensor | None = None,
+    fp4: bool = False,
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """Per-group-64 symmetric int4 quantization without smoothing or LoRA (reference:
+    nunchaku/ops/triton/gemm_w4a4.py:1568-1577): ``(codes (M, K/2) uint8, scales (K/64, M))``."""
+    out, scales, _ = quantize_w4a4_act_fuse_lora(input, output, oscales, fp4=fp4)
+    return out, scales
+
+
+def quantize_w4a4_wgt(
+    input: torch.Tensor,
+    output: torch.Tensor | None = None,
+    oscales: torch.Tensor | None = None,
+    fp4: bool = False,
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """The same arithmetic applied to a weight ``(N, K)`` (reference: nunchaku/ops/triton/gemm_w4a4.py:1580-1592): the
+    result ``(codes (N, K/2), scales (K/64, N))`` is the natural layout the GEMM reads as ``wgt`` / ``wscales``."""
+    out, scales, _ = quantize_w4a4_act_fuse_lora(input, output, oscales, fp4=fp4)
+    return out, scales
+
+
 def svdq_quantize_w4a4_act_fuse_lora_cuda(
     input: torch.Tensor,
     output: torch.Tensor | None = None,

@@ -150,3 +150,32 @@ def test_norm_modulate_prologue(dev, M, K, R, batches, dtype):
     q3, s3, _ = ops.svdq_quantize_w4a4_act_fuse_lora_cuda(x.to(dev), lora_down=None if ld is None else ld.to(dev),
                                                           smooth=lin["smooth_factor"].to(dev), norm=(emb[:, :, 1], emb[:, :, 0], st))  # fmt: skip
     assert torch.equal(q3[:M], q[:M]) and torch.equal(s3[:, :M].view(torch.int16), s[:, :M].view(torch.int16))
+
+
+def test_plain_aliases_and_quantized_product(dev):
+    """quantize_w4a4_act / quantize_w4a4_wgt (no smoothing, no LoRA): bit-equal to the oracle, and their outputs are the
+    GEMM's natural-layout operands: the int4 product tracks the dense one within the quantization noise."""
+    from nunchaku_rocm_amd import ops
+
+    g = torch.Generator().manual_seed(77)
+    M, N, K = 96, 160, 512
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (torch.randn(N, K, generator=g) * 0.05).to(torch.bfloat16)
+    qa, sa = ops.quantize_w4a4_act(x.to(dev))
+    qw, sw = ops.quantize_w4a4_wgt(w.to(dev))
+    torch.cuda.synchronize()
+    ra = O.quantize_act(x)
+    rw = O.quantize_act(w)
+    assert qa.shape == (M, K // 2) and sa.shape == (K // 64, M) and qw.shape == (N, K // 2) and sw.shape == (K // 64, N)
+    assert torch.equal(qa.cpu(), ra[0]) and torch.equal(sa.cpu(), ra[1])
+    assert torch.equal(qw.cpu(), rw[0]) and torch.equal(sw.cpu(), rw[1])
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+    ops.svdq_gemm_w4a4_cuda(qa, qw, out=out, ascales=sa, wscales=sw)
+    torch.cuda.synchronize()
+    ref = O.gemm_w4a4(ra[0], rw[0], ra[1], rw[1])
+    assert O.max_rel_err(out.cpu(), ref) <= 1e-2
+    dense = x.float() @ w.float().t()
+    # int4 x int4 with per-group absmax scales: relative error of a dot product of 512 terms is a few percent
+    assert O.cosine(out.cpu().float(), dense) >= 0.98
+    with pytest.raises(NotImplementedError):
+        ops.quantize_w4a4_wgt(w.to(dev), fp4=True)
