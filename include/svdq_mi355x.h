@@ -35,6 +35,7 @@ extern "C" {
 #define SVDQ_ABI_VERSION 3
 
 enum { SVDQ_BF16 = 0, SVDQ_FP16 = 1 };
+enum { SVDQ_PRE_NONE = 0, SVDQ_PRE_GLU = 1, SVDQ_PRE_GELU = 2 }; /* svdq_quantize_args.prologue */
 
 enum {
     SVDQ_OK = 0,
@@ -67,9 +68,11 @@ typedef struct {
     int32_t ld_x, ld_out, ld_scales, ld_lora_act;
     int32_t dtype;           /* SVDQ_BF16 / SVDQ_FP16                                                       */
     int32_t is_unsigned;     /* 0: codes in [-8, 7], absmax / 7;  1: codes in [0, 15], max / 15             */
-    int32_t fuse_glu;        /* 1: x is (M, 2K) and the quantized value is x[:, :K] * silu(x[:, K:])        */
+    int32_t prologue;        /* SVDQ_PRE_NONE; SVDQ_PRE_GLU: x is (M, 2K) and the quantized value is
+                              * x[:, :K] * silu(x[:, K:]) (fuse_glu); SVDQ_PRE_GELU: tanh-GELU of x (fuse_gelu,
+                              * ops/triton/gemm_w4a4.py:1403-1408): the LoRA-down sees the result rounded to T */
     float shift;             /* added before smoothing (0.171875 after GELU, else 0)                        */
-    /* Optional prologue (NULL norm_stats = off; not with fuse_glu): the quantized and LoRA-projected value is
+    /* Optional norm prologue (NULL norm_stats = off; only with SVDQ_PRE_NONE): the quantized and LoRA-projected value is
      * T(T(T((x - mean[m]) * rstd[m]) * norm_scale[k]) + norm_shift[k]), i.e. LayerNorm without affine followed by the
      * adaLN modulate, each step rounded to T as separate elementwise kernels would
      * (nunchaku/models/normalization.py:97-104, models/transformers/transformer_flux_v2.py:236-237). */

@@ -18,6 +18,7 @@ ABI_VERSION = 3
 
 BF16, FP16 = 0, 1
 EPI_PLAIN, EPI_QK_NORM_ROPE, EPI_GELU_QUANT, EPI_SWIGLU_QUANT = 0, 1, 2, 3
+PRE_NONE, PRE_GLU, PRE_GELU = 0, 1, 2
 E_INVALID, E_UNSUPPORTED, E_LAUNCH = -1, -2, -3
 
 EXPORTS = (
@@ -49,7 +50,7 @@ class QuantizeArgs(ctypes.Structure):
 
     _fields_ = (
         [(n, _vp) for n in ("x", "smooth", "lora_down_t", "out", "scales", "lora_act")]
-        + [(n, _i32) for n in ("M", "K", "R", "ld_x", "ld_out", "ld_scales", "ld_lora_act", "dtype", "is_unsigned", "fuse_glu")]
+        + [(n, _i32) for n in ("M", "K", "R", "ld_x", "ld_out", "ld_scales", "ld_lora_act", "dtype", "is_unsigned", "prologue")]
         + [("shift", _f32)]
         + [(n, _vp) for n in ("norm_stats", "norm_scale", "norm_shift")]
         + [(n, _i32) for n in ("norm_rows_per_batch", "norm_ld", "norm_stride")]

@@ -39,8 +39,9 @@ struct QVecs {
     uint16_t sm, ns, nh;  // smooth factor, norm scale, norm shift
 };
 
-template <typename T, bool UNSIGNED, bool GLU, bool HAS_LORA, bool HAS_SMOOTH, bool NORM>
+template <typename T, bool UNSIGNED, int PRE, bool HAS_LORA, bool HAS_SMOOTH, bool NORM>
 __global__ __launch_bounds__(Q_WAVES * 64, NORM ? 4 : 2) void quantize_act_kernel(svdq_quantize_args a) {
+    constexpr bool GLU = PRE == SVDQ_PRE_GLU, GELU = PRE == SVDQ_PRE_GELU;
     // per wavefront: two activation stages (16 rows, + the gate tile with GLU) and one LoRA-down tile (32 ranks), 128
     // bytes a row.  The LoRA-down tile is an L2 hit and the first thing a group consumes: one group ahead is enough.
     constexpr int XS_BYTES = (GLU ? 2 : 1) * Q_ROWS * Q_ROW_BYTES, G_OFF = Q_ROWS * Q_ROW_BYTES;
@@ -182,6 +183,16 @@ __global__ __launch_bounds__(Q_WAVES * 64, NORM ? 4 : 2) void quantize_act_kerne
                     v[8 + 2 * j] = v[8 + 2 * j] * (g2 / (1.0f + __expf(-g2)));
                     v[8 + 2 * j + 1] = v[8 + 2 * j + 1] * (g3 / (1.0f + __expf(-g3)));
                 }
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    cxlo[j] = (int)pack2<T>(v[2 * j], v[2 * j + 1]);
+                    cxhi[j] = (int)pack2<T>(v[8 + 2 * j], v[8 + 2 * j + 1]);
+                }
+            }
+            if (GELU) {
+                // tanh-GELU of the input (the unfused form of the GEMM's GELU epilogue); the LoRA-down sees it rounded to T
+#pragma unroll
+                for (int j = 0; j < 16; j++) v[j] = gelu_tanh(v[j]);
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
                     cxlo[j] = (int)pack2<T>(v[2 * j], v[2 * j + 1]);
@@ -432,7 +443,7 @@ __global__ void transpose_kr_kernel(const uint16_t *in, uint16_t *out, int K, in
     out[idx] = in[(size_t)k * ld_in + r];
 }
 
-template <typename T, bool U, bool G, bool NORM>
+template <typename T, bool U, int G, bool NORM>
 static void launch_quantize3(const svdq_quantize_args &a, hipStream_t s) {
     dim3 grid((a.M + Q_ROWS - 1) / Q_ROWS), block(Q_WAVES * 64);
     const bool lora = a.R > 0, sm = a.smooth != nullptr;
@@ -446,11 +457,11 @@ static void launch_quantize3(const svdq_quantize_args &a, hipStream_t s) {
         hipLaunchKernelGGL((quantize_act_kernel<T, U, G, false, false, NORM>), grid, block, 0, s, a);
 }
 
-template <typename T, bool U, bool G>
+template <typename T, bool U, int G>
 static void launch_quantize2(const svdq_quantize_args &a, hipStream_t s) {
-    if constexpr (!G) {
+    if constexpr (G == SVDQ_PRE_NONE) {
         if (a.norm_stats) {
-            launch_quantize3<T, U, false, true>(a, s);
+            launch_quantize3<T, U, SVDQ_PRE_NONE, true>(a, s);
             return;
         }
     }
@@ -459,16 +470,21 @@ static void launch_quantize2(const svdq_quantize_args &a, hipStream_t s) {
 
 template <typename T>
 static void launch_quantize(const svdq_quantize_args &a, hipStream_t s) {
-    if (a.fuse_glu) {
+    if (a.prologue == SVDQ_PRE_GLU) {
         if (a.is_unsigned)
-            launch_quantize2<T, true, true>(a, s);
+            launch_quantize2<T, true, SVDQ_PRE_GLU>(a, s);
         else
-            launch_quantize2<T, false, true>(a, s);
+            launch_quantize2<T, false, SVDQ_PRE_GLU>(a, s);
+    } else if (a.prologue == SVDQ_PRE_GELU) {
+        if (a.is_unsigned)
+            launch_quantize2<T, true, SVDQ_PRE_GELU>(a, s);
+        else
+            launch_quantize2<T, false, SVDQ_PRE_GELU>(a, s);
     } else {
         if (a.is_unsigned)
-            launch_quantize2<T, true, false>(a, s);
+            launch_quantize2<T, true, SVDQ_PRE_NONE>(a, s);
         else
-            launch_quantize2<T, false, false>(a, s);
+            launch_quantize2<T, false, SVDQ_PRE_NONE>(a, s);
     }
 }
 
@@ -502,7 +518,11 @@ extern "C" int svdq_quantize_act(const svdq_quantize_args *args, void *stream) {
         set_error("svdq_quantize_act: out rows must be 8-byte aligned (ld_out=%d)", a.ld_out);
         return SVDQ_E_INVALID;
     }
-    if (a.ld_x < (a.fuse_glu ? 2 : 1) * a.K || a.ld_out < a.K / 2 || a.ld_scales < a.M ||
+    if (a.prologue < SVDQ_PRE_NONE || a.prologue > SVDQ_PRE_GELU) {
+        set_error("svdq_quantize_act: unknown prologue %d", a.prologue);
+        return SVDQ_E_INVALID;
+    }
+    if (a.ld_x < (a.prologue == SVDQ_PRE_GLU ? 2 : 1) * a.K || a.ld_out < a.K / 2 || a.ld_scales < a.M ||
         (a.R > 0 && a.ld_lora_act < a.R)) {
         set_error("svdq_quantize_act: a leading dimension is smaller than its row");
         return SVDQ_E_INVALID;
@@ -512,8 +532,8 @@ extern "C" int svdq_quantize_act(const svdq_quantize_args *args, void *stream) {
         return SVDQ_E_INVALID;
     }
     if (a.norm_stats) {
-        if (a.fuse_glu) {
-            set_error("svdq_quantize_act: the norm prologue cannot be combined with fuse_glu");
+        if (a.prologue != SVDQ_PRE_NONE) {
+            set_error("svdq_quantize_act: the norm prologue cannot be combined with the GLU / GELU prologue");
             return SVDQ_E_UNSUPPORTED;
         }
         if (!a.norm_scale || !a.norm_shift || a.norm_rows_per_batch < 0 || a.norm_rows_per_batch % Q_ROWS ||

@@ -96,6 +96,26 @@ def svdq_gemm_w4a4_cuda(
         )
     if fuse_swiglu:
         assert out is None and want_quant, "fuse_swiglu writes qout/oscales, not out"
+    if want_quant and not want_qk and (N % 128 or M % 16 or qout.stride(-1) != 1 or (fuse_swiglu and N % 32)):
+        # shapes the requantizing epilogues do not take: the unfused form, as the reference's dispatcher does
+        # (nunchaku/ops/triton/gemm_w4a4.py:985-1000, 1298-1312): 16-bit GEMM output, then the activation quantizer
+        from .quantize import quantize_w4a4_act_fuse_lora
+
+        T = oscales.dtype
+        x = out.reshape(-1, N) if out is not None else torch.empty(M, N, dtype=T, device=dev)
+        svdq_gemm_w4a4_cuda(act, wgt, out=x, ascales=ascales, wscales=wscales, lora_act_in=lora_act_in, lora_up=lora_up,
+                            bias=bias, act_unsigned=act_unsigned)  # fmt: skip
+        rows = x.shape[0]
+        qout2d = qout.reshape(-1, qout.shape[-1])
+        la_out = lora_act_out if lora_down is not None else None
+        if fuse_swiglu:
+            x = x.view(rows, N // 32, 2, 16)
+            y = (torch.nn.functional.silu(x[:, :, 0]) * x[:, :, 1]).reshape(rows, N // 2)
+            quantize_w4a4_act_fuse_lora(y, qout2d, oscales, lora_down, la_out, smooth_factor)
+        else:
+            quantize_w4a4_act_fuse_lora(x, qout2d, oscales, lora_down, la_out, smooth_factor, fuse_gelu=True,
+                                        shift_value=GELU_SHIFT, unsigned=True)  # fmt: skip
+        return None
 
     T = out.dtype if out is not None else (oscales.dtype if oscales is not None else ascales.dtype)
     if out is None and not want_quant:
@@ -158,7 +178,7 @@ def svdq_gemm_w4a4_cuda(
     lib = _lib.load()
     if want_qk:
         if rotary_emb.dtype != torch.float32:
-            raise ValueError("rotary_emb must be float32")
+            rotary_emb = rotary_emb.float()  # the reference's unfused kernel reads any dtype and computes in fp32
         rot = rotary_emb.reshape(actual_m, HEAD_DIM)
         if rot.stride(1) != 1:
             rot = rot.contiguous()

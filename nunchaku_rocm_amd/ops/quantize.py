@@ -64,8 +64,8 @@ def quantize_w4a4_act_fuse_lora(
     """
     Backend-level quantizer with the reference's full option set (reference:
     nunchaku/ops/triton/gemm_w4a4.py:1521-1565): no row padding, outputs allocated when not given, ``unsigned`` /
-    ``shift_value`` for activations known to be non-negative after a shift.  ``fuse_gelu`` (the reference's unfused
-    fallback prologue) is not implemented: the GELU lives in the GEMM epilogue here.
+    ``shift_value`` for activations known to be non-negative after a shift, ``fuse_gelu`` = tanh-GELU of the input
+    first (what the GEMM's fused GELU epilogue computes, for outputs that were produced unfused).
 
     ``norm=(scale, shift)`` or ``(scale, shift, stats)`` (no counterpart in the reference, which runs these as separate
     torch kernels): what is quantized and LoRA-projected is ``layer_norm(input) * scale + shift`` (no affine,
@@ -74,8 +74,8 @@ def quantize_w4a4_act_fuse_lora(
     """
     if fp4:
         raise NotImplementedError("NVFP4 quantization is not implemented (int4 only)")
-    if fuse_gelu:
-        raise NotImplementedError("fuse_gelu: GELU is fused into the producing GEMM's epilogue instead")
+    if fuse_gelu and fuse_glu:
+        raise NotImplementedError("fuse_gelu together with fuse_glu")
     inp = input.reshape(-1, input.shape[-1])
     _lib.require_cuda(inp, output, oscales, lora_down, lora_act_out, smooth)
     M = inp.shape[0]
@@ -106,8 +106,8 @@ def quantize_w4a4_act_fuse_lora(
     nstats = nscale = nshift = None
     nrows, nld, nstride = 0, 0, 1
     if norm is not None:
-        if fuse_glu:
-            raise NotImplementedError("norm= cannot be combined with fuse_glu")
+        if fuse_glu or fuse_gelu:
+            raise NotImplementedError("norm= cannot be combined with fuse_glu / fuse_gelu")
         nstats, nscale, nshift, nrows, nld, nstride = _norm_args(norm, inp, M, K, norm_eps)
     args = _lib.QuantizeArgs(
         norm_stats=_lib.ptr(nstats),
@@ -131,7 +131,7 @@ def quantize_w4a4_act_fuse_lora(
         ld_lora_act=lora_act_out.stride(0) if rank else 0,
         dtype=_lib.dtype_code(inp.dtype),
         is_unsigned=int(unsigned),
-        fuse_glu=int(fuse_glu),
+        prologue=_lib.PRE_GLU if fuse_glu else (_lib.PRE_GELU if fuse_gelu else _lib.PRE_NONE),
         shift=float(shift_value),
     )
     with torch.cuda.device(inp.device):

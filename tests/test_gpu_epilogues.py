@@ -217,3 +217,73 @@ def test_fused_swiglu_mlp(dev):
     err = O.max_rel_err(y.cpu(), ref)
     print(f"fused_swiglu_mlp max rel err {err:.3e}", flush=True)
     assert err <= TOL
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,N,R2,swiglu", [(40, 192, 32, False), (144, 320, 0, False), (40, 256, 16, True)])
+def test_requantizing_gemm_on_shapes_the_fused_epilogues_do_not_take(dev, M, N, R2, swiglu, dtype):
+    """N not a multiple of 128 or M not a multiple of 16: the 16-bit GEMM output, then the quantizer with its GELU
+    prologue (or torch's SiLU product for SwiGLU), as the reference's dispatcher falls back."""
+    from nunchaku_rocm_amd import ops
+
+    print(f"case M={M} N={N} R2={R2} swiglu={swiglu} {dtype}", flush=True)
+    K, R = 256, 16
+    H = N // 2 if swiglu else N
+    p = _problem(M, N, K, R, dtype, seed=N + R2 + 7)
+    g = torch.Generator().manual_seed(96)
+    smooth = (torch.rand(H, generator=g) + 0.5).to(dtype)
+    ld = (torch.randn(H, max(R2, 16), generator=g) * 0.1).to(dtype)[:, :R2].contiguous() if R2 else None
+    d = lambda t: None if t is None else t.to(dev)  # noqa: E731
+    qout = torch.zeros(M + 16, H // 2, dtype=torch.uint8, device=dev)
+    osc = torch.empty(H // 64, M, dtype=dtype, device=dev)
+    lao = torch.empty(M, R2, dtype=torch.float32, device=dev) if R2 else None
+    out = None if swiglu else torch.empty(M, N, dtype=dtype, device=dev)
+    ops.svdq_gemm_w4a4_cuda(
+        act=d(p["act"]), wgt=d(p["wgt"]), out=out, qout=qout, ascales=d(p["asc"]), wscales=d(p["wsc"]), oscales=osc,
+        lora_act_in=d(p["la"]), lora_up=d(p["lu"]), lora_down=d(ld), lora_act_out=lao, bias=d(p["bias"]),
+        smooth_factor=d(smooth), fuse_swiglu=swiglu,
+    )  # fmt: skip
+    torch.cuda.synchronize()
+    assert (qout[M:] == 0).all()
+    lin = O.gemm_w4a4(p["act"], p["wgt"], p["asc"], p["wsc"], p["bias"], p["la"], p["lu"], False)
+    if swiglu:
+        x = lin.to(dtype).view(M, N // 32, 2, 16)
+        y = (torch.nn.functional.silu(x[:, :, 0]) * x[:, :, 1]).reshape(M, H)
+        rp, rs, rl, rc = O.quantize_act(y, ld, smooth)
+        tol_rate = 2e-2  # a 16-bit ulp of the GEMM output moves a code now and then
+    else:
+        assert O.max_rel_err(out.cpu(), lin) <= TOL
+        # the quantizer's part is checked on the very output the GPU produced
+        rp, rs, rl, rc = O.quantize_act(out.cpu(), ld, smooth, unsigned=True, shift=O.GELU_SHIFT, fuse_gelu=True)
+        tol_rate = 1e-3
+    codes = O.unpack_int4(qout[:M].cpu(), swiglu)
+    diff = (codes - rc).abs()
+    rate = (diff > 0).float().mean().item()
+    print(f"  code mismatch rate {rate:.2e}", flush=True)
+    assert diff.max() <= (2 if swiglu else 1) and rate < tol_rate
+    ulp = 2**-7 if dtype == torch.bfloat16 else 2**-10
+    assert ((osc.cpu().float() - rs.float()).abs() <= rs.float().abs() * (4 if swiglu else 1) * ulp + 1e-7).all()
+    if R2:
+        assert (lao.cpu() - rl).abs().max() <= TOL * rl.abs().max()
+
+
+def test_rotary_table_in_16_bit(dev):
+    """A rotary table that is not fp32 is read as the values it holds (the reference's unfused kernel does the same)."""
+    from nunchaku_rocm_amd import ops
+
+    M, H, K, R, dtype = 64, 1, 256, 16, torch.bfloat16
+    N = 3 * H * 128
+    p = _problem(M, N, K, R, dtype, seed=5)
+    g = torch.Generator().manual_seed(95)
+    nq = (torch.rand(128, generator=g) + 0.5).to(dtype)
+    nk = (torch.rand(128, generator=g) + 0.5).to(dtype)
+    theta = torch.rand(M, 64, generator=g) * 6.28
+    rot = torch.stack([torch.sin(theta), torch.cos(theta)], -1).reshape(M, 64, 1, 2).to(dtype)
+    d = lambda t: t.to(dev)  # noqa: E731
+    kw = dict(act=d(p["act"]), wgt=d(p["wgt"]), ascales=d(p["asc"]), wscales=d(p["wsc"]), norm_q=d(nq), norm_k=d(nk))
+    a = torch.empty(M, N, dtype=dtype, device=dev)
+    b = torch.empty(M, N, dtype=dtype, device=dev)
+    ops.svdq_gemm_w4a4_cuda(out=a, rotary_emb=d(rot), **kw)
+    ops.svdq_gemm_w4a4_cuda(out=b, rotary_emb=d(rot.float()), **kw)
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)

@@ -179,3 +179,31 @@ def test_plain_aliases_and_quantized_product(dev):
     assert O.cosine(out.cpu().float(), dense) >= 0.98
     with pytest.raises(NotImplementedError):
         ops.quantize_w4a4_wgt(w.to(dev), fp4=True)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,K,R", [(48, 256, 32), (130, 384, 0), (257, 1024, 48)])
+def test_gelu_prologue(dev, M, K, R, dtype):
+    """fuse_gelu: tanh-GELU, LoRA-down on its rounded value, + 0.171875, smoothing, unsigned codes.  exp() differs
+    between implementations by an ulp, so codes carry the reference's own bar: off by at most one, rarely."""
+    from nunchaku_rocm_amd.ops.quantize import quantize_w4a4_act_fuse_lora
+
+    print(f"case M={M} K={K} R={R} {dtype}", flush=True)
+    lin = O.make_svdq_linear(K, 64, R=max(R, 16), seed=K + R, dtype=dtype)
+    x = (O.make_activations(M, K, seed=M, dtype=dtype).float() * 0.3).to(dtype)
+    ld = lin["proj_down"][:, :R].contiguous() if R else None
+    sm = lin["smooth_factor"]
+    out, osc, la = quantize_w4a4_act_fuse_lora(x.to(dev), lora_down=ld.to(dev) if R else None, smooth=sm.to(dev),
+                                               fuse_gelu=True, shift_value=O.GELU_SHIFT, unsigned=True)  # fmt: skip
+    torch.cuda.synchronize()
+    rp, rs, rl, rc = O.quantize_act(x, ld, sm, unsigned=True, shift=O.GELU_SHIFT, fuse_gelu=True)
+    diff = (O.unpack_int4(out.cpu(), False) - rc).abs()
+    rate = (diff > 0).float().mean().item()
+    print(f"  code mismatch rate {rate:.2e}", flush=True)
+    assert diff.max() <= 1 and rate < 1e-3
+    ulp = 2**-7 if dtype == torch.bfloat16 else 2**-10
+    assert ((osc.cpu().float() - rs.float()).abs() <= rs.float().abs() * ulp + 1e-7).all()
+    if R:
+        assert (la.cpu() - rl).abs().max() <= 1e-2 * rl.abs().max()
+    with pytest.raises(NotImplementedError):
+        quantize_w4a4_act_fuse_lora(torch.zeros(16, 128, dtype=dtype, device=dev), fuse_gelu=True, fuse_glu=True)
