@@ -123,7 +123,7 @@ typedef struct {
     const void *lora_up;    /* (N, R) T, row stride ld_lora_up; NULL iff R = 0                                  */
     void *out;              /* (actual_m, N) T, row stride ld_out (rows 16-byte aligned: base and ld_out % 8);   */
                             /* may be NULL for the requantizing epilogues                                       */
-    int32_t M, N, K, R;     /* K % 128 == 0, N % 8 == 0, R % 16 == 0                                            */
+    int32_t M, N, K, R;     /* K % 64 == 0, N % 8 == 0, R % 16 == 0                                             */
     int32_t actual_m;       /* rows of out that exist (<= M); rows beyond are computed but never written       */
     int32_t ld_act, ld_wgt, ld_ascales, ld_wscales, ld_lora_act, ld_lora_up, ld_out;
     int32_t dtype;

@@ -88,7 +88,7 @@ __device__ inline void tile_ids(int tiles_m, int tiles_n, int &pid_m, int &pid_n
     pid_n = (id % band) / gm;
 }
 
-template <typename T, bool ACT_UNSIGNED, int EPI, bool WPL>
+template <typename T, bool ACT_UNSIGNED, int EPI, bool WPL, bool ODDG>  // ODDG: K / 64 is odd
 __global__ __launch_bounds__(NTHREADS, 4) void gemm_w4a4_kernel(svdq_gemm_args a) {
     __shared__ __align__(16) uint8_t smem[SMEM_BYTES];
 
@@ -113,7 +113,18 @@ __global__ __launch_bounds__(NTHREADS, 4) void gemm_w4a4_kernel(svdq_gemm_args a
     const uint8_t *gbase[PER_WAVE];
     uint32_t goff[PER_WAVE];
     int ldst[PER_WAVE], gstep[PER_WAVE];
+    uint32_t gcap[PER_WAVE];
     const int G = a.K / GROUP;
+    // K / 64 odd: the last stage has one group only.  The loads of its second group stop one stage earlier (they re-read
+    // valid memory) and its scales are staged as zero, so it adds nothing.  A load's stage offset is min(s * step, cap).
+    auto cap_of = [&](int gg, int step, const uint8_t *&base, int back) -> uint32_t {
+        if (gg == 0) return (uint32_t)(G / 2) * (uint32_t)step;  // G is odd: stages 0 .. G / 2
+        if (G == 1) {  // no earlier stage: read the first group's bytes instead
+            base -= back;
+            return 0u;
+        }
+        return (uint32_t)(G / 2 - 1) * (uint32_t)step;
+    };
 #pragma unroll
     for (int i = 0; i < PER_WAVE; i++) {
         const int q = wave * PER_WAVE + i;  // wave-uniform
@@ -123,6 +134,7 @@ __global__ __launch_bounds__(NTHREADS, 4) void gemm_w4a4_kernel(svdq_gemm_args a
             goff[i] = (uint32_t)(min(m0 + blk * 32 + l32, a.M - 1) - m0) * (uint32_t)a.ld_act + half * 16;
             ldst[i] = (blk * 2 + gg) * BLK_BYTES;
             gstep[i] = KSTAGE / 2;
+            if constexpr (ODDG) gcap[i] = cap_of(gg, gstep[i], gbase[i], 32);
         } else if (WPL) {                   // weight plane block j: (blk = j / 4, group (j / 2) % 2, plane j % 2)
             const int j = q - 8, blk = j >> 2, gg = (j >> 1) & 1, pl = j & 1;
             const int nblk = min(n0 / 32 + blk, (a.N + 31) / 32 - 1);
@@ -130,19 +142,24 @@ __global__ __launch_bounds__(NTHREADS, 4) void gemm_w4a4_kernel(svdq_gemm_args a
             goff[i] = lane * 16;
             ldst[i] = W_OFF + ((blk * 2 + gg) * 2 + pl) * BLK_BYTES;
             gstep[i] = 2 * 2 * BLK_BYTES;   // two groups x two planes per stage
+            if constexpr (ODDG) gcap[i] = cap_of(gg, gstep[i], gbase[i], 2 * BLK_BYTES);
         } else {                            // packed weight block j: (blk = j / 2, group j % 2)
             const int j = q - 8, blk = j >> 1, gg = j & 1;
             gbase[i] = (const uint8_t *)a.wgt + (size_t)n0 * a.ld_wgt + gg * 32;
             goff[i] = (uint32_t)(min(n0 + blk * 32 + l32, a.N - 1) - n0) * (uint32_t)a.ld_wgt + half * 16;
             ldst[i] = W_OFF + (blk * 2 + gg) * BLK_BYTES;
             gstep[i] = KSTAGE / 2;
+            if constexpr (ODDG) gcap[i] = cap_of(gg, gstep[i], gbase[i], 32);
         }
     }
     auto dma_one = [&](int s, int buf, int i) {  // block load i of stage s into staging buffer buf
-        // pre-split weights: SGPR base + 32-bit offset; the packed path has the registers for neither form to spare
-        // and fares better with a 64-bit address
-        const uint8_t *src = WPL ? gbase[i] + (goff[i] + (uint32_t)s * (uint32_t)gstep[i])
-                                 : gbase[i] + (size_t)s * gstep[i] + goff[i];
+        // SGPR base + 32-bit offset (lane part + scalar stage part); the packed path with all stages whole has the
+        // registers for neither form to spare and fares better with a 64-bit address
+        const uint8_t *src;
+        if constexpr (ODDG)
+            src = gbase[i] + (goff[i] + min((uint32_t)s * (uint32_t)gstep[i], gcap[i]));  // stage part wave-uniform
+        else
+            src = WPL ? gbase[i] + (goff[i] + (uint32_t)s * (uint32_t)gstep[i]) : gbase[i] + (size_t)s * gstep[i] + goff[i];
         __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)src, (SVDQ_AS3 void *)(smem + buf * BUF_BYTES + ldst[i]),
                                          16, 0, 0);
     };
@@ -162,8 +179,21 @@ __global__ __launch_bounds__(NTHREADS, 4) void gemm_w4a4_kernel(svdq_gemm_args a
     const float fold = ACT_UNSIGNED ? (1.0f / 16.0f) : (1.0f / 256.0f);
     // a plain load: its first use is the conversion at the top of the next stage, behind that stage's vmcnt(0)
     uint16_t rsc;
+    uint32_t sc_cap = 0;
+    if constexpr (ODDG) {
+        sc_cap = (uint32_t)(G / 2) * sc_step;
+        if (sgu == 1) {  // this wavefront's group of the last stage does not exist
+            if (G == 1) gSC -= loads_as ? a.ld_ascales : a.ld_wscales;
+            sc_cap = G == 1 ? 0u : (uint32_t)(G / 2 - 1) * sc_step;
+        }
+    }
     auto load_scales = [&](int s) {
-        rsc = *(const uint16_t *)((const uint8_t *)gSC + (sc_off + (uint32_t)s * (uint32_t)sc_step));
+        if (ODDG) {
+            const uint16_t v = *(const uint16_t *)((const uint8_t *)gSC + (sc_off + min((uint32_t)s * (uint32_t)sc_step, sc_cap)));
+            rsc = (s == G / 2 && sgu == 1) ? (uint16_t)0 : v;  // +0 in both 16-bit types
+        } else {
+            rsc = *(const uint16_t *)((const uint8_t *)gSC + (sc_off + (uint32_t)s * (uint32_t)sc_step));
+        }
     };
     auto store_scales = [&](int s) {
         uint8_t *base = smem + (s % NSTAGE) * BUF_BYTES;
@@ -185,7 +215,7 @@ __global__ __launch_bounds__(NTHREADS, 4) void gemm_w4a4_kernel(svdq_gemm_args a
             for (int i = 0; i < 16; i++) acc[bn][bm][i] = 0.0f;
 
     const v16i cmagic = magic_acc();
-    const int nstages = a.K / KSTAGE;
+    const int nstages = ODDG ? a.K / KSTAGE + 1 : a.K / KSTAGE;
     const int offW = W_OFF + (wn * 2) * 2 * (WPL ? 2 : 1) * BLK_BYTES + lane * 16;
     const int offA = (wm * NBM) * 2 * BLK_BYTES + lane * 16;
 
@@ -730,23 +760,31 @@ __global__ __launch_bounds__(64) void group_acc_kernel(const uint8_t *act, const
     }
 }
 
-template <typename T, bool U, bool WPL>
-static void launch_gemm_epi2(const svdq_gemm_args &a, hipStream_t s) {
+template <typename T, bool U, bool WPL, bool ODDG>
+static void launch_gemm_epi3(const svdq_gemm_args &a, hipStream_t s) {
     const dim3 grid(((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN)), block(NTHREADS);
     switch (a.epilogue) {
         case SVDQ_EPI_PLAIN:
-            hipLaunchKernelGGL((gemm_w4a4_kernel<T, U, SVDQ_EPI_PLAIN, WPL>), grid, block, 0, s, a);
+            hipLaunchKernelGGL((gemm_w4a4_kernel<T, U, SVDQ_EPI_PLAIN, WPL, ODDG>), grid, block, 0, s, a);
             break;
         case SVDQ_EPI_QK_NORM_ROPE:
-            hipLaunchKernelGGL((gemm_w4a4_kernel<T, U, SVDQ_EPI_QK_NORM_ROPE, WPL>), grid, block, 0, s, a);
+            hipLaunchKernelGGL((gemm_w4a4_kernel<T, U, SVDQ_EPI_QK_NORM_ROPE, WPL, ODDG>), grid, block, 0, s, a);
             break;
         case SVDQ_EPI_GELU_QUANT:
-            hipLaunchKernelGGL((gemm_w4a4_kernel<T, U, SVDQ_EPI_GELU_QUANT, WPL>), grid, block, 0, s, a);
+            hipLaunchKernelGGL((gemm_w4a4_kernel<T, U, SVDQ_EPI_GELU_QUANT, WPL, ODDG>), grid, block, 0, s, a);
             break;
         case SVDQ_EPI_SWIGLU_QUANT:
-            hipLaunchKernelGGL((gemm_w4a4_kernel<T, U, SVDQ_EPI_SWIGLU_QUANT, WPL>), grid, block, 0, s, a);
+            hipLaunchKernelGGL((gemm_w4a4_kernel<T, U, SVDQ_EPI_SWIGLU_QUANT, WPL, ODDG>), grid, block, 0, s, a);
             break;
     }
+}
+
+template <typename T, bool U, bool WPL>
+static void launch_gemm_epi2(const svdq_gemm_args &a, hipStream_t s) {
+    if ((a.K / GROUP) & 1)
+        launch_gemm_epi3<T, U, WPL, true>(a, s);
+    else
+        launch_gemm_epi3<T, U, WPL, false>(a, s);
 }
 
 template <typename T, bool U>
@@ -810,8 +848,8 @@ extern "C" int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream) {
         set_error("svdq_gemm_w4a4: dtype %d", a.dtype);
         return SVDQ_E_INVALID;
     }
-    if (a.M < 0 || a.N <= 0 || a.K <= 0 || a.K % KSTAGE || a.N % 8) {
-        set_error("svdq_gemm_w4a4: M=%d N=%d K=%d needs K %% 128 == 0 and N %% 8 == 0", a.M, a.N, a.K);
+    if (a.M < 0 || a.N <= 0 || a.K <= 0 || a.K % GROUP || a.N % 8) {
+        set_error("svdq_gemm_w4a4: M=%d N=%d K=%d needs K %% 64 == 0 and N %% 8 == 0", a.M, a.N, a.K);
         return SVDQ_E_INVALID;
     }
     if (!a.act || !a.wgt || !a.ascales || !a.wscales) {

@@ -64,8 +64,9 @@ def test_invalid_arguments_are_rejected_without_launch(lib):
     assert b"multiple of 64" in lib.svdq_last_error()
     with pytest.raises(ValueError):
         _lib.check(_lib.E_INVALID)
-    g = _lib.GemmArgs(act=16, wgt=16, ascales=16, wscales=16, out=16, M=8, N=8, K=64, ld_act=32, ld_wgt=32)
-    assert lib.svdq_gemm_w4a4(g, None) == _lib.E_INVALID  # K % 128
+    g = _lib.GemmArgs(act=16, wgt=16, ascales=16, wscales=16, out=16, M=8, N=8, K=96, ld_act=48, ld_wgt=48)
+    assert lib.svdq_gemm_w4a4(g, None) == _lib.E_INVALID  # K % 64
+    assert b"K %% 64".replace(b"%%", b"%") in lib.svdq_last_error()
     g = _lib.GemmArgs(act=16, wgt=16, ascales=16, wscales=16, out=16, M=8, N=8, K=128, ld_act=64, ld_wgt=64,
                       ld_ascales=8, ld_wscales=8, ld_out=8, actual_m=8, epilogue=_lib.EPI_SWIGLU_QUANT,
                       qout=16, oscales=16)  # fmt: skip

@@ -61,9 +61,10 @@ def test_group_accumulators_bit_exact(dev, M, N, K, unsigned):
 
 @pytest.mark.parametrize("unsigned", [False, True])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_unit_scales_exact_integer_gemm(dev, unsigned, dtype):
+@pytest.mark.parametrize("K", [256, 192])
+def test_unit_scales_exact_integer_gemm(dev, unsigned, dtype, K):
     """With all scales 1 every fp32 partial sum is an exact integer, so the output must equal the oracle's bit for bit."""
-    M, N, K = 136, 264, 256
+    M, N = 136, 264
     p = _rand_problem(M, N, K, 0, dtype, seed=1)
     p["asc"] = torch.ones_like(p["asc"])
     p["wsc"] = torch.ones_like(p["wsc"])
@@ -76,7 +77,8 @@ def test_unit_scales_exact_integer_gemm(dev, unsigned, dtype):
 @pytest.mark.parametrize("unsigned", [False, True])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M,N,K,R,actual_m", [(136, 264, 256, 16, 130), (256, 256, 512, 32, 256), (64, 128, 1024, 48, 64), (128, 512, 256, 0, 100),
-                                                   (160, 256, 256, 160, 150), (72, 136, 512, 288, 72)])  # ranks grown at run time (32 + sum of LoRA ranks)
+                                                   (160, 256, 256, 160, 150), (72, 136, 512, 288, 72),  # ranks grown at run time (32 + sum of LoRA ranks)
+                                                   (136, 264, 64, 16, 136), (130, 200, 192, 32, 130), (256, 128, 448, 0, 200)])  # K / 64 odd
 def test_scaled_gemm_bias_lora(dev, M, N, K, R, actual_m, unsigned, dtype):
     print(f"case M={M} N={N} K={K} R={R} actual_m={actual_m} unsigned={unsigned} {dtype}", flush=True)
     p = _rand_problem(M, N, K, R, dtype, seed=K + R)
@@ -181,7 +183,8 @@ def test_weight_planes_layout(dev, N, K):
 
 
 @pytest.mark.parametrize("unsigned", [False, True])
-@pytest.mark.parametrize("M,N,K,R", [(136, 264, 256, 16), (256, 512, 1024, 32), (64, 72, 128, 0), (300, 3072, 3072, 32)])
+@pytest.mark.parametrize("M,N,K,R", [(136, 264, 256, 16), (256, 512, 1024, 32), (64, 72, 128, 0), (300, 3072, 3072, 32),
+                                     (100, 136, 64, 16), (257, 264, 320, 0)])  # the last two: K / 64 odd
 def test_presplit_weights_same_bits_as_packed(dev, M, N, K, R, unsigned):
     """The GEMM gives identical bits whether it unpacks the weights itself or reads the pre-split planes."""
     print(f"case M={M} N={N} K={K} R={R} unsigned={unsigned}", flush=True)
