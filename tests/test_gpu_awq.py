@@ -113,3 +113,19 @@ def test_gemm_and_gemv_fallback_decode_then_matmul(dev, m, group_size):
     assert O.max_rel_err(out2.cpu(), ref) <= 1e-2
     if group_size == 128:
         assert torch.equal(ops.gemm_awq(x.to(dev), kern, s.to(dev), z.to(dev)), out)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("N,K,group_size", [(256, 512, 128), (128, 256, 64)])
+def test_dequantize_inverts_the_packing(dev, dtype, N, K, group_size):
+    """Unit scales and zero zero-points: the decoder returns the packed codes exactly (the reference's own round-trip
+    test, tests/triton/test_gemm.py:98-110), from the int16 view of the packed tensor as well as the int32 one."""
+    from nunchaku_rocm_amd import ops
+
+    q = torch.randint(0, 16, (N, K), generator=torch.Generator().manual_seed(N), dtype=torch.int32)
+    packed = O.awq_pack(q).to(dev)
+    ones = torch.ones(K // group_size, N, dtype=dtype, device=dev)
+    out = ops.awq_dequantize(packed, ones, torch.zeros_like(ones), N, K, group_size, dtype)
+    assert torch.equal(out.float().cpu(), q.float())
+    out32 = ops.awq_dequantize(packed.view(torch.int32), ones, torch.zeros_like(ones), N, K, group_size, dtype)
+    assert torch.equal(out32, out)
