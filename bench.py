@@ -299,7 +299,7 @@ def main():
             "unit": "TFLOP/s",
             "frac": round(achieved / INT8_MFMA_PEAK_TOPS, 4),
             "traffic": GEMM_QKV_HBM_BYTES,
-            "traffic_unit": "bytes per launch (rocprofv3 FETCH_SIZE + WRITE_SIZE, see profiles/)",
+            "traffic_unit": "bytes per launch (rocprofv3 2.00 x FETCH_SIZE + 1.00 x WRITE_SIZE, the factors from copy kernels of known size; see profiles/)",
             "ops_per_launch": ops_per_gemm,
             "avg_launch_ms": round(gemm_ms, 5),
             "note": "int8 MFMA ops (2*M*N*K), peak = published dense int8 5.0 POP/s",
