@@ -151,3 +151,37 @@ def test_flux_shape_sampled_queries(dev):
     o2 = torch.empty_like(o)
     ops.attention_fp16(qd, kd, (vd * 2).contiguous(), o2, 128**-0.5)
     assert torch.equal(o2.float(), o.float() * 2)
+
+
+def test_full_size_invariants(dev):
+    """Properties that hold at any size, on the FLUX shape (24 heads, 4608 tokens, D = 128) entirely on the GPU:
+    doubling v doubles the output exactly; a permutation of the queries permutes the output rows bit for bit; a
+    permutation of the keys (with their values) changes only the order of the fp32 sums."""
+    from nunchaku_rocm_amd import ops
+
+    B, H, T, D = 1, 24, 4608, 128
+    g = torch.Generator(device=dev).manual_seed(21)
+    q = torch.randn(B, H, T, D, generator=g, device=dev).to(torch.bfloat16)
+    k = torch.randn(B, H, T, D, generator=g, device=dev).to(torch.bfloat16)
+    v = torch.randn(B, H, T, D, generator=g, device=dev).to(torch.bfloat16)
+    scale = D**-0.5
+
+    def run(q, k, v):
+        o = torch.empty(B, q.shape[2], H * D, dtype=q.dtype, device=dev)
+        ops.attention_fp16(q, k, v, o, scale)
+        return o
+
+    base = run(q, k, v)
+    assert bool(torch.isfinite(base.float()).all())
+    assert torch.equal(run(q, k, v * 2), base * 2)
+    pq = torch.randperm(T, generator=g, device=dev)
+    moved = run(q[:, :, pq].contiguous(), k, v)
+    err_q = float((moved.float() - base[:, pq].float()).abs().max()) / float(base.float().abs().max())
+    pk = torch.randperm(T, generator=g, device=dev)
+    shuffled = run(q, k[:, :, pk].contiguous(), v[:, :, pk].contiguous())
+    err_k = float((shuffled.float() - base.float()).abs().max()) / float(base.float().abs().max())
+    print(f"query permutation: max rel diff {err_q:.2e}; key permutation: {err_k:.2e}", flush=True)
+    assert err_q == 0.0 and err_k <= TOL  # query rows are computed independently of each other
+    # each output row is a convex combination of value rows
+    vmax = v.float().abs().amax(dim=2)  # (B, H, D)
+    assert bool((base.view(B, T, H, D).float().abs() <= vmax[:, None] * (1 + 2**-6)).all())

@@ -137,6 +137,46 @@ def test_flux_qkv_shapes_quantizer_then_gemm(dev, M):
         assert torch.equal(got, O.group_acc_i32(rp, lin["qweight"], False, groups=[g])[0])
 
 
+def test_full_size_invariants(dev):
+    """Properties that hold at any size, checked on the whole QKV problem (M=4608, K=3072, N=9216, R=32) on the GPU:
+    doubling the activation scales doubles every output exactly (a power of two commutes with every rounding); a
+    permutation of the activation rows permutes the output rows; a permutation of the weight rows permutes the output
+    columns -- bit for bit, whatever tile a row or column lands in."""
+    from nunchaku_rocm_amd import ops
+
+    M, K, N, R = 4608, 3072, 9216, 32
+    g = torch.Generator(device=dev).manual_seed(11)
+    act = torch.randint(0, 256, (M, K // 2), generator=g, dtype=torch.uint8, device=dev)
+    wgt = torch.randint(0, 256, (N, K // 2), generator=g, dtype=torch.uint8, device=dev)
+    asc = (torch.rand(K // 64, M, generator=g, device=dev) * 0.02 + 0.01).to(torch.bfloat16)
+    wsc = (torch.rand(K // 64, N, generator=g, device=dev) * 0.02 + 0.01).to(torch.bfloat16)
+    bias = torch.randn(N, generator=g, device=dev).to(torch.bfloat16)
+    la = torch.randn(M, R, generator=g, device=dev)
+    lu = (torch.randn(N, R, generator=g, device=dev) * 0.1).to(torch.bfloat16)
+
+    def run(act, wgt, asc, wsc, bias=None, la=None, lu=None):
+        out = torch.empty(act.shape[0], wgt.shape[0], dtype=torch.bfloat16, device=dev)
+        ops.svdq_gemm_w4a4_cuda(act=act, wgt=wgt, out=out, ascales=asc, wscales=wsc, bias=bias, lora_act_in=la, lora_up=lu)
+        return out
+
+    base = run(act, wgt, asc, wsc)
+    assert bool(torch.isfinite(base.float()).all()) and float(base.float().abs().max()) > 0
+    assert torch.equal(run(act, wgt, asc * 2, wsc), base * 2)
+    assert torch.equal(run(act, wgt, asc, wsc * 0.5), base * 0.5)
+
+    full = run(act, wgt, asc, wsc, bias, la, lu)
+    pm = torch.randperm(M, generator=g, device=dev)
+    assert torch.equal(run(act[pm].contiguous(), wgt, asc[:, pm].contiguous(), wsc, bias, la[pm].contiguous(), lu), full[pm])
+    pn = torch.randperm(N, generator=g, device=dev)
+    got = run(act, wgt[pn].contiguous(), asc, wsc[:, pn].contiguous(), bias[pn].contiguous(), la, lu[pn].contiguous())
+    assert torch.equal(got, full[:, pn])
+    # the low-rank branch and the bias are additive terms of the fp32 accumulator: against the plain output they
+    # account for the difference up to the final rounding
+    extra = (la.to(torch.bfloat16).float() @ lu.float().t()) + bias.float()
+    diff = (full.float() - base.float() - extra).abs()
+    assert float(diff.max()) <= 2**-7 * float(full.float().abs().max())
+
+
 def test_linear_module_matches_dequantised_reference(dev):
     """SVDQW4A4Linear.forward against the SVDQuant formula y = (x / smooth) .q W^T + (x . down) . up^T + bias."""
     from nunchaku_rocm_amd.linear import SVDQW4A4Linear

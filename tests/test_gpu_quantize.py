@@ -207,3 +207,25 @@ def test_gelu_prologue(dev, M, K, R, dtype):
         assert (la.cpu() - rl).abs().max() <= 1e-2 * rl.abs().max()
     with pytest.raises(NotImplementedError):
         quantize_w4a4_act_fuse_lora(torch.zeros(16, 128, dtype=dtype, device=dev), fuse_gelu=True, fuse_glu=True)
+
+
+def test_full_size_invariants(dev):
+    """On the whole (4608, 3072) input, on the GPU: multiplying the input by two leaves the codes alone and doubles the
+    scales and the LoRA hidden state exactly; permuting the rows permutes every output."""
+    from nunchaku_rocm_amd.ops.quantize import quantize_w4a4_act_fuse_lora
+
+    M, K, R = 4608, 3072, 32
+    lin = O.make_svdq_linear(K, 64, R=R, seed=3)
+    x = O.make_activations(M, K, seed=4).to(dev)
+    ld, sm = lin["proj_down"].to(dev), lin["smooth_factor"].to(dev)
+    q0, s0, l0 = quantize_w4a4_act_fuse_lora(x, lora_down=ld, smooth=sm)
+    q1, s1, l1 = quantize_w4a4_act_fuse_lora(x * 2, lora_down=ld, smooth=sm)
+    assert torch.equal(q0, q1) and torch.equal(s1, s0 * 2) and torch.equal(l1, l0 * 2)
+    pm = torch.randperm(M, generator=torch.Generator(device=dev).manual_seed(5), device=dev)
+    q2, s2, l2 = quantize_w4a4_act_fuse_lora(x[pm].contiguous(), lora_down=ld, smooth=sm)
+    assert torch.equal(q2, q0[pm]) and torch.equal(s2, s0[:, pm]) and torch.equal(l2, l0[pm])
+    # every group uses its full range: the largest code magnitude of a group with a non-zero scale is 7 (or -8 never
+    # without a 7-magnitude partner: |x| / (absmax / 7) <= 7)
+    codes = O.unpack_int4(q0.cpu(), True).view(M, K // 64, 64)
+    nz = s0.cpu().t().float() != 0
+    assert bool((codes.abs().amax(dim=2)[nz] == 7).all()) and int(codes.min()) >= -7
