@@ -3,6 +3,9 @@
 The kernels read a LoRA-down weight ``(K, R)`` transposed, ``(R, K)``, so that MFMA operands are K-contiguous.  The
 operator signatures take the natural layout (as the reference does), so the transposed copy is made on first use and
 kept for as long as the weight tensor lives and is not modified in place.
+
+A copy is made on the stream that is current at its first use.  A later use on another stream waits for the event
+recorded behind that launch (until it has completed once); the copy itself stays allocated while it is cached.
 """
 
 from __future__ import annotations
@@ -16,26 +19,46 @@ from .. import _lib
 _cache: dict[int, tuple] = {}
 
 
+class _Ready:
+    """Orders the first uses of a freshly made copy on other streams behind the launch that made it."""
+
+    __slots__ = ("stream", "event")
+
+    def __init__(self, device: torch.device):
+        cur = torch.cuda.current_stream(device)
+        self.stream = cur.cuda_stream
+        self.event = torch.cuda.Event()
+        self.event.record(cur)
+
+    def wait(self, device: torch.device) -> None:
+        if self.event is None:
+            return
+        if self.event.query():
+            self.event = None
+            return
+        cur = torch.cuda.current_stream(device)
+        if cur.cuda_stream != self.stream:
+            cur.wait_event(self.event)
+
+
 def lora_down_t(lora_down: torch.Tensor) -> torch.Tensor:
     key = id(lora_down)
     hit = _cache.get(key)
     if hit is not None:
-        ref, version, data_ptr, t = hit
+        ref, version, data_ptr, t, ready = hit
         if ref() is lora_down and version == lora_down._version and data_ptr == lora_down.data_ptr():
+            ready.wait(t.device)
             return t
     K, R = lora_down.shape
-    if lora_down.stride(1) != 1:
-        lora_down = lora_down.contiguous()
+    src = lora_down if lora_down.stride(1) == 1 else lora_down.contiguous()
     t = torch.empty(R, K, dtype=lora_down.dtype, device=lora_down.device)
     lib = _lib.load()
-    _lib.check(
-        lib.svdq_transpose_lora_down(
-            lora_down.data_ptr(), t.data_ptr(), K, R, lora_down.stride(0), _lib.stream_of(lora_down)
-        )
-    )
+    with torch.cuda.device(t.device):
+        _lib.check(lib.svdq_transpose_lora_down(src.data_ptr(), t.data_ptr(), K, R, src.stride(0), _lib.stream_of(src)))
+        ready = _Ready(t.device)
     try:
         ref = weakref.ref(lora_down, lambda _r, k=key: _cache.pop(k, None))
-        _cache[key] = (ref, lora_down._version, lora_down.data_ptr(), t)
+        _cache[key] = (ref, lora_down._version, lora_down.data_ptr(), t, ready)
     except TypeError:
         pass
     return t
@@ -51,16 +74,19 @@ def weight_planes(qweight: torch.Tensor) -> torch.Tensor:
     key = id(qweight)
     hit = _planes_cache.get(key)
     if hit is not None:
-        ref, version, data_ptr, t = hit
+        ref, version, data_ptr, t, ready = hit
         if ref() is qweight and version == qweight._version and data_ptr == qweight.data_ptr():
+            ready.wait(t.device)
             return t
     N, K = qweight.shape[0], qweight.shape[1] * 2
     lib = _lib.load()
     t = torch.empty(lib.svdq_weight_planes_bytes(N, K), dtype=torch.uint8, device=qweight.device)
-    _lib.check(lib.svdq_split_weight_planes(qweight.data_ptr(), t.data_ptr(), N, K, qweight.stride(0), _lib.stream_of(qweight)))
+    with torch.cuda.device(t.device):
+        _lib.check(lib.svdq_split_weight_planes(qweight.data_ptr(), t.data_ptr(), N, K, qweight.stride(0), _lib.stream_of(qweight)))
+        ready = _Ready(t.device)
     try:
         ref = weakref.ref(qweight, lambda _r, k=key: _planes_cache.pop(k, None))
-        _planes_cache[key] = (ref, qweight._version, qweight.data_ptr(), t)
+        _planes_cache[key] = (ref, qweight._version, qweight.data_ptr(), t, ready)
     except TypeError:
         pass
     return t

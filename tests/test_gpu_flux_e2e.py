@@ -89,3 +89,34 @@ def test_flux1_schnell_shape_four_steps(dev):
     cos = O.cosine(out, ref)
     print(f"FLUX.1-shaped 4-step latent cosine {cos:.6f}", flush=True)
     assert cos >= 0.999
+
+
+def test_relayout_made_on_one_stream_is_ordered_before_its_use_on_another(dev):
+    """The cached weight re-layouts are launched on the stream of their first use; a first use elsewhere right after
+    must wait for them (same bits as a run where everything happens on one stream)."""
+    from nunchaku_rocm_amd.linear import SVDQW4A4Linear
+
+    K, N, M = 3072, 3072, 512
+    lin = O.make_svdq_linear(K, N, seed=9)
+    x = O.make_activations(M, K, seed=10).view(1, M, K).to(dev)
+
+    def fresh():
+        mod = SVDQW4A4Linear(K, N, rank=32, device=dev)
+        with torch.no_grad():
+            for name in ("qweight", "wscales", "smooth_factor", "proj_down", "proj_up", "bias"):
+                getattr(mod, name).copy_(lin[name])
+        return mod
+
+    ref = fresh()(x)
+    torch.cuda.synchronize()
+    mod = fresh()
+    side = torch.cuda.Stream()
+    busy = torch.empty(64 << 20, device=dev)
+    torch.cuda.synchronize()
+    for _ in range(8):
+        busy.normal_()  # keeps the main stream busy, so the re-layouts queued behind it are still pending below
+    y_main = mod(x)  # first use: re-layouts and this call on the main stream
+    with torch.cuda.stream(side):
+        y_side = mod(x)  # cache hits on another stream
+    torch.cuda.synchronize()
+    assert torch.equal(y_main, ref) and torch.equal(y_side, ref)
