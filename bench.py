@@ -264,6 +264,17 @@ def main():
         model.denoise(lat, txt, pooled, rot, steps=4)
         torch.cuda.synchronize()
         kernels["flux1_schnell_shaped 19+38 blocks 4608 tokens"] = {"s_per_step": round((time.perf_counter() - t1) / 4, 4), "steps": 4}
+        if not args.eager:
+            # the same steps with each forward pass replayed from one recorded HIP graph (both streams' launches)
+            step_fn = model.capture(lat, txt, pooled, rot)
+            model.denoise(lat, txt, pooled, rot, steps=1, step_fn=step_fn)
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            model.denoise(lat, txt, pooled, rot, steps=4, step_fn=step_fn)
+            torch.cuda.synchronize()
+            kernels["flux1_schnell_shaped 19+38 blocks 4608 tokens, HIP graph"] = {
+                "s_per_step": round((time.perf_counter() - t1) / 4, 4), "steps": 4}  # fmt: skip
+            del step_fn
         del model
         # plain elementwise kernel of known size: the scale reference for the FETCH_SIZE / WRITE_SIZE counters
         # (random data, and a second buffer written in between so that the read comes from HBM, not from cache)

@@ -345,11 +345,43 @@ class FluxShapedTransformer(nn.Module):
         return self.proj_out(x)
 
     @torch.no_grad()
-    def denoise(self, latents, text, pooled, rot, steps: int = 4, backend=None):
-        """Euler steps of the rectified flow from t = 1 to t = 0 (FLUX.1-schnell runs 4)."""
+    def capture(self, latents, text, pooled, rot, backend=None):
+        """Record one forward pass (all of its launches on both streams) into a HIP graph.  Returns
+        ``step(latents, timestep) -> velocity``: it copies its arguments into the recorded input buffers, replays the
+        graph and returns the recorded output buffer (overwritten by the next call).  ``text``, ``pooled`` and ``rot``
+        are fixed at capture.  The ~1100 launches of a step then cost the host one call."""
+        dev = latents.device
+        s_lat, s_t = latents.clone(), torch.zeros(latents.shape[0], device=dev)
+        warm = torch.cuda.Stream(dev)
+        warm.wait_stream(torch.cuda.current_stream(dev))
+        with torch.cuda.stream(warm):  # first uses (weight re-layouts, library workspaces) happen outside the graph
+            for _ in range(2):
+                self.forward(s_lat, text, pooled, s_t, rot, backend=backend)
+        torch.cuda.current_stream(dev).wait_stream(warm)
+        torch.cuda.synchronize(dev)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            out = self.forward(s_lat, text, pooled, s_t, rot, backend=backend)
+
+        def step(lat, timestep):
+            s_lat.copy_(lat)
+            s_t.copy_(timestep)
+            graph.replay()
+            return out
+
+        step.graph = graph  # keeps the recording (and its memory pool) alive with the callable
+        return step
+
+    @torch.no_grad()
+    def denoise(self, latents, text, pooled, rot, steps: int = 4, backend=None, step_fn=None):
+        """Euler steps of the rectified flow from t = 1 to t = 0 (FLUX.1-schnell runs 4).  ``step_fn``: a callable from
+        :meth:`capture` to run the forward passes from a recorded HIP graph."""
         sig = torch.linspace(1.0, 0.0, steps + 1, device=latents.device)
         for i in range(steps):
             t = sig[i].expand(latents.shape[0])
-            v = self.forward(latents, text, pooled, t, rot, backend=backend)
+            if step_fn is not None:
+                v = step_fn(latents, t)
+            else:
+                v = self.forward(latents, text, pooled, t, rot, backend=backend)
             latents = (latents.float() + (sig[i + 1] - sig[i]) * v.float()).to(latents.dtype)
         return latents
