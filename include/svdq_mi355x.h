@@ -95,10 +95,12 @@ int svdq_row_stats(const void *x, float *stats, int32_t M, int32_t K, int32_t ld
  * nunchaku/models/transformers/transformer_flux_v2.py:233-234, :241-243 and :326-330, each step rounded to T), and,
  * when stats is not NULL, the (mean, rstd) row statistics of out for the next layer's norm prologue.  gate element
  * (b, k) is at b * gate_ld + k * gate_stride with b = m / rows_per_batch (rows_per_batch 0 = one vector).
+ * clip > 0: out is limited to [-clip, clip] before it is stored and before the statistics (the model's
+ * `hidden_states.clip(-65504, 65504)` of fp16 runs, transformer_flux_v2.py:255-256, :340-341); 0 = off.
  * K % 8 == 0, K <= 8192; x, y, y2, out rows 16-byte aligned with the row strides ld_* in elements; out may be x. */
 int svdq_gated_residual(const void *x, const void *gate, const void *y, const void *y2, void *out, float *stats,
                         int32_t M, int32_t K, int32_t ld_x, int32_t ld_y, int32_t ld_out, int32_t rows_per_batch,
-                        int32_t gate_ld, int32_t gate_stride, int32_t dtype, float eps, void *stream);
+                        int32_t gate_ld, int32_t gate_stride, int32_t dtype, float eps, float clip, void *stream);
 
 /* (K, R) row-major T  ->  (R, K) row-major T.  Done once per weight; the quantizer and the fused
  * requantizing epilogues read the transposed form so their MFMA operands are K-contiguous. */

@@ -119,7 +119,7 @@ def load() -> ctypes.CDLL:
     lib.svdq_weight_planes_bytes.restype = ctypes.c_size_t
     lib.svdq_weight_planes_bytes.argtypes = [_i32, _i32]
     lib.svdq_split_weight_planes.argtypes = [_vp, _vp, _i32, _i32, _i32, _vp]
-    lib.svdq_gated_residual.argtypes = [_vp] * 6 + [_i32] * 9 + [_f32, _vp]
+    lib.svdq_gated_residual.argtypes = [_vp] * 6 + [_i32] * 9 + [_f32, _f32, _vp]
     lib.svdq_row_stats.argtypes = [_vp, _vp, _i32, _i32, _i32, _i32, _f32, _vp]
     lib.svdq_quantize_act.argtypes = [ctypes.POINTER(QuantizeArgs), _vp]
     lib.svdq_gemm_w4a4.argtypes = [ctypes.POINTER(GemmArgs), _vp]

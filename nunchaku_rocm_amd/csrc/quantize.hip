@@ -367,7 +367,7 @@ template <typename T, bool SUM2, bool STATS>
 __global__ __launch_bounds__(256) void gated_residual_kernel(const uint16_t *x, const uint16_t *gate, const uint16_t *y,
                                                              const uint16_t *y2, uint16_t *out, float *stats, int M, int K,
                                                              long ld_x, long ld_y, long ld_out, int rows_per_batch,
-                                                             long gate_ld, int gate_stride, float eps) {
+                                                             long gate_ld, int gate_stride, float eps, float clip) {
     constexpr int MAXC = 16;  // 16-byte chunks per lane: K <= 64 * 8 * 16
     const int lane = threadIdx.x & 63, m = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (m >= M) return;
@@ -408,8 +408,12 @@ __global__ __launch_bounds__(256) void gated_residual_kernel(const uint16_t *x, 
                     t0 = rnd(t0 + T::lo_f32((uint32_t)zv[e]));
                     t1 = rnd(t1 + T::hi_f32((uint32_t)zv[e]));
                 }
-                const float o0 = rnd(T::lo_f32((uint32_t)xv[e]) + rnd(g[2 * e] * t0));
-                const float o1 = rnd(T::hi_f32((uint32_t)xv[e]) + rnd(g[2 * e + 1] * t1));
+                float o0 = rnd(T::lo_f32((uint32_t)xv[e]) + rnd(g[2 * e] * t0));
+                float o1 = rnd(T::hi_f32((uint32_t)xv[e]) + rnd(g[2 * e + 1] * t1));
+                if (clip > 0.0f) {  // x.clip(-clip, clip): infinities become the limit, NaN stays
+                    o0 = o0 > clip ? clip : (o0 < -clip ? -clip : o0);
+                    o1 = o1 > clip ? clip : (o1 < -clip ? -clip : o1);
+                }
                 s += o0 + o1;
                 res[c][e] = (int)pack2<T>(o0, o1);
             }
@@ -573,12 +577,12 @@ extern "C" int svdq_row_stats(const void *x, float *stats, int32_t M, int32_t K,
 template <typename T>
 static void launch_gated_residual(const void *x, const void *gate, const void *y, const void *y2, void *out, float *stats,
                                   int M, int K, long ld_x, long ld_y, long ld_out, int rpb, long gate_ld, int gate_stride,
-                                  float eps, hipStream_t s) {
+                                  float eps, float clip, hipStream_t s) {
     const dim3 grid((M + 3) / 4), block(256);
 #define SVDQ_GR(S2, ST)                                                                                                   \
     hipLaunchKernelGGL((gated_residual_kernel<T, S2, ST>), grid, block, 0, s, (const uint16_t *)x, (const uint16_t *)gate, \
                        (const uint16_t *)y, (const uint16_t *)y2, (uint16_t *)out, stats, M, K, ld_x, ld_y, ld_out, rpb,   \
-                       gate_ld, gate_stride, eps)
+                       gate_ld, gate_stride, eps, clip)
     if (y2 && stats)
         SVDQ_GR(true, true);
     else if (y2)
@@ -592,7 +596,7 @@ static void launch_gated_residual(const void *x, const void *gate, const void *y
 
 extern "C" int svdq_gated_residual(const void *x, const void *gate, const void *y, const void *y2, void *out, float *stats,
                                    int32_t M, int32_t K, int32_t ld_x, int32_t ld_y, int32_t ld_out, int32_t rows_per_batch,
-                                   int32_t gate_ld, int32_t gate_stride, int32_t dtype, float eps, void *stream) {
+                                   int32_t gate_ld, int32_t gate_stride, int32_t dtype, float eps, float clip, void *stream) {
     if (!x || !gate || !y || !out || M < 0 || K <= 0 || K % 8) {
         set_error("svdq_gated_residual: x, gate, y and out are required and K=%d must be a positive multiple of 8 (M=%d)", K, M);
         return SVDQ_E_INVALID;
@@ -611,11 +615,15 @@ extern "C" int svdq_gated_residual(const void *x, const void *gate, const void *
         set_error("svdq_gated_residual: dtype %d", dtype);
         return SVDQ_E_INVALID;
     }
+    if (!(clip >= 0.0f)) {
+        set_error("svdq_gated_residual: clip must be 0 (off) or a positive limit");
+        return SVDQ_E_INVALID;
+    }
     if (M == 0) return SVDQ_OK;
     if (dtype == SVDQ_BF16)
-        launch_gated_residual<BF16>(x, gate, y, y2, out, stats, M, K, ld_x, ld_y, ld_out, rows_per_batch, gate_ld, gate_stride, eps, (hipStream_t)stream);
+        launch_gated_residual<BF16>(x, gate, y, y2, out, stats, M, K, ld_x, ld_y, ld_out, rows_per_batch, gate_ld, gate_stride, eps, clip, (hipStream_t)stream);
     else
-        launch_gated_residual<FP16>(x, gate, y, y2, out, stats, M, K, ld_x, ld_y, ld_out, rows_per_batch, gate_ld, gate_stride, eps, (hipStream_t)stream);
+        launch_gated_residual<FP16>(x, gate, y, y2, out, stats, M, K, ld_x, ld_y, ld_out, rows_per_batch, gate_ld, gate_stride, eps, clip, (hipStream_t)stream);
     return check_launch("svdq_gated_residual");
 }
 

@@ -85,9 +85,9 @@ class HipBackend:
         return _ops.fused_qkv_norm_rottary(x, proj, norm_q, norm_k, rot, output=out, norm=mod)
 
     @staticmethod
-    def gated_residual(x, gate, y, y2=None, want_stats=False):
-        """``(x + gate[:, None] * (y [+ y2]), row statistics of the result or None)``"""
-        return _ops.gated_residual(x, gate, y, y2, want_stats=want_stats)
+    def gated_residual(x, gate, y, y2=None, want_stats=False, clip=0.0):
+        """``(x + gate[:, None] * (y [+ y2]), row statistics of the result or None)``; ``clip``: limit of the result"""
+        return _ops.gated_residual(x, gate, y, y2, want_stats=want_stats, clip=clip)
 
     @staticmethod
     def norm_stats(x):
@@ -101,6 +101,12 @@ class HipBackend:
     @staticmethod
     def attention(q, k, v):
         return _ops.scaled_dot_product_attention(q, k, v)
+
+
+def _fp16_clip(x: torch.Tensor) -> float:
+    """The reference limits fp16 hidden states to the finite range at the end of the text stream of a dual-stream block
+    and at the end of a single-stream block (nunchaku/models/transformers/transformer_flux_v2.py:255-256, :340-341)."""
+    return 65504.0 if x.dtype == torch.float16 else 0.0
 
 
 def rope_table(ids: torch.Tensor, axes_dim, theta: float) -> torch.Tensor:
@@ -236,7 +242,7 @@ class _DoubleBlock(nn.Module):
         side.wait_stream(main)
         with torch.cuda.stream(side):
             ctx, st = be.gated_residual(ctx, cg_a, be.linear(o[:, :t_txt], at.to_add_out), want_stats=True)
-            ctx, _ = be.gated_residual(ctx, cg_m, be.gelu_mlp(ctx, self.ffc_fc1, self.ffc_fc2, mod=(csc_m, csh_m, st)))
+            ctx, _ = be.gated_residual(ctx, cg_m, be.gelu_mlp(ctx, self.ffc_fc1, self.ffc_fc2, mod=(csc_m, csh_m, st)), clip=_fp16_clip(ctx))
         x, st = be.gated_residual(x, g_a, be.linear(o[:, t_txt:], at.to_out), want_stats=True)
         x, _ = be.gated_residual(x, g_m, be.gelu_mlp(x, self.ff_fc1, self.ff_fc2, mod=(sc_m, sh_m, st)))
         ctx.record_stream(main)  # read next on either stream
@@ -255,7 +261,7 @@ class _DoubleBlock(nn.Module):
         x, st = be.gated_residual(x, g_a, ax, want_stats=True)
         x, _ = be.gated_residual(x, g_m, be.gelu_mlp(x, self.ff_fc1, self.ff_fc2, mod=(sc_m, sh_m, st)))
         ctx, st = be.gated_residual(ctx, cg_a, ac, want_stats=True)
-        ctx, _ = be.gated_residual(ctx, cg_m, be.gelu_mlp(ctx, self.ffc_fc1, self.ffc_fc2, mod=(csc_m, csh_m, st)))
+        ctx, _ = be.gated_residual(ctx, cg_m, be.gelu_mlp(ctx, self.ffc_fc1, self.ffc_fc2, mod=(csc_m, csh_m, st)), clip=_fp16_clip(ctx))
         return ctx, x
 
 
@@ -290,7 +296,7 @@ class _SingleBlock(nn.Module):
             att = self.attn(be, x, None, rot, None, mod_x=mod)
             main.wait_stream(side)
             mlp.record_stream(main)
-        return be.gated_residual(x, gate, att, mlp, want_stats=True)
+        return be.gated_residual(x, gate, att, mlp, want_stats=True, clip=_fp16_clip(x))
 
 
 class FluxShapedTransformer(nn.Module):

@@ -17,12 +17,14 @@ def gated_residual(
     out: torch.Tensor | None = None,
     want_stats: bool = False,
     eps: float = 1e-6,
+    clip: float = 0.0,
 ) -> tuple[torch.Tensor, torch.Tensor | None]:
     """
     ``out = x + gate[:, None] * (y [+ y2])`` for ``x``, ``y`` of shape ``(B, S, C)`` and ``gate`` ``(B, C)`` (any element
     stride), every step rounded to the 16-bit dtype as the separate torch kernels would.  With ``want_stats`` also
     returns the ``(B * S, 2)`` float32 row statistics ``(mean, 1 / sqrt(var + eps))`` of ``out``, ready for the ``norm=``
-    prologue of the next quantizer.  Returns ``(out, stats)``.
+    prologue of the next quantizer.  ``clip > 0`` limits ``out`` to ``[-clip, clip]`` first (the reference model's
+    ``clip(-65504, 65504)`` of fp16 runs).  Returns ``(out, stats)``.
     """
     _lib.require_cuda(x, gate, y, y2, out)
     B, S, C = x.shape
@@ -49,5 +51,5 @@ def gated_residual(
         _lib.check(_lib.load().svdq_gated_residual(
             x2.data_ptr(), gate.data_ptr(), ya.data_ptr(), _lib.ptr(yb), o2.data_ptr(), _lib.ptr(stats), B * S, C,
             x2.stride(0), ya.stride(0), o2.stride(0), S if B > 1 else 0, gate.stride(0), gate.stride(1),
-            _lib.dtype_code(x.dtype), float(eps), _lib.stream_of(x)))  # fmt: skip
+            _lib.dtype_code(x.dtype), float(eps), float(clip), _lib.stream_of(x)))  # fmt: skip
     return out, stats

@@ -33,8 +33,8 @@ class OracleBackend:
         return None
 
     @staticmethod
-    def gated_residual(x, gate, y, y2=None, want_stats=False):
-        return O.gated_residual(x, gate, y, y2), None
+    def gated_residual(x, gate, y, y2=None, want_stats=False, clip=0.0):
+        return O.gated_residual(x, gate, y, y2, clip), None
 
     def gelu_mlp(self, x, fc1, fc2, mod=None):
         B, S, C = x.shape

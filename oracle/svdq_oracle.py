@@ -346,14 +346,16 @@ def layernorm_modulate(x: torch.Tensor, scale: torch.Tensor, shift: torch.Tensor
     return (y.float() + sh.float()).to(dt)
 
 
-def gated_residual(x: torch.Tensor, gate: torch.Tensor, y: torch.Tensor, y2: torch.Tensor | None = None) -> torch.Tensor:
+def gated_residual(x: torch.Tensor, gate: torch.Tensor, y: torch.Tensor, y2: torch.Tensor | None = None,
+                   clip: float = 0.0) -> torch.Tensor:  # fmt: skip
     """nunchaku/models/transformers/transformer_flux_v2.py:233-234, :241-243 (``x + gate.unsqueeze(1) * y``) and
     :326-330 (``x + gate.unsqueeze(1) * (y + y2)``) as 16-bit elementwise steps: every +, * rounded to the dtype.
-    x, y (B, S, C); gate (B, C)."""
+    x, y (B, S, C); gate (B, C).  ``clip``: the ``.clip(-65504, 65504)`` that follows in fp16 runs (:255-256, :340-341)."""
     dt = x.dtype
     t = y if y2 is None else (y.float() + y2.float()).to(dt)
     g = (gate.float()[:, None, :] * t.float()).to(dt)
-    return (x.float() + g.float()).to(dt)
+    out = (x.float() + g.float()).to(dt)
+    return out.clip(-clip, clip) if clip > 0 else out
 
 
 # --------------------------------------------------------------------------------------

@@ -56,3 +56,34 @@ def test_rejects_bad_arguments(dev):
         ops.gated_residual(x, torch.zeros(1, 16384, dtype=torch.bfloat16, device=dev), x)
     with pytest.raises(ValueError):
         ops.gated_residual(x, torch.zeros(2, 16384, dtype=torch.bfloat16, device=dev), x)
+
+
+@pytest.mark.parametrize("two", [False, True])
+def test_fp16_clip_like_the_model(dev, two):
+    """fp16 hidden states that overflow are limited to +-65504 as ``.clip(-65504, 65504)`` does in the reference model
+    (infinities become the limit, NaN stays), and the statistics are those of the limited values."""
+    from nunchaku_rocm_amd import ops
+
+    g = torch.Generator().manual_seed(4)
+    B, S, C = 1, 40, 256
+    x = (torch.randn(B, S, C, generator=g) * 3e4).to(torch.float16)
+    y = (torch.randn(B, S, C, generator=g) * 3e4).to(torch.float16)
+    y2 = (torch.randn(B, S, C, generator=g) * 3e4).to(torch.float16)
+    gate = (torch.randn(B, C, generator=g) * 2).to(torch.float16)
+    x[0, 3, 5] = float("nan")
+    free, _ = ops.gated_residual(x.to(dev), gate.to(dev), y.to(dev), y2.to(dev) if two else None)
+    assert bool(torch.isinf(free).any())  # the case does overflow
+    out, stats = ops.gated_residual(x.to(dev), gate.to(dev), y.to(dev), y2.to(dev) if two else None, want_stats=True, clip=65504.0)
+    torch.cuda.synchronize()
+    ref = O.gated_residual(x, gate, y, y2 if two else None, clip=65504.0)
+    plain = O.gated_residual(x, gate, y, y2 if two else None).clip(-65504, 65504)
+    assert torch.equal(ref.nan_to_num(0.0), plain.nan_to_num(0.0))
+    got = out.cpu()
+    assert bool(torch.isnan(got[0, 3, 5])) and bool(torch.isnan(ref[0, 3, 5]))
+    assert torch.equal(got.isnan(), ref.isnan())  # inf - inf where x itself overflowed, and the planted NaN
+    assert torch.equal(got.nan_to_num(0.0).view(torch.int16), ref.nan_to_num(0.0).view(torch.int16))
+    assert float(got.nan_to_num(0.0).float().abs().max()) == 65504.0
+    rows = [r for r in range(S) if not bool(ref[0, r].isnan().any())]
+    assert rows
+    r64 = ref.double().reshape(S, C)[rows]
+    assert ((stats[rows, 0].cpu().double() - r64.mean(dim=1)).abs() <= 1e-5 * r64.abs().amax(dim=1)).all()
