@@ -17,23 +17,24 @@ from oracle.flux_backend import OracleBackend
 pytestmark = pytest.mark.gpu
 
 
-def _inputs(cfg, t_txt, gh, gw, dev, seed=7):
+def _inputs(cfg, t_txt, gh, gw, dev, seed=7, dtype=torch.bfloat16):
     from nunchaku_rocm_amd.flux_shaped import flux_ids, rope_table
 
     g = torch.Generator().manual_seed(seed)
-    lat = torch.randn(1, gh * gw, cfg.in_channels, generator=g).to(torch.bfloat16).to(dev)
-    txt = torch.randn(1, t_txt, cfg.text_dim, generator=g).to(torch.bfloat16).to(dev)
-    pooled = torch.randn(1, cfg.pooled_dim, generator=g).to(torch.bfloat16).to(dev)
+    lat = torch.randn(1, gh * gw, cfg.in_channels, generator=g).to(dtype).to(dev)
+    txt = torch.randn(1, t_txt, cfg.text_dim, generator=g).to(dtype).to(dev)
+    pooled = torch.randn(1, cfg.pooled_dim, generator=g).to(dtype).to(dev)
     rot = rope_table(flux_ids(t_txt, gh, gw, device=dev), cfg.axes_dim, cfg.theta)
     return lat, txt, pooled, rot
 
 
-def test_small_config_against_cpu_oracle(dev):
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_small_config_against_cpu_oracle(dev, dtype):
     from nunchaku_rocm_amd.flux_shaped import FluxShapedConfig, FluxShapedTransformer
 
     cfg = FluxShapedConfig(hidden=512, heads=4, mlp=2048, text_dim=256, pooled_dim=64, n_double=2, n_single=3)
-    model = FluxShapedTransformer(cfg, device=dev, seed=3)
-    lat, txt, pooled, rot = _inputs(cfg, 32, 16, 16, dev)
+    model = FluxShapedTransformer(cfg, device=dev, dtype=dtype, seed=3)
+    lat, txt, pooled, rot = _inputs(cfg, 32, 16, 16, dev, dtype=dtype)
     out = model.denoise(lat, txt, pooled, rot, steps=4).cpu()
     cpu_model = copy.deepcopy(model).to("cpu")
     ref = cpu_model.denoise(lat.cpu(), txt.cpu(), pooled.cpu(), rot.cpu(), steps=4, backend=OracleBackend())
