@@ -401,7 +401,9 @@ __global__ __launch_bounds__(NTHREADS, 4) void gemm_w4a4_kernel(svdq_gemm_args a
         for (int pass = 0; pass < BM * 16 / NTHREADS; pass++) {
             const int row = pass * (NTHREADS / 16) + (tid >> 4), m = m0 + row;
             if (m < a.actual_m && n < a.N)
-                *(v4i *)(out + (size_t)m * a.ld_out + n) = *(const v4i *)(smem + row * PITCH + c * 16);
+                // streamed: the 85 MB of a QKV output do not fit any cache level of the CU, and lines left dirty in L2 have
+                // to be written back before the next kernel on the stream starts (measured: 1 % of the launch)
+                __builtin_nontemporal_store(*(const v4i *)(smem + row * PITCH + c * 16), (v4i *)(out + (size_t)m * a.ld_out + n));
         }
     };
 
