@@ -25,8 +25,11 @@
 //    free by construction; one raw s_barrier per stage with explicit s_waitcnt.  The four wavefronts of a SIMD issue
 //    their block loads at four different points of the stage (a wavefront blocks at issue while the memory pipe is
 //    full; the others keep computing).
+//  * The epilogue's operands (bias, the first 32 ranks of lora_up and lora_act of the tile: 24.25 KB) are fetched into
+//    LDS together with stage 0, in MFMA lane order, so that the LoRA-up section does not wait for memory; with them
+//    a workgroup holds 78.25 KB of LDS, two workgroups still share a CU's 160 KB.
 //  * The 16-bit output tile leaves through LDS as 256-byte row segments (a lane's own accumulators are 8-byte pieces
-//    of 32 different rows, which the memory pipe takes one lane per cycle).
+//    of 32 different rows, which the memory pipe takes one lane per cycle), stored non-temporally.
 //  * Weights can be given pre-split (svdq_split_weight_planes: int8 even / odd planes stored block by block in MFMA
 //    lane order); their half of the unpack then disappears from the inner loop.
 //  * Workgroup ids are first regrouped so that each XCD (ids are dealt round-robin over 8 XCDs) works on a
@@ -49,6 +52,10 @@ constexpr int NM_OFF = AS_OFF + 2 * BM * 4;               // float -magic*as'[2]
 constexpr int WS_OFF = NM_OFF + 2 * BM * 4;               // float ws[2][BN]
 constexpr int BUF_BYTES = WS_OFF + 2 * BN * 4;            // 27648
 constexpr int SMEM_BYTES = NSTAGE * BUF_BYTES;            // 55296
+// the first 32 ranks of the tile's LoRA operands, fetched next to stage 0: lora_up [2 c][4 blocks] and lora_act
+// [2 c][4 blocks][2 halves of 8 floats] 1 KB blocks in MFMA lane order
+constexpr int LORA_BYTES = (8 + 16) * BLK_BYTES;          // 24576
+constexpr int BIAS_BYTES = BN * 2;                        // the tile's 128 bias values
 constexpr int NWAVES = 8, NTHREADS = NWAVES * 64;  // 2 wavefronts along n x 4 along m
 constexpr int NBM = 1, WROWS = NBM * 32;            // activation rows per wavefront (its 64 weight rows are 2 blocks)
 constexpr int GROUP_M_TILES = 8;      // m-tiles per raster band
@@ -90,7 +97,7 @@ __device__ inline void tile_ids(int tiles_m, int tiles_n, int &pid_m, int &pid_n
 
 template <typename T, bool ACT_UNSIGNED, int EPI, bool WPL, bool ODDG>  // ODDG: K / 64 is odd
 __global__ __launch_bounds__(NTHREADS, 4) void gemm_w4a4_kernel(svdq_gemm_args a) {
-    __shared__ __align__(16) uint8_t smem[SMEM_BYTES];
+    __shared__ __align__(16) uint8_t smem[SMEM_BYTES + LORA_BYTES + BIAS_BYTES];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -221,6 +228,30 @@ __global__ __launch_bounds__(NTHREADS, 4) void gemm_w4a4_kernel(svdq_gemm_args a
 
     load_scales(0);
     dma_stage(0);
+    // epilogue operands, fetched now so that the epilogue does not wait for memory
+    if (a.bias != nullptr && wave == 7) {  // 64 lanes x 4 bytes = the tile's 128 bias values
+        const uint8_t *src = (const uint8_t *)a.bias + (size_t)min(n0 + 2 * lane, a.N - 2) * 2;
+        __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)src, (SVDQ_AS3 void *)(smem + SMEM_BYTES + LORA_BYTES), 4, 0, 0);
+    }
+    if (a.R > 0) {
+#pragma unroll
+        for (int i = 0; i < 3; i++) {
+            const int q = wave * 3 + i;  // wave-uniform
+            const uint8_t *src;
+            bool on = true;
+            if (q < 8) {
+                const int c = q >> 2, blk = q & 3;
+                on = 16 * c < a.R;
+                src = (const uint8_t *)a.lora_up + ((size_t)min(n0 + blk * 32 + l32, a.N - 1) * a.ld_lora_up + 16 * c + 8 * half) * 2;
+            } else {
+                const int j = q - 8, c = j >> 3, blk = (j >> 1) & 3, part = j & 1;
+                on = 16 * c < a.R;
+                src = (const uint8_t *)a.lora_act + ((size_t)min(m0 + blk * 32 + l32, a.M - 1) * a.ld_lora_act + 16 * c + 8 * half + 4 * part) * 4;
+            }
+            if (on)
+                __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)src, (SVDQ_AS3 void *)(smem + SMEM_BYTES + q * BLK_BYTES), 16, 0, 0);
+        }
+    }
     // One copy of the loop per position (0..3) at which the wavefront issues its loads within a stage: the four
     // wavefronts that share a SIMD take different positions, so that one of them at a time waits for room in the
     // memory pipeline while the others compute.  (A run-time test of the position inside one loop costs registers.)
@@ -295,23 +326,22 @@ __global__ __launch_bounds__(NTHREADS, 4) void gemm_w4a4_kernel(svdq_gemm_args a
         default: main_loop(std::integral_constant<int, 3>{}); break;
     }
     // The last stage's (redundant) block loads of this wavefront have landed.  No barrier here: the LoRA-up / bias section
-    // does not touch LDS, and every epilogue starts its first use of the staging memory with a barrier of its own.
+    // only reads the LDS blocks that arrived before the first stage's barrier, and every epilogue starts its first use
+    // of the staging memory with a barrier of its own.
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
 
     // ---- epilogue: LoRA-up and bias ----------------------------------------------------------------
     const int nw0 = n0 + wn * 64, mw0 = m0 + wm * WROWS;
-    // All global loads of this section (bias, then 32 ranks of both LoRA operands at a time) are issued before their
-    // first use: the section costs one memory latency per 32 ranks rather than one per load group.
+    // The bias and the first 32 ranks of both LoRA operands were fetched into LDS next to stage 0 and arrived long ago;
+    // ranks beyond 32 come from global memory, all loads of a 32-rank pass issued before their first use.  Rows past
+    // N / M hold copies of the last row: they only reach outputs that are never stored.
     uint2 bb[2][4];
     if (a.bias != nullptr) {
-        const uint16_t *bias = (const uint16_t *)a.bias;
 #pragma unroll
         for (int bn = 0; bn < 2; bn++)
 #pragma unroll
             for (int j = 0; j < 4; j++) {
-                const int n = nw0 + bn * 32 + 8 * j + 4 * half;
-                bb[bn][j] = make_uint2(0u, 0u);
-                if (n < a.N) bb[bn][j] = *(const uint2 *)(bias + n);
+                bb[bn][j] = *(const uint2 *)(smem + SMEM_BYTES + LORA_BYTES + (wn * 64 + bn * 32 + 8 * j + 4 * half) * 2);
             }
     }
     if (a.R > 0) {
@@ -327,13 +357,20 @@ __global__ __launch_bounds__(NTHREADS, 4) void gemm_w4a4_kernel(svdq_gemm_args a
                 for (int blk = 0; blk < 2; blk++) {
                     const int n = nw0 + blk * 32 + l32;
                     ua[c][blk] = (v4i){0, 0, 0, 0};
-                    if (n < a.N) ua[c][blk] = *(const v4i *)(lu + (size_t)n * a.ld_lora_up + r0 + 16 * c + half * 8);
+                    if (r0 == 0)
+                        ua[c][blk] = *(const v4i *)(smem + SMEM_BYTES + (c * 4 + wn * 2 + blk) * BLK_BYTES + lane * 16);
+                    else if (n < a.N)
+                        ua[c][blk] = *(const v4i *)(lu + (size_t)n * a.ld_lora_up + r0 + 16 * c + half * 8);
                 }
 #pragma unroll
                 for (int blk = 0; blk < NBM; blk++) {
                     const int m = mw0 + blk * 32 + l32;
                     uf[c][blk][0] = uf[c][blk][1] = (v4f){0.f, 0.f, 0.f, 0.f};
-                    if (m < a.M) {
+                    if (r0 == 0) {
+                        const uint8_t *lp = smem + SMEM_BYTES + 8 * BLK_BYTES + ((c * 4 + wm * NBM + blk) * 2) * BLK_BYTES + lane * 16;
+                        uf[c][blk][0] = *(const v4f *)lp;
+                        uf[c][blk][1] = *(const v4f *)(lp + BLK_BYTES);
+                    } else if (m < a.M) {
                         const float *lp = a.lora_act + (size_t)m * a.ld_lora_act + r0 + 16 * c + half * 8;
                         uf[c][blk][0] = *(const v4f *)lp;
                         uf[c][blk][1] = *(const v4f *)(lp + 4);
