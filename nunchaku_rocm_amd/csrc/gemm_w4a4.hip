@@ -498,8 +498,27 @@ __global__ __launch_bounds__(NTHREADS, 4) void gemm_w4a4_kernel(svdq_gemm_args a
     }
 
     if (EPI == SVDQ_EPI_GELU_QUANT) {
-        if (a.out != nullptr) store_out();  // pre-GELU output, when asked for
         const uint16_t *ldt = (const uint16_t *)a.lora_down_t;
+        // loads whose values are needed further down, issued before the GELU arithmetic: the next layer's smoothing
+        // factor of this thread's column and the first 32 ranks of its LoRA-down weight
+        uint16_t smv = 0;
+        const bool has_sm = a.smooth_next != nullptr && tid < BN && n0 + tid < a.N;
+        if (has_sm) smv = ((const uint16_t *)a.smooth_next)[n0 + tid];
+        uint2 lq[2][2][2];
+        if (a.R2 > 0) {
+#pragma unroll
+            for (int bn = 0; bn < 2; bn++)
+#pragma unroll
+                for (int s = 0; s < 2; s++) {
+                    lq[bn][s][0] = lq[bn][s][1] = make_uint2(0u, 0u);
+                    if (l32 < a.R2) {
+                        const uint16_t *lp = ldt + (size_t)l32 * a.N + nw0 + bn * 32 + 16 * s + 4 * half;
+                        lq[bn][s][0] = *(const uint2 *)lp;
+                        lq[bn][s][1] = *(const uint2 *)(lp + 8);
+                    }
+                }
+        }
+        if (a.out != nullptr) store_out();  // pre-GELU output, when asked for
         float *lds_part = (float *)smem;  // [4 (wm)][16 regs][64 lanes] floats = 16 KB
         __syncthreads();
 #pragma unroll
@@ -523,7 +542,9 @@ __global__ __launch_bounds__(NTHREADS, 4) void gemm_w4a4_kernel(svdq_gemm_args a
 #pragma unroll
                 for (int s = 0; s < 2; s++) {
                     v4i la = (v4i){0, 0, 0, 0};
-                    if (r < a.R2) {
+                    if (rc == 0) {
+                        la = (v4i){(int)lq[bn][s][0].x, (int)lq[bn][s][0].y, (int)lq[bn][s][1].x, (int)lq[bn][s][1].y};
+                    } else if (r < a.R2) {
                         const uint16_t *lp = ldt + (size_t)r * a.N + nw0 + bn * 32 + 16 * s + 4 * half;
                         const uint2 q0 = *(const uint2 *)lp, q1 = *(const uint2 *)(lp + 8);
                         la = (v4i){(int)q0.x, (int)q0.y, (int)q1.x, (int)q1.y};
@@ -566,12 +587,7 @@ __global__ __launch_bounds__(NTHREADS, 4) void gemm_w4a4_kernel(svdq_gemm_args a
 
         // +shift, * 1/smooth, unsigned per-64 quantization: the wavefront's 64 columns are one group
         float *lds_rs = (float *)smem;  // [BN]
-        if (tid < BN) {
-            float rs = 1.0f;
-            if (a.smooth_next != nullptr && n0 + tid < a.N)
-                rs = 1.0f / T::to_f32(((const uint16_t *)a.smooth_next)[n0 + tid]);
-            lds_rs[tid] = rs;
-        }
+        if (tid < BN) lds_rs[tid] = has_sm ? 1.0f / T::to_f32(smv) : 1.0f;
         __syncthreads();
         const int g = nw0 / GROUP;
 #pragma unroll
