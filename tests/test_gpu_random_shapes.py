@@ -92,3 +92,91 @@ def test_attention_random_shapes(dev):
         ref = O.attention_fp16(q, k, v, D**-0.5)
         assert bool(torch.isfinite(o.float()).all())
         assert O.max_rel_err(o.cpu(), ref) <= 1e-2
+
+
+def test_epilogue_random_shapes(dev):
+    from nunchaku_rocm_amd import ops
+
+    rnd = random.Random(77)
+    for case in range(16):
+        M = 16 * rnd.randint(1, 18)
+        N = 128 * rnd.randint(1, 4)
+        K = 64 * rnd.randint(1, 6)
+        R, R2 = rnd.choice([0, 16, 32]), rnd.choice([0, 16, 32, 48])
+        smooth_on, store_out = rnd.random() < 0.7, rnd.random() < 0.5
+        dtype = rnd.choice([torch.bfloat16, torch.float16])
+        print(f"case {case}: gelu M={M} N={N} K={K} R={R} R2={R2} smooth={smooth_on} out={store_out} {dtype}", flush=True)
+        g = torch.Generator().manual_seed(1000 + case)
+        act = torch.randint(0, 256, (M, K // 2), generator=g, dtype=torch.uint8)
+        wgt = torch.randint(0, 256, (N, K // 2), generator=g, dtype=torch.uint8)
+        asc = (torch.rand(K // 64, M, generator=g) * 0.02 + 0.01).to(dtype)
+        wsc = (torch.rand(K // 64, N, generator=g) * 0.02 + 0.01).to(dtype)
+        b = torch.randn(N, generator=g).to(dtype)
+        la = torch.randn(M, R, generator=g) if R else None
+        lu = (torch.randn(N, R, generator=g) * 0.1).to(dtype) if R else None
+        sm = (torch.rand(N, generator=g) + 0.5).to(dtype) if smooth_on else None
+        ld = (torch.randn(N, R2, generator=g) * 0.1).to(dtype) if R2 else None
+        d = lambda t: None if t is None else t.to(dev)  # noqa: E731
+        qout = torch.zeros(M + 16, N // 2, dtype=torch.uint8, device=dev)
+        osc = torch.empty(N // 64, M, dtype=dtype, device=dev)
+        lao = torch.empty(M, R2, dtype=torch.float32, device=dev) if R2 else None
+        out = torch.empty(M, N, dtype=dtype, device=dev) if store_out else None
+        ops.svdq_gemm_w4a4_cuda(act=d(act), wgt=d(wgt), out=out, qout=qout, ascales=d(asc), wscales=d(wsc), oscales=osc,
+                                lora_act_in=d(la), lora_up=d(lu), lora_down=d(ld), lora_act_out=lao, bias=d(b),
+                                smooth_factor=d(sm))  # fmt: skip
+        torch.cuda.synchronize()
+        assert (qout[M:] == 0).all()
+        lin = O.gemm_w4a4(act, wgt, asc, wsc, b, la, lu, False)
+        rp, rs, rl, rc = O.gelu_quant(lin, sm, ld, dtype)
+        diff = (O.unpack_int4(qout[:M].cpu(), False) - rc).abs()
+        assert diff.max() <= 1 and (diff > 0).float().mean() < 2e-3
+        ulp = 2**-7 if dtype == torch.bfloat16 else 2**-10
+        assert ((osc.cpu().float() - rs.float()).abs() <= rs.float().abs() * ulp + 1e-7).all()
+        if R2:
+            assert (lao.cpu() - rl).abs().max() <= 1e-2 * rl.abs().max()
+        if store_out:
+            assert O.max_rel_err(out.cpu(), lin) <= 1e-2
+
+    for case in range(10):
+        H = rnd.randint(1, 3)
+        M = rnd.choice([8, 64, 100, 136, 256, 300])
+        am = rnd.randint(1, M)
+        K, N = 64 * rnd.randint(1, 5), 3 * H * 128
+        dtype = rnd.choice([torch.bfloat16, torch.float16])
+        print(f"case {case}: rope M={M} H={H} K={K} actual_m={am} {dtype}", flush=True)
+        g = torch.Generator().manual_seed(2000 + case)
+        act = torch.randint(0, 256, (M, K // 2), generator=g, dtype=torch.uint8)
+        wgt = torch.randint(0, 256, (N, K // 2), generator=g, dtype=torch.uint8)
+        asc = (torch.rand(K // 64, M, generator=g) * 0.02 + 0.01).to(dtype)
+        wsc = (torch.rand(K // 64, N, generator=g) * 0.02 + 0.01).to(dtype)
+        b = torch.randn(N, generator=g).to(dtype)
+        nq = (torch.rand(128, generator=g) + 0.5).to(dtype)
+        nk = (torch.rand(128, generator=g) + 0.5).to(dtype)
+        theta = torch.rand(am, 64, generator=g) * 6.28
+        rot = torch.stack([torch.sin(theta), torch.cos(theta)], -1).reshape(am, 64, 1, 2).float()
+        d = lambda t: t.to(dev)  # noqa: E731
+        buf = torch.full((am + 2, N), float("nan"), dtype=dtype, device=dev)
+        ops.svdq_gemm_w4a4_cuda(act=d(act), wgt=d(wgt), out=buf[:am], ascales=d(asc), wscales=d(wsc), bias=d(b),
+                                norm_q=d(nq), norm_k=d(nk), rotary_emb=d(rot))  # fmt: skip
+        torch.cuda.synchronize()
+        assert bool(buf[am:].isnan().all())
+        lin = O.gemm_w4a4(act, wgt, asc, wsc, b)[:am]
+        ref = O.qk_norm_rope(lin, nq, nk, rot.reshape(am, 128))
+        assert O.max_rel_err(buf[:am].cpu(), ref) <= 1e-2
+
+
+def test_awq_random_shapes(dev):
+    from nunchaku_rocm_amd import ops
+
+    rnd = random.Random(5)
+    for case in range(16):
+        m = rnd.choice([1, 2, 3, 8, 9, 17, 32, 33, 40])
+        N, K = 32 * rnd.randint(1, 12), 64 * rnd.randint(1, 10)
+        dtype = rnd.choice([torch.bfloat16, torch.float16])
+        print(f"case {case}: m={m} N={N} K={K} {dtype}", flush=True)
+        lin = O.make_awq_linear(K, N, seed=case, dtype=dtype)
+        x = torch.randn(m, K, generator=torch.Generator().manual_seed(300 + case)).to(dtype)
+        out = ops.awq_gemv_w4a16_cuda(x.to(dev), lin["qweight"].to(dev), lin["wscales"].to(dev), lin["wzeros"].to(dev), m, N, K)
+        torch.cuda.synchronize()
+        ref = O.awq_gemv(x, lin["qweight"].view(torch.int16).reshape(N // 4, K), lin["wscales"], lin["wzeros"])
+        assert O.max_rel_err(out.cpu(), ref) <= 1e-2
