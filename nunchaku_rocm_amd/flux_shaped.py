@@ -341,6 +341,8 @@ class FluxShapedTransformer(nn.Module):
         rot_txt, rot_img = rot[:t_txt].contiguous(), rot[t_txt:].contiguous()
         for blk in self.double_blocks:
             ctx, x = blk(be, x, ctx, temb, rot_img, rot_txt)
+        if hasattr(be, "join"):
+            be.join(x.device)  # the last block's text stream was produced on the side stream
         x = torch.cat([ctx, x], dim=1)
         stats = None
         for blk in self.single_blocks:
