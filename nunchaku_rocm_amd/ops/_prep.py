@@ -2,7 +2,12 @@
 
 The kernels read a LoRA-down weight ``(K, R)`` transposed, ``(R, K)``, so that MFMA operands are K-contiguous.  The
 operator signatures take the natural layout (as the reference does), so the transposed copy is made on first use and
-kept for as long as the weight tensor lives and is not modified in place.
+kept for as long as the weight tensor lives, is not modified in place and keeps its storage.
+
+A cache entry holds a reference to the storage it was made from.  Assigning ``param.data = other`` changes neither the
+parameter object nor its version counter, and without that reference the allocator could hand the freed block to the
+next tensor of the same size, which would then look like the cached source; with it, an equal storage address means
+the same storage.
 
 A copy is made on the stream that is current at its first use.  A later use on another stream waits for the event
 recorded behind that launch (until it has completed once); the copy itself stays allocated while it is cached.
@@ -41,12 +46,29 @@ class _Ready:
             cur.wait_event(self.event)
 
 
+def _source_of(t: torch.Tensor) -> tuple:
+    """What identifies the bytes a copy was derived from: version counter, the storage (kept alive) and the view."""
+    return (t._version, t.untyped_storage(), t.storage_offset(), tuple(t.shape), tuple(t.stride()))
+
+
+def _same_source(src: tuple, t: torch.Tensor) -> bool:
+    version, storage, offset, shape, stride = src
+    return (version == t._version and storage.data_ptr() == t.untyped_storage().data_ptr() and offset == t.storage_offset()
+            and shape == tuple(t.shape) and stride == tuple(t.stride()))  # fmt: skip
+
+
+def invalidate(t: torch.Tensor) -> None:
+    """Drop the derived copies of ``t`` (for callers that rewrite a weight through a path the version counter misses)."""
+    _cache.pop(id(t), None)
+    _planes_cache.pop(id(t), None)
+
+
 def lora_down_t(lora_down: torch.Tensor) -> torch.Tensor:
     key = id(lora_down)
     hit = _cache.get(key)
     if hit is not None:
-        ref, version, data_ptr, t, ready = hit
-        if ref() is lora_down and version == lora_down._version and data_ptr == lora_down.data_ptr():
+        ref, src, t, ready = hit
+        if ref() is lora_down and _same_source(src, lora_down):
             ready.wait(t.device)
             return t
     K, R = lora_down.shape
@@ -58,7 +80,7 @@ def lora_down_t(lora_down: torch.Tensor) -> torch.Tensor:
         ready = _Ready(t.device)
     try:
         ref = weakref.ref(lora_down, lambda _r, k=key: _cache.pop(k, None))
-        _cache[key] = (ref, lora_down._version, lora_down.data_ptr(), t, ready)
+        _cache[key] = (ref, _source_of(lora_down), t, ready)
     except TypeError:
         pass
     return t
@@ -74,8 +96,8 @@ def weight_planes(qweight: torch.Tensor) -> torch.Tensor:
     key = id(qweight)
     hit = _planes_cache.get(key)
     if hit is not None:
-        ref, version, data_ptr, t, ready = hit
-        if ref() is qweight and version == qweight._version and data_ptr == qweight.data_ptr():
+        ref, src, t, ready = hit
+        if ref() is qweight and _same_source(src, qweight):
             ready.wait(t.device)
             return t
     N, K = qweight.shape[0], qweight.shape[1] * 2
@@ -86,7 +108,7 @@ def weight_planes(qweight: torch.Tensor) -> torch.Tensor:
         ready = _Ready(t.device)
     try:
         ref = weakref.ref(qweight, lambda _r, k=key: _planes_cache.pop(k, None))
-        _planes_cache[key] = (ref, qweight._version, qweight.data_ptr(), t, ready)
+        _planes_cache[key] = (ref, _source_of(qweight), t, ready)
     except TypeError:
         pass
     return t

@@ -1,6 +1,7 @@
-"""Run-time LoRA on single layers: the widened low-rank branch of an SVDQuant linear (ranks 32 + sum r, padded to a
-multiple of 16) against the oracle on the concatenated factors, the base layer's bits restored on detach, and the
-forward hook of layers without a low-rank branch."""
+"""Low-rank branch widened at run time: ranks 32 + sum r (padded to a multiple of 16) through the same two kernels,
+against the oracle on the concatenated factors; swapping one set of factors for another of the same rank (the
+re-laid-out copy of ``proj_down`` must follow); the base layer's bits restored when the original tensors come back.
+The reference's own ``attach_lora`` (nunchaku/lora/runtime.py:476-525) does exactly this to the two parameters."""
 
 import pytest
 import torch
@@ -21,26 +22,38 @@ def _module(dev, K, N):
     return mod, lin
 
 
-@pytest.mark.parametrize("ranks", [(16,), (8, 20), (64, 64, 128)])
-def test_attach_widens_the_low_rank_branch(dev, ranks):
-    from nunchaku_rocm_amd.lora import attach_lora, detach_lora
+def _factors(K, N, ranks, seed):
+    g = torch.Generator().manual_seed(seed)
+    return [((torch.randn(r, K, generator=g) * 0.05).to(torch.bfloat16), (torch.randn(N, r, generator=g) * 0.2).to(torch.bfloat16))
+            for r in ranks]  # fmt: skip
 
+
+def _widen(mod, lin, pairs, dev):
+    """What a run-time LoRA loader does to the layer: append the factors to the two low-rank parameters, zero-padded
+    to a multiple of 16, by assigning ``.data``."""
+    down = torch.cat([lin["proj_down"]] + [d.t() for d, _ in pairs], 1)
+    up = torch.cat([lin["proj_up"]] + [u for _, u in pairs], 1)
+    R = down.shape[1]
+    pad = -R % 16
+    if pad:
+        down = torch.cat([down, down.new_zeros(down.shape[0], pad)], 1)
+        up = torch.cat([up, up.new_zeros(up.shape[0], pad)], 1)
+    mod.proj_down.data = down.to(dev).contiguous()
+    mod.proj_up.data = up.to(dev).contiguous()
+    mod.rank = R + pad
+    return down, up
+
+
+@pytest.mark.parametrize("ranks", [(16,), (8, 20), (64, 64, 128)])
+def test_widened_low_rank_branch(dev, ranks):
     print(f"case ranks={ranks}", flush=True)
     K, N, M = 512, 384, 150
     mod, lin = _module(dev, K, N)
     x = O.make_activations(M, K, seed=6).view(1, M, K)
     base = mod(x.to(dev)).cpu()
-    g = torch.Generator().manual_seed(sum(ranks))
-    pairs = [((torch.randn(r, K, generator=g) * 0.05).to(torch.bfloat16), (torch.randn(N, r, generator=g) * 0.2).to(torch.bfloat16))
-             for r in ranks]  # fmt: skip
-    attach_lora(mod, pairs)
-    R = 32 + sum(ranks)
-    Rp = (R + 15) // 16 * 16
-    assert mod.proj_down.shape == (K, Rp) and mod.proj_up.shape == (N, Rp) and mod.rank == Rp
-    assert bool((mod.proj_down[:, R:] == 0).all()) and bool((mod.proj_up[:, R:] == 0).all())
+    pairs = _factors(K, N, ranks, seed=sum(ranks))
+    down, up = _widen(mod, lin, pairs, dev)
     y = mod(x.to(dev)).cpu()
-    down = torch.cat([lin["proj_down"]] + [d.t() for d, _ in pairs], 1)
-    up = torch.cat([lin["proj_up"]] + [u for _, u in pairs], 1)
     rp, rs, rl, _ = O.quantize_act(x.view(-1, K), down, lin["smooth_factor"])
     ref = O.gemm_w4a4(rp, lin["qweight"], rs, lin["wscales"], lin["bias"], rl, up)
     assert O.max_rel_err(y.view(-1, N), ref) <= 1e-2
@@ -48,33 +61,29 @@ def test_attach_widens_the_low_rank_branch(dev, ranks):
     xd = x.view(-1, K).double()
     extra = sum((xd @ d.double().t()) @ u.double().t() for d, u in pairs)
     assert O.cosine((y.view(-1, N).double() - base.view(-1, N).double()), extra) > 0.99
-    detach_lora(mod)
-    assert mod.proj_down.shape == (K, 32) and mod.rank == 32
+    # back to the base tensors: the base layer's bits
+    mod.proj_down.data = lin["proj_down"].to(dev)
+    mod.proj_up.data = lin["proj_up"].to(dev)
+    mod.rank = 32
     assert torch.equal(mod(x.to(dev)).cpu(), base)
-    detach_lora(mod)  # nothing attached: no-op
 
 
-def test_hook_on_a_layer_without_low_rank_branch(dev):
-    from nunchaku_rocm_amd.linear import AWQW4A16Linear
-    from nunchaku_rocm_amd.lora import attach_lora, detach_lora
+def test_swapping_factors_of_the_same_rank(dev):
+    """Assigning ``.data`` changes neither the parameter object nor its version counter, and the allocator likes to hand
+    the block just freed to the next tensor of the same size: the cached transposed ``proj_down`` must not survive it."""
+    K, N, M = 512, 384, 150
+    mod, lin = _module(dev, K, N)
+    x = O.make_activations(M, K, seed=7).view(1, M, K)
+    for round_, seed in enumerate((11, 12, 13)):
+        pairs = _factors(K, N, (16,), seed=seed)
+        down, up = _widen(mod, lin, pairs, dev)
+        y = mod(x.to(dev)).cpu()
+        rp, rs, rl, _ = O.quantize_act(x.view(-1, K), down, lin["smooth_factor"])
+        ref = O.gemm_w4a4(rp, lin["qweight"], rs, lin["wscales"], lin["bias"], rl, up)
+        assert O.max_rel_err(y.view(-1, N), ref) <= 1e-2, f"round {round_}: stale low-rank factors"
+        # the quantizer's LoRA hidden state itself, not just the output
+        from nunchaku_rocm_amd import ops
 
-    K, N = 256, 128
-    lin = O.make_awq_linear(K, N, seed=31)
-    mod = AWQW4A16Linear(K, N, bias=False, device=dev)
-    with torch.no_grad():
-        mod.qweight.copy_(lin["qweight"])
-        mod.wscales.copy_(lin["wscales"])
-        mod.wzeros.copy_(lin["wzeros"])
-    g = torch.Generator().manual_seed(3)
-    x = torch.randn(2, K, generator=g).to(torch.bfloat16)
-    d = (torch.randn(8, K, generator=g) * 0.05).to(torch.bfloat16)
-    u = (torch.randn(N, 8, generator=g) * 0.2).to(torch.bfloat16)
-    base = mod(x.to(dev)).cpu()
-    attach_lora(mod, [(d, u)])
-    y = mod(x.to(dev)).cpu()
-    extra = (x.double() @ d.double().t()) @ u.double().t()
-    assert O.max_rel_err((y.double() - base.double()).float(), extra.float()) <= 3e-2
-    detach_lora(mod)
-    assert torch.equal(mod(x.to(dev)).cpu(), base)
-    with pytest.raises(NotImplementedError):
-        attach_lora(mod, [((d, (3, 3)), u)])
+        _, _, la = ops.svdq_quantize_w4a4_act_fuse_lora_cuda(x.view(-1, K).to(dev), lora_down=mod.proj_down,
+                                                             smooth=mod.smooth_factor)  # fmt: skip
+        assert O.max_rel_err(la[:M].cpu(), rl) <= 1e-2, f"round {round_}: LoRA-down read a stale transposed copy"
