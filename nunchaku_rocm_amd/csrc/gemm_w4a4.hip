@@ -47,17 +47,19 @@ constexpr int BLK_BYTES = 64 * 16;    // one MFMA operand block (32 rows x 16 by
 // stage layout: activation blocks [4 blocks of 32 rows][2 groups] packed (1 KB each), weight blocks
 // [4 blocks][2 groups][2 planes] (pre-split weights) or [4 blocks][2 groups] (packed), then the scales
 constexpr int W_OFF = 4 * 2 * BLK_BYTES;                  // 8192
-constexpr int AS_OFF = W_OFF + 4 * 2 * 2 * BLK_BYTES;     // 24576: float as'[2][BM]
-constexpr int NM_OFF = AS_OFF + 2 * BM * 4;               // float -magic*as'[2][BM]
-constexpr int WS_OFF = NM_OFF + 2 * BM * 4;               // float ws[2][BN]
-constexpr int BUF_BYTES = WS_OFF + 2 * BN * 4;            // 27648
+constexpr int AS_OFF = W_OFF + 4 * 2 * 2 * BLK_BYTES;     // 24576: float as[2][BM]
+constexpr int WS_OFF = AS_OFF + 2 * BM * 4;               // 25600: float2 (ws', -magic * ws')[2][BN]
+constexpr int BUF_BYTES = WS_OFF + 2 * BN * 8;            // 27648
 constexpr int SMEM_BYTES = NSTAGE * BUF_BYTES;            // 55296
 // the first 32 ranks of the tile's LoRA operands, fetched next to stage 0: lora_up [2 c][4 blocks] and lora_act
 // [2 c][4 blocks][2 halves of 8 floats] 1 KB blocks in MFMA lane order
 constexpr int LORA_BYTES = (8 + 16) * BLK_BYTES;          // 24576
 constexpr int BIAS_BYTES = BN * 2;                        // the tile's 128 bias values
-constexpr int NWAVES = 8, NTHREADS = NWAVES * 64;  // 2 wavefronts along n x 4 along m
-constexpr int NBM = 1, WROWS = NBM * 32;            // activation rows per wavefront (its 64 weight rows are 2 blocks)
+constexpr int NWAVES = 4, NTHREADS = NWAVES * 64;  // one wavefront per 32 activation rows
+constexpr int NBN = BN / 32;                        // 32-row weight blocks per wavefront: it owns 32 x 128 outputs
+constexpr int TP_PITCH = 36;                        // floats per row of the accumulator transposition tile
+constexpr int TP_WAVE_BYTES = 2 * 32 * TP_PITCH * 4;  // two 32x32 blocks at a time
+static_assert(2 * TP_WAVE_BYTES <= BUF_BYTES, "transposition tiles do not fit");
 constexpr int GROUP_M_TILES = 8;      // m-tiles per raster band
 constexpr int NUM_XCD = 8;
 
@@ -96,13 +98,16 @@ __device__ inline void tile_ids(int tiles_m, int tiles_n, int &pid_m, int &pid_n
 }
 
 template <typename T, bool ACT_UNSIGNED, int EPI, bool WPL, bool ODDG>  // ODDG: K / 64 is odd
-__global__ __launch_bounds__(NTHREADS, 4) void gemm_w4a4_kernel(svdq_gemm_args a) {
-    __shared__ __align__(16) uint8_t smem[SMEM_BYTES + LORA_BYTES + BIAS_BYTES];
+__global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a) {
+    // Three separate LDS objects: the compiler then knows that a block load into one staging buffer cannot touch what
+    // is being read from the other (one object would make every LDS read wait for the loads in flight).
+    __shared__ __align__(16) uint8_t sbuf0[BUF_BYTES];
+    __shared__ __align__(16) uint8_t sbuf1[BUF_BYTES];
+    __shared__ __align__(16) uint8_t sepi[LORA_BYTES + BIAS_BYTES];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keep it in an SGPR
-    const int wn = wave & 1, wm = wave >> 1;  // wavefront position: 2 along n (64 columns each) x 4 along m (32 rows each)
+    const int wm = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: the wavefront's 32-row block of the tile
     const int l32 = lane & 31, half = lane >> 5;
 
     int pid_m, pid_n;
@@ -114,7 +119,7 @@ __global__ __launch_bounds__(NTHREADS, 4) void gemm_w4a4_kernel(svdq_gemm_args a
     // 16 bytes MFMA lane l will read and the hardware writes them to LDS slot l of the block: the layout the operand
     // read wants, free of bank conflicts by construction.  Packed operands: lane l = (row l % 32, half l / 32) of a
     // row-major tile.  Pre-split weights are already stored block by block in that order (1 KB contiguous per load).
-    // The 8 activation + (WPL ? 16 : 8) weight block loads of a stage are dealt in runs to the eight wavefronts.
+    // The 8 activation + (WPL ? 16 : 8) weight block loads of a stage are dealt in runs to the four wavefronts.
     constexpr int NLOADS = WPL ? 24 : 16, PER_WAVE = NLOADS / NWAVES;
     // each load's address = wave-uniform base (SGPRs) + a 32-bit offset (lane part + stage * step; operands < 4 GiB)
     const uint8_t *gbase[PER_WAVE];
@@ -134,15 +139,15 @@ __global__ __launch_bounds__(NTHREADS, 4) void gemm_w4a4_kernel(svdq_gemm_args a
     };
 #pragma unroll
     for (int i = 0; i < PER_WAVE; i++) {
-        const int q = wave * PER_WAVE + i;  // wave-uniform
-        if (q < 8) {                        // activation block q: (blk = q / 2, group q % 2)
+        const int q = wm * PER_WAVE + i;  // wave-uniform
+        if (q < 8) {                      // activation block q: (blk = q / 2, group q % 2)
             const int blk = q >> 1, gg = q & 1;
             gbase[i] = (const uint8_t *)a.act + (size_t)m0 * a.ld_act + gg * 32;
             goff[i] = (uint32_t)(min(m0 + blk * 32 + l32, a.M - 1) - m0) * (uint32_t)a.ld_act + half * 16;
             ldst[i] = (blk * 2 + gg) * BLK_BYTES;
             gstep[i] = KSTAGE / 2;
             if constexpr (ODDG) gcap[i] = cap_of(gg, gstep[i], gbase[i], 32);
-        } else if (WPL) {                   // weight plane block j: (blk = j / 4, group (j / 2) % 2, plane j % 2)
+        } else if (WPL) {                 // weight plane block j: (blk = j / 4, group (j / 2) % 2, plane j % 2)
             const int j = q - 8, blk = j >> 2, gg = (j >> 1) & 1, pl = j & 1;
             const int nblk = min(n0 / 32 + blk, (a.N + 31) / 32 - 1);
             gbase[i] = (const uint8_t *)a.wgt_planes + (((size_t)nblk * G + gg) * 2 + pl) * BLK_BYTES;
@@ -150,7 +155,7 @@ __global__ __launch_bounds__(NTHREADS, 4) void gemm_w4a4_kernel(svdq_gemm_args a
             ldst[i] = W_OFF + ((blk * 2 + gg) * 2 + pl) * BLK_BYTES;
             gstep[i] = 2 * 2 * BLK_BYTES;   // two groups x two planes per stage
             if constexpr (ODDG) gcap[i] = cap_of(gg, gstep[i], gbase[i], 2 * BLK_BYTES);
-        } else {                            // packed weight block j: (blk = j / 2, group j % 2)
+        } else {                          // packed weight block j: (blk = j / 2, group j % 2)
             const int j = q - 8, blk = j >> 1, gg = j & 1;
             gbase[i] = (const uint8_t *)a.wgt + (size_t)n0 * a.ld_wgt + gg * 32;
             goff[i] = (uint32_t)(min(n0 + blk * 32 + l32, a.N - 1) - n0) * (uint32_t)a.ld_wgt + half * 16;
@@ -159,84 +164,81 @@ __global__ __launch_bounds__(NTHREADS, 4) void gemm_w4a4_kernel(svdq_gemm_args a
             if constexpr (ODDG) gcap[i] = cap_of(gg, gstep[i], gbase[i], 32);
         }
     }
-    auto dma_one = [&](int s, int buf, int i) {  // block load i of stage s into staging buffer buf
-        // SGPR base + 32-bit offset (lane part + scalar stage part); the packed path with all stages whole has the
-        // registers for neither form to spare and fares better with a 64-bit address
+    auto dma_one = [&](int s, uint8_t *dstbuf, int i) {  // block load i of stage s into a staging buffer
         const uint8_t *src;
         if constexpr (ODDG)
             src = gbase[i] + (goff[i] + min((uint32_t)s * (uint32_t)gstep[i], gcap[i]));  // stage part wave-uniform
         else
-            src = WPL ? gbase[i] + (goff[i] + (uint32_t)s * (uint32_t)gstep[i]) : gbase[i] + (size_t)s * gstep[i] + goff[i];
-        __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)src, (SVDQ_AS3 void *)(smem + buf * BUF_BYTES + ldst[i]),
-                                         16, 0, 0);
+            src = gbase[i] + (goff[i] + (uint32_t)s * (uint32_t)gstep[i]);
+        __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)src, (SVDQ_AS3 void *)(dstbuf + ldst[i]), 16, 0, 0);
     };
-    auto dma_stage = [&](int s) {
-#pragma unroll
-        for (int i = 0; i < PER_WAVE; i++) dma_one(s, s % NSTAGE, i);
-    };
-    // scales go through registers (they are converted to fp32 and pre-multiplied on the way), one stage ahead
-    // wavefronts 0-3 fetch the activation scales of the stage (2 groups x 128 rows), wavefronts 4-7 the weight scales
-    const int sg = (tid >> 7) & 1, sr = tid & 127;  // scale loader: group within stage, row within tile
-    const bool loads_as = wave < 4;                 // wave-uniform
+    // Scales go through registers (converted to fp32 and pre-multiplied on the way), one stage ahead: thread
+    // (group sg of the stage, row sr of the tile) fetches one activation scale and one weight scale.
+    const int sg = tid >> 7, sr = tid & 127;
     const int sgu = __builtin_amdgcn_readfirstlane(sg);
-    const uint16_t *gSC = loads_as ? (const uint16_t *)a.ascales + (size_t)sgu * a.ld_ascales + m0
-                                   : (const uint16_t *)a.wscales + (size_t)sgu * a.ld_wscales + n0;  // wave-uniform
-    const uint32_t sc_off = 2 * (uint32_t)(loads_as ? min(m0 + sr, a.M - 1) - m0 : min(n0 + sr, a.N - 1) - n0);
-    const uint32_t sc_step = 4 * (uint32_t)(loads_as ? a.ld_ascales : a.ld_wscales);  // bytes per stage (two groups)
+    const uint16_t *gAS = (const uint16_t *)a.ascales + (size_t)sgu * a.ld_ascales + m0;  // wave-uniform
+    const uint16_t *gWS = (const uint16_t *)a.wscales + (size_t)sgu * a.ld_wscales + n0;
+    const uint32_t as_off = 2 * (uint32_t)(min(m0 + sr, a.M - 1) - m0), ws_off = 2 * (uint32_t)(min(n0 + sr, a.N - 1) - n0);
+    const uint32_t as_step = 4 * (uint32_t)a.ld_ascales, ws_step = 4 * (uint32_t)a.ld_wscales;  // bytes per stage
     const float fold = ACT_UNSIGNED ? (1.0f / 16.0f) : (1.0f / 256.0f);
-    // a plain load: its first use is the conversion at the top of the next stage, behind that stage's vmcnt(0)
-    uint16_t rsc;
-    uint32_t sc_cap = 0;
+    uint16_t ras, rws;
+    uint32_t as_cap = 0, ws_cap = 0;
     if constexpr (ODDG) {
-        sc_cap = (uint32_t)(G / 2) * sc_step;
+        as_cap = (uint32_t)(G / 2) * as_step;
+        ws_cap = (uint32_t)(G / 2) * ws_step;
         if (sgu == 1) {  // this wavefront's group of the last stage does not exist
-            if (G == 1) gSC -= loads_as ? a.ld_ascales : a.ld_wscales;
-            sc_cap = G == 1 ? 0u : (uint32_t)(G / 2 - 1) * sc_step;
+            if (G == 1) {
+                gAS -= a.ld_ascales;
+                gWS -= a.ld_wscales;
+            }
+            as_cap = G == 1 ? 0u : (uint32_t)(G / 2 - 1) * as_step;
+            ws_cap = G == 1 ? 0u : (uint32_t)(G / 2 - 1) * ws_step;
         }
     }
     auto load_scales = [&](int s) {
         if (ODDG) {
-            const uint16_t v = *(const uint16_t *)((const uint8_t *)gSC + (sc_off + min((uint32_t)s * (uint32_t)sc_step, sc_cap)));
-            rsc = (s == G / 2 && sgu == 1) ? (uint16_t)0 : v;  // +0 in both 16-bit types
+            const uint16_t va = *(const uint16_t *)((const uint8_t *)gAS + (as_off + min((uint32_t)s * as_step, as_cap)));
+            const uint16_t vw = *(const uint16_t *)((const uint8_t *)gWS + (ws_off + min((uint32_t)s * ws_step, ws_cap)));
+            const bool off = s == G / 2 && sgu == 1;
+            ras = off ? (uint16_t)0 : va;  // +0 in both 16-bit types
+            rws = off ? (uint16_t)0 : vw;
         } else {
-            rsc = *(const uint16_t *)((const uint8_t *)gSC + (sc_off + (uint32_t)s * (uint32_t)sc_step));
+            ras = *(const uint16_t *)((const uint8_t *)gAS + (as_off + (uint32_t)s * as_step));
+            rws = *(const uint16_t *)((const uint8_t *)gWS + (ws_off + (uint32_t)s * ws_step));
         }
     };
-    auto store_scales = [&](int s) {
-        uint8_t *base = smem + (s % NSTAGE) * BUF_BYTES;
-        const float v = T::to_f32(rsc);
-        if (loads_as) {
-            ((float *)(base + AS_OFF))[sg * BM + sr] = v * fold;
-            ((float *)(base + NM_OFF))[sg * BM + sr] = -RNE_MAGIC * (v * fold);
-        } else {
-            ((float *)(base + WS_OFF))[sg * BN + sr] = v;
-        }
+    auto store_scales = [&](uint8_t *base) {
+        ((float *)(base + AS_OFF))[sg * BM + sr] = T::to_f32(ras);
+        const float w = T::to_f32(rws) * fold;
+        ((float2 *)(base + WS_OFF))[sg * BN + sr] = make_float2(w, -RNE_MAGIC * w);
     };
 
-    v16f acc[2][NBM];
+    // Main-loop accumulators: MFMA A operand = activations, B operand = weights, so a lane owns one weight row n and its
+    // registers walk the wavefront's 32 activation rows: the weight scale is a per-lane scalar and the 16 activation
+    // scales a lane needs per group are shared by the wavefront's four weight blocks.
+    v16f acc[NBN];
 #pragma unroll
-    for (int bn = 0; bn < 2; bn++)
+    for (int bn = 0; bn < NBN; bn++)
 #pragma unroll
-        for (int bm = 0; bm < NBM; bm++)
-#pragma unroll
-            for (int i = 0; i < 16; i++) acc[bn][bm][i] = 0.0f;
+        for (int i = 0; i < 16; i++) acc[bn][i] = 0.0f;
 
     const v16i cmagic = magic_acc();
     const int nstages = ODDG ? a.K / KSTAGE + 1 : a.K / KSTAGE;
-    const int offW = W_OFF + (wn * 2) * 2 * (WPL ? 2 : 1) * BLK_BYTES + lane * 16;
-    const int offA = (wm * NBM) * 2 * BLK_BYTES + lane * 16;
+    const int offW = W_OFF + lane * 16;
+    const int offA = wm * 2 * BLK_BYTES + lane * 16;
 
     load_scales(0);
-    dma_stage(0);
+#pragma unroll
+    for (int i = 0; i < PER_WAVE; i++) dma_one(0, sbuf0, i);
     // epilogue operands, fetched now so that the epilogue does not wait for memory
-    if (a.bias != nullptr && wave == 7) {  // 64 lanes x 4 bytes = the tile's 128 bias values
+    if (a.bias != nullptr && wm == 3) {  // 64 lanes x 4 bytes = the tile's 128 bias values
         const uint8_t *src = (const uint8_t *)a.bias + (size_t)min(n0 + 2 * lane, a.N - 2) * 2;
-        __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)src, (SVDQ_AS3 void *)(smem + SMEM_BYTES + LORA_BYTES), 4, 0, 0);
+        __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)src, (SVDQ_AS3 void *)(sepi + LORA_BYTES), 4, 0, 0);
     }
     if (a.R > 0) {
 #pragma unroll
-        for (int i = 0; i < 3; i++) {
-            const int q = wave * 3 + i;  // wave-uniform
+        for (int i = 0; i < 6; i++) {
+            const int q = wm * 6 + i;  // wave-uniform
             const uint8_t *src;
             bool on = true;
             if (q < 8) {
@@ -249,168 +251,178 @@ __global__ __launch_bounds__(NTHREADS, 4) void gemm_w4a4_kernel(svdq_gemm_args a
                 src = (const uint8_t *)a.lora_act + ((size_t)min(m0 + blk * 32 + l32, a.M - 1) * a.ld_lora_act + 16 * c + 8 * half + 4 * part) * 4;
             }
             if (on)
-                __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)src, (SVDQ_AS3 void *)(smem + SMEM_BYTES + q * BLK_BYTES), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)src, (SVDQ_AS3 void *)(sepi + q * BLK_BYTES), 16, 0, 0);
         }
     }
-    // One copy of the loop per position (0..3) at which the wavefront issues its loads within a stage: the four
-    // wavefronts that share a SIMD take different positions, so that one of them at a time waits for room in the
-    // memory pipeline while the others compute.  (A run-time test of the position inside one loop costs registers.)
-    auto main_loop = [&](auto pos_tag) {
-    constexpr int POS = decltype(pos_tag)::value;
-    for (int s = 0; s < nstages; s++) {
+    // One stage = eight (group, weight block) steps, software-pipelined inside the wavefront: the MFMAs of step b + 1
+    // are issued before the dequantisation FMAs of step b, and the operands of step b + 2 are read from LDS behind
+    // them, so the VALU work of a step runs while the matrix pipe works on the next one.
+    auto stage = [&](auto par_tag, int s) {
+        constexpr int P = decltype(par_tag)::value;
+        uint8_t *base = P ? sbuf1 : sbuf0;   // this stage's operands
+        uint8_t *other = P ? sbuf0 : sbuf1;  // being refilled for the next stage
         // everything issued for stage s (scale registers, then operand blocks) has landed
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
-        store_scales(s);
+        store_scales(base);
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));  // scale writes visible before the barrier
         __builtin_amdgcn_s_barrier();
-        // The other buffer was last read in iteration s - 1, before the barrier: refill it during this stage.  The last
+        // The other buffer was last read in the previous stage, before the barrier: refill it during this stage.  The last
         // stage re-fetches itself into the idle buffer (harmless, and keeps the stage one basic block).
         const int sn = min(s + 1, nstages - 1);
-        const uint8_t *base = smem + (s % NSTAGE) * BUF_BYTES;
-#pragma unroll
-        for (int gg = 0; gg < 2; gg++) {
-            v4i we[2], wo[2], ae[NBM], ao[NBM];
-#pragma unroll
-            for (int blk = 0; blk < 2; blk++) {
-                if (WPL) {
-                    we[blk] = *(const v4i *)(base + offW + ((blk * 2 + gg) * 2 + 0) * BLK_BYTES);
-                    wo[blk] = *(const v4i *)(base + offW + ((blk * 2 + gg) * 2 + 1) * BLK_BYTES);
-                } else {
-                    const v4i wp = *(const v4i *)(base + offW + (blk * 2 + gg) * BLK_BYTES);
-                    unpack_signed(wp, we[blk], wo[blk]);
-                }
+        load_scales(sn);
+        auto read_w = [&](int b, v4i &we, v4i &wo, float2 &wsp) {
+            const int gg = b >> 2, bn = b & 3;
+            if (WPL) {
+                we = *(const v4i *)(base + offW + ((bn * 2 + gg) * 2 + 0) * BLK_BYTES);
+                wo = *(const v4i *)(base + offW + ((bn * 2 + gg) * 2 + 1) * BLK_BYTES);
+            } else {
+                const v4i wp = *(const v4i *)(base + offW + (bn * 2 + gg) * BLK_BYTES);
+                unpack_signed(wp, we, wo);
             }
+            wsp = ((const float2 *)(base + WS_OFF))[gg * BN + bn * 32 + l32];
+        };
+        auto read_a = [&](int gg, v4i &ae, v4i &ao) {
+            const v4i ap = *(const v4i *)(base + offA + gg * BLK_BYTES);
+            if (ACT_UNSIGNED)
+                unpack_unsigned(ap, ae, ao);
+            else
+                unpack_signed(ap, ae, ao);
+        };
+        auto read_as = [&](int gg, v4f (&asv)[4]) {
 #pragma unroll
-            for (int blk = 0; blk < NBM; blk++) {
-                const v4i ap = *(const v4i *)(base + offA + (blk * 2 + gg) * BLK_BYTES);
-                if (ACT_UNSIGNED)
-                    unpack_unsigned(ap, ae[blk], ao[blk]);
-                else
-                    unpack_signed(ap, ae[blk], ao[blk]);
+            for (int j = 0; j < 4; j++)
+                asv[j] = *(const v4f *)((const float *)(base + AS_OFF) + gg * BM + wm * 32 + 8 * j + 4 * half);
+        };
+        v4i ae[2], ao[2], we[2], wo[2];
+        float2 wsp[2];
+        v4f asv[2][4];
+        v16i t[2];
+        read_a(0, ae[0], ao[0]);
+        read_w(0, we[0], wo[0], wsp[0]);
+        read_as(0, asv[0]);
+        read_w(1, we[1], wo[1], wsp[1]);
+        t[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ae[0], we[0], cmagic, 0, 0, 0);
+        t[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ao[0], wo[0], t[0], 0, 0, 0);
+        read_a(1, ae[1], ao[1]);
+        read_as(1, asv[1]);
+#pragma unroll
+        for (int b = 0; b < 8; b++) {
+            const int cur = b & 1, nxt = cur ^ 1;
+            float2 wcur = wsp[cur];
+            if (b + 1 < 8) {
+                const int g1 = (b + 1) >> 2;
+                t[nxt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ae[g1], we[nxt], cmagic, 0, 0, 0);
+                t[nxt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ao[g1], wo[nxt], t[nxt], 0, 0, 0);
             }
-            float asl[NBM], nml[NBM];
+            if (b + 2 < 8) read_w(b + 2, we[cur], wo[cur], wsp[cur]);
+            if (b < PER_WAVE) dma_one(sn, other, b);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int bm = 0; bm < NBM; bm++) {
-                asl[bm] = ((const float *)(base + AS_OFF))[gg * BM + wm * WROWS + bm * 32 + l32];
-                nml[bm] = ((const float *)(base + NM_OFF))[gg * BM + wm * WROWS + bm * 32 + l32];
+            for (int i = 0; i < 16; i++) {
+                const float u = __builtin_fmaf(__int_as_float(t[cur][i]), wcur.x, wcur.y);
+                acc[b & 3][i] = __builtin_fmaf(u, asv[b >> 2][i >> 2][i & 3], acc[b & 3][i]);
             }
-#pragma unroll
-            for (int bn = 0; bn < 2; bn++) {
-                if (POS == gg * 2 + bn) {
-                    load_scales(sn);
-#pragma unroll
-                    for (int i = 0; i < PER_WAVE; i++) dma_one(sn, (s + 1) % NSTAGE, i);
-                }
-                v4f wsr[4];
-#pragma unroll
-                for (int j = 0; j < 4; j++)
-                    wsr[j] = *(const v4f *)((const float *)(base + WS_OFF) + gg * BN + wn * 64 + bn * 32 + 8 * j + 4 * half);
-#pragma unroll
-                for (int bm = 0; bm < NBM; bm++) {
-                    v16i t = __builtin_amdgcn_mfma_i32_32x32x32_i8(we[bn], ae[bm], cmagic, 0, 0, 0);
-                    t = __builtin_amdgcn_mfma_i32_32x32x32_i8(wo[bn], ao[bm], t, 0, 0, 0);
-#pragma unroll
-                    for (int i = 0; i < 16; i++) {
-                        const float u = __builtin_fmaf(__int_as_float(t[i]), asl[bm], nml[bm]);
-                        acc[bn][bm][i] = __builtin_fmaf(u, wsr[i >> 2][i & 3], acc[bn][bm][i]);
-                    }
-                }
-            }
+            __builtin_amdgcn_sched_barrier(0);
         }
-    }
     };
-    switch (wm) {  // wave-uniform
-        case 0: main_loop(std::integral_constant<int, 0>{}); break;
-        case 1: main_loop(std::integral_constant<int, 1>{}); break;
-        case 2: main_loop(std::integral_constant<int, 2>{}); break;
-        default: main_loop(std::integral_constant<int, 3>{}); break;
+    {
+        int s = 0;
+        for (; s + 1 < nstages; s += 2) {
+            stage(std::integral_constant<int, 0>{}, s);
+            stage(std::integral_constant<int, 1>{}, s + 1);
+        }
+        if (s < nstages) stage(std::integral_constant<int, 0>{}, s);
     }
-    // The last stage's (redundant) block loads of this wavefront have landed.  No barrier here: the LoRA-up / bias section
-    // only reads the LDS blocks that arrived before the first stage's barrier, and every epilogue starts its first use
-    // of the staging memory with a barrier of its own.
+    // The last stage's (redundant) block loads of this wavefront have landed.
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
 
-    // ---- epilogue: LoRA-up and bias ----------------------------------------------------------------
-    const int nw0 = n0 + wn * 64, mw0 = m0 + wm * WROWS;
+    // ---- LoRA-up and bias, still in the main loop's orientation (lane = weight row, registers = activation rows) ----
     // The bias and the first 32 ranks of both LoRA operands were fetched into LDS next to stage 0 and arrived long ago;
     // ranks beyond 32 come from global memory, all loads of a 32-rank pass issued before their first use.  Rows past
     // N / M hold copies of the last row: they only reach outputs that are never stored.
-    uint2 bb[2][4];
-    if (a.bias != nullptr) {
-#pragma unroll
-        for (int bn = 0; bn < 2; bn++)
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                bb[bn][j] = *(const uint2 *)(smem + SMEM_BYTES + LORA_BYTES + (wn * 64 + bn * 32 + 8 * j + 4 * half) * 2);
-            }
-    }
+    const int mw0 = m0 + wm * 32;
     if (a.R > 0) {
         const uint16_t *lu = (const uint16_t *)a.lora_up;
         for (int r0 = 0; r0 < a.R; r0 += 32) {
             const bool two = r0 + 16 < a.R;  // uniform: the second 16 ranks of this pass exist
-            v4i ua[2][2];
-            v4f uf[2][NBM][2];
+            v4i ua[2][NBN];
+            v4f uf[2][2];
 #pragma unroll
             for (int c = 0; c < 2; c++) {
                 if (c == 1 && !two) break;
 #pragma unroll
-                for (int blk = 0; blk < 2; blk++) {
-                    const int n = nw0 + blk * 32 + l32;
+                for (int blk = 0; blk < NBN; blk++) {
+                    const int n = n0 + blk * 32 + l32;
                     ua[c][blk] = (v4i){0, 0, 0, 0};
                     if (r0 == 0)
-                        ua[c][blk] = *(const v4i *)(smem + SMEM_BYTES + (c * 4 + wn * 2 + blk) * BLK_BYTES + lane * 16);
+                        ua[c][blk] = *(const v4i *)(sepi + (c * 4 + blk) * BLK_BYTES + lane * 16);
                     else if (n < a.N)
                         ua[c][blk] = *(const v4i *)(lu + (size_t)n * a.ld_lora_up + r0 + 16 * c + half * 8);
                 }
-#pragma unroll
-                for (int blk = 0; blk < NBM; blk++) {
-                    const int m = mw0 + blk * 32 + l32;
-                    uf[c][blk][0] = uf[c][blk][1] = (v4f){0.f, 0.f, 0.f, 0.f};
-                    if (r0 == 0) {
-                        const uint8_t *lp = smem + SMEM_BYTES + 8 * BLK_BYTES + ((c * 4 + wm * NBM + blk) * 2) * BLK_BYTES + lane * 16;
-                        uf[c][blk][0] = *(const v4f *)lp;
-                        uf[c][blk][1] = *(const v4f *)(lp + BLK_BYTES);
-                    } else if (m < a.M) {
-                        const float *lp = a.lora_act + (size_t)m * a.ld_lora_act + r0 + 16 * c + half * 8;
-                        uf[c][blk][0] = *(const v4f *)lp;
-                        uf[c][blk][1] = *(const v4f *)(lp + 4);
-                    }
+                const int m = mw0 + l32;
+                uf[c][0] = uf[c][1] = (v4f){0.f, 0.f, 0.f, 0.f};
+                if (r0 == 0) {
+                    const uint8_t *lp = sepi + 8 * BLK_BYTES + ((c * 4 + wm) * 2) * BLK_BYTES + lane * 16;
+                    uf[c][0] = *(const v4f *)lp;
+                    uf[c][1] = *(const v4f *)(lp + BLK_BYTES);
+                } else if (m < a.M) {
+                    const float *lp = a.lora_act + (size_t)m * a.ld_lora_act + r0 + 16 * c + half * 8;
+                    uf[c][0] = *(const v4f *)lp;
+                    uf[c][1] = *(const v4f *)(lp + 4);
                 }
             }
 #pragma unroll
             for (int c = 0; c < 2; c++) {
                 if (c == 1 && !two) break;
-                v4i ub[NBM];
+                const v4f f0 = uf[c][0], f1 = uf[c][1];
+                v4i ub;
+                ub[0] = (int)pack2<T>(f0[0], f0[1]);
+                ub[1] = (int)pack2<T>(f0[2], f0[3]);
+                ub[2] = (int)pack2<T>(f1[0], f1[1]);
+                ub[3] = (int)pack2<T>(f1[2], f1[3]);
 #pragma unroll
-                for (int blk = 0; blk < NBM; blk++) {
-                    const v4f f0 = uf[c][blk][0], f1 = uf[c][blk][1];
-                    ub[blk][0] = (int)pack2<T>(f0[0], f0[1]);
-                    ub[blk][1] = (int)pack2<T>(f0[2], f0[3]);
-                    ub[blk][2] = (int)pack2<T>(f1[0], f1[1]);
-                    ub[blk][3] = (int)pack2<T>(f1[2], f1[3]);
-                }
-#pragma unroll
-                for (int bn = 0; bn < 2; bn++)
-#pragma unroll
-                    for (int bm = 0; bm < NBM; bm++) acc[bn][bm] = mfma32_16bit<T>(ua[c][bn], ub[bm], acc[bn][bm]);
+                for (int bn = 0; bn < NBN; bn++) acc[bn] = mfma32_16bit<T>(ub, ua[c][bn], acc[bn]);
             }
         }
     }
     if (a.bias != nullptr) {
 #pragma unroll
-        for (int bn = 0; bn < 2; bn++)
+        for (int bn = 0; bn < NBN; bn++) {
+            const float b = T::to_f32(*(const uint16_t *)(sepi + LORA_BYTES + (bn * 32 + l32) * 2));
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const float b0 = T::lo_f32(bb[bn][j].x), b1 = T::hi_f32(bb[bn][j].x);
-                const float b2 = T::lo_f32(bb[bn][j].y), b3 = T::hi_f32(bb[bn][j].y);
+            for (int i = 0; i < 16; i++) acc[bn][i] += b;
+        }
+    }
+
+    // ---- transposition: lane = weight row -> lane = activation row ---------------------------------------------
+    // Each wavefront turns its four 32x32 blocks through a private LDS tile (the staging memory is free once every
+    // wavefront has left the main loop and read its LoRA operands).  Afterwards lane (m = lane % 32, half) holds
+    // columns 32 bn + 8 j + 4 half + e of row m in acc[bn][4 j + e]: row-wise epilogue work (RMSNorm sum of squares,
+    // RoPE pairs, group absmax, nibble packing, the next layer's LoRA-down B operand) is in-lane plus one exchange
+    // with lane ^ 32, and no epilogue needs another wavefront's data.
+    __syncthreads();
+    {
+        // wavefronts 0, 1 use the first staging buffer, 2, 3 the second; two blocks per round
+        float *tp = (float *)((wm < 2 ? sbuf0 : sbuf1) + (wm & 1) * TP_WAVE_BYTES);
 #pragma unroll
-                for (int bm = 0; bm < NBM; bm++) {
-                    acc[bn][bm][4 * j + 0] += b0;
-                    acc[bn][bm][4 * j + 1] += b1;
-                    acc[bn][bm][4 * j + 2] += b2;
-                    acc[bn][bm][4 * j + 3] += b3;
+        for (int rnd = 0; rnd < NBN / 2; rnd++) {
+#pragma unroll
+            for (int b2 = 0; b2 < 2; b2++)
+#pragma unroll
+                for (int i = 0; i < 16; i++)
+                    tp[(b2 * 32 + 8 * (i >> 2) + 4 * half + (i & 3)) * TP_PITCH + l32] = acc[2 * rnd + b2][i];
+            // the same wavefront writes and reads: the LDS operations of one wavefront complete in order
+#pragma unroll
+            for (int b2 = 0; b2 < 2; b2++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const v4f v = *(const v4f *)(tp + (b2 * 32 + l32) * TP_PITCH + 8 * j + 4 * half);
+                    acc[2 * rnd + b2][4 * j + 0] = v[0];
+                    acc[2 * rnd + b2][4 * j + 1] = v[1];
+                    acc[2 * rnd + b2][4 * j + 2] = v[2];
+                    acc[2 * rnd + b2][4 * j + 3] = v[3];
                 }
-            }
+        }
     }
 
     // Output rows go out through LDS: in registers a lane holds 4 consecutive columns of one row, which stored directly
@@ -418,29 +430,30 @@ __global__ __launch_bounds__(NTHREADS, 4) void gemm_w4a4_kernel(svdq_gemm_args a
     // contiguous 256-byte row segments instead.
     auto store_out = [&]() {
         constexpr int PITCH = BN * 2 + 16;  // bytes per staged row (16-byte aligned, off the power of two)
-        static_assert(BM * PITCH <= SMEM_BYTES, "output tile does not fit the staging memory");
+        static_assert(BM / 2 * PITCH <= BUF_BYTES, "half an output tile does not fit a staging buffer");
         __syncthreads();  // earlier users of the staging memory are done
+        uint8_t *mine = (wm < 2 ? sbuf0 : sbuf1) + ((wm & 1) * 32 + l32) * PITCH;  // rows 0-63 | rows 64-127
 #pragma unroll
-        for (int bm = 0; bm < NBM; bm++)
+        for (int bn = 0; bn < NBN; bn++)
 #pragma unroll
-            for (int bn = 0; bn < 2; bn++)
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    uint2 v;
-                    v.x = pack2<T>(acc[bn][bm][4 * j], acc[bn][bm][4 * j + 1]);
-                    v.y = pack2<T>(acc[bn][bm][4 * j + 2], acc[bn][bm][4 * j + 3]);
-                    *(uint2 *)(smem + (wm * WROWS + bm * 32 + l32) * PITCH + (wn * 64 + bn * 32 + 8 * j + 4 * half) * 2) = v;
-                }
+            for (int j = 0; j < 4; j++) {
+                uint2 v;
+                v.x = pack2<T>(acc[bn][4 * j], acc[bn][4 * j + 1]);
+                v.y = pack2<T>(acc[bn][4 * j + 2], acc[bn][4 * j + 3]);
+                *(uint2 *)(mine + (bn * 32 + 8 * j + 4 * half) * 2) = v;
+            }
         __syncthreads();
         uint16_t *out = (uint16_t *)a.out;
         const int c = tid & 15, n = n0 + c * 8;
+        constexpr int PASSES = BM * 16 / NTHREADS;
 #pragma unroll
-        for (int pass = 0; pass < BM * 16 / NTHREADS; pass++) {
+        for (int pass = 0; pass < PASSES; pass++) {
             const int row = pass * (NTHREADS / 16) + (tid >> 4), m = m0 + row;
+            const uint8_t *src = (pass < PASSES / 2 ? sbuf0 : sbuf1) + (row & 63) * PITCH + c * 16;
             if (m < a.actual_m && n < a.N)
                 // streamed: the 85 MB of a QKV output do not fit any cache level of the CU, and lines left dirty in L2 have
                 // to be written back before the next kernel on the stream starts (measured: 1 % of the launch)
-                __builtin_nontemporal_store(*(const v4i *)(smem + row * PITCH + c * 16), (v4i *)(out + (size_t)m * a.ld_out + n));
+                __builtin_nontemporal_store(*(const v4i *)src, (v4i *)(out + (size_t)m * a.ld_out + n));
         }
     };
 
@@ -450,48 +463,36 @@ __global__ __launch_bounds__(NTHREADS, 4) void gemm_w4a4_kernel(svdq_gemm_args a
     }
 
     if (EPI == SVDQ_EPI_QK_NORM_ROPE) {
-        // the 128-wide tile is one head; part 0 = Q, 1 = K, 2 = V (untouched)
+        // the 128-wide tile is one head, all of it in this wavefront; part 0 = Q, 1 = K, 2 = V (untouched)
         const int part = n0 / (a.N / 3);
         if (part < 2) {
-            float *red = (float *)smem;  // [2 (wn)][BM]
-            __syncthreads();             // main-loop LDS reads are done
+            float ss = 0.0f;
 #pragma unroll
-            for (int bm = 0; bm < NBM; bm++) {
-                float ss = 0.0f;
+            for (int bn = 0; bn < NBN; bn++)
 #pragma unroll
-                for (int bn = 0; bn < 2; bn++)
-#pragma unroll
-                    for (int i = 0; i < 16; i++) ss += acc[bn][bm][i] * acc[bn][bm][i];
-                ss += __shfl_xor(ss, 32);
-                if (half == 0) red[wn * BM + wm * WROWS + bm * 32 + l32] = ss;
-            }
-            __syncthreads();
+                for (int i = 0; i < 16; i++) ss += acc[bn][i] * acc[bn][i];
+            ss += __shfl_xor(ss, 32);
             const uint16_t *nw = (const uint16_t *)(part == 0 ? a.norm_q : a.norm_k);
+            const int m = mw0 + l32;
+            const float rstd = 1.0f / sqrtf(ss / 128.0f + a.eps);
+            const bool rok = m < a.actual_m;
+            const float *rot = a.rotary + (size_t)(rok ? m : 0) * a.ld_rotary;
 #pragma unroll
-            for (int bm = 0; bm < NBM; bm++) {
-                const int ml = wm * WROWS + bm * 32 + l32;
-                const int m = m0 + ml;
-                const float tot = red[ml] + red[BM + ml];
-                const float rstd = 1.0f / sqrtf(tot / 128.0f + a.eps);
-                const bool rok = m < a.actual_m;
-                const float *rot = a.rotary + (size_t)(rok ? m : 0) * a.ld_rotary;
+            for (int bn = 0; bn < NBN; bn++)
 #pragma unroll
-                for (int bn = 0; bn < 2; bn++)
-#pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        const int d = wn * 64 + bn * 32 + 8 * j + 4 * half;  // channel within the head
-                        const uint2 wb = *(const uint2 *)(nw + d);
-                        const v4f sc = *(const v4f *)(rot + d);  // (sin, cos, sin, cos)
-                        const float x0 = acc[bn][bm][4 * j + 0] * rstd * T::lo_f32(wb.x);
-                        const float x1 = acc[bn][bm][4 * j + 1] * rstd * T::hi_f32(wb.x);
-                        const float x2 = acc[bn][bm][4 * j + 2] * rstd * T::lo_f32(wb.y);
-                        const float x3 = acc[bn][bm][4 * j + 3] * rstd * T::hi_f32(wb.y);
-                        acc[bn][bm][4 * j + 0] = x0 * sc[1] - x1 * sc[0];
-                        acc[bn][bm][4 * j + 1] = x0 * sc[0] + x1 * sc[1];
-                        acc[bn][bm][4 * j + 2] = x2 * sc[3] - x3 * sc[2];
-                        acc[bn][bm][4 * j + 3] = x2 * sc[2] + x3 * sc[3];
-                    }
-            }
+                for (int j = 0; j < 4; j++) {
+                    const int d = bn * 32 + 8 * j + 4 * half;  // channel within the head
+                    const uint2 wb = *(const uint2 *)(nw + d);
+                    const v4f sc = *(const v4f *)(rot + d);  // (sin, cos, sin, cos)
+                    const float x0 = acc[bn][4 * j + 0] * rstd * T::lo_f32(wb.x);
+                    const float x1 = acc[bn][4 * j + 1] * rstd * T::hi_f32(wb.x);
+                    const float x2 = acc[bn][4 * j + 2] * rstd * T::lo_f32(wb.y);
+                    const float x3 = acc[bn][4 * j + 3] * rstd * T::hi_f32(wb.y);
+                    acc[bn][4 * j + 0] = x0 * sc[1] - x1 * sc[0];
+                    acc[bn][4 * j + 1] = x0 * sc[0] + x1 * sc[1];
+                    acc[bn][4 * j + 2] = x2 * sc[3] - x3 * sc[2];
+                    acc[bn][4 * j + 3] = x2 * sc[2] + x3 * sc[3];
+                }
         }
         store_out();
         return;
@@ -504,105 +505,80 @@ __global__ __launch_bounds__(NTHREADS, 4) void gemm_w4a4_kernel(svdq_gemm_args a
         uint16_t smv = 0;
         const bool has_sm = a.smooth_next != nullptr && tid < BN && n0 + tid < a.N;
         if (has_sm) smv = ((const uint16_t *)a.smooth_next)[n0 + tid];
-        uint2 lq[2][2][2];
+        uint2 lq[NBN][2][2];
         if (a.R2 > 0) {
 #pragma unroll
-            for (int bn = 0; bn < 2; bn++)
+            for (int bn = 0; bn < NBN; bn++)
 #pragma unroll
                 for (int s = 0; s < 2; s++) {
                     lq[bn][s][0] = lq[bn][s][1] = make_uint2(0u, 0u);
                     if (l32 < a.R2) {
-                        const uint16_t *lp = ldt + (size_t)l32 * a.N + nw0 + bn * 32 + 16 * s + 4 * half;
+                        const uint16_t *lp = ldt + (size_t)l32 * a.N + n0 + bn * 32 + 16 * s + 4 * half;
                         lq[bn][s][0] = *(const uint2 *)lp;
                         lq[bn][s][1] = *(const uint2 *)(lp + 8);
                     }
                 }
         }
         if (a.out != nullptr) store_out();  // pre-GELU output, when asked for
-        float *lds_part = (float *)smem;  // [4 (wm)][16 regs][64 lanes] floats = 16 KB
-        __syncthreads();
 #pragma unroll
-        for (int bn = 0; bn < 2; bn++)
+        for (int bn = 0; bn < NBN; bn++)
 #pragma unroll
-            for (int bm = 0; bm < NBM; bm++)
-#pragma unroll
-                for (int i = 0; i < 16; i++) acc[bn][bm][i] = gelu_tanh(acc[bn][bm][i]);
+            for (int i = 0; i < 16; i++) acc[bn][i] = gelu_tanh(acc[bn][i]);
 
         // next layer's LoRA-down on the un-shifted, un-smoothed GELU output rounded to T:
-        // D[r][m] = sum_n ldT[r][n] * x[n][m]; registers [8 s, 8 s + 8) of a block are one MFMA's B operand
+        // D[r][m] = sum_n ldT[r][n] * x[n][m] over the tile's 128 columns; registers [8 s, 8 s + 8) of a block are one
+        // MFMA's B operand.  One partial per n-tile, summed in tile order by lora_part_reduce_kernel.
         for (int rc = 0; rc < a.R2; rc += 32) {
-            v16f d[NBM];
+            v16f d;
 #pragma unroll
-            for (int bm = 0; bm < NBM; bm++)
-#pragma unroll
-                for (int i = 0; i < 16; i++) d[bm][i] = 0.0f;
+            for (int i = 0; i < 16; i++) d[i] = 0.0f;
             const int r = rc + l32;
 #pragma unroll
-            for (int bn = 0; bn < 2; bn++)
+            for (int bn = 0; bn < NBN; bn++)
 #pragma unroll
                 for (int s = 0; s < 2; s++) {
                     v4i la = (v4i){0, 0, 0, 0};
                     if (rc == 0) {
                         la = (v4i){(int)lq[bn][s][0].x, (int)lq[bn][s][0].y, (int)lq[bn][s][1].x, (int)lq[bn][s][1].y};
                     } else if (r < a.R2) {
-                        const uint16_t *lp = ldt + (size_t)r * a.N + nw0 + bn * 32 + 16 * s + 4 * half;
+                        const uint16_t *lp = ldt + (size_t)r * a.N + n0 + bn * 32 + 16 * s + 4 * half;
                         const uint2 q0 = *(const uint2 *)lp, q1 = *(const uint2 *)(lp + 8);
                         la = (v4i){(int)q0.x, (int)q0.y, (int)q1.x, (int)q1.y};
                     }
+                    v4i xb;
 #pragma unroll
-                    for (int bm = 0; bm < NBM; bm++) {
-                        v4i xb;
-#pragma unroll
-                        for (int e = 0; e < 4; e++)
-                            xb[e] = (int)pack2<T>(acc[bn][bm][8 * s + 2 * e], acc[bn][bm][8 * s + 2 * e + 1]);
-                        d[bm] = mfma32_16bit<T>(la, xb, d[bm]);
-                    }
+                    for (int e = 0; e < 4; e++) xb[e] = (int)pack2<T>(acc[bn][8 * s + 2 * e], acc[bn][8 * s + 2 * e + 1]);
+                    d = mfma32_16bit<T>(la, xb, d);
                 }
-            // add the two n-wavefronts in a fixed order (wn = 0 first), then one partial per n-tile
-            if (wn == 1) {
+            const int m = mw0 + l32;
 #pragma unroll
-                for (int bm = 0; bm < NBM; bm++)
-#pragma unroll
-                    for (int i = 0; i < 16; i++) lds_part[((wm * NBM + bm) * 16 + i) * 64 + lane] = d[bm][i];
+            for (int j = 0; j < 4; j++) {
+                const int rr = rc + 8 * j + 4 * half;
+                if (m < a.M && rr < a.R2)
+                    *(v4f *)(a.scratch + ((size_t)pid_n * a.M + m) * a.R2 + rr) = (v4f){d[4 * j], d[4 * j + 1], d[4 * j + 2], d[4 * j + 3]};
             }
-            __syncthreads();
-            if (wn == 0) {
-#pragma unroll
-                for (int bm = 0; bm < NBM; bm++) {
-                    const int m = mw0 + bm * 32 + l32;
-#pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        v4f o;
-#pragma unroll
-                        for (int e = 0; e < 4; e++)
-                            o[e] = d[bm][4 * j + e] + lds_part[((wm * NBM + bm) * 16 + 4 * j + e) * 64 + lane];
-                        const int rr = rc + 8 * j + 4 * half;
-                        if (m < a.M && rr < a.R2)
-                            *(v4f *)(a.scratch + ((size_t)pid_n * a.M + m) * a.R2 + rr) = o;
-                    }
-                }
-            }
-            __syncthreads();
         }
 
-        // +shift, * 1/smooth, unsigned per-64 quantization: the wavefront's 64 columns are one group
-        float *lds_rs = (float *)smem;  // [BN]
+        // +shift, * 1/smooth, unsigned per-64 quantization: the wavefront's 128 columns are two groups
+        float *lds_rs = (float *)sbuf0;  // [BN]
+        __syncthreads();                // transposition tiles / staged output are no longer read
         if (tid < BN) lds_rs[tid] = has_sm ? 1.0f / T::to_f32(smv) : 1.0f;
         __syncthreads();
-        const int g = nw0 / GROUP;
+        const int m = mw0 + l32;
 #pragma unroll
-        for (int bm = 0; bm < NBM; bm++) {
-            const int m = mw0 + bm * 32 + l32;
+        for (int gi = 0; gi < 2; gi++) {
+            const int g = (n0 + 64 * gi) / GROUP;
             float gmax = 0.0f;
 #pragma unroll
-            for (int bn = 0; bn < 2; bn++)
+            for (int b2 = 0; b2 < 2; b2++)
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
-                    const v4f rs = *(const v4f *)(lds_rs + wn * 64 + bn * 32 + 8 * j + 4 * half);
+                    const int bn = 2 * gi + b2;
+                    const v4f rs = *(const v4f *)(lds_rs + bn * 32 + 8 * j + 4 * half);
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
-                        const float v = (acc[bn][bm][4 * j + e] + a.shift) * rs[e];
-                        acc[bn][bm][4 * j + e] = v;
+                        const float v = (acc[bn][4 * j + e] + a.shift) * rs[e];
+                        acc[bn][4 * j + e] = v;
                         gmax = fmaxf(gmax, v);
                     }
                 }
@@ -610,16 +586,17 @@ __global__ __launch_bounds__(NTHREADS, 4) void gemm_w4a4_kernel(svdq_gemm_args a
             const float scale = gmax / 15.0f;
             const float safe = (scale == 0.0f) ? 1.0f : scale;
             const float rq = 1.0f / safe;
-            if (half == 0 && m < a.M && nw0 < a.N) ((uint16_t *)a.oscales)[(size_t)g * a.ld_oscales + m] = T::from_f32(scale);
+            if (half == 0 && m < a.M && n0 + 64 * gi < a.N) ((uint16_t *)a.oscales)[(size_t)g * a.ld_oscales + m] = T::from_f32(scale);
 #pragma unroll
-            for (int bn = 0; bn < 2; bn++) {
+            for (int b2 = 0; b2 < 2; b2++) {
+                const int bn = 2 * gi + b2;
                 uint32_t mine[4];
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
                     uint32_t w = 0;
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
-                        const float q = __builtin_amdgcn_fmed3f(acc[bn][bm][4 * j + e] * rq, 0.0f, 15.0f) + RNE_MAGIC;
+                        const float q = __builtin_amdgcn_fmed3f(acc[bn][4 * j + e] * rq, 0.0f, 15.0f) + RNE_MAGIC;
                         w |= (__float_as_uint(q) & 0xFu) << (4 * e);
                     }
                     mine[j] = w;  // 16 bits: columns 8 j + 4 half + 0..3
@@ -636,7 +613,7 @@ __global__ __launch_bounds__(NTHREADS, 4) void gemm_w4a4_kernel(svdq_gemm_args a
                     dw[t] = half ? (theirs | (keep << 16)) : (keep | (theirs << 16));
                 }
                 if (m < a.M)
-                    *(uint2 *)((uint8_t *)a.qout + (size_t)m * a.ld_qout + (nw0 + bn * 32) / 2 + 8 * half) =
+                    *(uint2 *)((uint8_t *)a.qout + (size_t)m * a.ld_qout + (n0 + bn * 32) / 2 + 8 * half) =
                         make_uint2(dw[0], dw[1]);
             }
         }
@@ -646,133 +623,91 @@ __global__ __launch_bounds__(NTHREADS, 4) void gemm_w4a4_kernel(svdq_gemm_args a
     if (EPI == SVDQ_EPI_SWIGLU_QUANT) {
         // Output columns come in 16-blocks [gate | up]: registers j = 0, 1 of a 32-column block are gate values and
         // j = 2, 3 the matching up values, so y = silu(gate) * up is formed in-lane.  The tile's 128 columns give 64
-        // y columns = one quantization group, shared by the two n-wavefronts (32 y columns each).
+        // y columns = one quantization group, all of it in this wavefront.
         const int H = a.N / 2;
         const uint16_t *ldt = (const uint16_t *)a.lora_down_t;
-        float y[NBM][2][8];  // [bm][bn][4 j + e]: y column 16 bn + 8 j + 4 half + e of the wavefront's 32
+        float y[NBN][8];  // [bn][4 j + e]: y column 16 bn + 8 j + 4 half + e of the tile's 64
 #pragma unroll
-        for (int bm = 0; bm < NBM; bm++)
+        for (int bn = 0; bn < NBN; bn++)
 #pragma unroll
-            for (int bn = 0; bn < 2; bn++)
-#pragma unroll
-                for (int i = 0; i < 8; i++) y[bm][bn][i] = silu(acc[bn][bm][i]) * acc[bn][bm][8 + i];
-        const int yt0 = n0 / 2;          // first y column of the tile
-        const int yw0 = yt0 + 32 * wn;   // ... of this wavefront
-        float *lds_part = (float *)smem;  // [4 (wm)][16 regs][64 lanes] floats = 16 KB
-        __syncthreads();
+            for (int i = 0; i < 8; i++) y[bn][i] = silu(acc[bn][i]) * acc[bn][8 + i];
+        const int yt0 = n0 / 2;  // first y column of the tile
+        const int m = mw0 + l32;
         for (int rc = 0; rc < a.R2; rc += 32) {
-            v16f d[NBM];
+            v16f d;
 #pragma unroll
-            for (int bm = 0; bm < NBM; bm++)
-#pragma unroll
-                for (int i = 0; i < 16; i++) d[bm][i] = 0.0f;
+            for (int i = 0; i < 16; i++) d[i] = 0.0f;
             const int r = rc + l32;
 #pragma unroll
-            for (int s = 0; s < 2; s++) {
+            for (int s = 0; s < NBN; s++) {
                 v4i la = (v4i){0, 0, 0, 0};
                 if (r < a.R2) {
-                    const uint16_t *lp = ldt + (size_t)r * H + yw0 + 16 * s + 4 * half;
+                    const uint16_t *lp = ldt + (size_t)r * H + yt0 + 16 * s + 4 * half;
                     const uint2 q0 = *(const uint2 *)lp, q1 = *(const uint2 *)(lp + 8);
                     la = (v4i){(int)q0.x, (int)q0.y, (int)q1.x, (int)q1.y};
                 }
+                v4i xb;
 #pragma unroll
-                for (int bm = 0; bm < NBM; bm++) {
-                    v4i xb;
-#pragma unroll
-                    for (int e = 0; e < 4; e++) xb[e] = (int)pack2<T>(y[bm][s][2 * e], y[bm][s][2 * e + 1]);
-                    d[bm] = mfma32_16bit<T>(la, xb, d[bm]);
-                }
+                for (int e = 0; e < 4; e++) xb[e] = (int)pack2<T>(y[s][2 * e], y[s][2 * e + 1]);
+                d = mfma32_16bit<T>(la, xb, d);
             }
-            if (wn == 1) {
 #pragma unroll
-                for (int bm = 0; bm < NBM; bm++)
-#pragma unroll
-                    for (int i = 0; i < 16; i++) lds_part[((wm * NBM + bm) * 16 + i) * 64 + lane] = d[bm][i];
+            for (int j = 0; j < 4; j++) {
+                const int rr = rc + 8 * j + 4 * half;
+                if (m < a.M && rr < a.R2)
+                    *(v4f *)(a.scratch + ((size_t)pid_n * a.M + m) * a.R2 + rr) = (v4f){d[4 * j], d[4 * j + 1], d[4 * j + 2], d[4 * j + 3]};
             }
-            __syncthreads();
-            if (wn == 0) {
-#pragma unroll
-                for (int bm = 0; bm < NBM; bm++) {
-                    const int m = mw0 + bm * 32 + l32;
-#pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        v4f o;
-#pragma unroll
-                        for (int e = 0; e < 4; e++)
-                            o[e] = d[bm][4 * j + e] + lds_part[((wm * NBM + bm) * 16 + 4 * j + e) * 64 + lane];
-                        const int rr = rc + 8 * j + 4 * half;
-                        if (m < a.M && rr < a.R2)
-                            *(v4f *)(a.scratch + ((size_t)pid_n * a.M + m) * a.R2 + rr) = o;
-                    }
-                }
-            }
-            __syncthreads();
         }
 
         // * 1/smooth, signed per-64 quantization over the tile's 64 y columns
-        float *lds_rs = (float *)smem;        // [64]
-        float *lds_max = (float *)smem + 64;  // [2 (wn)][BM]
+        float *lds_rs = (float *)sbuf0;  // [64]
+        __syncthreads();                // transposition tiles are no longer read
         if (tid < 64) {
             float rs = 1.0f;
             if (a.smooth_next != nullptr) rs = 1.0f / T::to_f32(((const uint16_t *)a.smooth_next)[yt0 + tid]);
             lds_rs[tid] = rs;
         }
         __syncthreads();
-        float gm[2];
+        float gmax = 0.0f;
 #pragma unroll
-        for (int bm = 0; bm < NBM; bm++) {
-            float gmax = 0.0f;
+        for (int bn = 0; bn < NBN; bn++)
 #pragma unroll
-            for (int bn = 0; bn < 2; bn++)
+            for (int j = 0; j < 2; j++) {
+                const v4f rs = *(const v4f *)(lds_rs + 16 * bn + 8 * j + 4 * half);
 #pragma unroll
-                for (int j = 0; j < 2; j++) {
-                    const v4f rs = *(const v4f *)(lds_rs + 32 * wn + 16 * bn + 8 * j + 4 * half);
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        const float v = (y[bm][bn][4 * j + e] + a.shift) * rs[e];
-                        y[bm][bn][4 * j + e] = v;
-                        gmax = fmaxf(gmax, fabsf(v));
-                    }
+                for (int e = 0; e < 4; e++) {
+                    const float v = (y[bn][4 * j + e] + a.shift) * rs[e];
+                    y[bn][4 * j + e] = v;
+                    gmax = fmaxf(gmax, fabsf(v));
                 }
-            gmax = fmaxf(gmax, __shfl_xor(gmax, 32));
-            if (half == 0) lds_max[wn * BM + wm * WROWS + bm * 32 + l32] = gmax;
-            gm[bm] = gmax;
-        }
-        __syncthreads();
-#pragma unroll
-        for (int bm = 0; bm < NBM; bm++) {
-            const int ml = wm * WROWS + bm * 32 + l32;
-            const int m = m0 + ml;
-            const float gmax = fmaxf(lds_max[ml], lds_max[BM + ml]);
-            const float scale = gmax / 7.0f;
-            const float safe = (scale == 0.0f) ? 1.0f : scale;
-            const float rq = 1.0f / safe;
-            if (wn == 0 && half == 0 && m < a.M)
-                ((uint16_t *)a.oscales)[(size_t)(yt0 / GROUP) * a.ld_oscales + m] = T::from_f32(scale);
-#pragma unroll
-            for (int bn = 0; bn < 2; bn++) {
-                uint32_t mine[2];
-#pragma unroll
-                for (int j = 0; j < 2; j++) {
-                    uint32_t w = 0;
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        const float q = __builtin_amdgcn_fmed3f(y[bm][bn][4 * j + e] * rq, -8.0f, 7.0f) + RNE_MAGIC;
-                        w |= (__float_as_uint(q) & 0xFu) << (4 * e);
-                    }
-                    mine[j] = w;  // 16 bits: y columns 16 bn + 8 j + 4 half + 0..3
-                }
-                // dword j of the block's 8-byte run = piece of half 0 (low 16 bits) | piece of half 1 (high 16 bits);
-                // half h keeps dword h
-                const uint32_t keep = half ? mine[1] : mine[0];
-                const uint32_t send = half ? mine[0] : mine[1];
-                const uint32_t theirs = __shfl_xor(send, 32);
-                const uint32_t dw = half ? (theirs | (keep << 16)) : (keep | (theirs << 16));
-                if (m < a.M)
-                    *(uint32_t *)((uint8_t *)a.qout + (size_t)m * a.ld_qout + (yw0 + 16 * bn) / 2 + 4 * half) = dw;
             }
+        gmax = fmaxf(gmax, __shfl_xor(gmax, 32));
+        const float scale = gmax / 7.0f;
+        const float safe = (scale == 0.0f) ? 1.0f : scale;
+        const float rq = 1.0f / safe;
+        if (half == 0 && m < a.M) ((uint16_t *)a.oscales)[(size_t)(yt0 / GROUP) * a.ld_oscales + m] = T::from_f32(scale);
+#pragma unroll
+        for (int bn = 0; bn < NBN; bn++) {
+            uint32_t mine[2];
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                uint32_t w = 0;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const float q = __builtin_amdgcn_fmed3f(y[bn][4 * j + e] * rq, -8.0f, 7.0f) + RNE_MAGIC;
+                    w |= (__float_as_uint(q) & 0xFu) << (4 * e);
+                }
+                mine[j] = w;  // 16 bits: y columns 16 bn + 8 j + 4 half + 0..3
+            }
+            // dword j of the block's 8-byte run = piece of half 0 (low 16 bits) | piece of half 1 (high 16 bits);
+            // half h keeps dword h
+            const uint32_t keep = half ? mine[1] : mine[0];
+            const uint32_t send = half ? mine[0] : mine[1];
+            const uint32_t theirs = __shfl_xor(send, 32);
+            const uint32_t dw = half ? (theirs | (keep << 16)) : (keep | (theirs << 16));
+            if (m < a.M)
+                *(uint32_t *)((uint8_t *)a.qout + (size_t)m * a.ld_qout + (yt0 + 16 * bn) / 2 + 4 * half) = dw;
         }
-        (void)gm;
         return;
     }
 }
