@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define SVDQ_ABI_VERSION 3
+#define SVDQ_ABI_VERSION 4
 
 enum { SVDQ_BF16 = 0, SVDQ_FP16 = 1 };
 enum { SVDQ_PRE_NONE = 0, SVDQ_PRE_GLU = 1, SVDQ_PRE_GELU = 2 }; /* svdq_quantize_args.prologue */
@@ -161,6 +161,18 @@ size_t svdq_weight_planes_bytes(int32_t N, int32_t K);
 
 /* Bytes of `scratch` needed by a requantizing epilogue with LoRA-down (0 when R2 == 0). */
 size_t svdq_gemm_w4a4_scratch_bytes(int32_t M, int32_t N, int32_t R2, int32_t epilogue);
+
+/*
+ * svdq_gemm_w4a4 for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  No counterpart in the reference.  `args->scratch` is ignored: the LoRA-down partial
+ * sums go to a buffer of SVDQ_STATIC_SCRATCH_BYTES built into the library (one per GPU, held until the process
+ * ends).  Returns SVDQ_E_UNSUPPORTED when svdq_gemm_w4a4_scratch_bytes(M, N, R2, epilogue) exceeds it.  Calls no
+ * hipMalloc / hipFree.  All calls on one GPU share the buffer: calls that overlap in time on one GPU (two streams) race;
+ * calls on one stream are ordered.  Results are bit-identical to svdq_gemm_w4a4's.
+ */
+#define SVDQ_STATIC_SCRATCH_BYTES (16u << 20)
+int svdq_gemm_w4a4_static_scratch(const svdq_gemm_args *args, void *stream);
+size_t svdq_gemm_w4a4_static_scratch_capacity(void);
 
 /*
  * Debug: exact int32 accumulators of one scale group, p[m, n] = sum_{k in group g} a[m, k] * w[n, k], computed by

@@ -14,7 +14,7 @@ import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libsvdq_mi355x.so")
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 BF16, FP16 = 0, 1
 EPI_PLAIN, EPI_QK_NORM_ROPE, EPI_GELU_QUANT, EPI_SWIGLU_QUANT = 0, 1, 2, 3
@@ -28,6 +28,8 @@ EXPORTS = (
     "svdq_transpose_lora_down",
     "svdq_gemm_w4a4",
     "svdq_gemm_w4a4_scratch_bytes",
+    "svdq_gemm_w4a4_static_scratch",
+    "svdq_gemm_w4a4_static_scratch_capacity",
     "svdq_split_weight_planes",
     "svdq_weight_planes_bytes",
     "svdq_group_acc_i32",
@@ -123,6 +125,9 @@ def load() -> ctypes.CDLL:
     lib.svdq_row_stats.argtypes = [_vp, _vp, _i32, _i32, _i32, _i32, _f32, _vp]
     lib.svdq_quantize_act.argtypes = [ctypes.POINTER(QuantizeArgs), _vp]
     lib.svdq_gemm_w4a4.argtypes = [ctypes.POINTER(GemmArgs), _vp]
+    lib.svdq_gemm_w4a4_static_scratch.argtypes = [ctypes.POINTER(GemmArgs), _vp]
+    lib.svdq_gemm_w4a4_static_scratch_capacity.restype = ctypes.c_size_t
+    lib.svdq_gemm_w4a4_static_scratch_capacity.argtypes = []
     lib.svdq_awq_gemv_w4a16.argtypes = [ctypes.POINTER(AwqGemvArgs), _vp]
     lib.svdq_awq_dequantize.argtypes = [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _vp]
     lib.svdq_attention_fp16.argtypes = [ctypes.POINTER(AttentionArgs), _vp]

@@ -34,6 +34,7 @@
 //    lane order); their half of the unpack then disappears from the inner loop.
 //  * Workgroup ids are first regrouped so that each XCD (ids are dealt round-robin over 8 XCDs) works on a
 //    contiguous range of tiles, then swizzled in bands of m-tiles for L2 reuse of the weight tile.
+#include <atomic>
 #include <type_traits>
 
 #include "svdq_common.h"
@@ -828,12 +829,7 @@ extern "C" size_t svdq_gemm_w4a4_scratch_bytes(int32_t M, int32_t N, int32_t R2,
     return (size_t)((N + BN - 1) / BN) * (size_t)M * (size_t)R2 * sizeof(float);
 }
 
-extern "C" int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream) {
-    if (!args) {
-        set_error("svdq_gemm_w4a4: null args");
-        return SVDQ_E_INVALID;
-    }
-    const svdq_gemm_args &a = *args;
+static int gemm_w4a4_checked(const svdq_gemm_args &a, void *stream) {
     if (a.dtype != SVDQ_BF16 && a.dtype != SVDQ_FP16) {
         set_error("svdq_gemm_w4a4: dtype %d", a.dtype);
         return SVDQ_E_INVALID;
@@ -941,6 +937,59 @@ extern "C" int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream) {
         rc = check_launch("svdq_gemm_w4a4 (LoRA-down partial sum)");
     }
     return rc;
+}
+
+extern "C" int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream) {
+    if (!args) {
+        set_error("svdq_gemm_w4a4: null args");
+        return SVDQ_E_INVALID;
+    }
+    return gemm_w4a4_checked(*args, stream);
+}
+
+// ---- the same GEMM for callers that cannot allocate --------------------------------------------------------------
+// The LoRA-down partial sums of the requantizing epilogues live in a file-scope device array instead of a buffer the
+// caller brings.  In host code the array's name is only a stand-in; its device address is looked up once per device,
+// with that device current, and that pointer is what the kernels get.
+constexpr size_t STATIC_SCRATCH_BYTES = SVDQ_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+constexpr int MAX_DEVICES = 64;
+static std::atomic<void *> g_scratch_ptr[MAX_DEVICES];
+
+extern "C" size_t svdq_gemm_w4a4_static_scratch_capacity(void) { return STATIC_SCRATCH_BYTES; }
+
+extern "C" int svdq_gemm_w4a4_static_scratch(const svdq_gemm_args *args, void *stream) {
+    if (!args) {
+        set_error("svdq_gemm_w4a4_static_scratch: null args");
+        return SVDQ_E_INVALID;
+    }
+    svdq_gemm_args a = *args;
+    const size_t need = svdq_gemm_w4a4_scratch_bytes(a.M, a.N, a.R2, a.epilogue);
+    if (need > STATIC_SCRATCH_BYTES) {
+        set_error("svdq_gemm_w4a4_static_scratch: M=%d N=%d R2=%d needs %zu bytes of LoRA-down partial sums, the built-in "
+                  "buffer holds %zu; use svdq_gemm_w4a4 with a caller-provided scratch", a.M, a.N, a.R2, need,
+                  STATIC_SCRATCH_BYTES);
+        return SVDQ_E_UNSUPPORTED;
+    }
+    a.scratch = nullptr;
+    if (need > 0) {
+        int dev = -1;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
+            set_error("svdq_gemm_w4a4_static_scratch: no current device (or device index above %d)", MAX_DEVICES - 1);
+            return SVDQ_E_LAUNCH;
+        }
+        void *ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+        if (ptr == nullptr) {  // first call on this device: every device holds its own copy of the array
+            const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+            if (e != hipSuccess || ptr == nullptr) {
+                set_error("svdq_gemm_w4a4_static_scratch: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+                return SVDQ_E_LAUNCH;
+            }
+            g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+        }
+        a.scratch = (float *)ptr;  // every (tile, row, rank) entry the reduction reads is written first: nothing to clear
+    }
+    return gemm_w4a4_checked(a, stream);
 }
 
 extern "C" int svdq_group_acc_i32(const void *act, const void *wgt, int32_t *out, int32_t M, int32_t N, int32_t K,

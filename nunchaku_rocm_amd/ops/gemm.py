@@ -12,6 +12,12 @@ from ._prep import weight_planes as _weight_planes
 # streams those; False makes the GEMM unpack the packed weight itself (no extra memory, about 15% slower).
 USE_WEIGHT_PLANES = True
 
+# True sends the requantizing epilogues' LoRA-down partial sums to the buffer built into the library
+# (svdq_gemm_w4a4_static_scratch) instead of a torch allocation per call: for callers that may not allocate, e.g. while
+# a HIP graph is being captured.  The buffer holds 16 MiB (about M * N / 128 * R2 * 4 bytes are needed) and is shared
+# by every call on the GPU, so calls on two streams must not overlap.
+STATIC_SCRATCH = False
+
 HEAD_DIM = 128
 GELU_SHIFT = 0.171875
 
@@ -206,10 +212,13 @@ def svdq_gemm_w4a4_cuda(
                 raise ValueError("lora_act_out must be (>= M, R2) fp32")
             ldt = _lora_down_t(lora_down)
             epi = _lib.EPI_SWIGLU_QUANT if fuse_swiglu else _lib.EPI_GELU_QUANT
-            nbytes = lib.svdq_gemm_w4a4_scratch_bytes(M, N, R2, epi)
-            scratch = torch.empty(nbytes // 4, dtype=torch.float32, device=dev)
-            keep += [ldt, scratch]
-            args.lora_down_t, args.lora_act_out, args.scratch = ldt.data_ptr(), lora_act_out.data_ptr(), scratch.data_ptr()
+            keep.append(ldt)
+            args.lora_down_t, args.lora_act_out = ldt.data_ptr(), lora_act_out.data_ptr()
+            if not STATIC_SCRATCH:
+                nbytes = lib.svdq_gemm_w4a4_scratch_bytes(M, N, R2, epi)
+                scratch = torch.empty(nbytes // 4, dtype=torch.float32, device=dev)
+                keep.append(scratch)
+                args.scratch = scratch.data_ptr()
             args.ld_lora_act_out = lora_act_out.stride(0)
         args.epilogue = _lib.EPI_SWIGLU_QUANT if fuse_swiglu else _lib.EPI_GELU_QUANT
         args.qout, args.oscales, args.smooth_next = qout2d.data_ptr(), oscales.data_ptr(), _lib.ptr(smooth_factor)
@@ -217,7 +226,8 @@ def svdq_gemm_w4a4_cuda(
         args.shift = 0.0 if fuse_swiglu else GELU_SHIFT
 
     with torch.cuda.device(dev):
-        _lib.check(lib.svdq_gemm_w4a4(args, _lib.stream_of(act)))
+        entry = lib.svdq_gemm_w4a4_static_scratch if STATIC_SCRATCH else lib.svdq_gemm_w4a4
+        _lib.check(entry(args, _lib.stream_of(act)))
     return None
 
 
