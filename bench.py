@@ -126,7 +126,9 @@ def main():
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
     M, K, N, R = 4608, 3072, 9216, 32
-    lin = {k: v.to(dev) for k, v in O.make_svdq_linear(K, N, R, seed=0).items()}
+    # weights as module parameters, which is what the operators see in a model (the GEMM keeps its re-laid-out working
+    # copy per parameter)
+    lin = {k: torch.nn.Parameter(v.to(dev), requires_grad=False) for k, v in O.make_svdq_linear(K, N, R, seed=0).items()}
     x = O.make_activations(M, K, seed=1).to(dev)
     qx = torch.empty(M, K // 2, dtype=torch.uint8, device=dev)
     asc = torch.empty(K // 64, M, dtype=torch.bfloat16, device=dev)

@@ -108,7 +108,8 @@ int svdq_transpose_lora_down(const void *lora_down, void *lora_down_t, int32_t K
                              void *stream);
 
 /*
- * W4A4 GEMM: out[m, n] = sum_g as[g, m] * ws[g, n] * (sum_{k in g} a[m, k] w[n, k])  (int8 MFMA, exact int32 per group)
+ * W4A4 GEMM: out[m, n] = sum_g as[g, m] * ws[g, n] * (sum_{k in g} a[m, k] w[n, k])  (exact integer per group: int8 MFMA
+ *                        on packed weights, fp8 MFMA on int4-valued codes with pre-split weights)
  *                        + T(lora_act[m, :]) . lora_up[n, :] + bias[n],  then the epilogue.
  * Reference arithmetic: ops/triton/gemm_w4a4.py:447-488 (main loop), 156-209 (epilogue), 499-521 (QK), 730-778
  * (GELU + requantization), 998-1000 (SwiGLU semantics).
@@ -116,8 +117,9 @@ int svdq_transpose_lora_down(const void *lora_down, void *lora_down_t, int32_t K
 typedef struct {
     const void *act;        /* (M, K/2) packed int4, row stride ld_act bytes (multiple of 16, base 16-B aligned) */
     const void *wgt;        /* (N, K/2) packed signed int4, row stride ld_wgt bytes (same alignment)            */
-    const void *wgt_planes; /* optional: the same weights re-laid-out by svdq_split_weight_planes (then `wgt` is  */
-                            /* not read); NULL = unpack `wgt` inside the GEMM                                    */
+    const void *wgt_planes; /* optional: the same weights and `wscales` re-laid-out by svdq_split_weight_planes  */
+                            /* (then `wgt` is not read, fp8 main loop); NULL = unpack `wgt` inside the GEMM      */
+                            /* (int8 main loop)                                                                  */
     const void *ascales;    /* (K/64, >= M) T, group stride ld_ascales elements                                 */
     const void *wscales;    /* (K/64, >= N) T, group stride ld_wscales elements                                 */
     const void *bias;       /* (N,) T or NULL                                                                   */
@@ -151,12 +153,18 @@ typedef struct {
 int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream);
 
 /*
- * One-time re-layout of a weight for the GEMM: every (32-row block, scale group) becomes two 1 KB int8 planes (even and
- * odd nibbles, each value times 16) in the order the MFMA lanes read them, so the GEMM streams the weight tile into
- * LDS without touching it.  `planes` needs svdq_weight_planes_bytes(N, K) bytes (= ceil(N/32)*32 * K).  No
+ * One-time re-layout of a weight for the GEMM.  Every (32-row block, scale group) becomes two 1 KB planes (even and odd
+ * nibbles) of fp8 (e4m3) codes in the order the MFMA lanes read them: a signed int4 value v is stored as the byte
+ * sign | |v|, which the fp8 matrix instruction reads as v * 2^-9 exactly (v_mfma_scale_f32_32x32x64_f8f6f4 runs at
+ * the int8 rate, takes a whole 64-deep group per instruction and returns the integer dot product as fp32, which saves
+ * the GEMM one of its two scaling multiplies per output and group).  Behind the planes sit, per weight row, three T
+ * pieces per group that add up to -8 * ws[g, n] * (sum of the group's 64 weights): the GEMM offsets signed activations by
+ * +8 for the fp8 operand and takes that term out again.  `planes` needs svdq_weight_planes_bytes(N, K) bytes
+ * (= ceil(N/32)*32 * (K + 6 * ceil(K/1024)*16)).  The copy depends on `wgt` AND `wscales` (dtype = their type).  No
  * counterpart in the reference (its SwiGLU path re-orders weight rows at load in the same spirit, ops/fused.py:83-105).
  */
-int svdq_split_weight_planes(const void *wgt, void *planes, int32_t N, int32_t K, int32_t ld_wgt, void *stream);
+int svdq_split_weight_planes(const void *wgt, const void *wscales, void *planes, int32_t N, int32_t K, int32_t ld_wgt,
+                             int32_t ld_wscales, int32_t dtype, void *stream);
 size_t svdq_weight_planes_bytes(int32_t N, int32_t K);
 
 /* Bytes of `scratch` needed by a requantizing epilogue with LoRA-down (0 when R2 == 0). */
@@ -176,10 +184,12 @@ size_t svdq_gemm_w4a4_static_scratch_capacity(void);
 
 /*
  * Debug: exact int32 accumulators of one scale group, p[m, n] = sum_{k in group g} a[m, k] * w[n, k], computed by
- * the same nibble unpack + v_mfma_i32_32x32x32_i8 sequence the GEMM uses.  out (M, N) int32 row-major.
+ * the instruction sequence of one of the GEMM's two main loops: path 0 = nibble unpack + v_mfma_i32_32x32x32_i8 (packed
+ * weights), path 1 = fp8 codes + v_mfma_scale_f32_32x32x64_f8f6f4 with the +8 offset of signed activations taken out
+ * (pre-split weights).  out (M, N) int32 row-major.
  */
 int svdq_group_acc_i32(const void *act, const void *wgt, int32_t *out, int32_t M, int32_t N, int32_t K,
-                       int32_t ld_act, int32_t ld_wgt, int32_t group, int32_t act_unsigned, void *stream);
+                       int32_t ld_act, int32_t ld_wgt, int32_t group, int32_t act_unsigned, int32_t path, void *stream);
 
 /*
  * AWQ W4A16 GEMV, group 64, TinyChat packing (models/text_encoders/tinychat_utils.py:76-106):

@@ -120,7 +120,7 @@ def load() -> ctypes.CDLL:
     lib.svdq_gemm_w4a4_scratch_bytes.argtypes = [_i32, _i32, _i32, _i32]
     lib.svdq_weight_planes_bytes.restype = ctypes.c_size_t
     lib.svdq_weight_planes_bytes.argtypes = [_i32, _i32]
-    lib.svdq_split_weight_planes.argtypes = [_vp, _vp, _i32, _i32, _i32, _vp]
+    lib.svdq_split_weight_planes.argtypes = [_vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _vp]
     lib.svdq_gated_residual.argtypes = [_vp] * 6 + [_i32] * 9 + [_f32, _f32, _vp]
     lib.svdq_row_stats.argtypes = [_vp, _vp, _i32, _i32, _i32, _i32, _f32, _vp]
     lib.svdq_quantize_act.argtypes = [ctypes.POINTER(QuantizeArgs), _vp]
@@ -137,7 +137,7 @@ def load() -> ctypes.CDLL:
     lib.svdq_unpack_mma_scale.argtypes = [_vp, _vp, _i32, _i32, _i32, _vp]
     lib.svdq_unpack_mma_lowrank.argtypes = [_vp, _vp, _i32, _i32, _i32, _i32, _vp]
     lib.svdq_transpose_lora_down.argtypes = [_vp, _vp, _i32, _i32, _i32, _vp]
-    lib.svdq_group_acc_i32.argtypes = [_vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp]
+    lib.svdq_group_acc_i32.argtypes = [_vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp]
     if lib.svdq_abi_version() != ABI_VERSION:
         raise RuntimeError(f"{LIB_PATH} has ABI version {lib.svdq_abi_version()}, expected {ABI_VERSION}: rebuild it")
     _lib = lib

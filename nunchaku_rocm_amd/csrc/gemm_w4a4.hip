@@ -61,6 +61,7 @@ constexpr int NBN = BN / 32;                        // 32-row weight blocks per 
 constexpr int TP_PITCH = 36;                        // floats per row of the accumulator transposition tile
 constexpr int TP_WAVE_BYTES = 2 * 32 * TP_PITCH * 4;  // two 32x32 blocks at a time
 static_assert(2 * TP_WAVE_BYTES <= BUF_BYTES, "transposition tiles do not fit");
+constexpr int F8_SCALE = (int)0x88888888;  // e8m0 block scale 2^9 in every byte: an fp8 code c (value c * 2^-9) counts as c
 constexpr int GROUP_M_TILES = 8;      // m-tiles per raster band
 constexpr int NUM_XCD = 8;
 
@@ -75,6 +76,10 @@ __device__ inline void unpack_unsigned(v4i p, v4i &even, v4i &odd) {
     even = __builtin_bit_cast(v4i, u & 0x0F0F0F0Fu);
     odd = __builtin_bit_cast(v4i, (u >> 4) & 0x0F0F0F0Fu);
 }
+
+// fp8 (e4m3) code of a signed int4 value: sign bit | magnitude in the low four bits.  A code c <= 15 stands for
+// c * 2^-9 (subnormals and the first binade form one linear run).
+__device__ inline uint32_t f8_code(int v) { return (uint32_t)((v < 0 ? 0x80 : 0) | (v < 0 ? -v : v)); }
 
 __device__ inline v16i magic_acc() {
     v16i c;
@@ -213,6 +218,25 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
         const float w = T::to_f32(rws) * fold;
         ((float2 *)(base + WS_OFF))[sg * BN + sr] = make_float2(w, -RNE_MAGIC * w);
     };
+    // Pre-split weights (fp8 path): every lane fetches the scales its two rank-1 MFMA operands need, one stage ahead,
+    // straight into registers: the activation scale of row wm * 32 + l32 and the weight scales of columns lane and
+    // 64 + lane, for both groups of the stage.  Groups past the end (odd K / 64) are staged as zero.
+    uint16_t qa[2], qw[4];
+    const uint16_t *pA = (const uint16_t *)a.ascales + min(m0 + wm * 32 + l32, a.M - 1);
+    const uint16_t *pW0 = (const uint16_t *)a.wscales + min(n0 + lane, a.N - 1);
+    const uint16_t *pW1 = (const uint16_t *)a.wscales + min(n0 + 64 + lane, a.N - 1);
+    auto load_scales8 = [&](int s) {
+#pragma unroll
+        for (int gg = 0; gg < 2; gg++) {
+            const int gi = ODDG ? min(2 * s + gg, G - 1) : 2 * s + gg;
+            const uint16_t va = pA[(size_t)gi * a.ld_ascales];
+            const uint16_t v0 = pW0[(size_t)gi * a.ld_wscales], v1 = pW1[(size_t)gi * a.ld_wscales];
+            const bool on = !ODDG || 2 * s + gg < G;
+            qa[gg] = on ? va : (uint16_t)0;
+            qw[2 * gg] = on ? v0 : (uint16_t)0;
+            qw[2 * gg + 1] = on ? v1 : (uint16_t)0;
+        }
+    };
 
     // Main-loop accumulators: MFMA A operand = activations, B operand = weights, so a lane owns one weight row n and its
     // registers walk the wavefront's 32 activation rows: the weight scale is a per-lane scalar and the 16 activation
@@ -228,7 +252,10 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
     const int offW = W_OFF + lane * 16;
     const int offA = wm * 2 * BLK_BYTES + lane * 16;
 
-    load_scales(0);
+    if constexpr (WPL)
+        load_scales8(0);
+    else
+        load_scales(0);
 #pragma unroll
     for (int i = 0; i < PER_WAVE; i++) dma_one(0, sbuf0, i);
     // epilogue operands, fetched now so that the epilogue does not wait for memory
@@ -264,66 +291,123 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
         uint8_t *other = P ? sbuf0 : sbuf1;  // being refilled for the next stage
         // everything issued for stage s (scale registers, then operand blocks) has landed
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
-        store_scales(base);
-        __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));  // scale writes visible before the barrier
+        float fa[2], fw[4];
+        if constexpr (WPL) {
+#pragma unroll
+            for (int i = 0; i < 2; i++) fa[i] = T::to_f32(qa[i]);
+#pragma unroll
+            for (int i = 0; i < 4; i++) fw[i] = T::to_f32(qw[i]);
+        } else {
+            store_scales(base);
+            __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));  // scale writes visible before the barrier
+        }
         __builtin_amdgcn_s_barrier();
         // The other buffer was last read in the previous stage, before the barrier: refill it during this stage.  The last
         // stage re-fetches itself into the idle buffer (harmless, and keeps the stage one basic block).
         const int sn = min(s + 1, nstages - 1);
-        load_scales(sn);
-        auto read_w = [&](int b, v4i &we, v4i &wo, float2 &wsp) {
-            const int gg = b >> 2, bn = b & 3;
-            if (WPL) {
-                we = *(const v4i *)(base + offW + ((bn * 2 + gg) * 2 + 0) * BLK_BYTES);
-                wo = *(const v4i *)(base + offW + ((bn * 2 + gg) * 2 + 1) * BLK_BYTES);
-            } else {
+        if constexpr (WPL)
+            load_scales8(sn);
+        else
+            load_scales(sn);
+        if constexpr (WPL) {
+            // One stage = eight (group, weight block) steps.  The matrix instructions of step b + 1 (and, at every second
+            // step, the rank-1 product of the next pair's scales) are issued ahead of the sixteen FMAs of step b.
+            auto read_w8 = [&](int b) -> v8i {
+                const int gg = b >> 2, bn = b & 3;
+                const v4i lo = *(const v4i *)(base + offW + ((bn * 2 + gg) * 2 + 0) * BLK_BYTES);
+                const v4i hi = *(const v4i *)(base + offW + ((bn * 2 + gg) * 2 + 1) * BLK_BYTES);
+                return (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            };
+            auto read_a8 = [&](int gg) -> v8i {
+                typedef unsigned v4u __attribute__((ext_vector_type(4)));
+                v4u u = __builtin_bit_cast(v4u, *(const v4i *)(base + offA + gg * BLK_BYTES));
+                if (!ACT_UNSIGNED) u ^= 0x88888888u;  // two's complement nibble -> value + 8
+                const v4u e = u & 0x0F0F0F0Fu, o = (u >> 4) & 0x0F0F0F0Fu;
+                return (v8i){(int)e[0], (int)e[1], (int)e[2], (int)e[3], (int)o[0], (int)o[1], (int)o[2], (int)o[3]};
+            };
+            auto outer = [&](int p) -> v32f {  // as[m] * ws[n] of pair p: blocks 2 (p & 1), + 1 of group p >> 1
+                v32f z;
+#pragma unroll
+                for (int i = 0; i < 32; i++) z[i] = 0.0f;
+                // both 32x32 blocks take their rows from lanes 0-31 of the first operand
+                return __builtin_amdgcn_mfma_f32_32x32x1f32(fa[p >> 1], fw[p], z, 1, 0, 0);
+            };
+            const v16f z16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+            v8i a8[2], w8[3];
+            v32f S[2];
+            v16f P[2];
+            a8[0] = read_a8(0);
+            w8[0] = read_w8(0);
+            w8[1] = read_w8(1);
+            S[0] = outer(0);
+            P[0] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8[0], w8[0], z16, 0, 0, 0, F8_SCALE, 0, F8_SCALE);
+            a8[1] = read_a8(1);
+#pragma unroll
+            for (int b = 0; b < 8; b++) {
+                const int cur = b & 1, nxt = cur ^ 1;
+                if (b + 1 < 8) {
+                    if (((b + 1) & 1) == 0) S[((b + 1) >> 1) & 1] = outer((b + 1) >> 1);
+                    P[nxt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8[(b + 1) >> 2], w8[(b + 1) % 3], z16, 0, 0, 0,
+                                                                             F8_SCALE, 0, F8_SCALE);
+                }
+                if (b + 2 < 8) w8[(b + 2) % 3] = read_w8(b + 2);
+                if (b < PER_WAVE) dma_one(sn, other, b);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int i = 0; i < 16; i++)
+                    acc[b & 3][i] = __builtin_fmaf(P[cur][i], S[(b >> 1) & 1][16 * (b & 1) + i], acc[b & 3][i]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        } else {
+            auto read_w = [&](int b, v4i &we, v4i &wo, float2 &wsp) {
+                const int gg = b >> 2, bn = b & 3;
                 const v4i wp = *(const v4i *)(base + offW + (bn * 2 + gg) * BLK_BYTES);
                 unpack_signed(wp, we, wo);
+                wsp = ((const float2 *)(base + WS_OFF))[gg * BN + bn * 32 + l32];
+            };
+            auto read_a = [&](int gg, v4i &ae, v4i &ao) {
+                const v4i ap = *(const v4i *)(base + offA + gg * BLK_BYTES);
+                if (ACT_UNSIGNED)
+                    unpack_unsigned(ap, ae, ao);
+                else
+                    unpack_signed(ap, ae, ao);
+            };
+            auto read_as = [&](int gg, v4f (&asv)[4]) {
+    #pragma unroll
+                for (int j = 0; j < 4; j++)
+                    asv[j] = *(const v4f *)((const float *)(base + AS_OFF) + gg * BM + wm * 32 + 8 * j + 4 * half);
+            };
+            v4i ae[2], ao[2], we[2], wo[2];
+            float2 wsp[2];
+            v4f asv[2][4];
+            v16i t[2];
+            read_a(0, ae[0], ao[0]);
+            read_w(0, we[0], wo[0], wsp[0]);
+            read_as(0, asv[0]);
+            read_w(1, we[1], wo[1], wsp[1]);
+            t[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ae[0], we[0], cmagic, 0, 0, 0);
+            t[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ao[0], wo[0], t[0], 0, 0, 0);
+            read_a(1, ae[1], ao[1]);
+            read_as(1, asv[1]);
+    #pragma unroll
+            for (int b = 0; b < 8; b++) {
+                const int cur = b & 1, nxt = cur ^ 1;
+                float2 wcur = wsp[cur];
+                if (b + 1 < 8) {
+                    const int g1 = (b + 1) >> 2;
+                    t[nxt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ae[g1], we[nxt], cmagic, 0, 0, 0);
+                    t[nxt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ao[g1], wo[nxt], t[nxt], 0, 0, 0);
+                }
+                if (b + 2 < 8) read_w(b + 2, we[cur], wo[cur], wsp[cur]);
+                if (b < PER_WAVE) dma_one(sn, other, b);
+                __builtin_amdgcn_sched_barrier(0);
+    #pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    const float u = __builtin_fmaf(__int_as_float(t[cur][i]), wcur.x, wcur.y);
+                    acc[b & 3][i] = __builtin_fmaf(u, asv[b >> 2][i >> 2][i & 3], acc[b & 3][i]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
-            wsp = ((const float2 *)(base + WS_OFF))[gg * BN + bn * 32 + l32];
-        };
-        auto read_a = [&](int gg, v4i &ae, v4i &ao) {
-            const v4i ap = *(const v4i *)(base + offA + gg * BLK_BYTES);
-            if (ACT_UNSIGNED)
-                unpack_unsigned(ap, ae, ao);
-            else
-                unpack_signed(ap, ae, ao);
-        };
-        auto read_as = [&](int gg, v4f (&asv)[4]) {
-#pragma unroll
-            for (int j = 0; j < 4; j++)
-                asv[j] = *(const v4f *)((const float *)(base + AS_OFF) + gg * BM + wm * 32 + 8 * j + 4 * half);
-        };
-        v4i ae[2], ao[2], we[2], wo[2];
-        float2 wsp[2];
-        v4f asv[2][4];
-        v16i t[2];
-        read_a(0, ae[0], ao[0]);
-        read_w(0, we[0], wo[0], wsp[0]);
-        read_as(0, asv[0]);
-        read_w(1, we[1], wo[1], wsp[1]);
-        t[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ae[0], we[0], cmagic, 0, 0, 0);
-        t[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ao[0], wo[0], t[0], 0, 0, 0);
-        read_a(1, ae[1], ao[1]);
-        read_as(1, asv[1]);
-#pragma unroll
-        for (int b = 0; b < 8; b++) {
-            const int cur = b & 1, nxt = cur ^ 1;
-            float2 wcur = wsp[cur];
-            if (b + 1 < 8) {
-                const int g1 = (b + 1) >> 2;
-                t[nxt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ae[g1], we[nxt], cmagic, 0, 0, 0);
-                t[nxt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ao[g1], wo[nxt], t[nxt], 0, 0, 0);
-            }
-            if (b + 2 < 8) read_w(b + 2, we[cur], wo[cur], wsp[cur]);
-            if (b < PER_WAVE) dma_one(sn, other, b);
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int i = 0; i < 16; i++) {
-                const float u = __builtin_fmaf(__int_as_float(t[cur][i]), wcur.x, wcur.y);
-                acc[b & 3][i] = __builtin_fmaf(u, asv[b >> 2][i >> 2][i & 3], acc[b & 3][i]);
-            }
-            __builtin_amdgcn_sched_barrier(0);
         }
     };
     {
@@ -336,6 +420,36 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
     }
     // The last stage's (redundant) block loads of this wavefront have landed.
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
+
+    // ---- fp8 path, signed activations: take the +8 offset out again -------------------------------------------------
+    // sum_g as[g, m] ws[g, n] sum_k (a + 8) w  =  wanted  +  sum_g as[g, m] * (8 ws[g, n] W[g, n]),  W = the weights' group
+    // sums.  svdq_split_weight_planes stored D[g, n] = -8 ws[g, n] W[g, n] behind the planes as three 16-bit pieces
+    // that add up to the fp32 value exactly, K-contiguous per weight row like a LoRA-up matrix of rank 3 * G16; the
+    // activation scales are the other operand.  Products of two 16-bit values are exact, the sum is fp32.
+    if constexpr (WPL && !ACT_UNSIGNED) {
+        const int G16 = (G + 15) / 16 * 16, KC = 3 * G16;
+        const int npad = (a.N + 31) / 32 * 32;
+        const uint16_t *dp = (const uint16_t *)((const uint8_t *)a.wgt_planes + (size_t)npad * a.K);
+        const uint16_t *ap = (const uint16_t *)a.ascales + min(m0 + wm * 32 + l32, a.M - 1);
+        for (int g0 = 0; g0 < G16; g0 += 16) {
+            uint16_t av[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) av[j] = ap[(size_t)min(g0 + 8 * half + j, G - 1) * a.ld_ascales];
+            v4i db[3][NBN];
+#pragma unroll
+            for (int pc = 0; pc < 3; pc++)
+#pragma unroll
+                for (int bn = 0; bn < NBN; bn++)
+                    db[pc][bn] = *(const v4i *)(dp + (size_t)min(n0 + bn * 32 + l32, npad - 1) * KC + pc * G16 + g0 + 8 * half);
+            v4i ub;
+#pragma unroll
+            for (int e = 0; e < 4; e++) ub[e] = (int)((uint32_t)av[2 * e] | ((uint32_t)av[2 * e + 1] << 16));
+#pragma unroll
+            for (int pc = 0; pc < 3; pc++)
+#pragma unroll
+                for (int bn = 0; bn < NBN; bn++) acc[bn] = mfma32_16bit<T>(ub, db[pc][bn], acc[bn]);
+        }
+    }
 
     // ---- LoRA-up and bias, still in the main loop's orientation (lane = weight row, registers = activation rows) ----
     // The bias and the first 32 ranks of both LoRA operands were fetched into LDS next to stage 0 and arrived long ago;
@@ -751,6 +865,50 @@ __global__ __launch_bounds__(64) void group_acc_kernel(const uint8_t *act, const
     }
 }
 
+// The same read-out through the instruction sequence of the pre-split (fp8) path: nibbles as fp8 codes, activations
+// offset by 8 when signed, v_mfma_scale_f32_32x32x64_f8f6f4 with block scales 2^9, offset taken out with the weights'
+// group sum.  Every value involved is an integer below 2^24, so the fp32 result is exact.
+template <bool ACT_UNSIGNED>
+__global__ __launch_bounds__(64) void group_acc_f8_kernel(const uint8_t *act, const uint8_t *wgt, int32_t *out, int M,
+                                                          int N, int ld_act, int ld_wgt, int group) {
+    typedef unsigned v4u __attribute__((ext_vector_type(4)));
+    const int lane = threadIdx.x, l32 = lane & 31, half = lane >> 5;
+    const int nb = blockIdx.x * 32, mb = blockIdx.y * 32;
+    const v4i wp = *(const v4i *)(wgt + (size_t)min(nb + l32, N - 1) * ld_wgt + group * 32 + half * 16);
+    v4u u = __builtin_bit_cast(v4u, *(const v4i *)(act + (size_t)min(mb + l32, M - 1) * ld_act + group * 32 + half * 16));
+    if (!ACT_UNSIGNED) u ^= 0x88888888u;
+    const v4u e = u & 0x0F0F0F0Fu, o = (u >> 4) & 0x0F0F0F0Fu;
+    const v8i a8 = {(int)e[0], (int)e[1], (int)e[2], (int)e[3], (int)o[0], (int)o[1], (int)o[2], (int)o[3]};
+    v8i w8;
+    int wsum = 0;
+#pragma unroll
+    for (int d = 0; d < 4; d++) {
+        uint32_t we = 0, wo = 0;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int by = (wp[d] >> (8 * j)) & 0xFF;
+            const int lo = ((by & 0xF) ^ 8) - 8, hi = ((by >> 4) ^ 8) - 8;
+            wsum += lo + hi;
+            we |= f8_code(lo) << (8 * j);
+            wo |= f8_code(hi) << (8 * j);
+        }
+        w8[d] = (int)we;
+        w8[4 + d] = (int)wo;
+    }
+    wsum += __shfl_xor(wsum, 32);  // the other half of the group
+    const v16f z16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    v16f t = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8, w8, z16, 0, 0, 0, F8_SCALE, 0, F8_SCALE);
+    // The matrix instruction reads the operands of all 64 lanes: pin it here, ahead of the lane-dependent stores below
+    // (moved behind a divergent branch, it ran with some lanes' operands never loaded).
+    asm volatile("" : "+v"(t));
+    const int n = nb + l32;
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        const int m = mb + 8 * (i >> 2) + 4 * half + (i & 3);
+        if (m < M && n < N) out[(size_t)m * N + n] = (int)t[i] - (ACT_UNSIGNED ? 0 : 8 * wsum);
+    }
+}
+
 template <typename T, bool U, bool WPL, bool ODDG>
 static void launch_gemm_epi3(const svdq_gemm_args &a, hipStream_t s) {
     const dim3 grid(((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN)), block(NTHREADS);
@@ -786,7 +944,7 @@ static void launch_gemm_epi(const svdq_gemm_args &a, hipStream_t s) {
         launch_gemm_epi2<T, U, false>(a, s);
 }
 
-// weight re-layout: thread (block of 32 rows, group, lane) splits its 16 packed bytes into the even / odd planes
+// weight re-layout: thread (block of 32 rows, group, lane) turns its 16 packed bytes into the even / odd planes
 __global__ void split_weight_planes_kernel(const uint8_t *wgt, uint8_t *planes, int N, int G, int ld_wgt) {
     const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int lane = idx & 63;
@@ -796,9 +954,51 @@ __global__ void split_weight_planes_kernel(const uint8_t *wgt, uint8_t *planes, 
     const int row = min(nblk * 32 + (lane & 31), N - 1);
     const v4i p = *(const v4i *)(wgt + (size_t)row * ld_wgt + g * 32 + (lane >> 5) * 16);
     v4i even, odd;
-    unpack_signed(p, even, odd);
+#pragma unroll
+    for (int d = 0; d < 4; d++) {
+        uint32_t e = 0, o = 0;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int by = (p[d] >> (8 * j)) & 0xFF;
+            e |= f8_code(((by & 0xF) ^ 8) - 8) << (8 * j);
+            o |= f8_code(((by >> 4) ^ 8) - 8) << (8 * j);
+        }
+        even[d] = (int)e;
+        odd[d] = (int)o;
+    }
     *(v4i *)(planes + ((bg * 2 + 0) * 64 + lane) * 16) = even;
     *(v4i *)(planes + ((bg * 2 + 1) * 64 + lane) * 16) = odd;
+}
+
+// D[g, n] = -8 * ws[g, n] * (sum of the 64 weights of group g in row n), exact in fp32, written as three T values
+// that add up to it: dpieces[n][piece * G16 + g]; rows >= N and groups >= G are zero.
+template <typename T>
+__global__ void weight_group_sums_kernel(const uint8_t *wgt, const uint16_t *wscales, uint16_t *dpieces, int N, int npad,
+                                         int G, int G16, int ld_wgt, int ld_wscales) {
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int g = (int)(idx % G16), n = (int)(idx / G16);
+    if (n >= npad) return;
+    float d = 0.0f;
+    if (n < N && g < G) {
+        int w = 0;
+        const v4i *src = (const v4i *)(wgt + (size_t)n * ld_wgt + g * 32);
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const v4i p = src[h];
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+#pragma unroll
+                for (int j = 0; j < 8; j++) w += (((p[e] >> (4 * j)) & 0xF) ^ 8) - 8;
+        }
+        d = -8.0f * (T::to_f32(wscales[(size_t)g * ld_wscales + n]) * (float)w);
+    }
+    uint16_t *dst = dpieces + (size_t)n * 3 * G16 + g;
+#pragma unroll
+    for (int pc = 0; pc < 3; pc++) {
+        const uint16_t h = T::from_f32(d);
+        dst[pc * G16] = h;
+        d -= T::to_f32(h);
+    }
 }
 
 }  // namespace svdq
@@ -809,19 +1009,33 @@ static bool al16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
 extern "C" size_t svdq_weight_planes_bytes(int32_t N, int32_t K) {
     if (N <= 0 || K <= 0) return 0;
-    return (size_t)((N + 31) / 32) * 32 * (size_t)K;
+    const size_t npad = (size_t)((N + 31) / 32) * 32, g16 = (size_t)((K / GROUP + 15) / 16) * 16;
+    return npad * (size_t)K + npad * 3 * g16 * 2;  // fp8 planes, then the three 16-bit pieces of D[g, n]
 }
 
-extern "C" int svdq_split_weight_planes(const void *wgt, void *planes, int32_t N, int32_t K, int32_t ld_wgt, void *stream) {
-    if (!wgt || !planes || N <= 0 || K <= 0 || K % GROUP || ld_wgt % 16 || ld_wgt < K / 2 || ((uintptr_t)wgt & 15) ||
-        ((uintptr_t)planes & 15)) {
-        set_error("svdq_split_weight_planes: bad arguments (N=%d K=%d ld_wgt=%d; rows must be 16-byte aligned)", N, K, ld_wgt);
+extern "C" int svdq_split_weight_planes(const void *wgt, const void *wscales, void *planes, int32_t N, int32_t K,
+                                        int32_t ld_wgt, int32_t ld_wscales, int32_t dtype, void *stream) {
+    if (!wgt || !wscales || !planes || N <= 0 || K <= 0 || K % GROUP || ld_wgt % 16 || ld_wgt < K / 2 || ld_wscales < N ||
+        ((uintptr_t)wgt & 15) || ((uintptr_t)planes & 15) || (dtype != SVDQ_BF16 && dtype != SVDQ_FP16)) {
+        set_error("svdq_split_weight_planes: bad arguments (N=%d K=%d ld_wgt=%d ld_wscales=%d dtype=%d; rows must be 16-byte aligned)",
+                  N, K, ld_wgt, ld_wscales, dtype);
         return SVDQ_E_INVALID;
     }
-    const size_t n = (size_t)((N + 31) / 32) * (K / GROUP) * 64;
+    const int G = K / GROUP, G16 = (G + 15) / 16 * 16, npad = (N + 31) / 32 * 32;
+    const size_t n = (size_t)(npad / 32) * G * 64;
     hipLaunchKernelGGL(split_weight_planes_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
-                       (const uint8_t *)wgt, (uint8_t *)planes, N, K / GROUP, ld_wgt);
-    return check_launch("svdq_split_weight_planes");
+                       (const uint8_t *)wgt, (uint8_t *)planes, N, G, ld_wgt);
+    int rc = check_launch("svdq_split_weight_planes");
+    if (rc) return rc;
+    uint16_t *dpieces = (uint16_t *)((uint8_t *)planes + (size_t)npad * K);
+    const size_t nd = (size_t)npad * G16;
+    if (dtype == SVDQ_BF16)
+        hipLaunchKernelGGL(weight_group_sums_kernel<BF16>, dim3((unsigned)((nd + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                           (const uint8_t *)wgt, (const uint16_t *)wscales, dpieces, N, npad, G, G16, ld_wgt, ld_wscales);
+    else
+        hipLaunchKernelGGL(weight_group_sums_kernel<FP16>, dim3((unsigned)((nd + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                           (const uint8_t *)wgt, (const uint16_t *)wscales, dpieces, N, npad, G, G16, ld_wgt, ld_wscales);
+    return check_launch("svdq_split_weight_planes (group sums)");
 }
 
 extern "C" size_t svdq_gemm_w4a4_scratch_bytes(int32_t M, int32_t N, int32_t R2, int32_t epilogue) {
@@ -915,7 +1129,7 @@ static int gemm_w4a4_checked(const svdq_gemm_args &a, void *stream) {
         set_error("svdq_gemm_w4a4: unknown epilogue %d", a.epilogue);
         return SVDQ_E_INVALID;
     }
-    if (a.M == 0) return SVDQ_OK;
+    if (a.M == 0 || (a.actual_m == 0 && !quant)) return SVDQ_OK;  // nothing to write
     hipStream_t s = (hipStream_t)stream;
     if (a.dtype == SVDQ_BF16) {
         if (a.act_unsigned)
@@ -993,13 +1207,23 @@ extern "C" int svdq_gemm_w4a4_static_scratch(const svdq_gemm_args *args, void *s
 }
 
 extern "C" int svdq_group_acc_i32(const void *act, const void *wgt, int32_t *out, int32_t M, int32_t N, int32_t K,
-                                  int32_t ld_act, int32_t ld_wgt, int32_t group, int32_t act_unsigned, void *stream) {
+                                  int32_t ld_act, int32_t ld_wgt, int32_t group, int32_t act_unsigned, int32_t path,
+                                  void *stream) {
     if (!act || !wgt || !out || M <= 0 || N <= 0 || K <= 0 || K % GROUP || group < 0 || group >= K / GROUP ||
-        !al16(act) || !al16(wgt) || ld_act % 16 || ld_wgt % 16) {
+        !al16(act) || !al16(wgt) || ld_act % 16 || ld_wgt % 16 || path < 0 || path > 1) {
         set_error("svdq_group_acc_i32: bad arguments (M=%d N=%d K=%d group=%d)", M, N, K, group);
         return SVDQ_E_INVALID;
     }
     const dim3 grid((N + 31) / 32, (M + 31) / 32), block(64);
+    if (path == 1) {
+        if (act_unsigned)
+            hipLaunchKernelGGL(group_acc_f8_kernel<true>, grid, block, 0, (hipStream_t)stream, (const uint8_t *)act,
+                               (const uint8_t *)wgt, out, M, N, ld_act, ld_wgt, group);
+        else
+            hipLaunchKernelGGL(group_acc_f8_kernel<false>, grid, block, 0, (hipStream_t)stream, (const uint8_t *)act,
+                               (const uint8_t *)wgt, out, M, N, ld_act, ld_wgt, group);
+        return check_launch("svdq_group_acc_i32");
+    }
     if (act_unsigned)
         hipLaunchKernelGGL(group_acc_kernel<true>, grid, block, 0, (hipStream_t)stream, (const uint8_t *)act,
                            (const uint8_t *)wgt, out, M, N, ld_act, ld_wgt, group);

@@ -89,26 +89,28 @@ def lora_down_t(lora_down: torch.Tensor) -> torch.Tensor:
 _planes_cache: dict[int, tuple] = {}
 
 
-def weight_planes(qweight: torch.Tensor) -> torch.Tensor:
-    """Even / odd int8 nibble planes of a packed ``(N, K/2)`` weight in MFMA lane order (``svdq_split_weight_planes``),
-    made on first use and kept while the weight tensor lives unmodified.  Costs ``N * K`` bytes (twice the packed
-    weight) and removes the weight half of the nibble unpacking from the GEMM's inner loop."""
+def weight_planes(qweight: torch.Tensor, wscales: torch.Tensor) -> torch.Tensor:
+    """The GEMM's working copy of a packed ``(N, K/2)`` weight (``svdq_split_weight_planes``): even / odd nibble planes
+    as fp8 codes in MFMA lane order, followed by the per-group weight sums times ``-8 * wscales`` that take the offset
+    of signed activations out again.  Made on first use and kept while both tensors live unmodified.  Costs
+    ``N * K`` bytes (twice the packed weight) plus ``6 * N * K / 64`` bytes."""
     key = id(qweight)
     hit = _planes_cache.get(key)
     if hit is not None:
-        ref, src, t, ready = hit
-        if ref() is qweight and _same_source(src, qweight):
+        ref, src, src_s, t, ready = hit
+        if ref() is qweight and _same_source(src, qweight) and _same_source(src_s, wscales):
             ready.wait(t.device)
             return t
     N, K = qweight.shape[0], qweight.shape[1] * 2
     lib = _lib.load()
     t = torch.empty(lib.svdq_weight_planes_bytes(N, K), dtype=torch.uint8, device=qweight.device)
     with torch.cuda.device(t.device):
-        _lib.check(lib.svdq_split_weight_planes(qweight.data_ptr(), t.data_ptr(), N, K, qweight.stride(0), _lib.stream_of(qweight)))
+        _lib.check(lib.svdq_split_weight_planes(qweight.data_ptr(), wscales.data_ptr(), t.data_ptr(), N, K, qweight.stride(0),
+                                                wscales.stride(0), _lib.dtype_code(wscales.dtype), _lib.stream_of(qweight)))  # fmt: skip
         ready = _Ready(t.device)
     try:
         ref = weakref.ref(qweight, lambda _r, k=key: _planes_cache.pop(k, None))
-        _planes_cache[key] = (ref, _source_of(qweight), t, ready)
+        _planes_cache[key] = (ref, _source_of(qweight), _source_of(wscales), t, ready)
     except TypeError:
         pass
     return t

@@ -8,9 +8,11 @@ from .. import _lib
 from ._prep import lora_down_t as _lora_down_t
 from ._prep import weight_planes as _weight_planes
 
-# Weights are re-laid-out once into MFMA-ordered int8 planes (cached per tensor, see _prep.weight_planes) and the GEMM
-# streams those; False makes the GEMM unpack the packed weight itself (no extra memory, about 15% slower).
-USE_WEIGHT_PLANES = True
+# Which weights get the GEMM's working copy (fp8 nibble planes in MFMA lane order + group sums, cached per tensor, see
+# _prep.weight_planes; twice the packed weight's bytes on top of it, about 20 % faster GEMM): "parameters" = weights that
+# are nn.Parameter (module weights, which live long), "all" = any weight tensor (a temporary pays the re-layout on every
+# call), "none" = the GEMM unpacks the packed weight itself (int8 main loop, no extra memory).
+USE_WEIGHT_PLANES = "parameters"
 
 # True sends the requantizing epilogues' LoRA-down partial sums to the buffer built into the library
 # (svdq_gemm_w4a4_static_scratch) instead of a torch allocation per call: for callers that may not allocate, e.g. while
@@ -151,8 +153,8 @@ def svdq_gemm_w4a4_cuda(
     if out2d is not None and out2d.stride(1) != 1:
         raise ValueError("out not row-major")
 
-    # module weights (nn.Parameter) get the cached MFMA-ordered plane re-layout; ad-hoc tensors are unpacked in-kernel
-    planes = _weight_planes(wgt) if USE_WEIGHT_PLANES and wgt.stride(0) % 16 == 0 else None
+    want_planes = USE_WEIGHT_PLANES == "all" or (USE_WEIGHT_PLANES == "parameters" and isinstance(wgt, torch.nn.Parameter))
+    planes = _weight_planes(wgt, wscales) if want_planes and wgt.stride(0) % 16 == 0 else None
     args = _lib.GemmArgs(
         act=act.data_ptr(),
         wgt=wgt.data_ptr(),
@@ -231,8 +233,9 @@ def svdq_gemm_w4a4_cuda(
     return None
 
 
-def group_acc_i32(act: torch.Tensor, wgt: torch.Tensor, group: int, act_unsigned: bool = False) -> torch.Tensor:
-    """Debug read-out: exact int32 accumulators ``sum_{k in group} a[m, k] * w[n, k]`` from the GEMM's MFMA path."""
+def group_acc_i32(act: torch.Tensor, wgt: torch.Tensor, group: int, act_unsigned: bool = False, fp8_path: bool = False) -> torch.Tensor:
+    """Debug read-out: exact int32 accumulators ``sum_{k in group} a[m, k] * w[n, k]`` through the instruction sequence of
+    the GEMM's int8 main loop (packed weights) or of its fp8 main loop (pre-split weights)."""
     act = act.reshape(-1, act.shape[-1])
     dev = _lib.require_cuda(act, wgt)
     M, K, N = act.shape[0], act.shape[1] * 2, wgt.shape[0]
@@ -241,7 +244,7 @@ def group_acc_i32(act: torch.Tensor, wgt: torch.Tensor, group: int, act_unsigned
         _lib.check(
             _lib.load().svdq_group_acc_i32(
                 act.data_ptr(), wgt.data_ptr(), out.data_ptr(), M, N, K, act.stride(0), wgt.stride(0), group,
-                int(act_unsigned), _lib.stream_of(act),
+                int(act_unsigned), int(fp8_path), _lib.stream_of(act),
             )  # fmt: skip
         )
     return out

@@ -16,6 +16,16 @@ pytestmark = pytest.mark.gpu
 TOL = 1e-2  # max |out - ref| / max |ref| per layer
 
 
+@pytest.fixture(autouse=True, params=["none", "all"], ids=["int8-loop", "fp8-loop"])
+def main_loop(request):
+    """Every test runs through both main loops: packed weights (int8 MFMA) and pre-split weights (fp8 MFMA)."""
+    from nunchaku_rocm_amd.ops import gemm as G
+
+    old, G.USE_WEIGHT_PLANES = G.USE_WEIGHT_PLANES, request.param
+    yield request.param
+    G.USE_WEIGHT_PLANES = old
+
+
 def _rand_problem(M, N, K, R, dtype, seed, scale=0.02):
     g = torch.Generator().manual_seed(seed)
     p = {
@@ -48,14 +58,14 @@ def _gpu_gemm(p, dev, actual_m=None, unsigned=False, dtype=torch.bfloat16, canar
 
 @pytest.mark.parametrize("unsigned", [False, True])
 @pytest.mark.parametrize("M,N,K", [(32, 32, 64), (136, 264, 256), (257, 96, 384)])
-def test_group_accumulators_bit_exact(dev, M, N, K, unsigned):
+def test_group_accumulators_bit_exact(dev, M, N, K, unsigned, main_loop):
     from nunchaku_rocm_amd.ops.gemm import group_acc_i32
 
     print(f"case M={M} N={N} K={K} unsigned={unsigned}", flush=True)
     p = _rand_problem(M, N, K, 0, torch.bfloat16, seed=M + N)
     ref = O.group_acc_i32(p["act"], p["wgt"], unsigned)
     for g in range(K // 64):
-        got = group_acc_i32(p["act"].to(dev), p["wgt"].to(dev), g, unsigned).cpu()
+        got = group_acc_i32(p["act"].to(dev), p["wgt"].to(dev), g, unsigned, fp8_path=main_loop == "all").cpu()
         assert torch.equal(got, ref[g]), f"group {g}"
 
 
@@ -200,43 +210,59 @@ def test_linear_module_matches_dequantised_reference(dev):
     assert O.cosine(y.view(-1, N), truth) > 0.98
 
 
-def _planes_expected(wgt, N, K):
-    """Host restatement of the pre-split weight layout: [(block of 32 rows, group), plane, lane, 16 bytes], values x16."""
+def _planes_expected(wgt, wsc, N, K):
+    """Host restatement of the pre-split weight layout: [(block of 32 rows, group), plane, lane, 16 bytes] of fp8 codes
+    sign | magnitude, then per row three 16-bit pieces per group (piece-major, groups padded to 16) of
+    -8 * wscale * (sum of the group's weights)."""
     nb, G = (N + 31) // 32, K // 64
     q = O.unpack_int4(wgt, signed=True).to(torch.int16)  # (N, K) in [-8, 7]
     rows = torch.arange(nb * 32).clamp(max=N - 1)
-    q = q[rows].view(nb, 32, G, 2, 16, 2)  # (nblk, row in block, g, half, byte, even/odd)
-    v = ((q * 16) & 0xFF).to(torch.uint8)
-    # lane = half * 32 + row
-    return v.permute(0, 2, 5, 3, 1, 4).reshape(nb, G, 2, 64, 16).contiguous()
+    qb = q[rows].view(nb, 32, G, 2, 16, 2)  # (nblk, row in block, g, half, byte, even/odd)
+    v = (qb.abs() | ((qb < 0).to(torch.int16) << 7)).to(torch.uint8)
+    planes = v.permute(0, 2, 5, 3, 1, 4).reshape(nb, G, 2, 64, 16).contiguous()  # lane = half * 32 + row
+    G16 = (G + 15) // 16 * 16
+    d = torch.zeros(nb * 32, G16, dtype=torch.float32)
+    d[:N, :G] = -8.0 * (wsc.float().t()[:N] * q.view(N, G, 64).sum(-1).float())
+    pieces = torch.zeros(nb * 32, 3, G16, dtype=wsc.dtype)
+    for pc in range(3):
+        pieces[:, pc] = d.to(wsc.dtype)
+        d = d - pieces[:, pc].float()
+    assert bool((d[:N, :G].abs() <= 2.0**-20 * 1e-3).all())  # three pieces hold the fp32 value
+    return planes, pieces
 
 
-@pytest.mark.parametrize("N,K", [(32, 64), (264, 256), (100, 128)])
+@pytest.mark.parametrize("N,K", [(32, 64), (264, 256), (100, 128), (64, 2048)])
 def test_weight_planes_layout(dev, N, K):
     from nunchaku_rocm_amd.ops._prep import weight_planes
 
-    wgt = torch.randint(0, 256, (N, K // 2), generator=torch.Generator().manual_seed(N), dtype=torch.uint8)
-    got = weight_planes(wgt.to(dev)).cpu()
-    exp = _planes_expected(wgt, N, K)
-    assert got.numel() == exp.numel()
-    assert torch.equal(got.view(-1), exp.view(-1))
+    g = torch.Generator().manual_seed(N)
+    wgt = torch.randint(0, 256, (N, K // 2), generator=g, dtype=torch.uint8)
+    wsc = (torch.rand(K // 64, N, generator=g) * 0.02 + 0.005).to(torch.bfloat16)
+    got = weight_planes(wgt.to(dev), wsc.to(dev)).cpu()
+    planes, pieces = _planes_expected(wgt, wsc, N, K)
+    assert got.numel() == planes.numel() + pieces.numel() * 2
+    assert torch.equal(got[: planes.numel()], planes.view(-1))
+    assert torch.equal(got[planes.numel() :].view(torch.int16), pieces.view(torch.int16).view(-1))
 
 
 @pytest.mark.parametrize("unsigned", [False, True])
 @pytest.mark.parametrize("M,N,K,R", [(136, 264, 256, 16), (256, 512, 1024, 32), (64, 72, 128, 0), (300, 3072, 3072, 32),
                                      (100, 136, 64, 16), (257, 264, 320, 0)])  # the last two: K / 64 odd
-def test_presplit_weights_same_bits_as_packed(dev, M, N, K, R, unsigned):
-    """The GEMM gives identical bits whether it unpacks the weights itself or reads the pre-split planes."""
+def test_presplit_weights_against_packed(dev, M, N, K, R, unsigned):
+    """The two main loops (int8 MFMA on packed weights, fp8 MFMA on pre-split weights) compute the same integer group sums
+    and differ only in the order of fp32 roundings: outputs agree to one 16-bit ulp of the largest value."""
     print(f"case M={M} N={N} K={K} R={R} unsigned={unsigned}", flush=True)
     p = _rand_problem(M, N, K, R, torch.bfloat16, seed=7 + M)
     from nunchaku_rocm_amd.ops import gemm as gemm_mod
 
-    gemm_mod.USE_WEIGHT_PLANES = False
+    old = gemm_mod.USE_WEIGHT_PLANES
     try:
+        gemm_mod.USE_WEIGHT_PLANES = "none"
         packed = _gpu_gemm(p, dev, unsigned=unsigned)
+        gemm_mod.USE_WEIGHT_PLANES = "all"
+        split = _gpu_gemm(p, dev, unsigned=unsigned)
     finally:
-        gemm_mod.USE_WEIGHT_PLANES = True
-    split = _gpu_gemm(p, dev, unsigned=unsigned)
-    assert torch.equal(packed.view(torch.int16), split.view(torch.int16))
+        gemm_mod.USE_WEIGHT_PLANES = old
+    assert O.max_rel_err(split.float(), packed.float()) <= 2.0**-7
     ref = O.gemm_w4a4(p["act"], p["wgt"], p["asc"], p["wsc"], bias=p["bias"], lora_act=p["la"], lora_up=p["lu"], act_unsigned=unsigned)
     assert O.max_rel_err(split.float(), ref) <= TOL

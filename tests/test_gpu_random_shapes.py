@@ -12,6 +12,16 @@ from oracle import svdq_oracle as O
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True, params=["none", "all"], ids=["int8-loop", "fp8-loop"])
+def main_loop(request):
+    """Every test runs through both GEMM main loops: packed weights (int8 MFMA) and pre-split weights (fp8 MFMA)."""
+    from nunchaku_rocm_amd.ops import gemm as G
+
+    old, G.USE_WEIGHT_PLANES = G.USE_WEIGHT_PLANES, request.param
+    yield request.param
+    G.USE_WEIGHT_PLANES = old
+
+
 def test_gemm_random_shapes(dev):
     from nunchaku_rocm_amd import ops
 
