@@ -157,10 +157,10 @@ int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream);
  * nibbles) of fp8 (e4m3) codes in the order the MFMA lanes read them: a signed int4 value v is stored as the byte
  * sign | |v|, which the fp8 matrix instruction reads as v * 2^-9 exactly (v_mfma_scale_f32_32x32x64_f8f6f4 runs at
  * the int8 rate, takes a whole 64-deep group per instruction and returns the integer dot product as fp32, which saves
- * the GEMM one of its two scaling multiplies per output and group).  Behind the planes sit, per weight row, three T
- * pieces per group that add up to -8 * ws[g, n] * (sum of the group's 64 weights): the GEMM offsets signed activations by
+ * the GEMM one of its two scaling multiplies per output and group).  Behind the planes sit, per weight row, two T
+ * pieces per group (hi + lo) of -8 * ws[g, n] * (sum of the group's 64 weights): the GEMM offsets signed activations by
  * +8 for the fp8 operand and takes that term out again.  `planes` needs svdq_weight_planes_bytes(N, K) bytes
- * (= ceil(N/32)*32 * (K + 6 * ceil(K/1024)*16)).  The copy depends on `wgt` AND `wscales` (dtype = their type).  No
+ * (= ceil(N/32)*32 * (K + 4 * ceil(K/1024)*16)).  The copy depends on `wgt` AND `wscales` (dtype = their type).  No
  * counterpart in the reference (its SwiGLU path re-orders weight rows at load in the same spirit, ops/fused.py:83-105).
  */
 int svdq_split_weight_planes(const void *wgt, const void *wscales, void *planes, int32_t N, int32_t K, int32_t ld_wgt,

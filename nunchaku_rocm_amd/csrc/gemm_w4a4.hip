@@ -62,6 +62,8 @@ constexpr int TP_PITCH = 36;                        // floats per row of the acc
 constexpr int TP_WAVE_BYTES = 2 * 32 * TP_PITCH * 4;  // two 32x32 blocks at a time
 static_assert(2 * TP_WAVE_BYTES <= BUF_BYTES, "transposition tiles do not fit");
 constexpr int F8_SCALE = (int)0x88888888;  // e8m0 block scale 2^9 in every byte: an fp8 code c (value c * 2^-9) counts as c
+constexpr int NPIECE = 2;              // 16-bit pieces per group sum behind the weight planes (hi + lo: 16 / 22 significant bits)
+constexpr int CORR_LDS_G = 48;         // groups whose sums one staging buffer holds for the offset correction (24 blocks of 1 KB)
 constexpr int GROUP_M_TILES = 8;      // m-tiles per raster band
 constexpr int NUM_XCD = 8;
 
@@ -238,6 +240,53 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
         }
     };
 
+    // Operands of the offset correction that follows the main loop on the fp8 path with signed activations (see there).
+    // The group sums of the first CORR_LDS_G groups are fetched by the tile's last stage into the staging buffer that
+    // stage leaves idle, in MFMA lane order (block (weight block, piece, sixteen groups) = 1 KB, lane l's 16 bytes in
+    // slot l), one copy for the four wavefronts; the activation scales of those groups go to registers in the same
+    // stage.  Groups beyond that are read from global memory after the loop, sixteen at a time, two sets in flight.
+    const int G16 = (G + 15) / 16 * 16;
+    const int GL = min(G16, CORR_LDS_G);  // groups whose sums are staged in LDS
+    uint16_t cav[CORR_LDS_G / 16][8];
+    uint16_t cav2[2][8];
+    v4i cdb[2][NPIECE][NBN];
+    const uint16_t *cdp = nullptr, *cap = nullptr;
+    uint32_t cdrow[NBN];
+    const int cnpad = (a.N + 31) / 32 * 32;
+    static_assert(NBN * NPIECE * (CORR_LDS_G / 16) == NWAVES * 6 && NBN * NPIECE * (CORR_LDS_G / 16) * BLK_BYTES <= BUF_BYTES,
+                  "the staged group sums are dealt six blocks to a wavefront and must fit one staging buffer");
+    if constexpr (WPL && !ACT_UNSIGNED) {
+        const int npad = cnpad;
+        cdp = (const uint16_t *)((const uint8_t *)a.wgt_planes + (size_t)npad * a.K) + 8 * half;
+        cap = (const uint16_t *)a.ascales + min(m0 + wm * 32 + l32, a.M - 1);
+#pragma unroll
+        for (int bn = 0; bn < NBN; bn++) cdrow[bn] = (uint32_t)min(n0 + bn * 32 + l32, npad - 1) * (uint32_t)(NPIECE * G16);
+    }
+    auto corr_stage_lds = [&](uint8_t *dstbuf) {  // this wavefront's share of the (NBN x NPIECE x GL / 16) blocks
+#pragma unroll
+        for (int i = 0; i < PER_WAVE; i++) {
+            const int q = wm * PER_WAVE + i;  // wave-uniform: (sixteen groups gc, piece, weight block)
+            const int bn = q % NBN, pc = (q / NBN) % NPIECE, gc = q / (NBN * NPIECE);
+            const uint32_t row = (uint32_t)min(n0 + bn * 32 + l32, cnpad - 1) * (uint32_t)(NPIECE * G16);
+            if (gc * 16 < GL)
+                __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)(cdp + row + pc * G16 + gc * 16),
+                                                 (SVDQ_AS3 void *)(dstbuf + q * BLK_BYTES), 16, 0, 0);
+        }
+#pragma unroll
+        for (int gc = 0; gc < CORR_LDS_G / 16; gc++)
+            if (gc * 16 < GL) {
+#pragma unroll
+                for (int j = 0; j < 8; j++) cav[gc][j] = cap[(size_t)min(gc * 16 + 8 * half + j, G - 1) * a.ld_ascales];
+            }
+    };
+    auto corr_fetch = [&](int buf, int g0) {  // all loads issued before their first use
+#pragma unroll
+        for (int j = 0; j < 8; j++) cav2[buf][j] = cap[(size_t)min(g0 + 8 * half + j, G - 1) * a.ld_ascales];
+#pragma unroll
+        for (int pc = 0; pc < NPIECE; pc++)
+#pragma unroll
+            for (int bn = 0; bn < NBN; bn++) cdb[buf][pc][bn] = *(const v4i *)(cdp + cdrow[bn] + pc * G16 + g0);
+    };
     // Main-loop accumulators: MFMA A operand = activations, B operand = weights, so a lane owns one weight row n and its
     // registers walk the wavefront's 32 activation rows: the weight scale is a per-lane scalar and the 16 activation
     // scales a lane needs per group are shared by the wavefront's four weight blocks.
@@ -247,6 +296,19 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
 #pragma unroll
         for (int i = 0; i < 16; i++) acc[bn][i] = 0.0f;
 
+    auto pack8 = [&](const uint16_t (&v)[8]) -> v4i {
+        v4i ub;
+#pragma unroll
+        for (int e = 0; e < 4; e++) ub[e] = (int)((uint32_t)v[2 * e] | ((uint32_t)v[2 * e + 1] << 16));
+        return ub;
+    };
+    auto corr_apply = [&](int buf) {
+        const v4i ub = pack8(cav2[buf]);
+#pragma unroll
+        for (int pc = 0; pc < NPIECE; pc++)
+#pragma unroll
+            for (int bn = 0; bn < NBN; bn++) acc[bn] = mfma32_16bit<T>(ub, cdb[buf][pc][bn], acc[bn]);
+    };
     const v16i cmagic = magic_acc();
     const int nstages = ODDG ? a.K / KSTAGE + 1 : a.K / KSTAGE;
     const int offW = W_OFF + lane * 16;
@@ -285,8 +347,9 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
     // One stage = eight (group, weight block) steps, software-pipelined inside the wavefront: the MFMAs of step b + 1
     // are issued before the dequantisation FMAs of step b, and the operands of step b + 2 are read from LDS behind
     // them, so the VALU work of a step runs while the matrix pipe works on the next one.
-    auto stage = [&](auto par_tag, int s) {
+    auto stage = [&](auto par_tag, auto last_tag, int s) {
         constexpr int P = decltype(par_tag)::value;
+        constexpr bool LAST = decltype(last_tag)::value;  // the tile's last stage: the offset correction's first operands are fetched
         uint8_t *base = P ? sbuf1 : sbuf0;   // this stage's operands
         uint8_t *other = P ? sbuf0 : sbuf1;  // being refilled for the next stage
         // everything issued for stage s (scale registers, then operand blocks) has landed
@@ -302,6 +365,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
             __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));  // scale writes visible before the barrier
         }
         __builtin_amdgcn_s_barrier();
+        if constexpr (LAST && WPL && !ACT_UNSIGNED) corr_stage_lds(other);  // behind the wait above: lands while this stage computes
         // The other buffer was last read in the previous stage, before the barrier: refill it during this stage.  The last
         // stage re-fetches itself into the idle buffer (harmless, and keeps the stage one basic block).
         const int sn = min(s + 1, nstages - 1);
@@ -320,9 +384,11 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
             };
             auto read_a8 = [&](int gg) -> v8i {
                 typedef unsigned v4u __attribute__((ext_vector_type(4)));
-                v4u u = __builtin_bit_cast(v4u, *(const v4i *)(base + offA + gg * BLK_BYTES));
-                if (!ACT_UNSIGNED) u ^= 0x88888888u;  // two's complement nibble -> value + 8
-                const v4u e = u & 0x0F0F0F0Fu, o = (u >> 4) & 0x0F0F0F0Fu;
+                const v4u u = __builtin_bit_cast(v4u, *(const v4i *)(base + offA + gg * BLK_BYTES));
+                // two's complement nibble -> value + 8 is a flip of the nibble's top bit; written per plane so that mask
+                // and flip are one three-input bit operation
+                const unsigned flip = ACT_UNSIGNED ? 0u : 0x08080808u;
+                const v4u e = (u & 0x0F0F0F0Fu) ^ flip, o = ((u >> 4) & 0x0F0F0F0Fu) ^ flip;
                 return (v8i){(int)e[0], (int)e[1], (int)e[2], (int)e[3], (int)o[0], (int)o[1], (int)o[2], (int)o[3]};
             };
             auto outer = [&](int p) -> v32f {  // as[m] * ws[n] of pair p: blocks 2 (p & 1), + 1 of group p >> 1
@@ -351,7 +417,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
                                                                              F8_SCALE, 0, F8_SCALE);
                 }
                 if (b + 2 < 8) w8[(b + 2) % 3] = read_w8(b + 2);
-                if (b < PER_WAVE) dma_one(sn, other, b);
+                if (!(LAST && !ACT_UNSIGNED) && b < PER_WAVE) dma_one(sn, other, b);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int i = 0; i < 16; i++)
@@ -411,45 +477,52 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
         }
     };
     {
+        const int last = nstages - 1;
         int s = 0;
-        for (; s + 1 < nstages; s += 2) {
-            stage(std::integral_constant<int, 0>{}, s);
-            stage(std::integral_constant<int, 1>{}, s + 1);
+        for (; s + 1 < last; s += 2) {
+            stage(std::integral_constant<int, 0>{}, std::false_type{}, s);
+            stage(std::integral_constant<int, 1>{}, std::false_type{}, s + 1);
         }
-        if (s < nstages) stage(std::integral_constant<int, 0>{}, s);
+        if (s < last) {
+            stage(std::integral_constant<int, 0>{}, std::false_type{}, s);
+            s++;
+        }
+        if (s & 1)
+            stage(std::integral_constant<int, 1>{}, std::true_type{}, s);
+        else
+            stage(std::integral_constant<int, 0>{}, std::true_type{}, s);
     }
     // The last stage's (redundant) block loads of this wavefront have landed.
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
 
     // ---- fp8 path, signed activations: take the +8 offset out again -------------------------------------------------
     // sum_g as[g, m] ws[g, n] sum_k (a + 8) w  =  wanted  +  sum_g as[g, m] * (8 ws[g, n] W[g, n]),  W = the weights' group
-    // sums.  svdq_split_weight_planes stored D[g, n] = -8 ws[g, n] W[g, n] behind the planes as three 16-bit pieces
-    // that add up to the fp32 value exactly, K-contiguous per weight row like a LoRA-up matrix of rank 3 * G16; the
+    // sums.  svdq_split_weight_planes stored D[g, n] = -8 ws[g, n] W[g, n] behind the planes as two 16-bit pieces
+    // (hi + lo: 16 significant bits in bf16, 22 in fp16), K-contiguous per weight row like a LoRA-up matrix of rank 2 * G16; the
     // activation scales are the other operand.  Products of two 16-bit values are exact, the sum is fp32.
+#ifndef ABL_NOCORR
     if constexpr (WPL && !ACT_UNSIGNED) {
-        const int G16 = (G + 15) / 16 * 16, KC = 3 * G16;
-        const int npad = (a.N + 31) / 32 * 32;
-        const uint16_t *dp = (const uint16_t *)((const uint8_t *)a.wgt_planes + (size_t)npad * a.K);
-        const uint16_t *ap = (const uint16_t *)a.ascales + min(m0 + wm * 32 + l32, a.M - 1);
-        for (int g0 = 0; g0 < G16; g0 += 16) {
-            uint16_t av[8];
+        if (GL < G16) corr_fetch(0, GL);
+        __syncthreads();  // every wavefront's share of the staged blocks has landed (each waited for its own above)
+        const uint8_t *cl = (((nstages - 1) & 1) ? sbuf0 : sbuf1) + lane * 16;  // the buffer the last stage left idle
 #pragma unroll
-            for (int j = 0; j < 8; j++) av[j] = ap[(size_t)min(g0 + 8 * half + j, G - 1) * a.ld_ascales];
-            v4i db[3][NBN];
+        for (int gc = 0; gc < CORR_LDS_G / 16; gc++)
+            if (gc * 16 < GL) {
+                const v4i ub = pack8(cav[gc]);
 #pragma unroll
-            for (int pc = 0; pc < 3; pc++)
+                for (int pc = 0; pc < NPIECE; pc++)
 #pragma unroll
-                for (int bn = 0; bn < NBN; bn++)
-                    db[pc][bn] = *(const v4i *)(dp + (size_t)min(n0 + bn * 32 + l32, npad - 1) * KC + pc * G16 + g0 + 8 * half);
-            v4i ub;
-#pragma unroll
-            for (int e = 0; e < 4; e++) ub[e] = (int)((uint32_t)av[2 * e] | ((uint32_t)av[2 * e + 1] << 16));
-#pragma unroll
-            for (int pc = 0; pc < 3; pc++)
-#pragma unroll
-                for (int bn = 0; bn < NBN; bn++) acc[bn] = mfma32_16bit<T>(ub, db[pc][bn], acc[bn]);
+                    for (int bn = 0; bn < NBN; bn++)
+                        acc[bn] = mfma32_16bit<T>(ub, *(const v4i *)(cl + ((gc * NPIECE + pc) * NBN + bn) * BLK_BYTES), acc[bn]);
+            }
+        for (int g0 = GL; g0 < G16; g0 += 32) {  // two sets of operand registers, the next sixteen groups in flight
+            if (g0 + 16 < G16) corr_fetch(1, g0 + 16);
+            corr_apply(0);
+            if (g0 + 32 < G16) corr_fetch(0, g0 + 32);
+            if (g0 + 16 < G16) corr_apply(1);
         }
     }
+#endif
 
     // ---- LoRA-up and bias, still in the main loop's orientation (lane = weight row, registers = activation rows) ----
     // The bias and the first 32 ranks of both LoRA operands were fetched into LDS next to stage 0 and arrived long ago;
@@ -970,8 +1043,9 @@ __global__ void split_weight_planes_kernel(const uint8_t *wgt, uint8_t *planes, 
     *(v4i *)(planes + ((bg * 2 + 1) * 64 + lane) * 16) = odd;
 }
 
-// D[g, n] = -8 * ws[g, n] * (sum of the 64 weights of group g in row n), exact in fp32, written as three T values
-// that add up to it: dpieces[n][piece * G16 + g]; rows >= N and groups >= G are zero.
+// D[g, n] = -8 * ws[g, n] * (sum of the 64 weights of group g in row n), exact in fp32, written as NPIECE T values whose
+// sum is D to 16 (bf16) or 22 (fp16) significant bits, exactly when D is an integer below 2^16:
+// dpieces[n][piece * G16 + g]; rows >= N and groups >= G are zero.
 template <typename T>
 __global__ void weight_group_sums_kernel(const uint8_t *wgt, const uint16_t *wscales, uint16_t *dpieces, int N, int npad,
                                          int G, int G16, int ld_wgt, int ld_wscales) {
@@ -992,9 +1066,9 @@ __global__ void weight_group_sums_kernel(const uint8_t *wgt, const uint16_t *wsc
         }
         d = -8.0f * (T::to_f32(wscales[(size_t)g * ld_wscales + n]) * (float)w);
     }
-    uint16_t *dst = dpieces + (size_t)n * 3 * G16 + g;
+    uint16_t *dst = dpieces + (size_t)n * NPIECE * G16 + g;
 #pragma unroll
-    for (int pc = 0; pc < 3; pc++) {
+    for (int pc = 0; pc < NPIECE; pc++) {
         const uint16_t h = T::from_f32(d);
         dst[pc * G16] = h;
         d -= T::to_f32(h);
@@ -1010,7 +1084,7 @@ static bool al16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 extern "C" size_t svdq_weight_planes_bytes(int32_t N, int32_t K) {
     if (N <= 0 || K <= 0) return 0;
     const size_t npad = (size_t)((N + 31) / 32) * 32, g16 = (size_t)((K / GROUP + 15) / 16) * 16;
-    return npad * (size_t)K + npad * 3 * g16 * 2;  // fp8 planes, then the three 16-bit pieces of D[g, n]
+    return npad * (size_t)K + npad * NPIECE * g16 * 2;  // fp8 planes, then the 16-bit pieces of D[g, n]
 }
 
 extern "C" int svdq_split_weight_planes(const void *wgt, const void *wscales, void *planes, int32_t N, int32_t K,

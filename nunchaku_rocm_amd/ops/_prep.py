@@ -93,7 +93,7 @@ def weight_planes(qweight: torch.Tensor, wscales: torch.Tensor) -> torch.Tensor:
     """The GEMM's working copy of a packed ``(N, K/2)`` weight (``svdq_split_weight_planes``): even / odd nibble planes
     as fp8 codes in MFMA lane order, followed by the per-group weight sums times ``-8 * wscales`` that take the offset
     of signed activations out again.  Made on first use and kept while both tensors live unmodified.  Costs
-    ``N * K`` bytes (twice the packed weight) plus ``6 * N * K / 64`` bytes."""
+    ``N * K`` bytes (twice the packed weight) plus ``4 * N * K / 64`` bytes."""
     key = id(qweight)
     hit = _planes_cache.get(key)
     if hit is not None:
