@@ -1044,7 +1044,8 @@ __global__ void split_weight_planes_kernel(const uint8_t *wgt, uint8_t *planes, 
 }
 
 // D[g, n] = -8 * ws[g, n] * (sum of the 64 weights of group g in row n), exact in fp32, written as NPIECE T values whose
-// sum is D to 16 (bf16) or 22 (fp16) significant bits, exactly when D is an integer below 2^16:
+// sum is D to 16 (bf16) or 22 (fp16) significant bits, exactly when D is an integer below 2^16 (a third piece was
+// measured: it changes no requantized code at the FLUX fc1 shape and costs 4 % of the launch):
 // dpieces[n][piece * G16 + g]; rows >= N and groups >= G are zero.
 template <typename T>
 __global__ void weight_group_sums_kernel(const uint8_t *wgt, const uint16_t *wscales, uint16_t *dpieces, int N, int npad,

@@ -5,6 +5,7 @@ import pytest
 import torch
 
 from oracle import svdq_oracle as O
+from parity_bars import assert_requantized_like_the_reference
 
 pytestmark = pytest.mark.gpu
 
@@ -100,7 +101,7 @@ def test_fuse_glu_close_to_oracle(dev):
     rp, rs, _, rc = O.quantize_act(x, fuse_glu=True)
     codes = O.unpack_int4(out.cpu(), True)
     d = (codes - rc).abs()
-    assert d.max() <= 1 and (d > 0).float().mean() < 1e-3  # exp() differs between libraries
+    assert d.max() <= 1 and ((d > 0).float().mean() < 1e-5 or (d > 0).sum() <= 1)  # exp() differs between libraries
     assert ((osc.cpu().float() - rs.float()).abs() <= rs.float().abs() * 2**-7 + 1e-9).all()
 
 
@@ -126,15 +127,8 @@ def test_norm_modulate_prologue(dev, M, K, R, batches, dtype):
     torch.cuda.synchronize()
     xm = O.layernorm_modulate(x, scale, shift)
     rq, rs, rl, rc = O.quantize_act(xm, ld, lin["smooth_factor"])
-    codes = O.unpack_int4(q[:M].cpu(), True)
-    diff = (codes - rc).abs()
-    rate = (diff > 0).float().mean().item()
-    print(f"  code mismatch rate {rate:.2e}", flush=True)
-    assert diff.max() <= 1 and rate < 1e-3
     # a group maximum that flipped by one 16-bit step moves the stored scale by up to two of its own steps
-    ulp = 2**-7 if dtype == torch.bfloat16 else 2**-10
-    sdiff = (s[:, :M].cpu().float() - rs.float()).abs()
-    assert (sdiff <= rs.float().abs() * 2.01 * ulp + 1e-7).all() and (sdiff > 0).float().mean() < 1e-3
+    assert_requantized_like_the_reference(O.unpack_int4(q[:M].cpu(), True), rc, s[:, :M].cpu(), rs.to(dtype), dtype, scale_steps=2.01)
     if R:
         assert (la[:M].cpu() - rl).abs().max() <= 1e-2 * rl.abs().max()
     # statistics computed once and passed in give the same bits as computing them inside the call
@@ -197,12 +191,7 @@ def test_gelu_prologue(dev, M, K, R, dtype):
                                                fuse_gelu=True, shift_value=O.GELU_SHIFT, unsigned=True)  # fmt: skip
     torch.cuda.synchronize()
     rp, rs, rl, rc = O.quantize_act(x, ld, sm, unsigned=True, shift=O.GELU_SHIFT, fuse_gelu=True)
-    diff = (O.unpack_int4(out.cpu(), False) - rc).abs()
-    rate = (diff > 0).float().mean().item()
-    print(f"  code mismatch rate {rate:.2e}", flush=True)
-    assert diff.max() <= 1 and rate < 1e-3
-    ulp = 2**-7 if dtype == torch.bfloat16 else 2**-10
-    assert ((osc.cpu().float() - rs.float()).abs() <= rs.float().abs() * ulp + 1e-7).all()
+    assert_requantized_like_the_reference(O.unpack_int4(out.cpu(), False), rc, osc.cpu(), rs.to(dtype), dtype)
     if R:
         assert (la.cpu() - rl).abs().max() <= 1e-2 * rl.abs().max()
     with pytest.raises(NotImplementedError):
