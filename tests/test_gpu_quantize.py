@@ -66,6 +66,21 @@ def test_zero_groups_and_ties(dev):
     assert torch.equal(out, rp) and torch.equal(osc.view(torch.int16), rs.view(torch.int16))
 
 
+def test_kernel_multiplies_by_the_reciprocal(dev):
+    """Inputs on which ``x * (1 / scale)`` and ``x / scale`` give different codes; the expected codes come from exact
+    rational arithmetic (tests/golden/rcp_order_vectors.py)."""
+    from nunchaku_rocm_amd import ops
+    from test_oracle_pins import _rcp_order_input
+
+    xb, want = _rcp_order_input()
+    xp = torch.zeros(16, 64, dtype=torch.bfloat16)
+    xp[: xb.shape[0]] = xb
+    q, _, _ = ops.svdq_quantize_w4a4_act_fuse_lora_cuda(xp.to(dev))
+    codes = O.unpack_int4(q.cpu(), True)
+    for i, w in enumerate(want):
+        assert int(codes[i, 1 + i]) == w and int(codes[i, 0]) == 7
+
+
 def test_full_size_qkv_input_bit_exact_and_deterministic(dev):
     """The benchmark configuration: M=4608, K=3072, R=32, outlier channels, smooth U(0.5, 4)."""
     M, K = 4608, 3072

@@ -121,6 +121,39 @@ def test_quantizer_matches_c_restatement_bit_exact(unsigned, shift):
     assert (lora - c_lora).abs().max() <= 1e-5 * lora.abs().max()
 
 
+def _rcp_order_input():
+    import os
+    import sys
+
+    sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden"))
+    from rcp_order_vectors import VECTORS, expected
+
+    x = torch.zeros(len(VECTORS), 64, dtype=torch.float32)
+    want = []
+    for i, (v, gmax) in enumerate(VECTORS):
+        x[i, 0], x[i, 1 + i] = gmax, v
+        by_rcp, by_div = expected(v, gmax)
+        assert by_rcp != by_div  # the vector does tell the two orders apart
+        want.append(by_rcp)
+    xb = x.to(torch.bfloat16)
+    assert torch.equal(xb.float(), x)  # the values are bf16
+    return xb, want
+
+
+def test_quantizer_multiplies_by_the_reciprocal():
+    """``x * (1 / scale)``, not ``x / scale`` (nunchaku/ops/triton/gemm_w4a4.py:1440): on these inputs the two give
+    different codes, and the expected ones come from exact rational arithmetic (tests/golden/rcp_order_vectors.py), not from
+    a restatement of the formula in floating point."""
+    xb, want = _rcp_order_input()
+    _, _, _, codes = O.quantize_act(xb)
+    packed_c, _, _ = c_oracle.quantize_act(xb)
+    codes_c = O.unpack_int4(packed_c, True)
+    for i, w in enumerate(want):
+        assert int(codes[i, 1 + i]) == w, (i, int(codes[i, 1 + i]), w)
+        assert int(codes_c[i, 1 + i]) == w, (i, int(codes_c[i, 1 + i]), w)
+        assert int(codes[i, 0]) == 7
+
+
 # ----------------------------------------------------------------------------- integer group dots, GEMM
 @pytest.mark.parametrize("act_unsigned", [False, True])
 def test_group_acc_brute_force(act_unsigned):
