@@ -18,24 +18,18 @@
 //
 // One workgroup = 32 channels x all of K; its eight wavefronts take groups round-robin.  The small loads (activations,
 // the channels' scales and zeros) are issued first and staged in LDS while up to six weight loads per lane (all of a
-// wavefront's groups at K = 3072) are in flight; partial sums are added through LDS in a fixed order.
+// wavefront's groups at K = 3072) are in flight; partial sums are added through LDS in a fixed order.  Up to eight rows
+// of activations are staged in LDS as well when they fit next to the tables (M = 8 up to K = 3072, M = 2 up to
+// K = 12288); otherwise the MFMA operand is read from global memory.
 #include "svdq_common.h"
 
 namespace svdq {
 
-#ifndef SVDQ_AWQ_WAVES
-#define SVDQ_AWQ_WAVES 8
-#endif
-#ifndef SVDQ_AWQ_PF
-#define SVDQ_AWQ_PF 6
-#endif
-#ifndef SVDQ_AWQ_NT
-#define SVDQ_AWQ_NT 1
-#endif
-constexpr int AWQ_WAVES = SVDQ_AWQ_WAVES;
+constexpr int AWQ_WAVES = 8;  // wavefronts per workgroup (4 and 16 measured slower)
 constexpr int AWQ_NB = 32;    // channels per workgroup
-constexpr int AWQ_PF = SVDQ_AWQ_PF;    // weight loads in flight per lane (all of a wavefront's groups at K = 3072)
+constexpr int AWQ_PF = 6;     // weight loads in flight per lane (all of a wavefront's groups at K = 3072)
 constexpr int AWQ_XPAD = 8;   // 16-bit elements of padding per staged activation row
+constexpr size_t AWQ_LDS_MAX = 65536;  // dynamic LDS a launch may ask for
 
 template <typename T>
 struct AwqMagic;
@@ -56,19 +50,15 @@ __device__ inline int nibble_plane(int w, int sh, uint32_t mask, uint32_t magic)
 }
 
 __device__ inline v4i awq_wload(const v4i *p) {
-#if SVDQ_AWQ_NT
     return __builtin_nontemporal_load(p);  // streamed once: do not keep in cache
-#else
-    return *p;
-#endif
 }
 
-template <typename T, int MQ>  // MQ = ceil(M / 8): accumulator register quads that hold real rows
-__global__ __launch_bounds__(AWQ_WAVES * 64, AWQ_WAVES >= 16 ? 4 : (AWQ_WAVES >= 8 ? 6 : 4)) void awq_gemv_kernel(svdq_awq_gemv_args a) {
-    // xs[K/64][8*MQ] fp32 | red[AWQ_WAVES][8*MQ][32] fp32 | sz[K/64][2][32] 16-bit | (M <= 8 only) x[M][K + pad] 16-bit
+// MQ = ceil(M / 8): accumulator register quads that hold real rows; X_IN_LDS: the activations are staged in LDS
+template <typename T, int MQ, bool X_IN_LDS>
+__global__ __launch_bounds__(AWQ_WAVES * 64, 6) void awq_gemv_kernel(svdq_awq_gemv_args a) {
+    // xs[K/64][8*MQ] fp32 | red[AWQ_WAVES][8*MQ][32] fp32 | sz[K/64][2][32] 16-bit | (X_IN_LDS) x[M][K + pad] 16-bit
     extern __shared__ __align__(16) float lds[];
     constexpr int MR = 8 * MQ;
-    constexpr bool X_IN_LDS = MQ == 1;
     const int ngroups = a.K / GROUP;
     float *xs = lds;
     float *red = lds + (size_t)ngroups * MR;
@@ -254,24 +244,36 @@ __global__ __launch_bounds__(256) void awq_dequant_kernel(const v4i *__restrict_
     }
 }
 
+// LDS of a launch without the staged activations, and the bytes those would add
 static size_t awq_lds_bytes(int K, int M) {
     const int MQ = (M + 7) / 8;
     size_t b = ((size_t)(K / GROUP) * 8 * MQ + (size_t)AWQ_WAVES * 8 * MQ * AWQ_NB) * sizeof(float);
     b += (size_t)(K / GROUP) * 2 * AWQ_NB * 2;
-    if (MQ == 1) b += (size_t)M * (K + AWQ_XPAD) * 2;
     return b;
+}
+static size_t awq_x_lds_bytes(int K, int M) { return (size_t)M * (K + AWQ_XPAD) * 2; }
+static bool awq_stage_x(int K, int M) {
+    // wherever they fit: read from global memory instead, the eight rows of M = 8 cost 17.6 us against 12.6 us at the
+    // FLUX adaLN shape (four 16-byte activation loads per lane and group next to one weight load)
+    return M <= 8 && awq_lds_bytes(K, M) + awq_x_lds_bytes(K, M) <= AWQ_LDS_MAX;
 }
 
 template <typename T>
 static void launch_awq(const svdq_awq_gemv_args &a, hipStream_t s) {
     const int MQ = (a.M + 7) / 8;
     const dim3 grid(a.N / AWQ_NB), block(AWQ_WAVES * 64);
-    const size_t sh = awq_lds_bytes(a.K, a.M);
+    const bool xl = awq_stage_x(a.K, a.M);
+    const size_t sh = awq_lds_bytes(a.K, a.M) + (xl ? awq_x_lds_bytes(a.K, a.M) : 0);
     switch (MQ) {
-        case 1: hipLaunchKernelGGL((awq_gemv_kernel<T, 1>), grid, block, sh, s, a); break;
-        case 2: hipLaunchKernelGGL((awq_gemv_kernel<T, 2>), grid, block, sh, s, a); break;
-        case 3: hipLaunchKernelGGL((awq_gemv_kernel<T, 3>), grid, block, sh, s, a); break;
-        default: hipLaunchKernelGGL((awq_gemv_kernel<T, 4>), grid, block, sh, s, a); break;
+        case 1:
+            if (xl)
+                hipLaunchKernelGGL((awq_gemv_kernel<T, 1, true>), grid, block, sh, s, a);
+            else
+                hipLaunchKernelGGL((awq_gemv_kernel<T, 1, false>), grid, block, sh, s, a);
+            break;
+        case 2: hipLaunchKernelGGL((awq_gemv_kernel<T, 2, false>), grid, block, sh, s, a); break;
+        case 3: hipLaunchKernelGGL((awq_gemv_kernel<T, 3, false>), grid, block, sh, s, a); break;
+        default: hipLaunchKernelGGL((awq_gemv_kernel<T, 4, false>), grid, block, sh, s, a); break;
     }
 }
 
@@ -302,8 +304,9 @@ extern "C" int svdq_awq_gemv_w4a16(const svdq_awq_gemv_args *args, void *stream)
         set_error("svdq_awq_gemv_w4a16: x rows, qweight and scale / zero rows must be 16-byte aligned; leading dimensions >= row length");
         return SVDQ_E_INVALID;
     }
-    if (awq_lds_bytes(a.K, a.M) > 65536) {
-        set_error("svdq_awq_gemv_w4a16: K=%d too large for the LDS activation / group-sum tables", a.K);
+    if (awq_lds_bytes(a.K, a.M) > AWQ_LDS_MAX) {  // K = 12288 with M > 16, K > 16384 with M > 8
+        set_error("svdq_awq_gemv_w4a16: K=%d with M=%d needs %zu bytes of LDS tables (limit %zu)", a.K, a.M,
+                  awq_lds_bytes(a.K, a.M), AWQ_LDS_MAX);
         return SVDQ_E_UNSUPPORTED;
     }
     if (a.M == 0) return SVDQ_OK;

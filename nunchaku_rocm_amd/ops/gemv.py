@@ -59,7 +59,13 @@ def awq_gemv_w4a16_cuda(
                 ld_out=out.stride(0),
                 dtype=_lib.dtype_code(x.dtype),
             )
-            _lib.check(lib.svdq_awq_gemv_w4a16(args, _lib.stream_of(x)))
+            rc = lib.svdq_awq_gemv_w4a16(args, _lib.stream_of(x))
+            if rc == _lib.E_UNSUPPORTED:
+                # the kernel's per-group tables do not fit LDS (K = 12288 with more than 16 rows, longer K with fewer):
+                # decode the weight and multiply, the reference's route for everything but group size 64
+                w = awq_dequantize(kernel, scaling_factors, zeros, n, k, group_size, x.dtype)
+                return torch.matmul(x, w.t()).reshape(*in_feats.shape[:-1], n)
+            _lib.check(rc)
     return out.reshape(*in_feats.shape[:-1], n)
 
 

@@ -41,6 +41,17 @@ def test_flux_adaln_shape(dev, m):
     assert ((out.float() - ref).abs() <= ref.abs() * 2**-7 + 2e-2).all()
 
 
+@pytest.mark.parametrize("m", [2, 8, 32])
+@pytest.mark.parametrize("K", [3584, 4096, 12288])
+def test_long_k(dev, m, K):
+    """Row counts and lengths at which the activations no longer fit the kernel's LDS staging (they are then read from
+    global memory), and K = 12288 with 32 rows, where the per-group tables do not fit either and the operator decodes
+    the weight and multiplies instead."""
+    print(f"case m={m} K={K}", flush=True)
+    out, ref = _case(dev, m, 256, K, torch.bfloat16, seed=K + m)
+    assert O.max_rel_err(out, ref) <= 1e-2
+
+
 def test_linear_module_adds_bias_after_kernel(dev):
     from nunchaku_rocm_amd.linear import AWQW4A16Linear
 
