@@ -329,6 +329,73 @@ class FluxShapedTransformer(nn.Module):
                     m.weight.copy_((torch.rand(m.weight.shape, device=device, generator=gen) + 0.5).to(dtype))
         self.requires_grad_(False)
 
+    # names of nunchaku's FLUX model (what ``layout.convert_flux_state_dict`` produces, transformer_flux_v2.py:579-649)
+    # -> names of this harness; first match wins
+    _CHECKPOINT_NAMES = (
+        (r"^transformer_blocks\.(\d+)\.norm1\.linear\.", r"double_blocks.\1.norm1."),
+        (r"^transformer_blocks\.(\d+)\.norm1_context\.linear\.", r"double_blocks.\1.norm1_context."),
+        (r"^transformer_blocks\.(\d+)\.attn\.to_out\.0\.", r"double_blocks.\1.attn.to_out."),
+        (r"^transformer_blocks\.(\d+)\.attn\.", r"double_blocks.\1.attn."),
+        (r"^transformer_blocks\.(\d+)\.ff\.net\.0\.proj\.", r"double_blocks.\1.ff_fc1."),
+        (r"^transformer_blocks\.(\d+)\.ff\.net\.2\.", r"double_blocks.\1.ff_fc2."),
+        (r"^transformer_blocks\.(\d+)\.ff_context\.net\.0\.proj\.", r"double_blocks.\1.ffc_fc1."),
+        (r"^transformer_blocks\.(\d+)\.ff_context\.net\.2\.", r"double_blocks.\1.ffc_fc2."),
+        (r"^single_transformer_blocks\.(\d+)\.norm\.linear\.", r"single_blocks.\1.norm."),
+        (r"^single_transformer_blocks\.(\d+)\.", r"single_blocks.\1."),
+        (r"^time_text_embed\.timestep_embedder\.linear_1\.", "time_in.0."),
+        (r"^time_text_embed\.timestep_embedder\.linear_2\.", "time_in.2."),
+        (r"^time_text_embed\.text_embedder\.linear_1\.", "pooled_in.0."),
+        (r"^time_text_embed\.text_embedder\.linear_2\.", "pooled_in.2."),
+        (r"^norm_out\.linear\.", "norm_out_linear."),
+    )
+    # tensors a checkpoint may carry that the int4 path does not use (NVFP4 scales, the un-fused smoothing factors)
+    _CHECKPOINT_IGNORED = (".smooth_factor_orig", ".wtscale", ".wcscales")
+
+    @torch.no_grad()
+    def load_converted(self, state_dict: dict, strict: bool = True) -> None:
+        """Fill the model from a published int4 checkpoint: ``state_dict`` as ``layout.load_checkpoint`` reads it and
+        ``layout.convert_flux_state_dict`` renames it (tensors still in checkpoint layout).  Names are mapped onto this
+        harness, the tensors are loaded as they are, and every ``SVDQW4A4Linear`` is then turned into the natural layout
+        once (``convert_svdq_linear_to_natural_layout``); AWQ tensors stay in TinyChat packing.  What the reference's
+        ``from_pretrained`` does after building its model (transformer_flux_v2.py:419-435).  ``strict``: every tensor
+        of the model must be in the file and every tensor of the file must have a place (except the ones the int4 path
+        ignores)."""
+        import re
+
+        from .layout import convert_svdq_linear_to_natural_layout
+
+        own = dict(self.named_parameters())
+        own.update(dict(self.named_buffers()))
+        mapped, unexpected = {}, []
+        for key, value in state_dict.items():
+            if key.endswith(self._CHECKPOINT_IGNORED):
+                continue
+            name = key
+            for pat, rep in self._CHECKPOINT_NAMES:
+                name, n = re.subn(pat, rep, key)
+                if n:
+                    break
+            if name in own:
+                mapped[name] = value
+            else:
+                unexpected.append(key)
+        missing = [k for k in own if k not in mapped and not k.endswith(self._CHECKPOINT_IGNORED)]
+        if strict and (missing or unexpected):
+            raise KeyError(f"checkpoint does not match the model: missing {missing[:8]}{'...' if len(missing) > 8 else ''}, "
+                           f"unexpected {unexpected[:8]}{'...' if len(unexpected) > 8 else ''}")  # fmt: skip
+        for name, value in mapped.items():
+            dst = own[name]
+            if value.numel() != dst.numel():
+                raise ValueError(f"{name}: checkpoint tensor has {tuple(value.shape)}, the model {tuple(dst.shape)}")
+            # the checkpoint's 2-D views of the shuffled tensors differ from the logical shapes; the bytes are what counts
+            src = value.to(dst.device)
+            if src.dtype != dst.dtype:
+                src = src.view(dst.dtype) if src.element_size() == dst.element_size() and not src.is_floating_point() else src.to(dst.dtype)
+            dst.data = src.reshape(dst.shape).contiguous()
+        for m in self.modules():
+            if isinstance(m, SVDQW4A4Linear):
+                convert_svdq_linear_to_natural_layout(m)
+
     @torch.no_grad()
     def forward(self, latents, text, pooled, timestep, rot, backend=None):
         """latents (B, T_img, 64), text (B, T_txt, 4096), pooled (B, 768), timestep (B,) in [0, 1], rot the

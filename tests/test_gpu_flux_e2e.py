@@ -121,3 +121,105 @@ def test_relayout_made_on_one_stream_is_ordered_before_its_use_on_another(dev):
         y_side = mod(x)  # cache hits on another stream
     torch.cuda.synchronize()
     assert torch.equal(y_main, ref) and torch.equal(y_side, ref)
+
+
+# harness names -> nunchaku model names -> legacy checkpoint names: the inverse of what the loader applies
+_TO_MODEL = (
+    ("double_blocks.", "transformer_blocks."), ("single_blocks.", "single_transformer_blocks."),
+    (".norm1_context.", ".norm1_context.linear."), (".norm1.", ".norm1.linear."), (".norm.", ".norm.linear."),
+    (".ffc_fc1.", ".ff_context.net.0.proj."), (".ffc_fc2.", ".ff_context.net.2."),
+    (".ff_fc1.", ".ff.net.0.proj."), (".ff_fc2.", ".ff.net.2."),
+    ("time_in.0.", "time_text_embed.timestep_embedder.linear_1."), ("time_in.2.", "time_text_embed.timestep_embedder.linear_2."),
+    ("pooled_in.0.", "time_text_embed.text_embedder.linear_1."), ("pooled_in.2.", "time_text_embed.text_embedder.linear_2."),
+    ("norm_out_linear.", "norm_out.linear."),
+)  # fmt: skip
+_TO_LEGACY_DOUBLE = (
+    (".ff_context.net.0.proj.", ".mlp_context_fc1."), (".ff_context.net.2.", ".mlp_context_fc2."),
+    (".ff.net.0.proj.", ".mlp_fc1."), (".ff.net.2.", ".mlp_fc2."),
+    (".attn.add_qkv_proj.", ".qkv_proj_context."), (".attn.to_qkv.", ".qkv_proj."),
+    (".attn.to_add_out.", ".out_proj_context."), (".attn.to_out.", ".out_proj."),
+    (".attn.norm_added_q.", ".norm_added_q."), (".attn.norm_added_k.", ".norm_added_k."),
+    (".attn.norm_q.", ".norm_q."), (".attn.norm_k.", ".norm_k."),
+)  # fmt: skip
+_TO_LEGACY_SINGLE = (
+    (".attn.to_qkv.", ".qkv_proj."), (".attn.to_out.", ".out_proj."), (".attn.norm_q.", ".norm_q."), (".attn.norm_k.", ".norm_k."),
+)  # fmt: skip
+
+
+def _legacy_key(name: str) -> str:
+    for old, new in _TO_MODEL:
+        name = name.replace(old, new)
+    if name.startswith("transformer_blocks."):
+        for old, new in _TO_LEGACY_DOUBLE:
+            if old in name:
+                name = name.replace(old, new)
+                break
+    elif name.startswith("single_transformer_blocks."):
+        for old, new in _TO_LEGACY_SINGLE:
+            if old in name:
+                name = name.replace(old, new)
+                break
+    name = name.replace(".proj_down", ".lora_down").replace(".proj_up", ".lora_up")
+    if name.endswith(".smooth_factor"):
+        name = name[: -len(".smooth_factor")] + ".smooth"
+    return name
+
+
+def test_converted_checkpoint_runs(dev, tmp_path):
+    """A model written out the way the published int4 checkpoints are stored -- legacy module names, every SVDQuant tensor
+    shuffled into the mma fragment order by the packer restatement, one ``.safetensors`` file -- read back through
+    ``layout.load_checkpoint``, ``convert_flux_state_dict`` and ``FluxShapedTransformer.load_converted`` computes the
+    same bits as the model it was written from (reference: transformer_flux_v2.py:375-435)."""
+    from safetensors.torch import save_file
+
+    from nunchaku_rocm_amd import layout
+    from nunchaku_rocm_amd.flux_shaped import FluxShapedConfig, FluxShapedTransformer
+    from nunchaku_rocm_amd.linear import SVDQW4A4Linear
+    from oracle import mma_packer as P
+
+    cfg = FluxShapedConfig(hidden=256, heads=2, mlp=512, text_dim=128, pooled_dim=64, n_double=2, n_single=2)
+    src = FluxShapedTransformer(cfg, device=dev, seed=11)
+    svdq = {n for n, m in src.named_modules() if isinstance(m, SVDQW4A4Linear)}
+    as16 = lambda t: t.detach().cpu().contiguous().view(torch.int16).numpy()  # noqa: E731
+    bf = lambda a: torch.from_numpy(a).view(torch.bfloat16)  # noqa: E731
+    ckpt = {}
+    for name, t in src.state_dict().items():
+        mod, leaf = name.rsplit(".", 1) if "." in name else ("", name)
+        t = t.detach().cpu()
+        if mod in svdq:
+            if leaf == "smooth_factor_orig":
+                continue
+            if leaf == "qweight":
+                codes = O.unpack_int4(t, signed=False).to(torch.int32)
+                t = torch.from_numpy(P.pack_weight(codes.numpy())).view(torch.int8)
+            elif leaf == "wscales":
+                t = bf(P.pack_scale(as16(t.t()))).reshape(t.shape)
+            elif leaf in ("bias", "smooth_factor"):
+                t = bf(P.pack_scale(as16(t)))
+            elif leaf == "proj_down":
+                t = bf(P.pack_lowrank_weight(as16(t.t()), down=True))
+            elif leaf == "proj_up":
+                t = bf(P.pack_lowrank_weight(as16(t), down=False))
+        ckpt[_legacy_key(name)] = t.contiguous()
+    assert any(".qkv_proj_context.lora_down" in k for k in ckpt) and any(k.endswith(".mlp_fc2.smooth") for k in ckpt)
+    path = tmp_path / "svdq-int4-flux-shaped.safetensors"
+    save_file(ckpt, str(path), metadata={"config": "{\"num_layers\": 2}", "quantization_config": "{\"rank\": 32}"})
+
+    state, meta, config = layout.load_checkpoint(path)
+    assert config == {"num_layers": 2} and "quantization_config" in meta
+    dst = FluxShapedTransformer(cfg, device=dev, seed=99)  # other weights: everything must come from the file
+    dst.load_converted(layout.convert_flux_state_dict(state))
+    for (n1, t1), (n2, t2) in zip(src.state_dict().items(), dst.state_dict().items()):
+        if n1.endswith("smooth_factor_orig"):
+            continue
+        assert n1 == n2 and torch.equal(t1.view(torch.uint8), t2.view(torch.uint8)), n1
+    lat, txt, pooled, rot = _inputs(cfg, 32, 16, 16, dev)
+    a = src.denoise(lat, txt, pooled, rot, steps=2)
+    b = dst.denoise(lat, txt, pooled, rot, steps=2)
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+    # a file that lacks a tensor, or brings one with no place, is refused
+    broken = dict(layout.convert_flux_state_dict(state))
+    broken.pop("transformer_blocks.0.attn.to_qkv.qweight")
+    with pytest.raises(KeyError):
+        dst.load_converted(broken)
