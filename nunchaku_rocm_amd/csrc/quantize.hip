@@ -22,10 +22,11 @@
 
 namespace svdq {
 
-constexpr int Q_ROWS = 16;
+constexpr int Q_ROWS = 16;         // rows of one MFMA pass; a workgroup takes QR = 16 or 32 rows (one or two passes)
 constexpr int Q_WAVES = 8;
 constexpr int Q_ROW_BYTES = 128;  // one scale group of one row (64 x 16 bit)
 constexpr int Q_RCHUNK = 32;  // LoRA ranks per pass over the row block
+constexpr int Q32_ABOVE = 256, Q32_UPTO = 512;  // number of 16-row workgroups for which 32-row workgroups are used instead
 
 // sum_j (0x4B400000 << 4 j) mod 2^32: what eight magic-biased codes add up to besides their nibbles
 constexpr uint32_t pack_bias() {
@@ -39,28 +40,27 @@ struct QVecs {
     uint16_t sm, ns, nh;  // smooth factor, norm scale, norm shift
 };
 
-template <typename T, bool UNSIGNED, int PRE, bool HAS_LORA, bool HAS_SMOOTH, bool NORM>
-__global__ __launch_bounds__(Q_WAVES * 64, NORM ? 4 : 2) void quantize_act_kernel(svdq_quantize_args a) {
+template <typename T, bool UNSIGNED, int PRE, bool HAS_LORA, bool HAS_SMOOTH, bool NORM, int QR>
+__global__ __launch_bounds__(Q_WAVES * 64, QR == 32 ? 1 : (NORM ? 4 : 2)) void quantize_act_kernel(svdq_quantize_args a) {
     constexpr bool GLU = PRE == SVDQ_PRE_GLU, GELU = PRE == SVDQ_PRE_GELU;
+    constexpr int NH = QR / Q_ROWS;  // 16-row halves of the row block: each LoRA-down tile read serves all of them
     // per wavefront: two activation stages (16 rows, + the gate tile with GLU) and one LoRA-down tile (32 ranks), 128
     // bytes a row.  The LoRA-down tile is an L2 hit and the first thing a group consumes: one group ahead is enough.
-    constexpr int XS_BYTES = (GLU ? 2 : 1) * Q_ROWS * Q_ROW_BYTES, G_OFF = Q_ROWS * Q_ROW_BYTES;
+    constexpr int XS_BYTES = (GLU ? 2 : 1) * QR * Q_ROW_BYTES, G_OFF = QR * Q_ROW_BYTES;
     constexpr int L_OFF = 2 * XS_BYTES;
     constexpr int WAVE_BYTES = L_OFF + (HAS_LORA ? Q_RCHUNK * Q_ROW_BYTES : 0);
-    constexpr int ACC_BYTES = HAS_LORA ? Q_WAVES * Q_RCHUNK * (Q_ROWS + 1) * 4 : 0;  // cross-wave sum, after the loop
+    constexpr int ACC_BYTES = HAS_LORA ? Q_WAVES * Q_RCHUNK * (QR + 1) * 4 : 0;  // cross-wave sum, after the loop
     constexpr int STG_BYTES = Q_WAVES * WAVE_BYTES;
     __shared__ __align__(16) uint8_t smem[STG_BYTES > ACC_BYTES ? STG_BYTES : ACC_BYTES];
     __shared__ float lds_rs[Q_WAVES][64];
     __shared__ float lds_ns[NORM ? Q_WAVES : 1][64], lds_nh[NORM ? Q_WAVES : 1][64];
-    float (*lds_acc)[Q_RCHUNK][Q_ROWS + 1] = (float (*)[Q_RCHUNK][Q_ROWS + 1])smem;
+    float (*lds_acc)[Q_RCHUNK][QR + 1] = (float (*)[Q_RCHUNK][QR + 1])smem;
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: keep it in an SGPR
     const int ml = lane & 15;
     const int kq = lane >> 4;
-    const int m0 = blockIdx.x * Q_ROWS;
-    const int m = m0 + ml;
-    const bool row_ok = m < a.M;
+    const int m0 = blockIdx.x * QR;
     const int ngroups = a.K / GROUP;
     const int nmy = (ngroups - wave + Q_WAVES - 1) / Q_WAVES;  // groups g = wave + Q_WAVES * i
     // Block loads: lane l of load i fetches chunk (l % 8) ^ (l / 8) of tile row 8 i + l / 8 into LDS slot l of that
@@ -68,9 +68,9 @@ __global__ __launch_bounds__(Q_WAVES * 64, NORM ? 4 : 2) void quantize_act_kerne
     // memory; nothing is stored for them).  Addresses = uniform base + 32-bit lane offset (+ uniform group step).
     const int drow = lane >> 3, dchunk = (lane & 7) ^ drow;
     const uint8_t *__restrict__ xbase = (const uint8_t *)a.x + (size_t)m0 * a.ld_x * 2;
-    uint32_t xdma[2];
+    uint32_t xdma[2 * NH];
 #pragma unroll
-    for (int i = 0; i < 2; i++) xdma[i] = (uint32_t)(min(m0 + 8 * i + drow, a.M - 1) - m0) * a.ld_x * 2 + dchunk * 16;
+    for (int i = 0; i < 2 * NH; i++) xdma[i] = (uint32_t)(min(m0 + 8 * i + drow, a.M - 1) - m0) * a.ld_x * 2 + dchunk * 16;
     // read-back: lane (m, q) takes chunks 2 q and 2 q + 1 of tile row m (and of row m + 16 of the LoRA-down tile)
     const int rd_lo = ml * Q_ROW_BYTES + (((2 * kq) ^ (ml & 7)) * 16), rd_hi = ml * Q_ROW_BYTES + (((2 * kq + 1) ^ (ml & 7)) * 16);
     uint8_t *const wbase = smem + wave * WAVE_BYTES;
@@ -83,12 +83,15 @@ __global__ __launch_bounds__(Q_WAVES * 64, NORM ? 4 : 2) void quantize_act_kerne
     const float rmagic = UNSIGNED ? RNE_MAGIC : RNE_MAGIC + 8.0f;  // signed codes are packed as c + 8, then ^ 8
     const bool has_shift = a.shift != 0.0f;
     // norm prologue: this lane's row statistics, and the workgroup's scale / shift vectors (one batch per workgroup)
-    float n_mean = 0.0f, n_rstd = 1.0f;
+    float n_mean[NH], n_rstd[NH];
     const uint16_t *__restrict__ nscale = nullptr, *__restrict__ nshift = nullptr;
     if (NORM) {
-        const int mr = min(m, a.M - 1);
-        n_mean = a.norm_stats[2 * mr];
-        n_rstd = a.norm_stats[2 * mr + 1];
+#pragma unroll
+        for (int h = 0; h < NH; h++) {
+            const int mr = min(m0 + Q_ROWS * h + ml, a.M - 1);
+            n_mean[h] = a.norm_stats[2 * mr];
+            n_rstd[h] = a.norm_stats[2 * mr + 1];
+        }
         const size_t voff = a.norm_rows_per_batch > 0 ? (size_t)(m0 / a.norm_rows_per_batch) * a.norm_ld : 0;
         nscale = (const uint16_t *)a.norm_scale + voff;
         nshift = (const uint16_t *)a.norm_shift + voff;
@@ -96,7 +99,9 @@ __global__ __launch_bounds__(Q_WAVES * 64, NORM ? 4 : 2) void quantize_act_kerne
 
     const int nchunks = HAS_LORA ? (a.R + Q_RCHUNK - 1) / Q_RCHUNK : 1;
     for (int rc = 0; rc < nchunks; rc++) {
-        v4f acc0 = (v4f){0.f, 0.f, 0.f, 0.f}, acc1 = (v4f){0.f, 0.f, 0.f, 0.f};
+        v4f acc0[NH], acc1[NH];
+#pragma unroll
+        for (int h = 0; h < NH; h++) acc0[h] = acc1[h] = (v4f){0.f, 0.f, 0.f, 0.f};
         // ranks >= R re-read rank R - 1; their accumulator rows are never stored
         const uint8_t *__restrict__ lbase = (const uint8_t *)a.lora_down_t;
         uint32_t ldma[4] = {0, 0, 0, 0};
@@ -107,7 +112,7 @@ __global__ __launch_bounds__(Q_WAVES * 64, NORM ? 4 : 2) void quantize_act_kerne
         }
         const bool do_quant = rc == 0;
 
-        constexpr int NX = GLU ? 4 : 2;  // block loads of one activation stage
+        constexpr int NX = (GLU ? 4 : 2) * NH;  // block loads of one activation stage
         auto group_off = [&](int i) {  // byte offset of group wave + Q_WAVES * i in a row; past the end: the last group
             return (uint32_t)min(wave + Q_WAVES * i, ngroups - 1) * (GROUP * 2);
         };
@@ -122,12 +127,12 @@ __global__ __launch_bounds__(Q_WAVES * 64, NORM ? 4 : 2) void quantize_act_kerne
                 qv.nh = nshift[((k0 >> 1) + lane) * a.norm_stride];
             }
 #pragma unroll
-            for (int j = 0; j < 2; j++)
+            for (int j = 0; j < 2 * NH; j++)
                 __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)(xbase + (xdma[j] + k0)),
                                                  (SVDQ_AS3 void *)(dst + j * 1024), 16, 0, 0);
             if (GLU) {
 #pragma unroll
-                for (int j = 0; j < 2; j++)
+                for (int j = 0; j < 2 * NH; j++)
                     __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)(xbase + (size_t)a.K * 2 + (xdma[j] + k0)),
                                                      (SVDQ_AS3 void *)(dst + G_OFF + j * 1024), 16, 0, 0);
             }
@@ -142,15 +147,18 @@ __global__ __launch_bounds__(Q_WAVES * 64, NORM ? 4 : 2) void quantize_act_kerne
         };
 
         struct Ops {
-            v4i xlo, xhi, glo, ghi, l0lo, l0hi, l1lo, l1hi;
+            v4i xlo[NH], xhi[NH], glo[NH], ghi[NH], l0lo, l0hi, l1lo, l1hi;
         };
         auto fetch = [&](int i, Ops &o) {  // LDS -> registers, in the MFMA operand layout
             const uint8_t *src = wbase + (i & 1) * XS_BYTES;
-            o.xlo = *(const v4i *)(src + rd_lo);
-            o.xhi = *(const v4i *)(src + rd_hi);
-            if (GLU) {
-                o.glo = *(const v4i *)(src + G_OFF + rd_lo);
-                o.ghi = *(const v4i *)(src + G_OFF + rd_hi);
+#pragma unroll
+            for (int h = 0; h < NH; h++) {
+                o.xlo[h] = *(const v4i *)(src + h * Q_ROWS * Q_ROW_BYTES + rd_lo);
+                o.xhi[h] = *(const v4i *)(src + h * Q_ROWS * Q_ROW_BYTES + rd_hi);
+                if (GLU) {
+                    o.glo[h] = *(const v4i *)(src + G_OFF + h * Q_ROWS * Q_ROW_BYTES + rd_lo);
+                    o.ghi[h] = *(const v4i *)(src + G_OFF + h * Q_ROWS * Q_ROW_BYTES + rd_hi);
+                }
             }
             if (HAS_LORA) {
                 o.l0lo = *(const v4i *)(wbase + L_OFF + rd_lo);
@@ -162,8 +170,21 @@ __global__ __launch_bounds__(Q_WAVES * 64, NORM ? 4 : 2) void quantize_act_kerne
 
         auto process = [&](int i, const Ops &o, const QVecs qv) {
             const uint16_t smv = qv.sm;
-            v4i cxlo = o.xlo, cxhi = o.xhi;
-            const v4i glo = o.glo, ghi = o.ghi, l0lo = o.l0lo, l0hi = o.l0hi, l1lo = o.l1lo, l1hi = o.l1hi;
+            const v4i l0lo = o.l0lo, l0hi = o.l0hi, l1lo = o.l1lo, l1hi = o.l1hi;
+            // per-channel vectors of the group, once for all halves: 1/smooth (one IEEE divide per lane) and the norm
+            // prologue's scale / shift, shared through LDS
+            if (NORM) {
+                lds_ns[wave][lane] = T::to_f32(qv.ns);
+                lds_nh[wave][lane] = T::to_f32(qv.nh);
+            }
+            if (HAS_SMOOTH && do_quant) lds_rs[wave][lane] = 1.0f / T::to_f32(smv);
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int h = 0; h < NH; h++) {
+            const int m = m0 + Q_ROWS * h + ml;
+            const bool row_ok = m < a.M;
+            v4i cxlo = o.xlo[h], cxhi = o.xhi[h];
+            const v4i glo = o.glo[h], ghi = o.ghi[h];
             float v[16];
 #pragma unroll
             for (int j = 0; j < 4; j++) {
@@ -201,21 +222,17 @@ __global__ __launch_bounds__(Q_WAVES * 64, NORM ? 4 : 2) void quantize_act_kerne
             }
             if (NORM) {
                 // LayerNorm, scale, shift, each rounded to T; the LoRA-down sees the result
-                lds_ns[wave][lane] = T::to_f32(qv.ns);
-                lds_nh[wave][lane] = T::to_f32(qv.nh);
-                __builtin_amdgcn_wave_barrier();
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
                     const v4f sc = *(const v4f *)&lds_ns[wave][kq * 16 + 4 * j];
                     const v4f sh = *(const v4f *)&lds_nh[wave][kq * 16 + 4 * j];
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
-                        float t = T::to_f32(T::from_f32((v[4 * j + e] - n_mean) * n_rstd));
+                        float t = T::to_f32(T::from_f32((v[4 * j + e] - n_mean[h]) * n_rstd[h]));
                         t = T::to_f32(T::from_f32(t * sc[e]));
                         v[4 * j + e] = T::to_f32(T::from_f32(t + sh[e]));
                     }
                 }
-                __builtin_amdgcn_wave_barrier();
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
                     cxlo[j] = (int)pack2<T>(v[2 * j], v[2 * j + 1]);
@@ -223,27 +240,23 @@ __global__ __launch_bounds__(Q_WAVES * 64, NORM ? 4 : 2) void quantize_act_kerne
                 }
             }
             if (HAS_LORA) {
-                acc0 = mfma16_16bit<T>(l0lo, cxlo, acc0);
-                acc0 = mfma16_16bit<T>(l0hi, cxhi, acc0);
-                acc1 = mfma16_16bit<T>(l1lo, cxlo, acc1);
-                acc1 = mfma16_16bit<T>(l1hi, cxhi, acc1);
+                acc0[h] = mfma16_16bit<T>(l0lo, cxlo, acc0[h]);
+                acc0[h] = mfma16_16bit<T>(l0hi, cxhi, acc0[h]);
+                acc1[h] = mfma16_16bit<T>(l1lo, cxlo, acc1[h]);
+                acc1[h] = mfma16_16bit<T>(l1hi, cxhi, acc1[h]);
             }
-            if (!do_quant) return;
+            if (!do_quant) continue;
             if (has_shift) {
 #pragma unroll
                 for (int j = 0; j < 16; j++) v[j] = v[j] + a.shift;
             }
             if (HAS_SMOOTH) {
-                // 1/smooth for the group's 64 channels: one IEEE divide per lane, shared through LDS
-                lds_rs[wave][lane] = 1.0f / T::to_f32(smv);
-                __builtin_amdgcn_wave_barrier();
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
                     const v4f rs = *(const v4f *)&lds_rs[wave][kq * 16 + 4 * j];
 #pragma unroll
                     for (int e = 0; e < 4; e++) v[4 * j + e] = v[4 * j + e] * rs[e];
                 }
-                __builtin_amdgcn_wave_barrier();
             }
             float gmax = 0.0f;
 #pragma unroll
@@ -276,9 +289,11 @@ __global__ __launch_bounds__(Q_WAVES * 64, NORM ? 4 : 2) void quantize_act_kerne
                 w1 ^= 0x88888888u;
             }
             if (row_ok) {
-                if (kq == 0) (scales + (size_t)i * Q_WAVES * a.ld_scales)[ml] = T::from_f32(scale);
-                *(uint2 *)(outbase + (size_t)i * (GSTEP / 2) + outoff) = make_uint2(w0, w1);
+                if (kq == 0) (scales + (size_t)i * Q_WAVES * a.ld_scales)[Q_ROWS * h + ml] = T::from_f32(scale);
+                *(uint2 *)(outbase + (size_t)i * (GSTEP / 2) + (uint32_t)(Q_ROWS * h) * a.ld_out + outoff) = make_uint2(w0, w1);
             }
+            }  // halves
+            __builtin_amdgcn_wave_barrier();  // the shared vectors are rewritten by the next group
         };
 
         // Two groups of activations and one LoRA-down tile in flight per wavefront; each wavefront owns its LDS, so no
@@ -310,12 +325,14 @@ __global__ __launch_bounds__(Q_WAVES * 64, NORM ? 4 : 2) void quantize_act_kerne
             // fixed-order sum of the wavefronts' partial products
             __syncthreads();  // every wavefront is done with its stages: the sum reuses the memory
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                lds_acc[wave][4 * kq + i][ml] = acc0[i];
-                lds_acc[wave][16 + 4 * kq + i][ml] = acc1[i];
-            }
+            for (int h = 0; h < NH; h++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    lds_acc[wave][4 * kq + i][Q_ROWS * h + ml] = acc0[h][i];
+                    lds_acc[wave][16 + 4 * kq + i][Q_ROWS * h + ml] = acc1[h][i];
+                }
             __syncthreads();
-            for (int o = threadIdx.x; o < Q_ROWS * Q_RCHUNK; o += Q_WAVES * 64) {
+            for (int o = threadIdx.x; o < QR * Q_RCHUNK; o += Q_WAVES * 64) {
                 const int mm = o / Q_RCHUNK, r = o % Q_RCHUNK;
                 float s = lds_acc[0][r][mm];
 #pragma unroll
@@ -447,18 +464,42 @@ __global__ void transpose_kr_kernel(const uint16_t *in, uint16_t *out, int K, in
     out[idx] = in[(size_t)k * ld_in + r];
 }
 
+// Rows per workgroup.  A workgroup streams 4 KB of LoRA-down weight per group whatever its number of rows, and the
+// vector memory pipe of a CU is what that traffic is bound by: with 16-row workgroups, M = 4608 puts two of them on 32 of
+// the 256 CUs and the launch waits for those.  32-row workgroups (one LoRA-down tile read for two MFMA passes; a longer
+// chain per wavefront, 12 us even for one workgroup per CU) are faster where the 16-row grid needs between one and two
+// workgroups per CU: 13.4 against 14.2 us at M = 4608, 14.6 against 15.5 at 6144, 16.2 against 16.7 at 8192 (K = 3072,
+// R = 32); below and above that range the 16-row kernel wins.
+static int quantize_rows_per_workgroup(const svdq_quantize_args &a) {
+    if (a.R == 0 || a.prologue != SVDQ_PRE_NONE) return Q_ROWS;
+    if (a.norm_stats && a.norm_rows_per_batch % 32) return Q_ROWS;
+    const int wg16 = (a.M + 15) / 16;
+    return (wg16 > Q32_ABOVE && wg16 <= Q32_UPTO) ? 32 : Q_ROWS;
+}
+
 template <typename T, bool U, int G, bool NORM>
 static void launch_quantize3(const svdq_quantize_args &a, hipStream_t s) {
-    dim3 grid((a.M + Q_ROWS - 1) / Q_ROWS), block(Q_WAVES * 64);
+    const dim3 block(Q_WAVES * 64);
     const bool lora = a.R > 0, sm = a.smooth != nullptr;
+    if constexpr (G == SVDQ_PRE_NONE) {
+        if (quantize_rows_per_workgroup(a) == 32) {
+            const dim3 grid((a.M + 31) / 32);
+            if (sm)
+                hipLaunchKernelGGL((quantize_act_kernel<T, U, G, true, true, NORM, 32>), grid, block, 0, s, a);
+            else
+                hipLaunchKernelGGL((quantize_act_kernel<T, U, G, true, false, NORM, 32>), grid, block, 0, s, a);
+            return;
+        }
+    }
+    const dim3 grid((a.M + Q_ROWS - 1) / Q_ROWS);
     if (lora && sm)
-        hipLaunchKernelGGL((quantize_act_kernel<T, U, G, true, true, NORM>), grid, block, 0, s, a);
+        hipLaunchKernelGGL((quantize_act_kernel<T, U, G, true, true, NORM, 16>), grid, block, 0, s, a);
     else if (lora)
-        hipLaunchKernelGGL((quantize_act_kernel<T, U, G, true, false, NORM>), grid, block, 0, s, a);
+        hipLaunchKernelGGL((quantize_act_kernel<T, U, G, true, false, NORM, 16>), grid, block, 0, s, a);
     else if (sm)
-        hipLaunchKernelGGL((quantize_act_kernel<T, U, G, false, true, NORM>), grid, block, 0, s, a);
+        hipLaunchKernelGGL((quantize_act_kernel<T, U, G, false, true, NORM, 16>), grid, block, 0, s, a);
     else
-        hipLaunchKernelGGL((quantize_act_kernel<T, U, G, false, false, NORM>), grid, block, 0, s, a);
+        hipLaunchKernelGGL((quantize_act_kernel<T, U, G, false, false, NORM, 16>), grid, block, 0, s, a);
 }
 
 template <typename T, bool U, int G>
