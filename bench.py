@@ -28,11 +28,11 @@ sys.path.insert(0, ROOT)
 INT8_MFMA_PEAK_TOPS = 5000.0  # MI355X dense int8 MFMA, published
 BF16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 / fp16 MFMA, published
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
-# HBM bytes of one QKV GEMM launch: 2.00 x FETCH_SIZE + 1.00 x WRITE_SIZE (KiB per dispatch) of the grid-1327104 launches
+# HBM bytes of one QKV GEMM launch: 2.00 x FETCH_SIZE + 1.00 x WRITE_SIZE (KiB per dispatch) of the grid-663552 launches
 # in profiles/bench_all_kernels_hbm_traffic.txt, the factors being what the same counters read on plain copy kernels of
 # known size in the same run (FETCH_SIZE reads half the bytes of 16-byte-per-lane loads); counters cannot be read from
 # inside this process
-GEMM_QKV_HBM_BYTES = (2.0 * 97052.8 + 82944.0) * 1024
+GEMM_QKV_HBM_BYTES = (2.0 * 104572.7 + 82944.0) * 1024
 
 
 def _events(n):
