@@ -3,24 +3,22 @@
 // Arithmetic (reference: nunchaku/ops/triton/awq.py:160-182):
 //   out[m, n] = sum_c  s[c, n] * sum_{k in c} x[m, k] q[n, k]  +  z[c, n] * sum_{k in c} x[m, k]      (fp32)
 //
-// The kernel is HBM-bound: N*K/2 bytes of weights are read exactly once, for all M rows together (the reference
-// launches one pass over the weights per row).
+// N*K/2 bytes of weights are read exactly once, for all M rows together (the reference launches one pass over the
+// weights per row).
 //
 // Storage order is the access order.  Packed row a = n / 4 holds, for scale group c, 128 contiguous bytes =
 // 4 channels (b = n % 4) x 2 halves (h) x 16 bytes; the 16 bytes of (n, c, h) are eight int16 whose nibble j' holds
-// k = 64 c + 32 h + 8 j' + j (j = position of the int16).  Lane (n = lane % 32, h = lane / 32) of a wavefront loads
-// exactly that 16-byte piece, so one load instruction reads 8 packed rows x 128 contiguous bytes.  Nibble plane j' of
-// the loaded dwords, OR-ed with the bit pattern of 128.0 (bf16) / 1024.0 (fp16), is directly the B operand of one
-// 32x32x16 MFMA (exact: 128 + q and 1024 + q are representable); the A operand is the matching 16 bytes of x.  Four
-// MFMAs cover the group; the constant offset is folded into the zero-point term:
-//   s * (D - OFF * xs) + z * xs = s * D + (z - OFF * s) * xs,   xs = sum_{k in c} x[m, k]  (precomputed in LDS).
-// Only accumulator registers whose rows are < M are post-processed (rows m = 8 (i / 4) + 4 h + i % 4).
+// k = 64 c + 32 h + 8 j' + j (j = position of the int16).  A lane loads exactly one such piece per group, eight lanes
+// one contiguous 128-byte piece of a packed row, one load instruction 8 packed rows x 128 bytes.  Nibble plane j' of the
+// loaded dwords, OR-ed with the bit pattern of 128.0 (bf16) / 1024.0 (fp16), is directly an MFMA B operand (exact:
+// 128 + q and 1024 + q are representable); the A operand is the matching piece of x.  The constant offset is folded
+// into the zero-point term:
+//   s * (D - OFF * xs) + z * xs = s * D + (z - OFF * s) * xs,   xs = sum_{k in c} x[m, k]  (in LDS).
 //
-// One workgroup = 32 channels x all of K; its eight wavefronts take groups round-robin.  The small loads (activations,
-// the channels' scales and zeros) are issued first and staged in LDS while up to six weight loads per lane (all of a
-// wavefront's groups at K = 3072) are in flight; partial sums are added through LDS in a fixed order.  Up to eight rows
-// of activations are staged in LDS as well when they fit next to the tables (M = 8 up to K = 3072, M = 2 up to
-// K = 12288); otherwise the MFMA operand is read from global memory.
+// One workgroup = 32 channels x all of K; its eight wavefronts take groups round-robin with up to six weight loads per
+// lane in flight (all of a wavefront's groups at K = 3072); partial sums are added through LDS in a fixed order.
+#include <type_traits>
+
 #include "svdq_common.h"
 
 namespace svdq {
@@ -28,7 +26,6 @@ namespace svdq {
 constexpr int AWQ_WAVES = 8;  // wavefronts per workgroup (4 and 16 measured slower)
 constexpr int AWQ_NB = 32;    // channels per workgroup
 constexpr int AWQ_PF = 6;     // weight loads in flight per lane (all of a wavefront's groups at K = 3072)
-constexpr int AWQ_XPAD = 8;   // 16-bit elements of padding per staged activation row
 constexpr size_t AWQ_LDS_MAX = 65536;  // dynamic LDS a launch may ask for
 
 template <typename T>
@@ -53,18 +50,210 @@ __device__ inline v4i awq_wload(const v4i *p) {
     return __builtin_nontemporal_load(p);  // streamed once: do not keep in cache
 }
 
-// MQ = ceil(M / 8): accumulator register quads that hold real rows; X_IN_LDS: the activations are staged in LDS
-template <typename T, int MQ, bool X_IN_LDS>
-__global__ __launch_bounds__(AWQ_WAVES * 64, 6) void awq_gemv_kernel(svdq_awq_gemv_args a) {
-    // xs[K/64][8*MQ] fp32 | red[AWQ_WAVES][8*MQ][32] fp32 | sz[K/64][2][32] 16-bit | (X_IN_LDS) x[M][K + pad] 16-bit
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef short v4s __attribute__((ext_vector_type(4)));
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+
+// 4x4x4 MFMA in 16 independent blocks (block = lane / 4): D[block][row][col = lane % 4] += sum over 4 k of
+// A[block][row = lane % 4][k] * B[block][k][col]; four 16-bit values per lane, passed as raw bits
+template <typename T>
+__device__ inline v4f mfma4_16bit(v2i a, v2i b, v4f c);
+template <>
+__device__ inline v4f mfma4_16bit<BF16>(v2i a, v2i b, v4f c) {
+    return __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(v4s, a), __builtin_bit_cast(v4s, b), c, 0, 0, 0);
+}
+template <>
+__device__ inline v4f mfma4_16bit<FP16>(v2i a, v2i b, v4f c) {
+    return __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(v4h, a), __builtin_bit_cast(v4h, b), c, 0, 0, 0);
+}
+
+template <int CTRL>
+__device__ inline float dpp_f32(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xF, 0xF, false));
+}
+
+// M <= 8, RP = M rounded up to 1, 2, 4 or 8.
+//
+// The kernel is bound by instruction issue as much as by HBM (a wavefront has about 440 issue slots in the time its
+// share of the weights streams in), so every wavefront works alone until the final sum and with as few instructions as
+// possible: one global_load_lds for the activations of all its groups (RP = 1; one per 64 pieces otherwise), one for
+// their scales and zeros, then the weight pieces into registers, all issued back to back in straight-line code so
+// that each wait counts exactly the loads that must have returned; no workgroup barrier before the final sum.
+//
+// RP <= 4 uses the 4x4x4 MFMA (16 blocks of 4 channels x 4 rows, 8 cycles) in place of the 32x32x16 one (32 cycles for
+// the same number of weights): block 2 q + h holds channels 4 q .. 4 q + 3 over half h of the group, so that the eight
+// lanes of a channel quad still load one contiguous 128-byte piece of a packed row; the two halves are added in the
+// final sum.  RP = 8 keeps the 32x32x16 MFMA with lane = (channel, half).
+//
+// LDS of wavefront w:  x tiles of its AWQ_PF groups (RP rows x 128 bytes each; the 16-byte piece pc of row r sits in
+// slot pc ^ r, rows 128 bytes apart would otherwise meet in the same banks) | s of the groups (64 bytes each) | z;
+// after the tables of all wavefronts: xs[w][group][8] fp32 = sums of the activations per (half, row) (RP <= 4) or per
+// row (RP = 8).  The partial sums of the final reduction reuse the wavefront's own x tiles.
+template <int RP>
+constexpr int awq_wave_bytes() { return AWQ_PF * RP * 128 + 2 * AWQ_PF * 64; }
+
+template <typename T, int RP>
+__global__ __launch_bounds__(AWQ_WAVES * 64) __attribute__((amdgpu_waves_per_eu(RP <= 4 ? 6 : 4))) void awq_gemv_rows_kernel(svdq_awq_gemv_args a) {
+    extern __shared__ __align__(16) uint8_t lds8[];
+    constexpr bool SMALL = RP <= 4;
+    constexpr int WB = awq_wave_bytes<RP>(), XPIECES = AWQ_PF * 8 * RP, XPASSES = (XPIECES + 63) / 64;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int ngroups = a.K / GROUP;
+    const int nb0 = blockIdx.x * AWQ_NB;
+    uint8_t *xw = lds8 + wave * WB, *szw = xw + AWQ_PF * RP * 128;
+    float *xsw = (float *)(lds8 + AWQ_WAVES * WB) + wave * (AWQ_PF * 8);
+
+    // channel and half of the group this lane multiplies
+    const int ch = SMALL ? ((lane >> 3) << 2) | (lane & 3) : lane & 31;
+    const int half = SMALL ? (lane >> 2) & 1 : lane >> 5;
+    // weight piece: packed row n / 4, int16 column 64 c + 16 (n % 4) + 8 h  (byte offsets from the tensor, 32 bits)
+    const uint32_t woff = ((uint32_t)((nb0 + ch) >> 2) * (uint32_t)a.K + 16 * (ch & 3) + 8 * half) * 2;
+    // MFMA A operand: row min(lane % 4 or lane % 32, M - 1) (rows >= M land in accumulator rows nobody reads)
+    const int arow = min(SMALL ? lane & 3 : lane & 31, a.M - 1);
+    const uint8_t *aop = xw + arow * 128;
+    int aslot[4];
+#pragma unroll
+    for (int pl = 0; pl < 4; pl++) aslot[pl] = 16 * ((4 * half + pl) ^ arow);
+
+    uint32_t mask = 0x000F000Fu;
+    asm volatile("" : "+v"(mask));  // keep the mask in a VGPR: v_and_or_b32 takes only one literal
+    float acc[SMALL ? RP : 4];
+#pragma unroll
+    for (int i = 0; i < (SMALL ? RP : 4); i++) acc[i] = 0.0f;
+
+    // One batch: NV groups c = base + 8 u of this wavefront (NV < AWQ_PF only in the last batch of a ragged K)
+    auto batch = [&](auto nv_tag, int base) {
+        constexpr int NV = decltype(nv_tag)::value;
+        // activations: piece q = lane + 64 i is (group u = q / (8 RP), row r = (q / 8) % RP, slot q % 8)
+#pragma unroll
+        for (int i = 0; i < XPASSES; i++) {
+            const int q = lane + 64 * i, u = q / (8 * RP), r = (q >> 3) & (RP - 1), slot = q & 7;
+            const int c = min(base + AWQ_WAVES * u, ngroups - 1);
+            const uint32_t off = ((uint32_t)min(r, a.M - 1) * (uint32_t)a.ld_x + c * GROUP + 8 * (slot ^ r)) * 2;
+            if (XPIECES % 64 == 0 || i + 1 < XPASSES || q < XPIECES)
+                __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)((const uint8_t *)a.x + off), (SVDQ_AS3 void *)(xw + 1024 * i), 16, 0, 0);
+        }
+        {   // scales: lanes 0 .. 4 PF - 1 = (group, 16-byte piece of its 32 channels); zeros: the next 4 PF lanes
+            const bool z = lane >= 4 * AWQ_PF;
+            const int t = lane - (z ? 4 * AWQ_PF : 0), c = min(base + AWQ_WAVES * (t >> 2), ngroups - 1);
+            const uint32_t off = ((uint32_t)c * (uint32_t)a.ld_scales + nb0 + 8 * (t & 3)) * 2;
+            if (lane < 8 * AWQ_PF)
+                __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)((const uint8_t *)(z ? a.zeros : a.scales) + off), (SVDQ_AS3 void *)szw, 16, 0, 0);
+        }
+        v4i wreg[NV];
+#pragma unroll
+        for (int u = 0; u < NV; u++)
+            wreg[u] = awq_wload((const v4i *)((const uint8_t *)a.qweight + (woff + (uint32_t)(base + AWQ_WAVES * u) * (GROUP * 2))));
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(NV, 15));  // activations, scales and zeros have landed
+        // sums of the activations: every lane adds up its own piece, then the lanes of a (half) row are added
+#pragma unroll
+        for (int i = 0; i < XPASSES; i++) {
+            const int q = min(lane + 64 * i, XPIECES - 1), u = q / (8 * RP), r = (q >> 3) & (RP - 1), slot = q & 7;
+            const v4i v = *(const v4i *)(xw + 16 * q);
+            float s = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 4; e++) s += T::lo_f32((uint32_t)v[e]) + T::hi_f32((uint32_t)v[e]);
+            s += dpp_f32<0xB1>(s);  // quad_perm [1, 0, 3, 2]
+            s += dpp_f32<0x4E>(s);  // quad_perm [2, 3, 0, 1]
+            if (SMALL) {            // slots 4 h .. 4 h + 3 hold the pieces of half h (r < 4 permutes within them)
+                if ((slot & 3) == 0) xsw[u * 8 + (slot >> 2) * 4 + r] = s;
+            } else {
+                s += dpp_f32<0x141>(s);  // row_half_mirror: lane i <-> 7 - i of the octet
+                if (slot == 0) xsw[u * 8 + r] = s;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < NV; u++) {
+            const v4i w = wreg[u];
+            const float s = T::to_f32(((const uint16_t *)szw)[u * 32 + ch]);
+            const float zz = T::to_f32(((const uint16_t *)szw)[(AWQ_PF + u) * 32 + ch]) - AwqMagic<T>::off * s;
+            const uint8_t *at = aop + u * (RP * 128);
+            if constexpr (SMALL) {
+                v4f d0 = {0.0f, 0.0f, 0.0f, 0.0f}, d1 = d0;
+#pragma unroll
+                for (int pl = 0; pl < 4; pl++) {
+                    v4i wb;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) wb[e] = nibble_plane(w[e], 4 * pl, mask, AwqMagic<T>::bits);
+                    const v4i xa = *(const v4i *)(at + aslot[pl]);
+                    d0 = mfma4_16bit<T>(v2i{xa[0], xa[1]}, v2i{wb[0], wb[1]}, d0);
+                    d1 = mfma4_16bit<T>(v2i{xa[2], xa[3]}, v2i{wb[2], wb[3]}, d1);
+                }
+                const v4f xv = *(const v4f *)(xsw + u * 8 + 4 * half);
+#pragma unroll
+                for (int r = 0; r < RP; r++) {
+                    acc[r] = __builtin_fmaf(s, d0[r] + d1[r], acc[r]);
+                    acc[r] = __builtin_fmaf(zz, xv[r], acc[r]);
+                }
+            } else {
+                v16f d;
+#pragma unroll
+                for (int i = 0; i < 16; i++) d[i] = 0.0f;
+#pragma unroll
+                for (int pl = 0; pl < 4; pl++) {
+                    v4i wb;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) wb[e] = nibble_plane(w[e], 4 * pl, mask, AwqMagic<T>::bits);
+                    const v4i xa = *(const v4i *)(at + aslot[pl]);
+                    d = mfma32_16bit<T>(xa, wb, d);
+                }
+                const v4f xv = *(const v4f *)(xsw + u * 8 + 4 * half);
+#pragma unroll
+                for (int e = 0; e < 4; e++) {  // accumulator register e = row 4 h + e (rows 0 .. 7)
+                    acc[e] = __builtin_fmaf(s, d[e], acc[e]);
+                    acc[e] = __builtin_fmaf(zz, xv[e], acc[e]);
+                }
+            }
+        }
+    };
+    for (int base = wave; base < ngroups; base += AWQ_PF * AWQ_WAVES) {
+        const int nv = (ngroups - base + AWQ_WAVES - 1) / AWQ_WAVES;  // wave-uniform
+        if (nv >= AWQ_PF) batch(std::integral_constant<int, AWQ_PF>{}, base);
+        else if (nv == 5) batch(std::integral_constant<int, 5>{}, base);
+        else if (nv == 4) batch(std::integral_constant<int, 4>{}, base);
+        else if (nv == 3) batch(std::integral_constant<int, 3>{}, base);
+        else if (nv == 2) batch(std::integral_constant<int, 2>{}, base);
+        else batch(std::integral_constant<int, 1>{}, base);
+    }
+
+    // fixed-order sum over the wavefronts (and halves): partial sums [half][row][channel] (RP <= 4) or [row][channel]
+    // in the wavefront's own, now unused, x tiles; then store T
+    float *red = (float *)xw;
+    if constexpr (SMALL) {
+#pragma unroll
+        for (int r = 0; r < RP; r++) red[(half * RP + r) * AWQ_NB + ch] = acc[r];
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; e++) red[(4 * half + e) * AWQ_NB + ch] = acc[e];
+    }
+    __syncthreads();
+    if (tid < a.M * AWQ_NB) {
+        float s = 0.0f;
+#pragma unroll
+        for (int w = 0; w < AWQ_WAVES; w++) {
+            const float *rw = (const float *)(lds8 + w * WB);
+            if constexpr (SMALL)
+                s += rw[tid] + rw[RP * AWQ_NB + tid];
+            else
+                s += rw[tid];
+        }
+        ((uint16_t *)a.out)[(size_t)(tid / AWQ_NB) * a.ld_out + nb0 + tid % AWQ_NB] = T::from_f32(s);
+    }
+}
+
+// 8 < M <= 32, MQ = ceil(M / 8) accumulator register quads hold real rows.  One workgroup = 32 channels x all of K; its
+// wavefronts take groups round-robin; the scales and zeros of the channels and the group sums of the activations are
+// staged in LDS, the MFMA A operand is read from global memory (L2: every workgroup reads the same rows).
+template <typename T, int MQ>
+__global__ __launch_bounds__(AWQ_WAVES * 64) void awq_gemv_kernel(svdq_awq_gemv_args a) {
+    // xs[K/64][8*MQ] fp32 | red[AWQ_WAVES][8*MQ][32] fp32 | sz[K/64][2][32] 16-bit
     extern __shared__ __align__(16) float lds[];
     constexpr int MR = 8 * MQ;
     const int ngroups = a.K / GROUP;
     float *xs = lds;
     float *red = lds + (size_t)ngroups * MR;
     uint16_t *sz = (uint16_t *)(red + AWQ_WAVES * MR * AWQ_NB);
-    uint16_t *xl = sz + (size_t)ngroups * 2 * AWQ_NB;
-    const int xld = a.K + AWQ_XPAD;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keep it in an SGPR
@@ -73,68 +262,19 @@ __global__ __launch_bounds__(AWQ_WAVES * 64, 6) void awq_gemv_kernel(svdq_awq_ge
     const int n = nb0 + l32;
     const uint16_t *__restrict__ x = (const uint16_t *)a.x;
 
-    // 1. the small loads first (activations, scales, zeros), so that waiting for them does not wait for the weights
-    v4i xst[3];  // up to 3 x 16-byte pieces of activations per thread (M * K / 8 <= 3 * 256 covers M = 2 at K = 3072)
-    const int per_row = a.K / 8, xpieces = X_IN_LDS ? a.M * per_row : 0;
-    if (X_IN_LDS) {
-#pragma unroll
-        for (int u = 0; u < 3; u++) {
-            const int p = tid + u * AWQ_WAVES * 64;
-            if (p < xpieces) xst[u] = *(const v4i *)(x + (size_t)(p / per_row) * a.ld_x + 8 * (p % per_row));
-        }
-    }
     // scales / zeros of the 32 channels: group c, 64 bytes each -> thread (c = p / 4, piece = p % 4)
-    v4i sst[2], zst[2];
-#pragma unroll
-    for (int u = 0; u < 2; u++) {
-        const int p = tid + u * AWQ_WAVES * 64;
-        if (p < ngroups * 4) {
-            sst[u] = *(const v4i *)((const uint16_t *)a.scales + (size_t)(p >> 2) * a.ld_scales + nb0 + 8 * (p & 3));
-            zst[u] = *(const v4i *)((const uint16_t *)a.zeros + (size_t)(p >> 2) * a.ld_scales + nb0 + 8 * (p & 3));
-        }
-    }
-
-    // 2. this lane's weight stream: packed row n / 4, int16 column 64 c + 16 (n % 4) + 8 h, groups c = wave + 4 i
-    const uint16_t *__restrict__ wq =
-        (const uint16_t *)a.qweight + (size_t)(n >> 2) * a.K + 16 * (n & 3) + 8 * half + (size_t)wave * GROUP;
-    const int wstep = AWQ_WAVES * GROUP;
-    const int nmy = (ngroups - wave + AWQ_WAVES - 1) / AWQ_WAVES;
-    v4i wreg[AWQ_PF];
-#pragma unroll
-    for (int u = 0; u < AWQ_PF; u++)
-        if (u < nmy) wreg[u] = awq_wload((const v4i *)(wq + (size_t)u * wstep));
-
-    // 3. stage the small data in LDS
-    if (X_IN_LDS) {
-#pragma unroll
-        for (int u = 0; u < 3; u++) {
-            const int p = tid + u * AWQ_WAVES * 64;
-            if (p < xpieces) *(v4i *)(xl + (p / per_row) * xld + 8 * (p % per_row)) = xst[u];
-        }
-        for (int p = tid + 3 * AWQ_WAVES * 64; p < xpieces; p += AWQ_WAVES * 64)  // more rows: plain copy loop
-            *(v4i *)(xl + (p / per_row) * xld + 8 * (p % per_row)) = *(const v4i *)(x + (size_t)(p / per_row) * a.ld_x + 8 * (p % per_row));
-    }
-#pragma unroll
-    for (int u = 0; u < 2; u++) {
-        const int p = tid + u * AWQ_WAVES * 64;
-        if (p < ngroups * 4) {
-            *(v4i *)(sz + ((p >> 2) * 2 + 0) * AWQ_NB + 8 * (p & 3)) = sst[u];
-            *(v4i *)(sz + ((p >> 2) * 2 + 1) * AWQ_NB + 8 * (p & 3)) = zst[u];
-        }
-    }
-    for (int p = tid + 2 * AWQ_WAVES * 64; p < ngroups * 4; p += AWQ_WAVES * 64) {  // K > 8192
+    for (int p = tid; p < ngroups * 4; p += AWQ_WAVES * 64) {
         *(v4i *)(sz + ((p >> 2) * 2 + 0) * AWQ_NB + 8 * (p & 3)) =
             *(const v4i *)((const uint16_t *)a.scales + (size_t)(p >> 2) * a.ld_scales + nb0 + 8 * (p & 3));
         *(v4i *)(sz + ((p >> 2) * 2 + 1) * AWQ_NB + 8 * (p & 3)) =
             *(const v4i *)((const uint16_t *)a.zeros + (size_t)(p >> 2) * a.ld_scales + nb0 + 8 * (p & 3));
     }
-    __syncthreads();
     // xs[c][m] = sum of the group's 64 activations (fp32)
     for (int p = tid; p < ngroups * MR; p += AWQ_WAVES * 64) {
         const int c = p / MR, m = p % MR;
         float s = 0.0f;
         if (m < a.M) {
-            const v4i *xp = X_IN_LDS ? (const v4i *)(xl + m * xld + c * GROUP) : (const v4i *)(x + (size_t)m * a.ld_x + c * GROUP);
+            const v4i *xp = (const v4i *)(x + (size_t)m * a.ld_x + c * GROUP);
 #pragma unroll
             for (int q = 0; q < 8; q++) {
                 const v4i v = xp[q];
@@ -150,26 +290,31 @@ __global__ __launch_bounds__(AWQ_WAVES * 64, 6) void awq_gemv_kernel(svdq_awq_ge
 #pragma unroll
     for (int i = 0; i < 4 * MQ; i++) acc[i] = 0.0f;
 
+    // this lane's weight stream: packed row n / 4, int16 column 64 c + 16 (n % 4) + 8 h, groups c = wave + 8 i
+    const uint16_t *__restrict__ wq = (const uint16_t *)a.qweight + (size_t)(n >> 2) * a.K + 16 * (n & 3) + 8 * half;
     // A operand row of this lane; rows >= M repeat row M - 1 (their products land in accumulator rows nobody reads)
-    const int arow = min(l32, a.M - 1);
-    const uint16_t *xrow = (X_IN_LDS ? xl + arow * xld : x + (size_t)arow * a.ld_x) + 32 * half + wave * GROUP;
-    const float *xsp = xs + wave * MR + 4 * half;
-    const uint16_t *szp = sz + wave * 2 * AWQ_NB + l32;
+    const uint16_t *xrow = x + (size_t)min(l32, a.M - 1) * a.ld_x + 32 * half;
     uint32_t mask = 0x000F000Fu;
     asm volatile("" : "+v"(mask));  // keep the mask in a VGPR: v_and_or_b32 takes only one literal
     v16f zero16;
 #pragma unroll
     for (int i = 0; i < 16; i++) zero16[i] = 0.0f;
 
-    for (int base = 0;;) {
+    for (int base = wave; base < ngroups; base += AWQ_PF * AWQ_WAVES) {
+        // AWQ_PF weight loads in flight, issued without branches (past the end the last group is fetched again) so
+        // that every wait counts exactly the loads that must have returned
+        v4i wreg[AWQ_PF];
+#pragma unroll
+        for (int u = 0; u < AWQ_PF; u++)
+            wreg[u] = awq_wload((const v4i *)(wq + (size_t)min(base + AWQ_WAVES * u, ngroups - 1) * GROUP));
 #pragma unroll
         for (int u = 0; u < AWQ_PF; u++) {
-            const int idx = base + u;
-            if (idx < nmy) {
+            const int c = base + AWQ_WAVES * u;
+            if (c < ngroups) {
                 const v4i w = wreg[u];
-                const float s = T::to_f32(szp[idx * (AWQ_WAVES * 2 * AWQ_NB)]);
-                const float zz = T::to_f32(szp[idx * (AWQ_WAVES * 2 * AWQ_NB) + AWQ_NB]) - AwqMagic<T>::off * s;
-                const uint16_t *xg = xrow + idx * wstep;
+                const float s = T::to_f32(sz[(c * 2 + 0) * AWQ_NB + l32]);
+                const float zz = T::to_f32(sz[(c * 2 + 1) * AWQ_NB + l32]) - AwqMagic<T>::off * s;
+                const uint16_t *xg = xrow + c * GROUP;
                 v16f d;
 #pragma unroll
                 for (int pl = 0; pl < 4; pl++) {
@@ -181,7 +326,7 @@ __global__ __launch_bounds__(AWQ_WAVES * 64, 6) void awq_gemv_kernel(svdq_awq_ge
                 }
 #pragma unroll
                 for (int q = 0; q < MQ; q++) {
-                    const v4f xv = *(const v4f *)(xsp + idx * (AWQ_WAVES * MR) + 8 * q);
+                    const v4f xv = *(const v4f *)(xs + c * MR + 8 * q + 4 * half);
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
                         acc[4 * q + e] = __builtin_fmaf(s, d[4 * q + e], acc[4 * q + e]);
@@ -190,11 +335,6 @@ __global__ __launch_bounds__(AWQ_WAVES * 64, 6) void awq_gemv_kernel(svdq_awq_ge
                 }
             }
         }
-        base += AWQ_PF;
-        if (base >= nmy) break;
-#pragma unroll
-        for (int u = 0; u < AWQ_PF; u++)  // K > 3072: next batch of this wavefront's groups
-            if (base + u < nmy) wreg[u] = awq_wload((const v4i *)(wq + (size_t)(base + u) * wstep));
     }
 
     // fixed-order sum over the wavefronts, then store T
@@ -244,37 +384,34 @@ __global__ __launch_bounds__(256) void awq_dequant_kernel(const v4i *__restrict_
     }
 }
 
-// LDS of a launch without the staged activations, and the bytes those would add
+// LDS of a launch with more than eight rows (the kernels for up to eight rows need a fixed amount)
 static size_t awq_lds_bytes(int K, int M) {
+    if (M <= 8) return 0;
     const int MQ = (M + 7) / 8;
     size_t b = ((size_t)(K / GROUP) * 8 * MQ + (size_t)AWQ_WAVES * 8 * MQ * AWQ_NB) * sizeof(float);
     b += (size_t)(K / GROUP) * 2 * AWQ_NB * 2;
     return b;
 }
-static size_t awq_x_lds_bytes(int K, int M) { return (size_t)M * (K + AWQ_XPAD) * 2; }
-static bool awq_stage_x(int K, int M) {
-    // wherever they fit: read from global memory instead, the eight rows of M = 8 cost 17.6 us against 12.6 us at the
-    // FLUX adaLN shape (four 16-byte activation loads per lane and group next to one weight load)
-    return M <= 8 && awq_lds_bytes(K, M) + awq_x_lds_bytes(K, M) <= AWQ_LDS_MAX;
-}
 
 template <typename T>
 static void launch_awq(const svdq_awq_gemv_args &a, hipStream_t s) {
-    const int MQ = (a.M + 7) / 8;
     const dim3 grid(a.N / AWQ_NB), block(AWQ_WAVES * 64);
-    const bool xl = awq_stage_x(a.K, a.M);
-    const size_t sh = awq_lds_bytes(a.K, a.M) + (xl ? awq_x_lds_bytes(a.K, a.M) : 0);
-    switch (MQ) {
-        case 1:
-            if (xl)
-                hipLaunchKernelGGL((awq_gemv_kernel<T, 1, true>), grid, block, sh, s, a);
-            else
-                hipLaunchKernelGGL((awq_gemv_kernel<T, 1, false>), grid, block, sh, s, a);
-            break;
-        case 2: hipLaunchKernelGGL((awq_gemv_kernel<T, 2, false>), grid, block, sh, s, a); break;
-        case 3: hipLaunchKernelGGL((awq_gemv_kernel<T, 3, false>), grid, block, sh, s, a); break;
-        default: hipLaunchKernelGGL((awq_gemv_kernel<T, 4, false>), grid, block, sh, s, a); break;
-    }
+    constexpr size_t XS_BYTES = (size_t)AWQ_WAVES * AWQ_PF * 8 * sizeof(float);
+    const size_t sh = awq_lds_bytes(a.K, a.M);
+    if (a.M <= 1)
+        hipLaunchKernelGGL((awq_gemv_rows_kernel<T, 1>), grid, block, AWQ_WAVES * awq_wave_bytes<1>() + XS_BYTES, s, a);
+    else if (a.M <= 2)
+        hipLaunchKernelGGL((awq_gemv_rows_kernel<T, 2>), grid, block, AWQ_WAVES * awq_wave_bytes<2>() + XS_BYTES, s, a);
+    else if (a.M <= 4)
+        hipLaunchKernelGGL((awq_gemv_rows_kernel<T, 4>), grid, block, AWQ_WAVES * awq_wave_bytes<4>() + XS_BYTES, s, a);
+    else if (a.M <= 8)
+        hipLaunchKernelGGL((awq_gemv_rows_kernel<T, 8>), grid, block, AWQ_WAVES * awq_wave_bytes<8>() + XS_BYTES, s, a);
+    else if (a.M <= 16)
+        hipLaunchKernelGGL((awq_gemv_kernel<T, 2>), grid, block, sh, s, a);
+    else if (a.M <= 24)
+        hipLaunchKernelGGL((awq_gemv_kernel<T, 3>), grid, block, sh, s, a);
+    else
+        hipLaunchKernelGGL((awq_gemv_kernel<T, 4>), grid, block, sh, s, a);
 }
 
 }  // namespace svdq
