@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define SVDQ_ABI_VERSION 4
+#define SVDQ_ABI_VERSION 5
 
 enum { SVDQ_BF16 = 0, SVDQ_FP16 = 1 };
 enum { SVDQ_PRE_NONE = 0, SVDQ_PRE_GLU = 1, SVDQ_PRE_GELU = 2 }; /* svdq_quantize_args.prologue */
@@ -222,15 +222,13 @@ int svdq_awq_dequantize(const void *qweight, const void *scales, const void *zer
  * Unmasked scaled-dot-product attention, head dimension D = 128 or 64 (nunchaku/ops/dispatch.py:67-99 attention_fp16 /
  * ops/triton/attention.py:111-169): o[b, t, h*D + d] = softmax_k(scale * q[b,h,t,:] . k[b,h,k,:]) . v[b,h,k,d], fp32
  * softmax and accumulation, P rounded to T.  Strides are in elements; the last dimension of q, k, v, o is contiguous.
- * `vt` is a caller-owned workspace of svdq_attention_workspace_bytes(B, H, Tkv, D) bytes (a transposed copy of v made
- * by the call itself).
+ * No workspace: v is read in place (the kernel transposes its tiles on the way out of LDS).
  */
 typedef struct {
     const void *q;  /* (B, H, Tq, D) T  */
     const void *k;  /* (B, H, Tkv, D) T */
     const void *v;  /* (B, H, Tkv, D) T */
     void *o;        /* (B, Tq, H * D) T */
-    void *vt;       /* workspace          */
     int64_t sqb, sqh, sqm, skb, skh, skn, svb, svh, svn, sob, som;
     int32_t B, H, Tq, Tkv, D;
     int32_t dtype;
@@ -238,7 +236,6 @@ typedef struct {
 } svdq_attention_args;
 
 int svdq_attention_fp16(const svdq_attention_args *args, void *stream);
-size_t svdq_attention_workspace_bytes(int32_t B, int32_t H, int32_t Tkv, int32_t D);
 
 /*
  * Checkpoint ingestion.  The published SVDQuant int4 checkpoints hold every tensor of a quantized linear pre-shuffled

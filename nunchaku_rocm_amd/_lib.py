@@ -14,7 +14,7 @@ import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libsvdq_mi355x.so")
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 BF16, FP16 = 0, 1
 EPI_PLAIN, EPI_QK_NORM_ROPE, EPI_GELU_QUANT, EPI_SWIGLU_QUANT = 0, 1, 2, 3
@@ -36,7 +36,6 @@ EXPORTS = (
     "svdq_awq_gemv_w4a16",
     "svdq_awq_dequantize",
     "svdq_attention_fp16",
-    "svdq_attention_workspace_bytes",
     "svdq_unpack_mma_weight",
     "svdq_unpack_mma_scale",
     "svdq_unpack_mma_lowrank",
@@ -87,7 +86,7 @@ class AttentionArgs(ctypes.Structure):
     """``svdq_attention_args``"""
 
     _fields_ = (
-        [(n, _vp) for n in ("q", "k", "v", "o", "vt")]
+        [(n, _vp) for n in ("q", "k", "v", "o")]
         + [(n, _i64) for n in ("sqb", "sqh", "sqm", "skb", "skh", "skn", "svb", "svh", "svn", "sob", "som")]
         + [(n, _i32) for n in ("B", "H", "Tq", "Tkv", "D", "dtype")]
         + [("scale", _f32)]
@@ -131,8 +130,6 @@ def load() -> ctypes.CDLL:
     lib.svdq_awq_gemv_w4a16.argtypes = [ctypes.POINTER(AwqGemvArgs), _vp]
     lib.svdq_awq_dequantize.argtypes = [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _vp]
     lib.svdq_attention_fp16.argtypes = [ctypes.POINTER(AttentionArgs), _vp]
-    lib.svdq_attention_workspace_bytes.restype = ctypes.c_size_t
-    lib.svdq_attention_workspace_bytes.argtypes = [_i32, _i32, _i32, _i32]
     lib.svdq_unpack_mma_weight.argtypes = [_vp, _vp, _i32, _i32, _i32, _vp]
     lib.svdq_unpack_mma_scale.argtypes = [_vp, _vp, _i32, _i32, _i32, _vp]
     lib.svdq_unpack_mma_lowrank.argtypes = [_vp, _vp, _i32, _i32, _i32, _i32, _vp]

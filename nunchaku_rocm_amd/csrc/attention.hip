@@ -13,19 +13,20 @@
 //    maximum and row sum of the softmax are in-lane reductions plus one exchange with lane ^ 32
 //    (v_permlane32_swap), and the rescaling of the output accumulator is a per-lane scalar.  O^T = V^T P^T then
 //    takes P^T as its B operand straight from those accumulator registers (eight values of a lane are the eight
-//    k-slots the operand wants; the k order inside a 16-key chunk is the permutation 0-3, 8-11 | 4-7, 12-15, which
-//    V^T simply shares), with no trip through LDS.
+//    k-slots the operand wants: keys 4 h .. 4 h + 3 and 8 + 4 h .. 8 + 4 h + 3 of a 16-key chunk for the lanes of
+//    half h), with no trip through LDS.
 //  * The S^T accumulator starts at minus the row reference, so the scores leave the matrix instruction ready for
 //    exp2: no subtraction per score.
-//  * V^T is made once per call by a small transposing kernel (keys permuted as above, key count padded to 64); the
-//    main kernel then streams K tiles (64 keys x 2 D bytes) and V^T tiles (D rows x 128 bytes) buffer -> LDS
-//    directly (buffer_load_dwordx4 ... lds, whole rows per load, per-lane offsets fixed and the tile chosen by the
-//    scalar buffer base, 16-byte chunks XOR-swizzled so that the operand reads are conflict free), two tiles in
-//    flight, one barrier per 64 keys.
+//  * V is never transposed in memory: K and V tiles (64 keys x 2 D bytes each) stream buffer -> LDS directly
+//    (buffer_load_dwordx4 ... lds, whole rows per load, per-lane offsets fixed and the tile chosen by the scalar
+//    buffer base, 16-byte chunks XOR-swizzled so that the operand reads are conflict free), two tiles in flight, one
+//    barrier per 64 keys; the V^T operand comes out of the V tile through the transposing LDS read of gfx950
+//    (ds_read_b64_tr_b16: sixteen lanes pass the addresses of four rows x 16 columns and lane l receives column l
+//    of the four rows), two reads per operand.
 //  * 256 threads = 4 wavefronts of 32 queries, two workgroups per CU; Q stays in registers (pre-scaled), the output
 //    accumulator is D / 2 registers.  A tile is processed as two 32-key halves so that the softmax instructions of one
 //    half sit between the matrix instructions of the other (see the pipeline comment in the kernel).
-//  * Workgroups of one head run on one XCD (when the head count is a multiple of 8), so K and V^T of a head are
+//  * Workgroups of one head run on one XCD (when the head count is a multiple of 8), so K and V of a head are
 //    fetched into one L2 only.
 #include "svdq_common.h"
 
@@ -33,10 +34,12 @@ namespace svdq {
 
 constexpr int AT_BQ = 128, AT_BK = 64;     // queries per workgroup, keys per tile
 
-// Geometry for head dimension D (128 or 64).  A K tile is [key][2 D bytes], a V^T tile [d][128 bytes]; every block
-// load moves 1 KB (64 lanes x 16 bytes) = whole rows; 16-byte chunks are XOR-swizzled by the row so that the operand
-// reads (32 rows x one chunk per half-wave) touch every bank once: rows of 256 bytes by row & 15, rows of 128 bytes (two
-// rows span the 64 banks) by row / 2 & 7.
+// Geometry for head dimension D (128 or 64).  K and V tiles are [key][2 D bytes]; every block load moves 1 KB
+// (64 lanes x 16 bytes) = whole rows; 16-byte chunks are XOR-swizzled by the row so that the operand reads touch every
+// bank once.  K (32 rows x one chunk per half-wave): rows of 256 bytes by row & 15, rows of 128 bytes (two rows span
+// the 64 banks) by row / 2 & 7.  V (a transposing read = 4 rows x 32 bytes per 16 lanes): the four rows must land in
+// four different 32-byte slots of the banks, so chunk pairs are swizzled by row & 3 (256-byte rows) or row / 2 & 1
+// (128-byte rows, where rows r and r + 1 already differ by half the banks).
 template <int D>
 struct AtGeo {
     static constexpr int NC = D / 16;               // 16-wide k chunks of q k^T = matrix instructions per 32-key half
@@ -44,48 +47,13 @@ struct AtGeo {
     static constexpr int KROW = 2 * D;              // bytes per key row
     static constexpr int KCH = KROW / 16;           // chunks per key row (16 or 8)
     static constexpr int KT_BYTES = AT_BK * KROW;   // K tile
-    static constexpr int VT_BYTES = D * AT_BK * 2;  // V^T tile
+    static constexpr int VT_BYTES = KT_BYTES;       // V tile
     static constexpr int STAGE = KT_BYTES + VT_BYTES;
-    static constexpr int LOADS = KT_BYTES / 1024 / 4;  // block loads per wavefront and tile, of K and of V^T alike
+    static constexpr int LOADS = KT_BYTES / 1024 / 4;  // block loads per wavefront and tile, of K and of V alike
     static constexpr int OPITCH = 2 * D + 16;       // staged output row
     __host__ __device__ static constexpr int kswz(int row) { return KROW == 256 ? (row & 15) : ((row >> 1) & 7); }
+    __host__ __device__ static constexpr int vswz(int row) { return KROW == 256 ? ((row & 3) << 1) : (((row >> 1) & 1) << 1); }
 };
-
-// position p of a 16-key chunk holds key sigma(p)
-__device__ __host__ inline int at_sigma(int p) { return (p & 3) | ((p & 4) << 1) | ((p & 8) >> 1); }
-
-// V (B, H, Tkv, D) with arbitrary strides -> vt[(b * H + h) * D + d][Tpad], keys permuted inside 16-key chunks,
-// keys >= Tkv zero
-template <int D>
-__global__ __launch_bounds__(256) void transpose_v_kernel(const uint16_t *v, uint16_t *vt, int H, int Tkv, int Tpad,
-                                                          long svb, long svh, long svn) {
-    __shared__ uint16_t tile[AT_BK][D + 2];
-    const int k0 = blockIdx.x * AT_BK, h = blockIdx.y, b = blockIdx.z;
-    const uint16_t *vb = v + b * svb + h * svh;
-    for (int i = threadIdx.x; i < AT_BK * (D / 8); i += 256) {
-        const int key = i / (D / 8), c = i % (D / 8);
-        v4i x = {0, 0, 0, 0};
-        if (k0 + key < Tkv) x = *(const v4i *)(vb + (long)(k0 + key) * svn + 8 * c);
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-            tile[key][8 * c + 2 * e] = (uint16_t)((uint32_t)x[e] & 0xFFFFu);
-            tile[key][8 * c + 2 * e + 1] = (uint16_t)((uint32_t)x[e] >> 16);
-        }
-    }
-    __syncthreads();
-    uint16_t *ob = vt + ((size_t)(b * H + h) * D) * Tpad + k0;
-    for (int i = threadIdx.x; i < D * (AT_BK / 8); i += 256) {
-        const int d = i / (AT_BK / 8), c = i % (AT_BK / 8);  // 8 consecutive positions of row d
-        uint32_t w[4];
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-            const int p0 = 8 * c + 2 * e, p1 = p0 + 1;
-            const int key0 = (p0 & ~15) | at_sigma(p0 & 15), key1 = (p1 & ~15) | at_sigma(p1 & 15);
-            w[e] = (uint32_t)tile[key0][d] | ((uint32_t)tile[key1][d] << 16);
-        }
-        *(v4i *)(ob + (size_t)d * Tpad + 8 * c) = (v4i){(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
-    }
-}
 
 constexpr uint32_t AT_RSRC_FLAGS = 0x00020000;  // raw buffer, 32-bit data format (gfx9 family)
 
@@ -97,10 +65,17 @@ __device__ inline __amdgpu_buffer_rsrc_t at_buffer(const void *base, uint32_t by
 __device__ inline void at_load16_lds(__amdgpu_buffer_rsrc_t r, uint8_t *lds, uint32_t lane_off, uint32_t wave_off) {
     __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (SVDQ_AS3 void *)lds, 16, lane_off, wave_off, 0, 0);
 }
+// four rows x one column of a [row][col] 16-bit matrix in LDS: the sixteen lanes of a group pass the addresses of
+// (row r = lane % 16 / 4, columns 4 (lane % 4) .. + 3) and lane l of the group receives column l of rows 0 .. 3
+typedef short v4s16 __attribute__((ext_vector_type(4)));
+typedef int v2i32 __attribute__((ext_vector_type(2)));
+__device__ inline v2i32 at_read_tr(const uint8_t *p) {
+    return __builtin_bit_cast(v2i32, __builtin_amdgcn_ds_read_tr16_b64_v4i16((SVDQ_AS3 v4s16 *)p));
+}
 constexpr float AT_LAZY = 8.0f;                 // the accumulator is rescaled when a row maximum grew by more than this
 
 template <typename T, int D>
-__global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a, int Tpad, int ntile, int xcd_heads) {
+__global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a, int ntile, int xcd_heads) {
     using G = AtGeo<D>;
     constexpr int NC = G::NC, NDT = G::NDT, LOADS = G::LOADS;
     __shared__ __align__(16) uint8_t smem[2 * G::STAGE];
@@ -109,7 +84,7 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31, half = lane >> 5;
     // workgroup -> (batch * head, query tile).  Workgroups are dealt to the eight XCDs round-robin; when the head count
-    // allows it, a head's query tiles all land on one XCD so that its K and V^T stay in that XCD's L2.
+    // allows it, a head's query tiles all land on one XCD so that its K and V stay in that XCD's L2.
     int bh, qt;
     if (xcd_heads) {
         const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
@@ -135,39 +110,50 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a
             qop[c][e] = (int)pack2<T>(T::lo_f32((uint32_t)raw[e]) * qscale, T::hi_f32((uint32_t)raw[e]) * qscale);
     }
 
-    // ---- tile loads (buffer -> LDS, 16 bytes per lane): lane l of K load i fetches one chunk of key row
-    // (64 / KCH) i + l / KCH; of V^T load i, one chunk of d row 8 i + l / 8.  LOADS K and LOADS V^T loads per wavefront
-    // and tile.  The per-lane offsets never change; the tile is selected by the (scalar) buffer base, and key rows
-    // past the end lie outside the K buffer's range and arrive as zeros.
+    // ---- tile loads (buffer -> LDS, 16 bytes per lane): lane l of load i fetches one chunk of key row
+    // (64 / KCH) i + l / KCH of K and of V alike.  LOADS K and LOADS V loads per wavefront and tile.  The per-lane
+    // offsets never change; the tile is selected by the (scalar) buffer base, and key rows past the end lie outside
+    // the buffers' ranges and arrive as zeros.
     const uint8_t *kbase = (const uint8_t *)a.k + ((long)b * a.skb + (long)h * a.skh) * 2;
-    const uint8_t *vbase = (const uint8_t *)a.vt + ((size_t)bh * D) * Tpad * 2;
+    const uint8_t *vbase = (const uint8_t *)a.v + ((long)b * a.svb + (long)h * a.svh) * 2;
     const uint32_t kbytes = (uint32_t)(((long)(a.Tkv - 1) * a.skn + D) * 2);
-    const uint32_t ktile = (uint32_t)(AT_BK * a.skn * 2);
+    const uint32_t vbytes = (uint32_t)(((long)(a.Tkv - 1) * a.svn + D) * 2);
+    const uint32_t ktile = (uint32_t)(AT_BK * a.skn * 2), vtile = (uint32_t)(AT_BK * a.svn * 2);
     uint32_t kvo[LOADS], vvo[LOADS];
 #pragma unroll
     for (int j = 0; j < LOADS; j++) {
         const int i = wave * LOADS + j;
-        const int krow = (64 / G::KCH) * i + lane / G::KCH;
-        kvo[j] = (uint32_t)krow * (uint32_t)(a.skn * 2) + (uint32_t)(((lane % G::KCH) ^ G::kswz(krow)) * 16);
-        const int vrow = 8 * i + (lane >> 3);
-        vvo[j] = (uint32_t)vrow * (uint32_t)Tpad * 2 + (uint32_t)(((lane & 7) ^ ((vrow >> 1) & 7)) * 16);
+        const int row = (64 / G::KCH) * i + lane / G::KCH;
+        kvo[j] = (uint32_t)row * (uint32_t)(a.skn * 2) + (uint32_t)(((lane % G::KCH) ^ G::kswz(row)) * 16);
+        vvo[j] = (uint32_t)row * (uint32_t)(a.svn * 2) + (uint32_t)(((lane % G::KCH) ^ G::vswz(row)) * 16);
     }
-    const __amdgpu_buffer_rsrc_t vres = at_buffer(vbase, (uint32_t)(D * Tpad * 2));
     auto issue_k = [&](int blk, int stage, int j) {
         const uint32_t off = (uint32_t)blk * ktile;
         at_load16_lds(at_buffer(kbase + off, kbytes - off), smem + stage * G::STAGE + (wave * G::LOADS + j) * 1024, kvo[j], 0);
     };
     auto issue_v = [&](int blk, int stage, int j) {
-        at_load16_lds(vres, smem + stage * G::STAGE + G::KT_BYTES + (wave * G::LOADS + j) * 1024, vvo[j],
-                      (uint32_t)blk * (AT_BK * 2));
+        const uint32_t off = (uint32_t)blk * vtile;
+        at_load16_lds(at_buffer(vbase + off, vbytes - off), smem + stage * G::STAGE + G::KT_BYTES + (wave * G::LOADS + j) * 1024, vvo[j], 0);
     };
 
-    // operand read offsets: K rows 32 t + l32 (chunk 2 c + half), V^T rows 32 dt + l32 (chunk 2 c + half)
-    int koff[NC], vtoff[4];
+    // operand read offsets.  K rows 32 t + l32 (chunk 2 c + half).  V^T operand of d tile dt and 16-key chunk c: lane
+    // (half, dq = lane / 16 % 2, r = lane % 16 / 4, c4 = lane % 4) passes the address of V[16 c + 4 half + r (+ 8 for
+    // the second read)][32 dt + 16 dq + 4 c4] and receives d = 32 dt + lane % 32, keys 4 half .. + 3 (8 + 4 half .. + 3)
+    int koff[NC], vtoff[NDT];
 #pragma unroll
     for (int c = 0; c < NC; c++) koff[c] = l32 * G::KROW + (((2 * c + half) ^ G::kswz(l32)) * 16);
+    {
+        const int dq = (lane >> 4) & 1, r = (lane & 15) >> 2, c4 = lane & 3, key = 4 * half + r;
 #pragma unroll
-    for (int c = 0; c < 4; c++) vtoff[c] = G::KT_BYTES + l32 * 128 + (((2 * c + half) ^ ((l32 >> 1) & 7)) * 16);
+        for (int dt = 0; dt < NDT; dt++)
+            vtoff[dt] = G::KT_BYTES + key * G::KROW + (((4 * dt + 2 * dq + (c4 >> 1)) ^ G::vswz(key)) * 16) + 8 * (c4 & 1);
+    }
+    // (keys 16 c + 8 + key have the same swizzle as key: both leave key % 4 and, for 128-byte rows, key / 2 % 2 alone)
+    auto read_v = [&](const uint8_t *st, int dt, int c) {
+        const v2i32 lo = at_read_tr(st + vtoff[dt] + c * (16 * G::KROW));
+        const v2i32 hi = at_read_tr(st + vtoff[dt] + c * (16 * G::KROW) + 8 * G::KROW);
+        return v4i{lo[0], lo[1], hi[0], hi[1]};
+    };
 
     v16f acc_o[NDT];
 #pragma unroll
@@ -271,7 +257,7 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a
 #pragma unroll
         for (int c = 0; c < NC; c++) {
             s0 = mfma32_16bit<T>(rk[c], qop[c], c == 0 ? cinit : s0);
-            rv[4 * (c % NDT) + c / NDT] = *(const v4i *)(st + (c % NDT) * (32 * 128) + vtoff[c / NDT]);  // chunks 0, 1: keys 0..31
+            rv[4 * (c % NDT) + c / NDT] = read_v(st, c % NDT, c / NDT);  // chunks 0, 1: keys 0..31
             __builtin_amdgcn_sched_barrier(0);
         }
         if (ragged) {  // keys past the end count as -inf
@@ -285,7 +271,7 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a
 #pragma unroll
         for (int c = 0; c < NC; c++) {
             s1 = mfma32_16bit<T>(rk[NC + c], qop[c], c == 0 ? cinit : s1);
-            rv[4 * (c % NDT) + 2 + c / NDT] = *(const v4i *)(st + (c % NDT) * (32 * 128) + vtoff[2 + c / NDT]);  // keys 32..63
+            rv[4 * (c % NDT) + 2 + c / NDT] = read_v(st, c % NDT, 2 + c / NDT);  // keys 32..63
             if (c == 0) {
                 moved = row_max(s0);
                 rs = 0.0f;
@@ -366,23 +352,15 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a
 }
 
 template <typename T, int D>
-static void launch_attention(const svdq_attention_args &a, int Tpad, hipStream_t s) {
-    hipLaunchKernelGGL(transpose_v_kernel<D>, dim3(Tpad / AT_BK, a.H, a.B), dim3(256), 0, s, (const uint16_t *)a.v,
-                       (uint16_t *)a.vt, a.H, a.Tkv, Tpad, (long)a.svb, (long)a.svh, (long)a.svn);
+static void launch_attention(const svdq_attention_args &a, hipStream_t s) {
     const int ntile = (a.Tq + AT_BQ - 1) / AT_BQ;
     const int xcd_heads = (a.B * a.H) % 8 == 0;
-    hipLaunchKernelGGL((attention_kernel<T, D>), dim3((unsigned)(ntile * a.H * a.B)), dim3(256), 0, s, a, Tpad, ntile, xcd_heads);
+    hipLaunchKernelGGL((attention_kernel<T, D>), dim3((unsigned)(ntile * a.H * a.B)), dim3(256), 0, s, a, ntile, xcd_heads);
 }
 
 }  // namespace svdq
 
 using namespace svdq;
-
-extern "C" size_t svdq_attention_workspace_bytes(int32_t B, int32_t H, int32_t Tkv, int32_t D) {
-    if (B <= 0 || H <= 0 || Tkv <= 0 || (D != 128 && D != 64)) return 0;
-    const size_t Tpad = (size_t)((Tkv + AT_BK - 1) / AT_BK) * AT_BK;
-    return (size_t)B * H * D * Tpad * 2;
-}
 
 extern "C" int svdq_attention_fp16(const svdq_attention_args *args, void *stream) {
     if (!args) {
@@ -402,38 +380,39 @@ extern "C" int svdq_attention_fp16(const svdq_attention_args *args, void *stream
         set_error("svdq_attention_fp16: bad shape B=%d H=%d Tq=%d Tkv=%d", a.B, a.H, a.Tq, a.Tkv);
         return SVDQ_E_INVALID;
     }
-    if (!a.q || !a.k || !a.v || !a.o || !a.vt) {
-        set_error("svdq_attention_fp16: null tensor (q, k, v, o and the V^T workspace are required)");
+    if (!a.q || !a.k || !a.v || !a.o) {
+        set_error("svdq_attention_fp16: null tensor");
         return SVDQ_E_INVALID;
     }
     auto al = [](const void *p) { return ((uintptr_t)p & 15) == 0; };
-    if (!al(a.q) || !al(a.k) || !al(a.v) || !al(a.o) || !al(a.vt) || a.sqm % 8 || a.sqh % 8 || a.sqb % 8 || a.skn % 8 ||
+    if (!al(a.q) || !al(a.k) || !al(a.v) || !al(a.o) || a.sqm % 8 || a.sqh % 8 || a.sqb % 8 || a.skn % 8 ||
         a.skh % 8 || a.skb % 8 || a.svn % 8 || a.svh % 8 || a.svb % 8 || a.som % 8 || a.sob % 8) {
         set_error("svdq_attention_fp16: tensors and their row / head / batch strides must be 16-byte aligned");
         return SVDQ_E_INVALID;
     }
     if (a.Tq == 0) return SVDQ_OK;
     const int Tpad = (a.Tkv + AT_BK - 1) / AT_BK * AT_BK;
-    if ((size_t)a.D * Tpad * 2 >= ((size_t)1 << 31) || ((size_t)Tpad * a.skn + a.D) * 2 >= ((size_t)1 << 31) ||
+    if (((size_t)Tpad * a.svn + a.D) * 2 >= ((size_t)1 << 31) || ((size_t)Tpad * a.skn + a.D) * 2 >= ((size_t)1 << 31) ||
         (size_t)a.B * a.H * ((a.Tq + AT_BQ - 1) / AT_BQ) >= ((size_t)1 << 31)) {
-        set_error("svdq_attention_fp16: Tq=%d Tkv=%d key stride %lld: too large for 32-bit tile offsets", a.Tq, a.Tkv, (long long)a.skn);
+        set_error("svdq_attention_fp16: Tq=%d Tkv=%d key / value stride %lld / %lld: too large for 32-bit tile offsets", a.Tq, a.Tkv,
+                  (long long)a.skn, (long long)a.svn);
         return SVDQ_E_UNSUPPORTED;
     }
-    if (a.skn < a.D) {
-        set_error("svdq_attention_fp16: key rows overlap (stride %lld < head dimension)", (long long)a.skn);
+    if (a.skn < a.D || a.svn < a.D) {
+        set_error("svdq_attention_fp16: key or value rows overlap (stride %lld / %lld < head dimension)", (long long)a.skn, (long long)a.svn);
         return SVDQ_E_INVALID;
     }
     hipStream_t s = (hipStream_t)stream;
     if (a.D == 128) {
         if (a.dtype == SVDQ_BF16)
-            launch_attention<BF16, 128>(a, Tpad, s);
+            launch_attention<BF16, 128>(a, s);
         else
-            launch_attention<FP16, 128>(a, Tpad, s);
+            launch_attention<FP16, 128>(a, s);
     } else {
         if (a.dtype == SVDQ_BF16)
-            launch_attention<BF16, 64>(a, Tpad, s);
+            launch_attention<BF16, 64>(a, s);
         else
-            launch_attention<FP16, 64>(a, Tpad, s);
+            launch_attention<FP16, 64>(a, s);
     }
     return check_launch("svdq_attention_fp16");
 }

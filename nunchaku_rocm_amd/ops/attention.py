@@ -26,13 +26,11 @@ def attention_fp16(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, o: torch.T
         raise ValueError("q, k, v and o must share one dtype")
     if any(t.stride(-1) != 1 for t in (q, k, v, o)):
         raise ValueError("the last dimension of q, k, v and o must be contiguous")
-    lib = _lib.load()
-    ws = lib.svdq_attention_workspace_bytes(B, H, Tkv, D)
-    if ws == 0:
+    if D not in _HEAD_DIMS:
         raise NotImplementedError(f"attention_fp16: head dimension {D} is not supported (128 and 64 only)")
-    vt = torch.empty(ws, dtype=torch.uint8, device=q.device)
+    lib = _lib.load()
     args = _lib.AttentionArgs(
-        q=q.data_ptr(), k=k.data_ptr(), v=v.data_ptr(), o=o.data_ptr(), vt=vt.data_ptr(),
+        q=q.data_ptr(), k=k.data_ptr(), v=v.data_ptr(), o=o.data_ptr(),
         sqb=q.stride(0), sqh=q.stride(1), sqm=q.stride(2),
         skb=k.stride(0), skh=k.stride(1), skn=k.stride(2),
         svb=v.stride(0), svh=v.stride(1), svn=v.stride(2),

@@ -39,7 +39,7 @@ def test_struct_layouts_match_c(tmp_path):
         "svdq_gemm_args": ("GemmArgs", ["act", "M", "actual_m", "epilogue", "norm_q", "eps", "qout", "R2", "shift"]),
         "svdq_quantize_args": ("QuantizeArgs", ["x", "M", "ld_x", "dtype", "shift", "norm_stats", "norm_shift", "norm_rows_per_batch", "norm_stride"]),
         "svdq_awq_gemv_args": ("AwqGemvArgs", ["x", "M", "ld_out", "dtype"]),
-        "svdq_attention_args": ("AttentionArgs", ["q", "vt", "sqb", "som", "B", "D", "dtype", "scale"]),
+        "svdq_attention_args": ("AttentionArgs", ["q", "o", "sqb", "som", "B", "D", "dtype", "scale"]),
     }
     body = "".join(
         f'printf("{c} %zu\\n", sizeof({c}));' + "".join(f'printf("{c}.{f} %zu\\n", offsetof({c}, {f}));' for f in fs)
@@ -78,13 +78,12 @@ def test_invalid_arguments_are_rejected_without_launch(lib):
     assert lib.svdq_awq_dequantize(16, 16, 16, 16, 6, 64, 64, 8, 64, 0, None) == _lib.E_INVALID  # N % 4
     assert lib.svdq_awq_dequantize(16, 16, 16, 16, 8, 64, 64, 8, 32, 0, None) == _lib.E_INVALID  # ld_out < K
     assert lib.svdq_gemm_w4a4(None, None) == _lib.E_INVALID
-    at = _lib.AttentionArgs(q=16, k=16, v=16, o=16, vt=16, B=1, H=1, Tq=8, Tkv=8, D=32)
+    at = _lib.AttentionArgs(q=16, k=16, v=16, o=16, B=1, H=1, Tq=8, Tkv=8, D=32)
     assert lib.svdq_attention_fp16(at, None) == _lib.E_UNSUPPORTED  # head dimension
-    at = _lib.AttentionArgs(q=16, k=16, v=16, o=16, vt=0, B=1, H=1, Tq=8, Tkv=8, D=128)
-    assert lib.svdq_attention_fp16(at, None) == _lib.E_INVALID  # no workspace
-    assert lib.svdq_attention_workspace_bytes(2, 3, 65, 128) == 2 * 3 * 128 * 128 * 2
-    assert lib.svdq_attention_workspace_bytes(1, 1, 64, 64) == 64 * 64 * 2
-    assert lib.svdq_attention_workspace_bytes(1, 1, 64, 32) == 0
+    at = _lib.AttentionArgs(q=16, k=16, v=0, o=16, B=1, H=1, Tq=8, Tkv=8, D=128)
+    assert lib.svdq_attention_fp16(at, None) == _lib.E_INVALID  # null tensor
+    at = _lib.AttentionArgs(q=16, k=16, v=16, o=16, B=1, H=1, Tq=8, Tkv=8, D=128, skn=128, svn=64)
+    assert lib.svdq_attention_fp16(at, None) == _lib.E_INVALID  # value rows overlap
     assert lib.svdq_gemm_w4a4_scratch_bytes(256, 256, 32, _lib.EPI_GELU_QUANT) == 2 * 256 * 32 * 4
     assert lib.svdq_gemm_w4a4_scratch_bytes(256, 256, 32, _lib.EPI_PLAIN) == 0
 
