@@ -28,7 +28,8 @@ def _run(x, lin, dev, R, smooth=True, unsigned=False, shift=0.0, pad=0):
     return (out.cpu(), osc.cpu(), la.cpu() if R else None), ref
 
 
-@pytest.mark.parametrize("M,K,R", [(1, 128, 16), (16, 256, 32), (130, 384, 48), (257, 3072, 32), (64, 512, 0), (33, 1024, 288)])
+@pytest.mark.parametrize("M,K,R", [(1, 128, 16), (16, 256, 32), (130, 384, 48), (257, 3072, 32), (64, 512, 0), (33, 1024, 288),
+                                   (40, 640, 64), (18, 3072, 96), (50, 512, 160)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_codes_and_scales_bit_exact(dev, M, K, R, dtype):
     print(f"case M={M} K={K} R={R} {dtype}", flush=True)
@@ -121,7 +122,8 @@ def test_fuse_glu_close_to_oracle(dev):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("M,K,R,batches", [(48, 256, 32, 1), (130, 384, 48, 1), (64, 512, 16, 2), (4608, 3072, 32, 1), (96, 1024, 0, 3)])
+@pytest.mark.parametrize("M,K,R,batches", [(48, 256, 32, 1), (130, 384, 48, 1), (64, 512, 16, 2), (4608, 3072, 32, 1), (96, 1024, 0, 3),
+                                           (64, 512, 128, 2)])
 def test_norm_modulate_prologue(dev, M, K, R, batches, dtype):
     """LayerNorm + scale + shift applied inside the quantizer: codes, scales and the LoRA-down product are those of
     the oracle's quantizer fed with the oracle's layernorm_modulate output.  exp-free arithmetic, but the row
