@@ -37,9 +37,11 @@ constexpr int AT_BQ = 128, AT_BK = 64;     // queries per workgroup, keys per ti
 // Geometry for head dimension D (128 or 64).  K and V tiles are [key][2 D bytes]; every block load moves 1 KB
 // (64 lanes x 16 bytes) = whole rows; 16-byte chunks are XOR-swizzled by the row so that the operand reads touch every
 // bank once.  K (32 rows x one chunk per half-wave): rows of 256 bytes by row & 15, rows of 128 bytes (two rows span
-// the 64 banks) by row / 2 & 7.  V (a transposing read = 4 rows x 32 bytes per 16 lanes): the four rows must land in
-// four different 32-byte slots of the banks, so chunk pairs are swizzled by row & 3 (256-byte rows) or row / 2 & 1
-// (128-byte rows, where rows r and r + 1 already differ by half the banks).
+// the 64 banks) by row / 2 & 7.  V (a transposing read = 4 rows x 32 bytes per 16 lanes, two such groups with
+// neighbouring 32-byte column slots per half-wave): the eight (row, slot) pairs of a half-wave must land in eight
+// different 32-byte slots of the 256 bytes the banks span, so the 64-byte quarter of a row is swizzled by row & 3
+// (256-byte rows) or the 64-byte half by row / 2 & 1 (128-byte rows, where rows r and r + 1 already differ by half
+// the banks).
 template <int D>
 struct AtGeo {
     static constexpr int NC = D / 16;               // 16-wide k chunks of q k^T = matrix instructions per 32-key half
@@ -52,7 +54,7 @@ struct AtGeo {
     static constexpr int LOADS = KT_BYTES / 1024 / 4;  // block loads per wavefront and tile, of K and of V alike
     static constexpr int OPITCH = 2 * D + 16;       // staged output row
     __host__ __device__ static constexpr int kswz(int row) { return KROW == 256 ? (row & 15) : ((row >> 1) & 7); }
-    __host__ __device__ static constexpr int vswz(int row) { return KROW == 256 ? ((row & 3) << 1) : (((row >> 1) & 1) << 1); }
+    __host__ __device__ static constexpr int vswz(int row) { return KROW == 256 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); }
 };
 
 constexpr uint32_t AT_RSRC_FLAGS = 0x00020000;  // raw buffer, 32-bit data format (gfx9 family)
