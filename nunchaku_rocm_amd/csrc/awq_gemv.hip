@@ -447,6 +447,11 @@ extern "C" int svdq_awq_gemv_w4a16(const svdq_awq_gemv_args *args, void *stream)
         return SVDQ_E_UNSUPPORTED;
     }
     if (a.M == 0) return SVDQ_OK;
+    if (a.M <= 8 && ((size_t)a.N * a.K / 2 >= ((size_t)1 << 32) || (size_t)(a.K / GROUP) * a.ld_scales * 2 >= ((size_t)1 << 32) ||
+                     (size_t)a.M * a.ld_x * 2 >= ((size_t)1 << 32))) {  // the kernel for up to eight rows addresses with 32-bit byte offsets
+        set_error("svdq_awq_gemv_w4a16: N=%d K=%d ld_scales=%d ld_x=%d: a tensor of 4 GiB or more", a.N, a.K, a.ld_scales, a.ld_x);
+        return SVDQ_E_UNSUPPORTED;
+    }
     if (a.dtype == SVDQ_BF16)
         launch_awq<BF16>(a, (hipStream_t)stream);
     else
