@@ -49,12 +49,12 @@ __global__ __launch_bounds__(Q_WAVES * 64, QR == 32 ? 1 : (NORM ? 4 : 2)) void q
     constexpr int XS_BYTES = (GLU ? 2 : 1) * QR * Q_ROW_BYTES, G_OFF = QR * Q_ROW_BYTES;
     constexpr int L_OFF = 2 * XS_BYTES;
     constexpr int WAVE_BYTES = L_OFF + (HAS_LORA ? Q_RCHUNK * Q_ROW_BYTES : 0);
-    constexpr int ACC_BYTES = HAS_LORA ? Q_WAVES * Q_RCHUNK * (QR + 1) * 4 : 0;  // cross-wave sum, after the loop
-    constexpr int STG_BYTES = Q_WAVES * WAVE_BYTES;
-    __shared__ __align__(16) uint8_t smem[STG_BYTES > ACC_BYTES ? STG_BYTES : ACC_BYTES];
+    // the cross-wave sum after the loop keeps each wavefront's partial products in that wavefront's own (then idle) stages
+    static_assert(!HAS_LORA || Q_RCHUNK * (QR + 1) * 4 <= WAVE_BYTES, "partial products do not fit the wavefront's stages");
+    __shared__ __align__(16) uint8_t smem[Q_WAVES * WAVE_BYTES];
     __shared__ float lds_rs[Q_WAVES][64];
     __shared__ float lds_ns[NORM ? Q_WAVES : 1][64], lds_nh[NORM ? Q_WAVES : 1][64];
-    float (*lds_acc)[Q_RCHUNK][QR + 1] = (float (*)[Q_RCHUNK][QR + 1])smem;
+    auto lds_acc = [&](int w) { return (float (*)[QR + 1])(smem + w * WAVE_BYTES); };  // [Q_RCHUNK][QR + 1] of wavefront w
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform: keep it in an SGPR
@@ -322,25 +322,25 @@ __global__ __launch_bounds__(Q_WAVES * 64, QR == 32 ? 1 : (NORM ? 4 : 2)) void q
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
 
         if (HAS_LORA) {
-            // fixed-order sum of the wavefronts' partial products
-            __syncthreads();  // every wavefront is done with its stages: the sum reuses the memory
+            // fixed-order sum of the wavefronts' partial products (this wavefront is done with its own stages)
+            float (*mine)[QR + 1] = lds_acc(wave);
 #pragma unroll
             for (int h = 0; h < NH; h++)
 #pragma unroll
                 for (int i = 0; i < 4; i++) {
-                    lds_acc[wave][4 * kq + i][Q_ROWS * h + ml] = acc0[h][i];
-                    lds_acc[wave][16 + 4 * kq + i][Q_ROWS * h + ml] = acc1[h][i];
+                    mine[4 * kq + i][Q_ROWS * h + ml] = acc0[h][i];
+                    mine[16 + 4 * kq + i][Q_ROWS * h + ml] = acc1[h][i];
                 }
             __syncthreads();
             for (int o = threadIdx.x; o < QR * Q_RCHUNK; o += Q_WAVES * 64) {
                 const int mm = o / Q_RCHUNK, r = o % Q_RCHUNK;
-                float s = lds_acc[0][r][mm];
+                float s = lds_acc(0)[r][mm];
 #pragma unroll
-                for (int w = 1; w < Q_WAVES; w++) s += lds_acc[w][r][mm];
+                for (int w = 1; w < Q_WAVES; w++) s += lds_acc(w)[r][mm];
                 if (m0 + mm < a.M && rc * Q_RCHUNK + r < a.R)
                     a.lora_act[(size_t)(m0 + mm) * a.ld_lora_act + rc * Q_RCHUNK + r] = s;
             }
-            __syncthreads();
+            if (rc + 1 < nchunks) __syncthreads();  // the next pass refills the stages
         }
     }
 }
