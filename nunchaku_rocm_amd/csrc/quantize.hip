@@ -97,8 +97,15 @@ __global__ __launch_bounds__(Q_WAVES * 64, QR == 32 ? 1 : (NORM ? 4 : 2)) void q
         nshift = (const uint16_t *)a.norm_shift + voff;
     }
 
-    const int nchunks = HAS_LORA ? (a.R + Q_RCHUNK - 1) / Q_RCHUNK : 1;
-    for (int rc = 0; rc < nchunks; rc++) {
+    // Ranks beyond Q_RCHUNK: the grid's second axis.  Workgroup (row block, rc) projects onto ranks [32 rc, 32 rc + 32);
+    // only rc = 0 quantizes.  (The further workgroups read the activations again, from the memory-side cache, and
+    // run next to the others on CUs the row blocks alone leave idle.)
+    // With one more workgroup row than rank chunks, row 0 only quantizes and rows 1 .. project (the two kinds of work
+    // then run side by side on different CUs instead of one after the other in every wavefront).
+    {
+        const bool split = HAS_LORA && (int)gridDim.y > (a.R + Q_RCHUNK - 1) / Q_RCHUNK;
+        const int rc = split ? max((int)blockIdx.y - 1, 0) : (int)blockIdx.y;
+        const bool do_lora = HAS_LORA && !(split && blockIdx.y == 0);
         v4f acc0[NH], acc1[NH];
 #pragma unroll
         for (int h = 0; h < NH; h++) acc0[h] = acc1[h] = (v4f){0.f, 0.f, 0.f, 0.f};
@@ -110,7 +117,7 @@ __global__ __launch_bounds__(Q_WAVES * 64, QR == 32 ? 1 : (NORM ? 4 : 2)) void q
             for (int i = 0; i < 4; i++)
                 ldma[i] = (uint32_t)min(rc * Q_RCHUNK + 8 * i + drow, a.R - 1) * a.K * 2 + dchunk * 16;
         }
-        const bool do_quant = rc == 0;
+        const bool do_quant = split ? blockIdx.y == 0 : rc == 0;
 
         constexpr int NX = (GLU ? 4 : 2) * NH;  // block loads of one activation stage
         auto group_off = [&](int i) {  // byte offset of group wave + Q_WAVES * i in a row; past the end: the last group
@@ -138,7 +145,7 @@ __global__ __launch_bounds__(Q_WAVES * 64, QR == 32 ? 1 : (NORM ? 4 : 2)) void q
             }
         };
         auto issue_l = [&](int i) {
-            if (!HAS_LORA) return;
+            if (!do_lora) return;
             const uint32_t k0 = group_off(i);
 #pragma unroll
             for (int j = 0; j < 4; j++)
@@ -160,7 +167,7 @@ __global__ __launch_bounds__(Q_WAVES * 64, QR == 32 ? 1 : (NORM ? 4 : 2)) void q
                     o.ghi[h] = *(const v4i *)(src + G_OFF + h * Q_ROWS * Q_ROW_BYTES + rd_hi);
                 }
             }
-            if (HAS_LORA) {
+            if (do_lora) {
                 o.l0lo = *(const v4i *)(wbase + L_OFF + rd_lo);
                 o.l0hi = *(const v4i *)(wbase + L_OFF + rd_hi);
                 o.l1lo = *(const v4i *)(wbase + L_OFF + 16 * Q_ROW_BYTES + rd_lo);
@@ -239,7 +246,7 @@ __global__ __launch_bounds__(Q_WAVES * 64, QR == 32 ? 1 : (NORM ? 4 : 2)) void q
                     cxhi[j] = (int)pack2<T>(v[8 + 2 * j], v[8 + 2 * j + 1]);
                 }
             }
-            if (HAS_LORA) {
+            if (do_lora) {
                 acc0[h] = mfma16_16bit<T>(l0lo, cxlo, acc0[h]);
                 acc0[h] = mfma16_16bit<T>(l0hi, cxhi, acc0[h]);
                 acc1[h] = mfma16_16bit<T>(l1lo, cxlo, acc1[h]);
@@ -321,7 +328,7 @@ __global__ __launch_bounds__(Q_WAVES * 64, QR == 32 ? 1 : (NORM ? 4 : 2)) void q
         }
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
 
-        if (HAS_LORA) {
+        if (do_lora) {
             // fixed-order sum of the wavefronts' partial products (this wavefront is done with its own stages)
             float (*mine)[QR + 1] = lds_acc(wave);
 #pragma unroll
@@ -340,7 +347,6 @@ __global__ __launch_bounds__(Q_WAVES * 64, QR == 32 ? 1 : (NORM ? 4 : 2)) void q
                 if (m0 + mm < a.M && rc * Q_RCHUNK + r < a.R)
                     a.lora_act[(size_t)(m0 + mm) * a.ld_lora_act + rc * Q_RCHUNK + r] = s;
             }
-            if (rc + 1 < nchunks) __syncthreads();  // the next pass refills the stages
         }
     }
 }
@@ -477,13 +483,36 @@ static int quantize_rows_per_workgroup(const svdq_quantize_args &a) {
     return (wg16 > Q32_ABOVE && wg16 <= Q32_UPTO) ? 32 : Q_ROWS;
 }
 
+static int device_cus() {
+    static int cus = 0;
+    if (!cus) {
+        int dev = 0, n = 0;
+        cus = hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0 ? n : 256;
+    }
+    return cus;
+}
+
+// Second grid axis: one workgroup row per chunk of 32 ranks, plus one that only quantizes where that still leaves about
+// one workgroup per CU: quantizing and projecting then run side by side on different CUs (K = 3072, R = 32: 6.4
+// against 7.9 us at M = 512, 7.1 against 8.5 at 2048, 12.3 against 13.4 at 4608 with 32-row workgroups; slower once the
+// CUs are taken: 9.9 against 9.5 us at M = 4096, 17.2 against 14.5 at 6144).
+static int quantize_grid_y(const svdq_quantize_args &a, int row_blocks, int rows) {
+    if (a.R == 0) return 1;
+    const int chunks = (a.R + Q_RCHUNK - 1) / Q_RCHUNK, cus = device_cus();
+    // (with a prologue the workgroups that only project compute it a second time: only where half the CUs would idle
+    // anyway; norm prologue, M = 512: 10.4 against 11.8 us, M = 4608: 25.5 against 20.7)
+    const bool prologue = a.norm_stats || a.prologue != SVDQ_PRE_NONE;
+    const bool split = row_blocks * (chunks + 1) <= (prologue ? cus / 2 : cus + (rows == 32 ? cus / 8 : 0));
+    return chunks + (split ? 1 : 0);
+}
+
 template <typename T, bool U, int G, bool NORM>
 static void launch_quantize3(const svdq_quantize_args &a, hipStream_t s) {
     const dim3 block(Q_WAVES * 64);
     const bool lora = a.R > 0, sm = a.smooth != nullptr;
     if constexpr (G == SVDQ_PRE_NONE) {
         if (quantize_rows_per_workgroup(a) == 32) {
-            const dim3 grid((a.M + 31) / 32);
+            const dim3 grid((a.M + 31) / 32, quantize_grid_y(a, (a.M + 31) / 32, 32));
             if (sm)
                 hipLaunchKernelGGL((quantize_act_kernel<T, U, G, true, true, NORM, 32>), grid, block, 0, s, a);
             else
@@ -491,7 +520,7 @@ static void launch_quantize3(const svdq_quantize_args &a, hipStream_t s) {
             return;
         }
     }
-    const dim3 grid((a.M + Q_ROWS - 1) / Q_ROWS);
+    const dim3 grid((a.M + Q_ROWS - 1) / Q_ROWS, quantize_grid_y(a, (a.M + Q_ROWS - 1) / Q_ROWS, Q_ROWS));
     if (lora && sm)
         hipLaunchKernelGGL((quantize_act_kernel<T, U, G, true, true, NORM, 16>), grid, block, 0, s, a);
     else if (lora)
