@@ -6,7 +6,9 @@ A step is one pass of the hot path over one batch of synthetic input: the FLUX.1
 ``value`` is 2*M*N*K / step time in TOP/s (the reference's GEMM convention, tests/triton/bench_kernels.py:61, charged
 with the quantizer's time as well).  The step's two launches are recorded once into a HIP graph and the timed region
 replays it, so the figure is what the kernels take and not what Python needs to marshal two calls (about 15 us each,
-more than the quantizer runs); ``--eager`` times the eager calls instead.  The JSON line also carries the roofline of
+more than the quantizer runs); ``--eager`` times the eager calls instead.  Every timed region follows at least 0.12 s
+of the same work without a pause (the W warm-up steps and as many more as that takes): the GPU's clocks need about
+50 ms of continuous work to settle, and the settled rate is the one a denoising loop sees.  The JSON line also carries the roofline of
 the dominant kernel (the GEMM: HIP events on the launch stream around back-to-back launches of it, the figure the
 rocprofv3 kernel trace under profiles/ reproduces), a per-kernel table (quantizer GB/s, AWQ GEMV GB/s, GEMM M-sweep and fused
 epilogue shapes), and the CPU baseline (the oracle's pure-PyTorch restatement of the reference's CPU path).
@@ -32,7 +34,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # in profiles/bench_all_kernels_hbm_traffic.txt, the factors being what the same counters read on plain copy kernels of
 # known size in the same run (FETCH_SIZE reads half the bytes of 16-byte-per-lane loads); counters cannot be read from
 # inside this process
-GEMM_QKV_HBM_BYTES = (2.0 * 104572.7 + 82944.0) * 1024
+GEMM_QKV_HBM_BYTES = (2.0 * 104717.3 + 82944.1) * 1024
 
 
 def _events(n):
@@ -41,10 +43,26 @@ def _events(n):
     return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
 
 
+STEADY_S = 0.12  # continuous work before a timed region: the GPU's clocks take about 50 ms of it to settle
+
+
+def _steady(run, seconds=STEADY_S):
+    """Repeat ``run`` (a batch of launches) until ``seconds`` of wall time have passed without the GPU going idle for
+    longer than a host round trip.  After an idle period the QKV GEMM takes 240 us per launch and settles at 194 us
+    within 50 ms of continuous launches (measured in batches of 20 launches: 240, 229, 219, 213, 210, 206, 201, 198,
+    196, 194, then 193-195 for the next 1000 launches).  Every figure of this benchmark is the settled one."""
+    import torch
+
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        run()
+        torch.cuda.synchronize()
+
+
 def _time_kernel(fn, iters=50, warmup=10, graph=False):
-    """Average launch duration in ms: HIP events on the launch stream around ``iters`` back-to-back launches.
-    ``graph=True`` records the launches into one HIP graph first, which takes the host's launch cost (about 15 us per
-    call through ctypes, more than the small kernels run) out of the figure."""
+    """Average launch duration in ms at settled clocks: HIP events on the launch stream around ``iters`` back-to-back
+    launches.  ``graph=True`` records the launches into one HIP graph first, which takes the host's launch cost (about
+    15 us per call through ctypes, more than the small kernels run) out of the figure."""
     import torch
 
     for _ in range(warmup):
@@ -56,16 +74,20 @@ def _time_kernel(fn, iters=50, warmup=10, graph=False):
         with torch.cuda.graph(g):
             for _ in range(iters):
                 fn()
-        g.replay()
-        torch.cuda.synchronize()
+        _steady(g.replay)
         a.record()
         g.replay()
         b.record()
         torch.cuda.synchronize()
         return a.elapsed_time(b) / iters
+
+    def batch():
+        for _ in range(iters):
+            fn()
+
+    _steady(batch)
     a.record()
-    for _ in range(iters):
-        fn()
+    batch()
     b.record()
     torch.cuda.synchronize()
     return a.elapsed_time(b) / iters
@@ -160,6 +182,12 @@ def main():
         for _ in range(args.warmup):
             run_step()
     torch.cuda.synchronize()
+
+    def steps_back_to_back():
+        for _ in range(args.steps):
+            run_step()
+
+    _steady(steps_back_to_back)  # more untimed steps, until the clocks have settled (see _steady)
     t0 = time.perf_counter()
     for _ in range(args.steps):
         run_step()
