@@ -45,6 +45,23 @@ def test_codes_and_scales_bit_exact(dev, M, K, R, dtype):
         assert (la[M:] == 7.0).all()
 
 
+@pytest.mark.parametrize("M", [2064, 4112, 4640, 8208])
+def test_every_grid_layout_bit_exact(dev, M):
+    """The launcher picks 16- or 32-row workgroups and, where CUs would idle, a further workgroup row that only
+    quantizes while the others only project (see quantize_grid_y): 2064 rows = 16-row workgroups doing both, 4112 =
+    32-row doing both on a 256-CU part, 4640 = 32-row just past the split's limit, 8208 = 16-row again; the small
+    shapes of the other tests and M = 4608 take the split layouts."""
+    print(f"case M={M}", flush=True)
+    K, R = 128, 32
+    x = O.make_activations(M, K, seed=M, dtype=torch.bfloat16)
+    lin = O.make_svdq_linear(K, 64, R=R, seed=K)
+    (out, osc, la), (rp, rs, rl, _) = _run(x, lin, dev, R)
+    assert torch.equal(out[:M], rp)
+    assert torch.equal(osc[:, :M].view(torch.int16), rs.view(torch.int16))
+    ref64 = x.double() @ lin["proj_down"][:, :R].double()
+    assert (la[:M].double() - ref64).abs().max() <= 2e-5 * ref64.abs().max()
+
+
 @pytest.mark.parametrize("smooth", [True, False])
 def test_unsigned_with_shift_bit_exact(dev, smooth):
     M, K = 96, 512
