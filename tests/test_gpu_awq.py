@@ -41,12 +41,24 @@ def test_flux_adaln_shape(dev, m):
     assert ((out.float() - ref).abs() <= ref.abs() * 2**-7 + 2e-2).all()
 
 
+@pytest.mark.parametrize("m", [1, 3, 4, 7, 12])
+@pytest.mark.parametrize("K", [64, 192, 576, 1088, 3136, 3520, 6208])
+def test_ragged_k(dev, m, K):
+    """Group counts that leave wavefronts without work (K = 64: one group for eight wavefronts), batches that are not
+    full (1088 = 17 groups: three wavefronts get three, the others two), and a partial batch after full ones (3136 = 49
+    groups, 6208 = 97); every row-count variant of the kernel (1, 2, 4, 8 padded rows, and the one for more than 8)."""
+    print(f"case m={m} K={K}", flush=True)
+    out, ref = _case(dev, m, 96, K, torch.bfloat16, seed=K + m)
+    assert O.max_rel_err(out, ref) <= 1e-2
+    assert ((out.float() - ref).abs() <= ref.abs() * 2**-7 + 2e-2).all()
+
+
 @pytest.mark.parametrize("m", [2, 8, 32])
 @pytest.mark.parametrize("K", [3584, 4096, 12288])
 def test_long_k(dev, m, K):
-    """Row counts and lengths at which the activations no longer fit the kernel's LDS staging (they are then read from
-    global memory), and K = 12288 with 32 rows, where the per-group tables do not fit either and the operator decodes
-    the weight and multiplies instead."""
+    """Long rows for every kernel variant: up to eight rows the kernel's LDS use does not depend on K; K = 12288 with
+    32 rows, where the per-group tables of the kernel for more than eight rows do not fit LDS, goes to the operator's
+    decode-and-multiply route."""
     print(f"case m={m} K={K}", flush=True)
     out, ref = _case(dev, m, 256, K, torch.bfloat16, seed=K + m)
     assert O.max_rel_err(out, ref) <= 1e-2
