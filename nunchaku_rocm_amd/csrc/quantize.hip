@@ -397,7 +397,6 @@ __global__ __launch_bounds__(256) void gated_residual_kernel(const uint16_t *x, 
     const uint16_t *xr = x + (long)m * ld_x, *yr = y + (long)m * ld_y, *y2r = SUM2 ? y2 + (long)m * ld_y : nullptr;
     const uint16_t *gr = gate + (rows_per_batch > 0 ? (long)(m / rows_per_batch) * gate_ld : 0);
     uint16_t *orow = out + (long)m * ld_out;
-    auto rnd = [](float f) { return T::to_f32(T::from_f32(f)); };
     auto wave_sum = [](float s) {
 #pragma unroll
         for (int o = 32; o >= 1; o >>= 1) s += __shfl_xor(s, o);
@@ -425,20 +424,19 @@ __global__ __launch_bounds__(256) void gated_residual_kernel(const uint16_t *x, 
                 for (int e = 0; e < 8; e++) g[e] = T::to_f32(gr[(long)(k + e) * gate_stride]);
             }
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                float t0 = T::lo_f32((uint32_t)yv[e]), t1 = T::hi_f32((uint32_t)yv[e]);
-                if (SUM2) {
-                    t0 = rnd(t0 + T::lo_f32((uint32_t)zv[e]));
-                    t1 = rnd(t1 + T::hi_f32((uint32_t)zv[e]));
-                }
-                float o0 = rnd(T::lo_f32((uint32_t)xv[e]) + rnd(g[2 * e] * t0));
-                float o1 = rnd(T::hi_f32((uint32_t)xv[e]) + rnd(g[2 * e + 1] * t1));
+            for (int e = 0; e < 4; e++) {  // every step rounded to T, two values per rounding instruction
+                uint32_t w = (uint32_t)yv[e];
+                if (SUM2) w = pack2<T>(T::lo_f32(w) + T::lo_f32((uint32_t)zv[e]), T::hi_f32(w) + T::hi_f32((uint32_t)zv[e]));
+                w = pack2<T>(g[2 * e] * T::lo_f32(w), g[2 * e + 1] * T::hi_f32(w));
+                w = pack2<T>(T::lo_f32((uint32_t)xv[e]) + T::lo_f32(w), T::hi_f32((uint32_t)xv[e]) + T::hi_f32(w));
+                float o0 = T::lo_f32(w), o1 = T::hi_f32(w);
                 if (clip > 0.0f) {  // x.clip(-clip, clip): infinities become the limit, NaN stays
                     o0 = o0 > clip ? clip : (o0 < -clip ? -clip : o0);
                     o1 = o1 > clip ? clip : (o1 < -clip ? -clip : o1);
+                    w = pack2<T>(o0, o1);
                 }
                 s += o0 + o1;
-                res[c][e] = (int)pack2<T>(o0, o1);
+                res[c][e] = (int)w;
             }
             *(v4i *)(orow + k) = res[c];
         }
