@@ -351,31 +351,72 @@ __global__ __launch_bounds__(Q_WAVES * 64, QR == 32 ? 1 : (NORM ? 4 : 2)) void q
     }
 }
 
-// one wavefront per row: mean, then the centred sum of squares (second read from cache), fixed reduction order
+template <int CTRL>
+__device__ inline float q_dpp(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xF, 0xF, false));
+}
+// Sum over the wavefront, the same value in every lane, fixed order: pairs, quads, octets, rows of sixteen lanes (data
+// parallel primitives, no LDS round trips), then the four rows in order.
+__device__ inline float wave_sum(float s) {
+    s += q_dpp<0xB1>(s);   // quad_perm [1, 0, 3, 2]
+    s += q_dpp<0x4E>(s);   // quad_perm [2, 3, 0, 1]
+    s += q_dpp<0x141>(s);  // row_half_mirror
+    s += q_dpp<0x140>(s);  // row_mirror
+    const int b = __builtin_bit_cast(int, s);
+    const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 0)), r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 16));
+    const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 32)), r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(b, 48));
+    return ((r0 + r1) + r2) + r3;
+}
+
+// one wavefront per row: mean, then the centred sum of squares, fixed reduction order.  Rows of up to 8192 values are
+// read once and kept in registers, their loads issued eight at a time without branches (offsets past the end of the
+// row are clamped and those chunks not used), so that a wavefront has 8 KB in flight instead of 1; longer rows are read
+// twice, the second time from cache.
 template <typename T>
 __global__ __launch_bounds__(256) void row_stats_kernel(const uint16_t *x, float *stats, int M, int K, long ld_x, float eps) {
+    constexpr int MAXC = 16, BATCH = 8;  // 16-byte chunks per lane kept in registers; loads in flight
     const int lane = threadIdx.x & 63, m = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (m >= M) return;
     const uint16_t *row = x + (long)m * ld_x;
-    auto wave_sum = [](float s) {
+    float s = 0.0f, q = 0.0f, mean;
+    if (K <= 512 * MAXC) {
+        v4i r[MAXC];
 #pragma unroll
-        for (int o = 32; o >= 1; o >>= 1) s += __shfl_xor(s, o);
-        return s;
-    };
-    float s = 0.0f;
-    for (int k = 8 * lane; k < K; k += 512) {
-        const v4i w = *(const v4i *)(row + k);
+        for (int c0 = 0; c0 < MAXC; c0 += BATCH)
+            if (512 * c0 < K) {
 #pragma unroll
-        for (int e = 0; e < 4; e++) s += T::lo_f32((uint32_t)w[e]) + T::hi_f32((uint32_t)w[e]);
-    }
-    const float mean = wave_sum(s) / (float)K;
-    float q = 0.0f;
-    for (int k = 8 * lane; k < K; k += 512) {
-        const v4i w = *(const v4i *)(row + k);
+                for (int u = 0; u < BATCH; u++) r[c0 + u] = *(const v4i *)(row + min(8 * lane + 512 * (c0 + u), K - 8));
+            }
 #pragma unroll
-        for (int e = 0; e < 4; e++) {
-            const float d0 = T::lo_f32((uint32_t)w[e]) - mean, d1 = T::hi_f32((uint32_t)w[e]) - mean;
-            q += d0 * d0 + d1 * d1;
+        for (int c = 0; c < MAXC; c++)
+            if (8 * lane + 512 * c < K) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) s += T::lo_f32((uint32_t)r[c][e]) + T::hi_f32((uint32_t)r[c][e]);
+            }
+        mean = wave_sum(s) / (float)K;
+#pragma unroll
+        for (int c = 0; c < MAXC; c++)
+            if (8 * lane + 512 * c < K) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const float d0 = T::lo_f32((uint32_t)r[c][e]) - mean, d1 = T::hi_f32((uint32_t)r[c][e]) - mean;
+                    q += d0 * d0 + d1 * d1;
+                }
+            }
+    } else {
+        for (int k = 8 * lane; k < K; k += 512) {
+            const v4i w = *(const v4i *)(row + k);
+#pragma unroll
+            for (int e = 0; e < 4; e++) s += T::lo_f32((uint32_t)w[e]) + T::hi_f32((uint32_t)w[e]);
+        }
+        mean = wave_sum(s) / (float)K;
+        for (int k = 8 * lane; k < K; k += 512) {
+            const v4i w = *(const v4i *)(row + k);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const float d0 = T::lo_f32((uint32_t)w[e]) - mean, d1 = T::hi_f32((uint32_t)w[e]) - mean;
+                q += d0 * d0 + d1 * d1;
+            }
         }
     }
     const float var = wave_sum(q) / (float)K;
@@ -397,48 +438,54 @@ __global__ __launch_bounds__(256) void gated_residual_kernel(const uint16_t *x, 
     const uint16_t *xr = x + (long)m * ld_x, *yr = y + (long)m * ld_y, *y2r = SUM2 ? y2 + (long)m * ld_y : nullptr;
     const uint16_t *gr = gate + (rows_per_batch > 0 ? (long)(m / rows_per_batch) * gate_ld : 0);
     uint16_t *orow = out + (long)m * ld_out;
-    auto wave_sum = [](float s) {
-#pragma unroll
-        for (int o = 32; o >= 1; o >>= 1) s += __shfl_xor(s, o);
-        return s;
-    };
     v4i res[MAXC];
     float s = 0.0f;
+    constexpr int BATCH = 2;  // chunks whose loads (x, y, y2, gate: up to eight) are issued together, without branches
 #pragma unroll
-    for (int c = 0; c < MAXC; c++) {
-        const int k = 8 * lane + 512 * c;
-        if (k < K) {
-            const v4i xv = *(const v4i *)(xr + k), yv = *(const v4i *)(yr + k);
-            v4i zv = {0, 0, 0, 0};
-            if (SUM2) zv = *(const v4i *)(y2r + k);
-            float g[8];
-            if (gate_stride == 1) {
-                const v4i gv = *(const v4i *)(gr + k);
+    for (int c0 = 0; c0 < MAXC; c0 += BATCH) {
+        if (512 * c0 >= K) break;
+        v4i xb[BATCH], yb[BATCH], zb[BATCH], gb[BATCH];
 #pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    g[2 * e] = T::lo_f32((uint32_t)gv[e]);
-                    g[2 * e + 1] = T::hi_f32((uint32_t)gv[e]);
+        for (int u = 0; u < BATCH; u++) {
+            const int kk = min(8 * lane + 512 * (c0 + u), K - 8);  // past the end: the row's last chunk again, not used
+            xb[u] = *(const v4i *)(xr + kk);
+            yb[u] = *(const v4i *)(yr + kk);
+            zb[u] = SUM2 ? *(const v4i *)(y2r + kk) : (v4i){0, 0, 0, 0};
+            gb[u] = gate_stride == 1 ? *(const v4i *)(gr + kk) : (v4i){0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int u = 0; u < BATCH; u++) {
+            const int c = c0 + u, k = 8 * lane + 512 * c;
+            if (k < K) {
+                const v4i xv = xb[u], yv = yb[u], zv = zb[u];
+                float g[8];
+                if (gate_stride == 1) {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        g[2 * e] = T::lo_f32((uint32_t)gb[u][e]);
+                        g[2 * e + 1] = T::hi_f32((uint32_t)gb[u][e]);
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; e++) g[e] = T::to_f32(gr[(long)(k + e) * gate_stride]);
                 }
-            } else {
 #pragma unroll
-                for (int e = 0; e < 8; e++) g[e] = T::to_f32(gr[(long)(k + e) * gate_stride]);
-            }
-#pragma unroll
-            for (int e = 0; e < 4; e++) {  // every step rounded to T, two values per rounding instruction
-                uint32_t w = (uint32_t)yv[e];
-                if (SUM2) w = pack2<T>(T::lo_f32(w) + T::lo_f32((uint32_t)zv[e]), T::hi_f32(w) + T::hi_f32((uint32_t)zv[e]));
-                w = pack2<T>(g[2 * e] * T::lo_f32(w), g[2 * e + 1] * T::hi_f32(w));
-                w = pack2<T>(T::lo_f32((uint32_t)xv[e]) + T::lo_f32(w), T::hi_f32((uint32_t)xv[e]) + T::hi_f32(w));
-                float o0 = T::lo_f32(w), o1 = T::hi_f32(w);
-                if (clip > 0.0f) {  // x.clip(-clip, clip): infinities become the limit, NaN stays
-                    o0 = o0 > clip ? clip : (o0 < -clip ? -clip : o0);
-                    o1 = o1 > clip ? clip : (o1 < -clip ? -clip : o1);
-                    w = pack2<T>(o0, o1);
+                for (int e = 0; e < 4; e++) {  // every step rounded to T, two values per rounding instruction
+                    uint32_t w = (uint32_t)yv[e];
+                    if (SUM2) w = pack2<T>(T::lo_f32(w) + T::lo_f32((uint32_t)zv[e]), T::hi_f32(w) + T::hi_f32((uint32_t)zv[e]));
+                    w = pack2<T>(g[2 * e] * T::lo_f32(w), g[2 * e + 1] * T::hi_f32(w));
+                    w = pack2<T>(T::lo_f32((uint32_t)xv[e]) + T::lo_f32(w), T::hi_f32((uint32_t)xv[e]) + T::hi_f32(w));
+                    float o0 = T::lo_f32(w), o1 = T::hi_f32(w);
+                    if (clip > 0.0f) {  // x.clip(-clip, clip): infinities become the limit, NaN stays
+                        o0 = o0 > clip ? clip : (o0 < -clip ? -clip : o0);
+                        o1 = o1 > clip ? clip : (o1 < -clip ? -clip : o1);
+                        w = pack2<T>(o0, o1);
+                    }
+                    s += o0 + o1;
+                    res[c][e] = (int)w;
                 }
-                s += o0 + o1;
-                res[c][e] = (int)w;
+                *(v4i *)(orow + k) = res[c];
             }
-            *(v4i *)(orow + k) = res[c];
         }
     }
     if (!STATS) return;
