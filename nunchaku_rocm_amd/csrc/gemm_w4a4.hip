@@ -770,7 +770,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
                         gmax = fmaxf(gmax, v);
                     }
                 }
-            gmax = fmaxf(gmax, __shfl_xor(gmax, 32));
+            gmax = max_with_lane_xor32(gmax);
             const float scale = gmax / 15.0f;
             const float safe = (scale == 0.0f) ? 1.0f : scale;
             const float rq = 1.0f / safe;
@@ -869,7 +869,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
                     gmax = fmaxf(gmax, fabsf(v));
                 }
             }
-        gmax = fmaxf(gmax, __shfl_xor(gmax, 32));
+        gmax = max_with_lane_xor32(gmax);
         const float scale = gmax / 7.0f;
         const float safe = (scale == 0.0f) ? 1.0f : scale;
         const float rq = 1.0f / safe;

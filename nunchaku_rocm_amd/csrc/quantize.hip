@@ -270,8 +270,7 @@ __global__ __launch_bounds__(Q_WAVES * 64, QR == 32 ? 1 : (NORM ? 4 : 2)) void q
             for (int j = 0; j < 16; j += 2)
                 gmax = UNSIGNED ? __builtin_fmaxf(__builtin_fmaxf(v[j], v[j + 1]), gmax)
                                 : __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(v[j]), __builtin_fabsf(v[j + 1])), gmax);
-            gmax = fmaxf(gmax, __shfl_xor(gmax, 16));
-            gmax = fmaxf(gmax, __shfl_xor(gmax, 32));
+            gmax = max_with_lane_xor32(max_with_lane_xor16(gmax));
             const float scale = gmax / qmax;
             const float safe = (scale == 0.0f) ? 1.0f : scale;
             const float rq = 1.0f / safe;

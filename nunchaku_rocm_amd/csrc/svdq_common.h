@@ -106,6 +106,17 @@ __device__ inline v4f mfma16_16bit<FP16>(v4i a, v4i b, v4f c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0, 0, 0);
 }
 
+// Value of lane ^ 32 / lane ^ 16 by the lane-swap instructions of gfx950 (vector ALU, no LDS round trip): swapping a
+// register with itself leaves every lane's own value in one result and its partner's in the other.
+__device__ inline float max_with_lane_xor32(float v) {
+    const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+}
+__device__ inline float max_with_lane_xor16(float v) {
+    const auto sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+}
+
 __device__ inline float gelu_tanh(float x) {
     // 0.5 x (1 + tanh(u)), u = 0.79788456 (x + 0.044715 x^3), which the reference spells 0.5 x (1 + 2 / (1 + exp(-2 u)) - 1)
     // (nunchaku/ops/triton/_common.py:71-78).  That is x / (1 + exp(-2 u)); with the hardware reciprocal (1 ulp) it is 9
