@@ -50,9 +50,6 @@ __device__ inline v4i awq_wload(const v4i *p) {
     return __builtin_nontemporal_load(p);  // streamed once: do not keep in cache
 }
 
-typedef int v2i __attribute__((ext_vector_type(2)));
-typedef short v4s __attribute__((ext_vector_type(4)));
-typedef _Float16 v4h __attribute__((ext_vector_type(4)));
 
 // 4x4x4 MFMA in 16 independent blocks (block = lane / 4): D[block][row][col = lane % 4] += sum over 4 k of
 // A[block][row = lane % 4][k] * B[block][k][col]; four 16-bit values per lane, passed as raw bits

@@ -354,12 +354,22 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
         uint8_t *other = P ? sbuf0 : sbuf1;  // being refilled for the next stage
         // everything issued for stage s (scale registers, then operand blocks) has landed
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
-        float fa[2], fw[4];
+        // Operands of the scale products as[m] * ws[n] (see the loop below) for a 32x32x8 matrix instruction on 16-bit values:
+        // lanes 0-31 hold K 0-3 and lanes 32-63 hold K 4-7, two K slots to a register.  The first slot of a lane carries
+        // the stage's first group, the second slot its second group: the activation operand holds both activation scales,
+        // the weight operand one weight scale in the slot of its group and zero in the other.  A lane loaded the weight
+        // scales of column lane and column 64 + lane, so the even weight blocks find theirs in lanes 0-31 and the odd ones
+        // in lanes 32-63: sa[0] is zero in lanes 32-63, sa[1] in lanes 0-31.  Seven of the eight products are zero.
+        v2i sa[2], sw[2][2];
         if constexpr (WPL) {
+            const int both = (int)((uint32_t)qa[0] | ((uint32_t)qa[1] << 16));
+            sa[0] = (v2i){half ? 0 : both, 0};
+            sa[1] = (v2i){half ? both : 0, 0};
 #pragma unroll
-            for (int i = 0; i < 2; i++) fa[i] = T::to_f32(qa[i]);
-#pragma unroll
-            for (int i = 0; i < 4; i++) fw[i] = T::to_f32(qw[i]);
+            for (int j = 0; j < 2; j++) {
+                sw[0][j] = (v2i){(int)qw[j], 0};
+                sw[1][j] = (v2i){(int)((uint32_t)qw[2 + j] << 16), 0};
+            }
         } else {
             store_scales(base);
             __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));  // scale writes visible before the barrier
@@ -391,28 +401,23 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
                 const v4u e = (u & 0x0F0F0F0Fu) ^ flip, o = ((u >> 4) & 0x0F0F0F0Fu) ^ flip;
                 return (v8i){(int)e[0], (int)e[1], (int)e[2], (int)e[3], (int)o[0], (int)o[1], (int)o[2], (int)o[3]};
             };
-            auto outer = [&](int p) -> v32f {  // as[m] * ws[n] of pair p: blocks 2 (p & 1), + 1 of group p >> 1
-                v32f z;
-#pragma unroll
-                for (int i = 0; i < 32; i++) z[i] = 0.0f;
-                // both 32x32 blocks take their rows from lanes 0-31 of the first operand
-                return __builtin_amdgcn_mfma_f32_32x32x1f32(fa[p >> 1], fw[p], z, 1, 0, 0);
-            };
             const v16f z16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+            // as[m] * ws[n] of step b, exact (two 16-bit values, one non-zero product): a 16-bit matrix instruction, which
+            // runs beside the vector FMAs; the fp32 rank-1 matrix instruction shares the vector ALUs and does not
+            auto scales = [&](int b) -> v16f { return mfma32_16bit_k8<T>(sa[b & 1], sw[b >> 2][(b >> 1) & 1], z16); };
             v8i a8[2], w8[3];
-            v32f S[2];
-            v16f P[2];
+            v16f S[2], P[2];
             a8[0] = read_a8(0);
             w8[0] = read_w8(0);
             w8[1] = read_w8(1);
-            S[0] = outer(0);
+            S[0] = scales(0);
             P[0] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8[0], w8[0], z16, 0, 0, 0, F8_SCALE, 0, F8_SCALE);
             a8[1] = read_a8(1);
 #pragma unroll
             for (int b = 0; b < 8; b++) {
                 const int cur = b & 1, nxt = cur ^ 1;
                 if (b + 1 < 8) {
-                    if (((b + 1) & 1) == 0) S[((b + 1) >> 1) & 1] = outer((b + 1) >> 1);
+                    S[nxt] = scales(b + 1);
                     P[nxt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8[(b + 1) >> 2], w8[(b + 1) % 3], z16, 0, 0, 0,
                                                                              F8_SCALE, 0, F8_SCALE);
                 }
@@ -420,8 +425,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
                 if (!(LAST && !ACT_UNSIGNED) && b < PER_WAVE) dma_one(sn, other, b);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int i = 0; i < 16; i++)
-                    acc[b & 3][i] = __builtin_fmaf(P[cur][i], S[(b >> 1) & 1][16 * (b & 1) + i], acc[b & 3][i]);
+                for (int i = 0; i < 16; i++) acc[b & 3][i] = __builtin_fmaf(P[cur][i], S[cur][i], acc[b & 3][i]);
                 __builtin_amdgcn_sched_barrier(0);
             }
         } else {

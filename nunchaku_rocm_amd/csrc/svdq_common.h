@@ -8,6 +8,7 @@
 
 namespace svdq {
 
+typedef int v2i __attribute__((ext_vector_type(2)));
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef int v16i __attribute__((ext_vector_type(16)));
@@ -17,6 +18,8 @@ typedef float v32f __attribute__((ext_vector_type(32)));
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef short v8s __attribute__((ext_vector_type(8)));
+typedef short v4s __attribute__((ext_vector_type(4)));
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
 
 #define SVDQ_AS1 __attribute__((address_space(1)))
 #define SVDQ_AS3 __attribute__((address_space(3)))
@@ -94,6 +97,17 @@ __device__ inline v16f mfma32_16bit<BF16>(v4i a, v4i b, v16f c) {
 template <>
 __device__ inline v16f mfma32_16bit<FP16>(v4i a, v4i b, v16f c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(v8h, a), __builtin_bit_cast(v8h, b), c, 0, 0, 0);
+}
+// The same on four 16-bit values per lane (32x32, K = 8).
+template <typename T>
+__device__ inline v16f mfma32_16bit_k8(v2i a, v2i b, v16f c);
+template <>
+__device__ inline v16f mfma32_16bit_k8<BF16>(v2i a, v2i b, v16f c) {
+    return __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(__builtin_bit_cast(v4s, a), __builtin_bit_cast(v4s, b), c, 0, 0, 0);
+}
+template <>
+__device__ inline v16f mfma32_16bit_k8<FP16>(v2i a, v2i b, v16f c) {
+    return __builtin_amdgcn_mfma_f32_32x32x8f16(__builtin_bit_cast(v4h, a), __builtin_bit_cast(v4h, b), c, 0, 0, 0);
 }
 template <typename T>
 __device__ inline v4f mfma16_16bit(v4i a, v4i b, v4f c);

@@ -101,6 +101,30 @@ def test_scaled_gemm_bias_lora(dev, M, N, K, R, actual_m, unsigned, dtype):
     assert torch.equal(out.view(torch.int16), out2.view(torch.int16))
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_scale_products_are_exact_over_the_exponent_range(dev, dtype):
+    """as * ws is formed from the 16-bit scales themselves: subnormal fp16 activation scales (|x| < 4e-4 in a group),
+    tiny and large bf16 scales and zero scales must give the oracle's fp32 product.  One group: the output is p * as * ws
+    with p an exact integer, so a flushed or rounded scale shows as a wrong output.  Unsigned activations: the signed
+    fp8 loop adds its offset correction, whose 16-bit pieces are not exact at these magnitudes."""
+    M, N, K = 64, 128, 64
+    p = _rand_problem(M, N, K, 0, dtype, seed=5)
+    p["bias"] = None
+    if dtype == torch.float16:  # products from 2^-14 to 2^2: every output is a normal fp16 number or zero
+        asc = torch.tensor([2.0**-24, 3 * 2.0**-24, 1023 * 2.0**-24, 2.0**-14, 2.0**-15, 0.0, 2.0**-12, 2.0**-20], dtype=torch.float32)
+        wsc = torch.tensor([2.0**10, 1.5 * 2.0**10, 2.0**11, 2.0**12, 1.25 * 2.0**11, 2.0**14, 0.0, 2054.0], dtype=torch.float32)
+    else:  # products from 2^-115 to 2^60
+        asc = torch.tensor([2.0**-60, 1.5 * 2.0**-40, 2.0**-14, 1.0, 2.0**20, 0.0, 255 * 2.0**-30, 2.0**-50], dtype=torch.float32)
+        wsc = torch.tensor([1.0, 2.0**30, 2.0**-20, 1.9921875, 2.0**-30, 2.0**40, 0.0, 2.0**-55], dtype=torch.float32)
+    p["asc"] = asc.repeat(M // 8).reshape(1, M).to(dtype)
+    p["wsc"] = wsc.repeat_interleave(N // 8).reshape(1, N).to(dtype)
+    assert torch.equal(p["asc"].float()[0, :8], asc) and torch.equal(p["wsc"].float()[0, :: N // 8], wsc), "not representable"
+    out = _gpu_gemm(p, dev, unsigned=True, dtype=dtype)
+    ref = O.gemm_w4a4(p["act"], p["wgt"], p["asc"], p["wsc"], act_unsigned=True).to(dtype)
+    assert torch.isfinite(ref.float()).all() and (ref != 0).any()
+    assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
+
+
 def test_strided_row_views(dev):
     """act/wgt/out may be row slices of wider buffers as long as rows stay 16-byte aligned."""
     from nunchaku_rocm_amd import ops
