@@ -5,33 +5,33 @@
 // with p_g the exact int32 dot product of the group's 64 int4 pairs.
 //
 // How it maps to CDNA4:
-//  * p_g comes from two v_mfma_i32_32x32x32_i8 per 32x32 block.  A 16-byte LDS read holds 32 nibbles; the even and
-//    the odd nibbles are split into two int8 planes with shift/mask only (signed values land in the high nibble of
-//    each byte, i.e. times 16; unsigned activations in the low nibble, times 1).  Both operands use the same split,
-//    so the K order inside a group is a shared permutation and the dot product is unchanged.  The power-of-two
-//    factor (256 signed, 16 unsigned) is folded exactly into the fp32 activation scale.
-//  * The MFMA accumulator starts at the bit pattern of 1.5*2^23, so the int32 result read as fp32 is (2^23*1.5 + p)
-//    exactly and  fma(bits, as', -1.5*2^23*as')  gives p*as' with one rounding and no int->float convert; a second
-//    fma applies ws[g, n] and accumulates.  Two VALU ops per accumulator element per group.
-//  * The MFMA's A operand is the weight tile and its B operand the activation tile, so a lane owns one activation
-//    row m and its registers walk n in runs of four.  Row-wise epilogue work (RMSNorm sum of squares, RoPE pairs,
-//    group absmax, nibble packing, the next layer's LoRA-down B operand) is therefore in-lane plus one exchange with
-//    lane ^ 32.
-//  * 512 threads = 2 (n) x 4 (m) wavefronts of 64 weight rows x 32 activation rows on a 128x128 tile, two workgroups
-//    per CU = four wavefronts per SIMD: at half that occupancy the loop runs at about half the speed, its waits
-//    (LDS, MFMA results, barrier) exposed.  K is staged through LDS 128 at a time (two scale groups), two stages.
-//    Operands go global -> LDS directly (global_load_lds_dwordx4, no registers), one stage ahead, into a lane-linear
-//    layout (LDS slot l of a 1 KB block = the 16 bytes MFMA lane l needs), so the operand reads are bank-conflict
-//    free by construction; one raw s_barrier per stage with explicit s_waitcnt.  The four wavefronts of a SIMD issue
-//    their block loads at four different points of the stage (a wavefront blocks at issue while the memory pipe is
-//    full; the others keep computing).
+//  * 256 threads = four wavefronts, each 32 activation rows x all 128 weight rows of a 128x128 tile; two workgroups per
+//    CU = two wavefronts per SIMD.  The MFMA's A operand is the activation tile and its B operand the weight tile, so
+//    in the main loop a lane owns one weight row n and its registers walk the wavefront's 32 activation rows.
+//  * Packed weights (int8 loop): a 16-byte LDS read holds 32 nibbles; the even and the odd nibbles are split into two
+//    int8 planes with shift/mask only (signed values land in the high nibble of each byte, i.e. times 16; unsigned
+//    activations in the low nibble, times 1).  Both operands use the same split, so the K order inside a group is a
+//    shared permutation and the dot product is unchanged; the power-of-two factor is folded exactly into the weight
+//    scale.  p_g comes from two v_mfma_i32_32x32x32_i8 whose accumulator starts at the bit pattern of 1.5*2^23, so
+//    the int32 result read as fp32 is (1.5*2^23 + p) exactly and  fma(bits, ws', -1.5*2^23*ws')  gives p*ws' with one
+//    rounding and no int->float convert; a second fma applies as[g, m] and accumulates: two VALU ops per output and
+//    group.
+//  * Pre-split weights (fp8 loop, svdq_split_weight_planes): an int4 value is carried as the fp8 (e4m3) code of
+//    value * 2^-9, a signed activation as value + 8 (one three-input bit operation per plane; the offset is taken out
+//    after the loop with the weights' group sums).  One v_mfma_scale_f32_32x32x64_f8f6f4 with block scales 2^9 gives
+//    the exact p_g of a whole group as fp32; as[g, m] * ws[g, n] of the block comes from a 16-bit matrix instruction
+//    on the scales themselves (exact: one non-zero product); one FMA per output and group is left for the VALU.
+//  * K is staged through LDS 128 at a time (two scale groups), two stages.  Operands go global -> LDS directly
+//    (global_load_lds_dwordx4, no registers), one stage ahead, into a lane-linear layout (LDS slot l of a 1 KB block =
+//    the 16 bytes MFMA lane l needs), so the operand reads are bank-conflict free by construction; one raw s_barrier
+//    per stage with explicit s_waitcnt.  A wavefront issues its block loads one per step of the stage.
 //  * The epilogue's operands (bias, the first 32 ranks of lora_up and lora_act of the tile: 24.25 KB) are fetched into
 //    LDS together with stage 0, in MFMA lane order, so that the LoRA-up section does not wait for memory; with them
 //    a workgroup holds 78.25 KB of LDS, two workgroups still share a CU's 160 KB.
-//  * The 16-bit output tile leaves through LDS as 256-byte row segments (a lane's own accumulators are 8-byte pieces
-//    of 32 different rows, which the memory pipe takes one lane per cycle), stored non-temporally.
-//  * Weights can be given pre-split (svdq_split_weight_planes: int8 even / odd planes stored block by block in MFMA
-//    lane order); their half of the unpack then disappears from the inner loop.
+//  * After LoRA-up and bias each wavefront turns its four 32x32 blocks through a private LDS tile into "lane =
+//    activation row": row-wise epilogue work (RMSNorm sum of squares, RoPE pairs, group absmax, nibble packing, the
+//    next layer's LoRA-down operand) is then in-lane plus one exchange with lane ^ 32.
+//  * The 16-bit output tile leaves through LDS as 256-byte row segments, stored non-temporally.
 //  * Workgroup ids are first regrouped so that each XCD (ids are dealt round-robin over 8 XCDs) works on a
 //    contiguous range of tiles, then swizzled in bands of m-tiles for L2 reuse of the weight tile.
 #include <atomic>
@@ -220,7 +220,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
         const float w = T::to_f32(rws) * fold;
         ((float2 *)(base + WS_OFF))[sg * BN + sr] = make_float2(w, -RNE_MAGIC * w);
     };
-    // Pre-split weights (fp8 path): every lane fetches the scales its two rank-1 MFMA operands need, one stage ahead,
+    // Pre-split weights (fp8 path): every lane fetches the scales its scale-product MFMA operands need, one stage ahead,
     // straight into registers: the activation scale of row wm * 32 + l32 and the weight scales of columns lane and
     // 64 + lane, for both groups of the stage.  Groups past the end (odd K / 64) are staged as zero.
     uint16_t qa[2], qw[4];
@@ -384,8 +384,8 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
         else
             load_scales(sn);
         if constexpr (WPL) {
-            // One stage = eight (group, weight block) steps.  The matrix instructions of step b + 1 (and, at every second
-            // step, the rank-1 product of the next pair's scales) are issued ahead of the sixteen FMAs of step b.
+            // One stage = eight (group, weight block) steps.  The two matrix instructions of step b + 1 (scale product and
+            // group dot product) are issued ahead of the sixteen FMAs of step b.
             auto read_w8 = [&](int b) -> v8i {
                 const int gg = b >> 2, bn = b & 3;
                 const v4i lo = *(const v4i *)(base + offW + ((bn * 2 + gg) * 2 + 0) * BLK_BYTES);
