@@ -421,6 +421,9 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
                     P[nxt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8[(b + 1) >> 2], w8[(b + 1) % 3], z16, 0, 0, 0,
                                                                              F8_SCALE, 0, F8_SCALE);
                 }
+                // the operand reads of step b + 2 stay behind the matrix instructions: hoisted above them, the wait for step
+                // b + 1's operands would also wait for these
+                __builtin_amdgcn_sched_barrier(0);
                 if (b + 2 < 8) w8[(b + 2) % 3] = read_w8(b + 2);
                 if (!(LAST && !ACT_UNSIGNED) && b < PER_WAVE) dma_one(sn, other, b);
                 __builtin_amdgcn_sched_barrier(0);
@@ -504,7 +507,6 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
     // sums.  svdq_split_weight_planes stored D[g, n] = -8 ws[g, n] W[g, n] behind the planes as two 16-bit pieces
     // (hi + lo: 16 significant bits in bf16, 22 in fp16), K-contiguous per weight row like a LoRA-up matrix of rank 2 * G16; the
     // activation scales are the other operand.  Products of two 16-bit values are exact, the sum is fp32.
-#ifndef ABL_NOCORR
     if constexpr (WPL && !ACT_UNSIGNED) {
         if (GL < G16) corr_fetch(0, GL);
         __syncthreads();  // every wavefront's share of the staged blocks has landed (each waited for its own above)
@@ -526,7 +528,6 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
             if (g0 + 16 < G16) corr_apply(1);
         }
     }
-#endif
 
     // ---- LoRA-up and bias, still in the main loop's orientation (lane = weight row, registers = activation rows) ----
     // The bias and the first 32 ranks of both LoRA operands were fetched into LDS next to stage 0 and arrived long ago;
