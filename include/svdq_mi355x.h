@@ -153,14 +153,16 @@ typedef struct {
 int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream);
 
 /*
- * One-time re-layout of a weight for the GEMM.  Every (32-row block, scale group) becomes two 1 KB planes (even and odd
- * nibbles) of fp8 (e4m3) codes in the order the MFMA lanes read them: a signed int4 value v is stored as the byte
- * sign | |v|, which the fp8 matrix instruction reads as v * 2^-9 exactly (v_mfma_scale_f32_32x32x64_f8f6f4 runs at
- * the int8 rate, takes a whole 64-deep group per instruction and returns the integer dot product as fp32, which saves
- * the GEMM one of its two scaling multiplies per output and group).  Behind the planes sit, per weight row, two T
+ * One-time re-layout of a weight for the GEMM.  Every (32-row block, pair of scale groups) becomes three 1 KB blocks of
+ * fp6 (e2m3) codes in the order the MFMA lanes read them: a signed int4 value v is stored as the six bits
+ * sign | |v|, which the matrix instruction reads as v / 8 exactly; a lane's 32 weights of a group are six registers
+ * (blocks 0 and 1: registers 0-3 of the pair's first and second group, block 2: registers 4-5 of both; a missing second
+ * group is zeros).  v_mfma_scale_f32_32x32x64_f8f6f4 takes them next to fp8 activation codes at the int8 rate, a whole
+ * 64-deep group per instruction, and returns the integer dot product as fp32, which saves the GEMM one of its two
+ * scaling multiplies per output and group.  Behind the codes sit, per weight row, two T
  * pieces per group (hi + lo) of -8 * ws[g, n] * (sum of the group's 64 weights): the GEMM offsets signed activations by
  * +8 for the fp8 operand and takes that term out again.  `planes` needs svdq_weight_planes_bytes(N, K) bytes
- * (= ceil(N/32)*32 * (K + 4 * ceil(K/1024)*16)).  The copy depends on `wgt` AND `wscales` (dtype = their type).  No
+ * (= ceil(N/32) * (ceil(K/128) * 3072 + 32 * 4 * ceil(K/1024)*16): three quarters of a byte per weight).  The copy depends on `wgt` AND `wscales` (dtype = their type).  No
  * counterpart in the reference (its SwiGLU path re-orders weight rows at load in the same spirit, ops/fused.py:83-105).
  */
 int svdq_split_weight_planes(const void *wgt, const void *wscales, void *planes, int32_t N, int32_t K, int32_t ld_wgt,

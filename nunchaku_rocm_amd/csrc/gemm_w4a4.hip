@@ -16,10 +16,11 @@
 //    the int32 result read as fp32 is (1.5*2^23 + p) exactly and  fma(bits, ws', -1.5*2^23*ws')  gives p*ws' with one
 //    rounding and no int->float convert; a second fma applies as[g, m] and accumulates: two VALU ops per output and
 //    group.
-//  * Pre-split weights (fp8 loop, svdq_split_weight_planes): an int4 value is carried as the fp8 (e4m3) code of
-//    value * 2^-9, a signed activation as value + 8 (one three-input bit operation per plane; the offset is taken out
-//    after the loop with the weights' group sums).  One v_mfma_scale_f32_32x32x64_f8f6f4 with block scales 2^9 gives
-//    the exact p_g of a whole group as fp32; as[g, m] * ws[g, n] of the block comes from a 16-bit matrix instruction
+//  * Pre-split weights (fp8 loop, svdq_split_weight_planes): an activation is carried as the fp8 (e4m3) code of
+//    value * 2^-9, a signed one as value + 8 (one three-input bit operation per plane; the offset is taken out after
+//    the loop with the weights' group sums); a weight as the fp6 (e2m3) code of value / 8, 24 bytes per lane and group
+//    instead of 32.  One v_mfma_scale_f32_32x32x64_f8f6f4 with block scales 2^9 and 2^3 gives the exact p_g of a
+//    whole group as fp32; as[g, m] * ws[g, n] of the block comes from a 16-bit matrix instruction
 //    on the scales themselves (exact: one non-zero product); one FMA per output and group is left for the VALU.
 //  * K is staged through LDS 128 at a time (two scale groups), two stages.  Operands go global -> LDS directly
 //    (global_load_lds_dwordx4, no registers), one stage ahead, into a lane-linear layout (LDS slot l of a 1 KB block =
@@ -46,7 +47,7 @@ constexpr int KSTAGE = 128;           // K per LDS stage = two scale groups
 constexpr int NSTAGE = 2;             // LDS stages: one being computed on, one being filled
 constexpr int BLK_BYTES = 64 * 16;    // one MFMA operand block (32 rows x 16 bytes per lane) of one group, lane-linear
 // stage layout: activation blocks [4 blocks of 32 rows][2 groups] packed (1 KB each), weight blocks
-// [4 blocks][2 groups][2 planes] (pre-split weights) or [4 blocks][2 groups] (packed), then the scales
+// [4 blocks][group 0 low, group 1 low, both high] (pre-split weights) or [4 blocks][2 groups] (packed), then the scales
 constexpr int W_OFF = 4 * 2 * BLK_BYTES;                  // 8192
 constexpr int AS_OFF = W_OFF + 4 * 2 * 2 * BLK_BYTES;     // 24576: float as[2][BM]
 constexpr int WS_OFF = AS_OFF + 2 * BM * 4;               // 25600: float2 (ws', -magic * ws')[2][BN]
@@ -62,6 +63,12 @@ constexpr int TP_PITCH = 36;                        // floats per row of the acc
 constexpr int TP_WAVE_BYTES = 2 * 32 * TP_PITCH * 4;  // two 32x32 blocks at a time
 static_assert(2 * TP_WAVE_BYTES <= BUF_BYTES, "transposition tiles do not fit");
 constexpr int F8_SCALE = (int)0x88888888;  // e8m0 block scale 2^9 in every byte: an fp8 code c (value c * 2^-9) counts as c
+constexpr int F6_SCALE = (int)0x82828282;  // e8m0 block scale 2^3: an fp6 (e2m3) code c <= 15 (value c / 8) counts as c
+// Pre-split weights, per (block of 32 rows, stage of two groups): three 1 KB blocks in MFMA lane order.  A lane's 32
+// weights of a group are 32 six-bit codes = six registers: blocks 0 and 1 hold registers 0-3 of the stage's first and
+// second group (16 bytes per lane), block 2 registers 4-5 of both (8 + 8 bytes per lane).
+constexpr int WPL_BLOCKS = 3;
+constexpr int CORR_PER_WAVE = 6;       // staged group-sum blocks fetched per wavefront
 constexpr int NPIECE = 2;              // 16-bit pieces per group sum behind the weight planes (hi + lo: 16 / 22 significant bits)
 constexpr int CORR_LDS_G = 48;         // groups whose sums one staging buffer holds for the offset correction (24 blocks of 1 KB)
 constexpr int GROUP_M_TILES = 8;      // m-tiles per raster band
@@ -82,6 +89,24 @@ __device__ inline void unpack_unsigned(v4i p, v4i &even, v4i &odd) {
 // fp8 (e4m3) code of a signed int4 value: sign bit | magnitude in the low four bits.  A code c <= 15 stands for
 // c * 2^-9 (subnormals and the first binade form one linear run).
 __device__ inline uint32_t f8_code(int v) { return (uint32_t)((v < 0 ? 0x80 : 0) | (v < 0 ? -v : v)); }
+// fp6 (e2m3) code of a signed int4 value: sign bit | magnitude in the low four bits; a code c <= 15 stands for c / 8.
+__device__ inline uint32_t f6_code(int v) { return (uint32_t)((v < 0 ? 0x20 : 0) | (v < 0 ? -v : v)); }
+// The six registers of a lane's fp6 operand: 32 six-bit codes, code p in bits 6 p .. 6 p + 5.  The matrix instruction
+// numbers K differently per format: an fp8 lane of half h holds K 16 h .. 16 h + 15 and 32 + 16 h .. 47 + 16 h (the even,
+// then the odd nibbles of the lane's 16 packed activation bytes), an fp6 lane of half h holds K 32 h .. 32 h + 31.  So
+// the weight lanes of half 0 carry the even nibbles of all 32 packed bytes of the row's group, those of half 1 the odd.
+__device__ inline void f6_pack(const v4i lo16, const v4i hi16, int odd, uint32_t (&d)[6]) {
+#pragma unroll
+    for (int i = 0; i < 6; i++) d[i] = 0;
+#pragma unroll
+    for (int p = 0; p < 32; p++) {
+        const int by = ((p < 16 ? lo16 : hi16)[(p & 15) >> 2] >> (8 * (p & 3))) & 0xFF;
+        const uint32_t c = f6_code((((odd ? by >> 4 : by) & 0xF) ^ 8) - 8);
+        const int bit = 6 * p;
+        d[bit >> 5] |= c << (bit & 31);
+        if ((bit & 31) > 26) d[(bit >> 5) + 1] |= c >> (32 - (bit & 31));
+    }
+}
 
 __device__ inline v16i magic_acc() {
     v16i c;
@@ -127,8 +152,8 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
     // 16 bytes MFMA lane l will read and the hardware writes them to LDS slot l of the block: the layout the operand
     // read wants, free of bank conflicts by construction.  Packed operands: lane l = (row l % 32, half l / 32) of a
     // row-major tile.  Pre-split weights are already stored block by block in that order (1 KB contiguous per load).
-    // The 8 activation + (WPL ? 16 : 8) weight block loads of a stage are dealt in runs to the four wavefronts.
-    constexpr int NLOADS = WPL ? 24 : 16, PER_WAVE = NLOADS / NWAVES;
+    // The 8 activation + (WPL ? 12 : 8) weight block loads of a stage are dealt in runs to the four wavefronts.
+    constexpr int NLOADS = WPL ? 8 + 4 * WPL_BLOCKS : 16, PER_WAVE = NLOADS / NWAVES;
     // each load's address = wave-uniform base (SGPRs) + a 32-bit offset (lane part + stage * step; operands < 4 GiB)
     const uint8_t *gbase[PER_WAVE];
     uint32_t goff[PER_WAVE];
@@ -155,14 +180,14 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
             ldst[i] = (blk * 2 + gg) * BLK_BYTES;
             gstep[i] = KSTAGE / 2;
             if constexpr (ODDG) gcap[i] = cap_of(gg, gstep[i], gbase[i], 32);
-        } else if (WPL) {                 // weight plane block j: (blk = j / 4, group (j / 2) % 2, plane j % 2)
-            const int j = q - 8, blk = j >> 2, gg = (j >> 1) & 1, pl = j & 1;
+        } else if (WPL) {                 // pre-split weight block j: (blk = j / 3, part j % 3)
+            const int j = q - 8, blk = j / WPL_BLOCKS, part = j % WPL_BLOCKS;
             const int nblk = min(n0 / 32 + blk, (a.N + 31) / 32 - 1);
-            gbase[i] = (const uint8_t *)a.wgt_planes + (((size_t)nblk * G + gg) * 2 + pl) * BLK_BYTES;
+            gbase[i] = (const uint8_t *)a.wgt_planes + ((size_t)nblk * ((G + 1) / 2) * WPL_BLOCKS + part) * BLK_BYTES;
             goff[i] = lane * 16;
-            ldst[i] = W_OFF + ((blk * 2 + gg) * 2 + pl) * BLK_BYTES;
-            gstep[i] = 2 * 2 * BLK_BYTES;   // two groups x two planes per stage
-            if constexpr (ODDG) gcap[i] = cap_of(gg, gstep[i], gbase[i], 2 * BLK_BYTES);
+            ldst[i] = W_OFF + (blk * WPL_BLOCKS + part) * BLK_BYTES;
+            gstep[i] = WPL_BLOCKS * BLK_BYTES;
+            if constexpr (ODDG) gcap[i] = 0xFFFFFFFFu;  // a last stage of one group is stored with zeros for the other
         } else {                          // packed weight block j: (blk = j / 2, group j % 2)
             const int j = q - 8, blk = j >> 1, gg = j & 1;
             gbase[i] = (const uint8_t *)a.wgt + (size_t)n0 * a.ld_wgt + gg * 32;
@@ -253,19 +278,19 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
     const uint16_t *cdp = nullptr, *cap = nullptr;
     uint32_t cdrow[NBN];
     const int cnpad = (a.N + 31) / 32 * 32;
-    static_assert(NBN * NPIECE * (CORR_LDS_G / 16) == NWAVES * 6 && NBN * NPIECE * (CORR_LDS_G / 16) * BLK_BYTES <= BUF_BYTES,
+    static_assert(NBN * NPIECE * (CORR_LDS_G / 16) == NWAVES * CORR_PER_WAVE && NBN * NPIECE * (CORR_LDS_G / 16) * BLK_BYTES <= BUF_BYTES,
                   "the staged group sums are dealt six blocks to a wavefront and must fit one staging buffer");
     if constexpr (WPL && !ACT_UNSIGNED) {
         const int npad = cnpad;
-        cdp = (const uint16_t *)((const uint8_t *)a.wgt_planes + (size_t)npad * a.K) + 8 * half;
+        cdp = (const uint16_t *)((const uint8_t *)a.wgt_planes + (size_t)(npad / 32) * ((G + 1) / 2) * (WPL_BLOCKS * BLK_BYTES)) + 8 * half;
         cap = (const uint16_t *)a.ascales + min(m0 + wm * 32 + l32, a.M - 1);
 #pragma unroll
         for (int bn = 0; bn < NBN; bn++) cdrow[bn] = (uint32_t)min(n0 + bn * 32 + l32, npad - 1) * (uint32_t)(NPIECE * G16);
     }
     auto corr_stage_lds = [&](uint8_t *dstbuf) {  // this wavefront's share of the (NBN x NPIECE x GL / 16) blocks
 #pragma unroll
-        for (int i = 0; i < PER_WAVE; i++) {
-            const int q = wm * PER_WAVE + i;  // wave-uniform: (sixteen groups gc, piece, weight block)
+        for (int i = 0; i < CORR_PER_WAVE; i++) {
+            const int q = wm * CORR_PER_WAVE + i;  // wave-uniform: (sixteen groups gc, piece, weight block)
             const int bn = q % NBN, pc = (q / NBN) % NPIECE, gc = q / (NBN * NPIECE);
             const uint32_t row = (uint32_t)min(n0 + bn * 32 + l32, cnpad - 1) * (uint32_t)(NPIECE * G16);
             if (gc * 16 < GL)
@@ -386,11 +411,11 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
         if constexpr (WPL) {
             // One stage = eight (group, weight block) steps.  The two matrix instructions of step b + 1 (scale product and
             // group dot product) are issued ahead of the sixteen FMAs of step b.
-            auto read_w8 = [&](int b) -> v8i {
+            auto read_w8 = [&](int b) -> v8i {  // six registers of fp6 codes (the matrix instruction ignores the last two)
                 const int gg = b >> 2, bn = b & 3;
-                const v4i lo = *(const v4i *)(base + offW + ((bn * 2 + gg) * 2 + 0) * BLK_BYTES);
-                const v4i hi = *(const v4i *)(base + offW + ((bn * 2 + gg) * 2 + 1) * BLK_BYTES);
-                return (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                const v4i lo = *(const v4i *)(base + offW + (bn * WPL_BLOCKS + gg) * BLK_BYTES);
+                const v2i hi = *(const v2i *)(base + offW + (bn * WPL_BLOCKS + 2) * BLK_BYTES + gg * 8);
+                return (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], 0, 0};
             };
             auto read_a8 = [&](int gg) -> v8i {
                 typedef unsigned v4u __attribute__((ext_vector_type(4)));
@@ -411,15 +436,15 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
             w8[0] = read_w8(0);
             w8[1] = read_w8(1);
             S[0] = scales(0);
-            P[0] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8[0], w8[0], z16, 0, 0, 0, F8_SCALE, 0, F8_SCALE);
+            P[0] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8[0], w8[0], z16, 0, 2, 0, F8_SCALE, 0, F6_SCALE);
             a8[1] = read_a8(1);
 #pragma unroll
             for (int b = 0; b < 8; b++) {
                 const int cur = b & 1, nxt = cur ^ 1;
                 if (b + 1 < 8) {
                     S[nxt] = scales(b + 1);
-                    P[nxt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8[(b + 1) >> 2], w8[(b + 1) % 3], z16, 0, 0, 0,
-                                                                             F8_SCALE, 0, F8_SCALE);
+                    P[nxt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8[(b + 1) >> 2], w8[(b + 1) % 3], z16, 0, 2, 0,
+                                                                             F8_SCALE, 0, F6_SCALE);
                 }
                 // the operand reads of step b + 2 stay behind the matrix instructions: hoisted above them, the wait for step
                 // b + 1's operands would also wait for these
@@ -943,9 +968,9 @@ __global__ __launch_bounds__(64) void group_acc_kernel(const uint8_t *act, const
     }
 }
 
-// The same read-out through the instruction sequence of the pre-split (fp8) path: nibbles as fp8 codes, activations
-// offset by 8 when signed, v_mfma_scale_f32_32x32x64_f8f6f4 with block scales 2^9, offset taken out with the weights'
-// group sum.  Every value involved is an integer below 2^24, so the fp32 result is exact.
+// The same read-out through the instruction sequence of the pre-split (fp8) path: activation nibbles as fp8 codes,
+// offset by 8 when signed, weights as fp6 codes, v_mfma_scale_f32_32x32x64_f8f6f4 with block scales 2^9 and 2^3, offset
+// taken out with the weights' group sum.  Every value involved is an integer below 2^24, so the fp32 result is exact.
 template <bool ACT_UNSIGNED>
 __global__ __launch_bounds__(64) void group_acc_f8_kernel(const uint8_t *act, const uint8_t *wgt, int32_t *out, int M,
                                                           int N, int ld_act, int ld_wgt, int group) {
@@ -957,25 +982,20 @@ __global__ __launch_bounds__(64) void group_acc_f8_kernel(const uint8_t *act, co
     if (!ACT_UNSIGNED) u ^= 0x88888888u;
     const v4u e = u & 0x0F0F0F0Fu, o = (u >> 4) & 0x0F0F0F0Fu;
     const v8i a8 = {(int)e[0], (int)e[1], (int)e[2], (int)e[3], (int)o[0], (int)o[1], (int)o[2], (int)o[3]};
-    v8i w8;
+    uint32_t w6[6];
+    {
+        const uint8_t *wrow = wgt + (size_t)min(nb + l32, N - 1) * ld_wgt + group * 32;
+        f6_pack(*(const v4i *)wrow, *(const v4i *)(wrow + 16), half, w6);
+    }
+    const v8i w8 = {(int)w6[0], (int)w6[1], (int)w6[2], (int)w6[3], (int)w6[4], (int)w6[5], 0, 0};
     int wsum = 0;
 #pragma unroll
-    for (int d = 0; d < 4; d++) {
-        uint32_t we = 0, wo = 0;
+    for (int d = 0; d < 4; d++)
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int by = (wp[d] >> (8 * j)) & 0xFF;
-            const int lo = ((by & 0xF) ^ 8) - 8, hi = ((by >> 4) ^ 8) - 8;
-            wsum += lo + hi;
-            we |= f8_code(lo) << (8 * j);
-            wo |= f8_code(hi) << (8 * j);
-        }
-        w8[d] = (int)we;
-        w8[4 + d] = (int)wo;
-    }
+        for (int j = 0; j < 8; j++) wsum += (((wp[d] >> (4 * j)) & 0xF) ^ 8) - 8;
     wsum += __shfl_xor(wsum, 32);  // the other half of the group
     const v16f z16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-    v16f t = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8, w8, z16, 0, 0, 0, F8_SCALE, 0, F8_SCALE);
+    v16f t = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8, w8, z16, 0, 2, 0, F8_SCALE, 0, F6_SCALE);
     // The matrix instruction reads the operands of all 64 lanes: pin it here, ahead of the lane-dependent stores below
     // (moved behind a divergent branch, it ran with some lanes' operands never loaded).
     asm volatile("" : "+v"(t));
@@ -1022,30 +1042,28 @@ static void launch_gemm_epi(const svdq_gemm_args &a, hipStream_t s) {
         launch_gemm_epi2<T, U, false>(a, s);
 }
 
-// weight re-layout: thread (block of 32 rows, group, lane) turns its 16 packed bytes into the even / odd planes
+// weight re-layout: thread (block of 32 rows, stage of two groups, lane) turns the nibbles of its parity of each group's
+// 32 packed bytes into six registers of fp6 codes; a group past the end (K / 64 odd) is stored as zeros
 __global__ void split_weight_planes_kernel(const uint8_t *wgt, uint8_t *planes, int N, int G, int ld_wgt) {
     const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int lane = idx & 63;
-    const size_t bg = idx >> 6;  // nblk * G + g
-    const int g = (int)(bg % G), nblk = (int)(bg / G);
+    const size_t bs = idx >> 6;  // nblk * nst + s
+    const int nst = (G + 1) / 2;
+    const int s = (int)(bs % nst), nblk = (int)(bs / nst);
     if (nblk >= (N + 31) / 32) return;
     const int row = min(nblk * 32 + (lane & 31), N - 1);
-    const v4i p = *(const v4i *)(wgt + (size_t)row * ld_wgt + g * 32 + (lane >> 5) * 16);
-    v4i even, odd;
+    uint8_t *dst = planes + bs * (WPL_BLOCKS * BLK_BYTES) + lane * 16;
 #pragma unroll
-    for (int d = 0; d < 4; d++) {
-        uint32_t e = 0, o = 0;
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int by = (p[d] >> (8 * j)) & 0xFF;
-            e |= f8_code(((by & 0xF) ^ 8) - 8) << (8 * j);
-            o |= f8_code(((by >> 4) ^ 8) - 8) << (8 * j);
+    for (int gg = 0; gg < 2; gg++) {
+        const int g = 2 * s + gg;
+        uint32_t d[6] = {0, 0, 0, 0, 0, 0};
+        if (g < G) {
+            const uint8_t *src = wgt + (size_t)row * ld_wgt + g * 32;
+            f6_pack(*(const v4i *)src, *(const v4i *)(src + 16), lane >> 5, d);
         }
-        even[d] = (int)e;
-        odd[d] = (int)o;
+        *(v4i *)(dst + gg * BLK_BYTES) = (v4i){(int)d[0], (int)d[1], (int)d[2], (int)d[3]};
+        *(v2i *)(dst + 2 * BLK_BYTES + gg * 8) = (v2i){(int)d[4], (int)d[5]};
     }
-    *(v4i *)(planes + ((bg * 2 + 0) * 64 + lane) * 16) = even;
-    *(v4i *)(planes + ((bg * 2 + 1) * 64 + lane) * 16) = odd;
 }
 
 // D[g, n] = -8 * ws[g, n] * (sum of the 64 weights of group g in row n), exact in fp32, written as NPIECE T values whose
@@ -1090,7 +1108,8 @@ static bool al16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 extern "C" size_t svdq_weight_planes_bytes(int32_t N, int32_t K) {
     if (N <= 0 || K <= 0) return 0;
     const size_t npad = (size_t)((N + 31) / 32) * 32, g16 = (size_t)((K / GROUP + 15) / 16) * 16;
-    return npad * (size_t)K + npad * NPIECE * g16 * 2;  // fp8 planes, then the 16-bit pieces of D[g, n]
+    const size_t nst = (size_t)(K / GROUP + 1) / 2;
+    return npad / 32 * nst * (WPL_BLOCKS * BLK_BYTES) + npad * NPIECE * g16 * 2;  // fp6 codes, then the 16-bit pieces of D[g, n]
 }
 
 extern "C" int svdq_split_weight_planes(const void *wgt, const void *wscales, void *planes, int32_t N, int32_t K,
@@ -1102,12 +1121,12 @@ extern "C" int svdq_split_weight_planes(const void *wgt, const void *wscales, vo
         return SVDQ_E_INVALID;
     }
     const int G = K / GROUP, G16 = (G + 15) / 16 * 16, npad = (N + 31) / 32 * 32;
-    const size_t n = (size_t)(npad / 32) * G * 64;
+    const size_t n = (size_t)(npad / 32) * ((G + 1) / 2) * 64;
     hipLaunchKernelGGL(split_weight_planes_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
                        (const uint8_t *)wgt, (uint8_t *)planes, N, G, ld_wgt);
     int rc = check_launch("svdq_split_weight_planes");
     if (rc) return rc;
-    uint16_t *dpieces = (uint16_t *)((uint8_t *)planes + (size_t)npad * K);
+    uint16_t *dpieces = (uint16_t *)((uint8_t *)planes + (size_t)(npad / 32) * ((G + 1) / 2) * (WPL_BLOCKS * BLK_BYTES));
     const size_t nd = (size_t)npad * G16;
     if (dtype == SVDQ_BF16)
         hipLaunchKernelGGL(weight_group_sums_kernel<BF16>, dim3((unsigned)((nd + 255) / 256)), dim3(256), 0, (hipStream_t)stream,

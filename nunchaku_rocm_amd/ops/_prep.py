@@ -90,10 +90,10 @@ _planes_cache: dict[int, tuple] = {}
 
 
 def weight_planes(qweight: torch.Tensor, wscales: torch.Tensor) -> torch.Tensor:
-    """The GEMM's working copy of a packed ``(N, K/2)`` weight (``svdq_split_weight_planes``): even / odd nibble planes
-    as fp8 codes in MFMA lane order, followed by the per-group weight sums times ``-8 * wscales`` that take the offset
-    of signed activations out again.  Made on first use and kept while both tensors live unmodified.  Costs
-    ``N * K`` bytes (twice the packed weight) plus ``4 * N * K / 64`` bytes."""
+    """The GEMM's working copy of a packed ``(N, K/2)`` weight (``svdq_split_weight_planes``): six-bit fp6 codes in
+    MFMA lane order, followed by the per-group weight sums times ``-8 * wscales`` that take the offset of signed
+    activations out again.  Made on first use and kept while both tensors live unmodified.  Costs ``0.75 * N * K``
+    bytes (one and a half times the packed weight) plus ``4 * N * K / 64`` bytes."""
     key = id(qweight)
     hit = _planes_cache.get(key)
     if hit is not None:

@@ -8,8 +8,8 @@ from .. import _lib
 from ._prep import lora_down_t as _lora_down_t
 from ._prep import weight_planes as _weight_planes
 
-# Which weights get the GEMM's working copy (fp8 nibble planes in MFMA lane order + group sums, cached per tensor, see
-# _prep.weight_planes; twice the packed weight's bytes on top of it, about 20 % faster GEMM): "parameters" = weights that
+# Which weights get the GEMM's working copy (fp6 codes in MFMA lane order + group sums, cached per tensor, see
+# _prep.weight_planes; one and a half times the packed weight's bytes on top of it, about 22 % faster GEMM): "parameters" = weights that
 # are nn.Parameter (module weights, which live long), "all" = any weight tensor (a temporary pays the re-layout on every
 # call), "none" = the GEMM unpacks the packed weight itself (int8 main loop, no extra memory).
 USE_WEIGHT_PLANES = "parameters"

@@ -235,15 +235,29 @@ def test_linear_module_matches_dequantised_reference(dev):
 
 
 def _planes_expected(wgt, wsc, N, K):
-    """Host restatement of the pre-split weight layout: [(block of 32 rows, group), plane, lane, 16 bytes] of fp8 codes
-    sign | magnitude, then per row two 16-bit pieces (hi, lo) per group (piece-major, groups padded to 16) of
-    -8 * wscale * (sum of the group's weights)."""
+    """Host restatement of the pre-split weight layout.  Per (block of 32 rows, stage of two groups) three 1 KB blocks:
+    a lane (= parity * 32 + row) holds, per group, 32 six-bit codes sign | magnitude (position p = the nibble of its parity
+    of the row's packed byte p of the group; code p in bits 6 p .. 6 p + 5 of 24 little-endian bytes); blocks 0 and 1 = bytes
+    0-15 of the stage's two groups, block 2 = bytes 16-23 of both.  A group past the end is zeros.  Then per row two 16-bit
+    pieces (hi, lo) per group (piece-major, groups padded to 16) of -8 * wscale * (sum of the group's weights)."""
+    import numpy as np
+
     nb, G = (N + 31) // 32, K // 64
+    nst = (G + 1) // 2
     q = O.unpack_int4(wgt, signed=True).to(torch.int16)  # (N, K) in [-8, 7]
     rows = torch.arange(nb * 32).clamp(max=N - 1)
-    qb = q[rows].view(nb, 32, G, 2, 16, 2)  # (nblk, row in block, g, half, byte, even/odd)
-    v = (qb.abs() | ((qb < 0).to(torch.int16) << 7)).to(torch.uint8)
-    planes = v.permute(0, 2, 5, 3, 1, 4).reshape(nb, G, 2, 64, 16).contiguous()  # lane = half * 32 + row
+    qb = q[rows].view(nb, 32, G, 32, 2)  # (nblk, row in block, g, packed byte, even/odd nibble)
+    code = (qb.abs() | ((qb < 0).to(torch.int16) << 5)).to(torch.uint8)
+    code = code.permute(0, 2, 4, 1, 3).reshape(nb, G, 64, 32)  # (nblk, g, lane = parity * 32 + row, position = byte)
+    full = torch.zeros(nb, nst * 2, 64, 32, dtype=torch.uint8)
+    full[:, :G] = code
+    bits = ((full.numpy()[..., None] >> np.arange(6, dtype=np.uint8)) & 1).reshape(nb, nst, 2, 64, 192)
+    by = torch.from_numpy(np.packbits(bits, axis=-1, bitorder="little"))  # (nblk, stage, group of the stage, lane, 24)
+    planes = torch.zeros(nb, nst, 3, 64, 16, dtype=torch.uint8)
+    planes[:, :, 0] = by[:, :, 0, :, :16]
+    planes[:, :, 1] = by[:, :, 1, :, :16]
+    planes[:, :, 2, :, :8] = by[:, :, 0, :, 16:]
+    planes[:, :, 2, :, 8:] = by[:, :, 1, :, 16:]
     G16 = (G + 15) // 16 * 16
     d = torch.zeros(nb * 32, G16, dtype=torch.float32)
     d[:N, :G] = -8.0 * (wsc.float().t()[:N] * q.view(N, G, 64).sum(-1).float())
@@ -254,7 +268,7 @@ def _planes_expected(wgt, wsc, N, K):
     return planes, pieces
 
 
-@pytest.mark.parametrize("N,K", [(32, 64), (264, 256), (100, 128), (64, 2048)])
+@pytest.mark.parametrize("N,K", [(32, 64), (264, 256), (100, 128), (64, 2048), (72, 320)])
 def test_weight_planes_layout(dev, N, K):
     from nunchaku_rocm_amd.ops._prep import weight_planes
 
