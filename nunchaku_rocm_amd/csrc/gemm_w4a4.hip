@@ -152,8 +152,10 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
     // 16 bytes MFMA lane l will read and the hardware writes them to LDS slot l of the block: the layout the operand
     // read wants, free of bank conflicts by construction.  Packed operands: lane l = (row l % 32, half l / 32) of a
     // row-major tile.  Pre-split weights are already stored block by block in that order (1 KB contiguous per load).
-    // The 8 activation + (WPL ? 12 : 8) weight block loads of a stage are dealt in runs to the four wavefronts.
-    constexpr int NLOADS = WPL ? 8 + 4 * WPL_BLOCKS : 16, PER_WAVE = NLOADS / NWAVES;
+    // Packed weights: the 8 activation + 8 weight block loads of a stage are dealt in runs to the four wavefronts.
+    // Pre-split weights: only the 12 weight blocks go through LDS; a wavefront's 32 activation rows are read by nobody
+    // else, so it fetches them straight into registers (see load_act below).
+    constexpr int NLOADS = WPL ? 4 * WPL_BLOCKS : 16, PER_WAVE = NLOADS / NWAVES, NABLK = WPL ? 0 : 8;
     // each load's address = wave-uniform base (SGPRs) + a 32-bit offset (lane part + stage * step; operands < 4 GiB)
     const uint8_t *gbase[PER_WAVE];
     uint32_t goff[PER_WAVE];
@@ -173,7 +175,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
 #pragma unroll
     for (int i = 0; i < PER_WAVE; i++) {
         const int q = wm * PER_WAVE + i;  // wave-uniform
-        if (q < 8) {                      // activation block q: (blk = q / 2, group q % 2)
+        if (q < NABLK) {                  // activation block q: (blk = q / 2, group q % 2)
             const int blk = q >> 1, gg = q & 1;
             gbase[i] = (const uint8_t *)a.act + (size_t)m0 * a.ld_act + gg * 32;
             goff[i] = (uint32_t)(min(m0 + blk * 32 + l32, a.M - 1) - m0) * (uint32_t)a.ld_act + half * 16;
@@ -181,7 +183,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
             gstep[i] = KSTAGE / 2;
             if constexpr (ODDG) gcap[i] = cap_of(gg, gstep[i], gbase[i], 32);
         } else if (WPL) {                 // pre-split weight block j: (blk = j / 3, part j % 3)
-            const int j = q - 8, blk = j / WPL_BLOCKS, part = j % WPL_BLOCKS;
+            const int j = q, blk = j / WPL_BLOCKS, part = j % WPL_BLOCKS;
             const int nblk = min(n0 / 32 + blk, (a.N + 31) / 32 - 1);
             gbase[i] = (const uint8_t *)a.wgt_planes + ((size_t)nblk * ((G + 1) / 2) * WPL_BLOCKS + part) * BLK_BYTES;
             goff[i] = lane * 16;
@@ -189,7 +191,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
             gstep[i] = WPL_BLOCKS * BLK_BYTES;
             if constexpr (ODDG) gcap[i] = 0xFFFFFFFFu;  // a last stage of one group is stored with zeros for the other
         } else {                          // packed weight block j: (blk = j / 2, group j % 2)
-            const int j = q - 8, blk = j >> 1, gg = j & 1;
+            const int j = q - NABLK, blk = j >> 1, gg = j & 1;
             gbase[i] = (const uint8_t *)a.wgt + (size_t)n0 * a.ld_wgt + gg * 32;
             goff[i] = (uint32_t)(min(n0 + blk * 32 + l32, a.N - 1) - n0) * (uint32_t)a.ld_wgt + half * 16;
             ldst[i] = W_OFF + (blk * 2 + gg) * BLK_BYTES;
@@ -252,6 +254,17 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
     const uint16_t *pA = (const uint16_t *)a.ascales + min(m0 + wm * 32 + l32, a.M - 1);
     const uint16_t *pW0 = (const uint16_t *)a.wscales + min(n0 + lane, a.N - 1);
     const uint16_t *pW1 = (const uint16_t *)a.wscales + min(n0 + 64 + lane, a.N - 1);
+    // ... and the 16 packed bytes of its activation row (row wm * 32 + l32, K half lane / 32) for both groups: exactly
+    // what the lane holds as MFMA operand after the unpack.
+    v4i araw[2];
+    const uint8_t *pAct = (const uint8_t *)a.act + (size_t)min(m0 + wm * 32 + l32, a.M - 1) * a.ld_act + half * 16;
+    auto load_act = [&](int s) {
+#pragma unroll
+        for (int gg = 0; gg < 2; gg++) {
+            const int gi = ODDG ? min(2 * s + gg, G - 1) : 2 * s + gg;  // a group past the end re-reads the last one (scales zero)
+            araw[gg] = *(const v4i *)(pAct + (size_t)gi * 32);
+        }
+    };
     auto load_scales8 = [&](int s) {
 #pragma unroll
         for (int gg = 0; gg < 2; gg++) {
@@ -339,10 +352,12 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
     const int offW = W_OFF + lane * 16;
     const int offA = wm * 2 * BLK_BYTES + lane * 16;
 
-    if constexpr (WPL)
+    if constexpr (WPL) {
         load_scales8(0);
-    else
+        load_act(0);
+    } else {
         load_scales(0);
+    }
 #pragma unroll
     for (int i = 0; i < PER_WAVE; i++) dma_one(0, sbuf0, i);
     // epilogue operands, fetched now so that the epilogue does not wait for memory
@@ -386,7 +401,18 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
         // scales of column lane and column 64 + lane, so the even weight blocks find theirs in lanes 0-31 and the odd ones
         // in lanes 32-63: sa[0] is zero in lanes 32-63, sa[1] in lanes 0-31.  Seven of the eight products are zero.
         v2i sa[2], sw[2][2];
+        v8i a8[2];  // fp8 path: the wavefront's activation operands of the stage's two groups
         if constexpr (WPL) {
+            // two's complement nibble -> value + 8 is a flip of the nibble's top bit; written per plane so that mask and
+            // flip are one three-input bit operation
+#pragma unroll
+            for (int gg = 0; gg < 2; gg++) {
+                typedef unsigned v4u __attribute__((ext_vector_type(4)));
+                const v4u u = __builtin_bit_cast(v4u, araw[gg]);
+                const unsigned flip = ACT_UNSIGNED ? 0u : 0x08080808u;
+                const v4u e = (u & 0x0F0F0F0Fu) ^ flip, o = ((u >> 4) & 0x0F0F0F0Fu) ^ flip;
+                a8[gg] = (v8i){(int)e[0], (int)e[1], (int)e[2], (int)e[3], (int)o[0], (int)o[1], (int)o[2], (int)o[3]};
+            }
             const int both = (int)((uint32_t)qa[0] | ((uint32_t)qa[1] << 16));
             sa[0] = (v2i){half ? 0 : both, 0};
             sa[1] = (v2i){half ? both : 0, 0};
@@ -404,10 +430,12 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
         // The other buffer was last read in the previous stage, before the barrier: refill it during this stage.  The last
         // stage re-fetches itself into the idle buffer (harmless, and keeps the stage one basic block).
         const int sn = min(s + 1, nstages - 1);
-        if constexpr (WPL)
+        if constexpr (WPL) {
             load_scales8(sn);
-        else
+            load_act(sn);
+        } else {
             load_scales(sn);
+        }
         if constexpr (WPL) {
             // One stage = eight (group, weight block) steps.  The two matrix instructions of step b + 1 (scale product and
             // group dot product) are issued ahead of the sixteen FMAs of step b.
@@ -417,27 +445,16 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
                 const v2i hi = *(const v2i *)(base + offW + (bn * WPL_BLOCKS + 2) * BLK_BYTES + gg * 8);
                 return (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], 0, 0};
             };
-            auto read_a8 = [&](int gg) -> v8i {
-                typedef unsigned v4u __attribute__((ext_vector_type(4)));
-                const v4u u = __builtin_bit_cast(v4u, *(const v4i *)(base + offA + gg * BLK_BYTES));
-                // two's complement nibble -> value + 8 is a flip of the nibble's top bit; written per plane so that mask
-                // and flip are one three-input bit operation
-                const unsigned flip = ACT_UNSIGNED ? 0u : 0x08080808u;
-                const v4u e = (u & 0x0F0F0F0Fu) ^ flip, o = ((u >> 4) & 0x0F0F0F0Fu) ^ flip;
-                return (v8i){(int)e[0], (int)e[1], (int)e[2], (int)e[3], (int)o[0], (int)o[1], (int)o[2], (int)o[3]};
-            };
             const v16f z16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
             // as[m] * ws[n] of step b, exact (two 16-bit values, one non-zero product): a 16-bit matrix instruction, which
             // runs beside the vector FMAs; the fp32 rank-1 matrix instruction shares the vector ALUs and does not
             auto scales = [&](int b) -> v16f { return mfma32_16bit_k8<T>(sa[b & 1], sw[b >> 2][(b >> 1) & 1], z16); };
-            v8i a8[2], w8[3];
+            v8i w8[3];
             v16f S[2], P[2];
-            a8[0] = read_a8(0);
             w8[0] = read_w8(0);
             w8[1] = read_w8(1);
             S[0] = scales(0);
             P[0] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8[0], w8[0], z16, 0, 2, 0, F8_SCALE, 0, F6_SCALE);
-            a8[1] = read_a8(1);
 #pragma unroll
             for (int b = 0; b < 8; b++) {
                 const int cur = b & 1, nxt = cur ^ 1;
