@@ -22,10 +22,12 @@
 //    instead of 32.  One v_mfma_scale_f32_32x32x64_f8f6f4 with block scales 2^9 and 2^3 gives the exact p_g of a
 //    whole group as fp32; as[g, m] * ws[g, n] of the block comes from a 16-bit matrix instruction
 //    on the scales themselves (exact: one non-zero product); one FMA per output and group is left for the VALU.
-//  * K is staged through LDS 128 at a time (two scale groups), two stages.  Operands go global -> LDS directly
-//    (global_load_lds_dwordx4, no registers), one stage ahead, into a lane-linear layout (LDS slot l of a 1 KB block =
-//    the 16 bytes MFMA lane l needs), so the operand reads are bank-conflict free by construction; one raw s_barrier
-//    per stage with explicit s_waitcnt.  A wavefront issues its block loads one per step of the stage.
+//  * K is staged through LDS 128 at a time (two scale groups), two stages.  Operands that several wavefronts read (the
+//    weights; with packed weights also the activations) go global -> LDS directly (global_load_lds_dwordx4, no
+//    registers), one stage ahead, into a lane-linear layout (LDS slot l of a 1 KB block = the 16 bytes MFMA lane l
+//    needs), so the operand reads are bank-conflict free by construction; one raw s_barrier per stage with explicit
+//    s_waitcnt.  A wavefront issues its block loads one per step of the stage.  In the fp8 loop a wavefront's own 32
+//    activation rows and its scales go to registers, one stage ahead.
 //  * The epilogue's operands (bias, the first 32 ranks of lora_up and lora_act of the tile: 24.25 KB) are fetched into
 //    LDS together with stage 0, in MFMA lane order, so that the LoRA-up section does not wait for memory; with them
 //    a workgroup holds 78.25 KB of LDS, two workgroups still share a CU's 160 KB.
