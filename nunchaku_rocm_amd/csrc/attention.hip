@@ -28,6 +28,8 @@
 //    half sit between the matrix instructions of the other (see the pipeline comment in the kernel).
 //  * Workgroups of one head run on one XCD (when the head count is a multiple of 8), so K and V of a head are
 //    fetched into one L2 only.
+#include <type_traits>
+
 #include "svdq_common.h"
 
 namespace svdq {
@@ -80,7 +82,12 @@ template <typename T, int D>
 __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a, int ntile, int xcd_heads) {
     using G = AtGeo<D>;
     constexpr int NC = G::NC, NDT = G::NDT, LOADS = G::LOADS;
-    __shared__ __align__(16) uint8_t smem[2 * G::STAGE];
+    // Two separate LDS objects, one per stage, and a main loop unrolled over them: the compiler then knows that a tile
+    // load into one stage cannot touch what is being read from the other.  With one object and a run-time stage offset
+    // it made every LDS read wait for all loads in flight, i.e. for the tile that was requested just before.
+    static_assert(AT_BQ == 128 && 64 * G::OPITCH <= G::STAGE, "the output tile is staged as two halves of 64 rows, one per stage");
+    __shared__ __align__(16) uint8_t smem0[G::STAGE];
+    __shared__ __align__(16) uint8_t smem1[G::STAGE];
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -129,13 +136,13 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a
         kvo[j] = (uint32_t)row * (uint32_t)(a.skn * 2) + (uint32_t)(((lane % G::KCH) ^ G::kswz(row)) * 16);
         vvo[j] = (uint32_t)row * (uint32_t)(a.svn * 2) + (uint32_t)(((lane % G::KCH) ^ G::vswz(row)) * 16);
     }
-    auto issue_k = [&](int blk, int stage, int j) {
+    auto issue_k = [&](int blk, uint8_t *stage, int j) {
         const uint32_t off = (uint32_t)blk * ktile;
-        at_load16_lds(at_buffer(kbase + off, kbytes - off), smem + stage * G::STAGE + (wave * G::LOADS + j) * 1024, kvo[j], 0);
+        at_load16_lds(at_buffer(kbase + off, kbytes - off), stage + (wave * G::LOADS + j) * 1024, kvo[j], 0);
     };
-    auto issue_v = [&](int blk, int stage, int j) {
+    auto issue_v = [&](int blk, uint8_t *stage, int j) {
         const uint32_t off = (uint32_t)blk * vtile;
-        at_load16_lds(at_buffer(vbase + off, vbytes - off), smem + stage * G::STAGE + G::KT_BYTES + (wave * G::LOADS + j) * 1024, vvo[j], 0);
+        at_load16_lds(at_buffer(vbase + off, vbytes - off), stage + G::KT_BYTES + (wave * G::LOADS + j) * 1024, vvo[j], 0);
     };
 
     // operand read offsets.  K rows 32 t + l32 (chunk 2 c + half).  V^T operand of d tile dt and 16-key chunk c: lane
@@ -182,23 +189,23 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a
     //                                                     the stage tile t has left
     // The compiler is kept from regrouping the slots (one matrix instruction plus its share of the rest).
 #pragma unroll
-    for (int j = 0; j < LOADS; j++) issue_k(0, 0, j);
+    for (int j = 0; j < LOADS; j++) issue_k(0, smem0, j);
 #pragma unroll
-    for (int j = 0; j < LOADS; j++) issue_v(0, 0, j);
+    for (int j = 0; j < LOADS; j++) issue_v(0, smem0, j);
     {
         const int t1 = min(1, nblk - 1);
 #pragma unroll
-        for (int j = 0; j < LOADS; j++) issue_k(t1, 1, j);
+        for (int j = 0; j < LOADS; j++) issue_k(t1, smem1, j);
 #pragma unroll
-        for (int j = 0; j < LOADS; j++) issue_v(t1, 1, j);
+        for (int j = 0; j < LOADS; j++) issue_v(t1, smem1, j);
     }
     __builtin_amdgcn_s_waitcnt(waitcnt_imm(2 * LOADS, 15));  // tile 0 (the older half of the loads)
     __builtin_amdgcn_s_barrier();
     v4i rk[2 * NC], rv[4 * NDT];  // rk[NC t + c]: K rows 32 t.., chunk c;  rv[4 dt + c]: V^T rows 32 dt.., 16-key chunk c
 #pragma unroll
     for (int c = 0; c < NC; c++) {
-        rk[c] = *(const v4i *)(smem + koff[c]);
-        rk[NC + c] = *(const v4i *)(smem + 32 * G::KROW + koff[c]);
+        rk[c] = *(const v4i *)(smem0 + koff[c]);
+        rk[NC + c] = *(const v4i *)(smem0 + 32 * G::KROW + koff[c]);
     }
 
     float shift, alpha, rs;  // rs: this half's row sum, at the new reference
@@ -247,9 +254,10 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a
         shift16(cinit);
     };
 
-    for (int blk = 0; blk < nblk; blk++) {
-        const uint8_t *st = smem + (blk & 1) * G::STAGE;
-        const uint8_t *sn = smem + ((blk + 1) & 1) * G::STAGE;
+    auto tile = [&](auto par_tag, int blk) {  // tile blk, which lives in stage par_tag
+        constexpr int PAR = decltype(par_tag)::value;
+        uint8_t *st = PAR ? smem1 : smem0;
+        const uint8_t *sn = PAR ? smem0 : smem1;
         const int nxt = min(blk + 2, nblk - 1);  // past the end: the last tile again, into a stage nobody reads
         const bool ragged = blk == nblk - 1 && (a.Tkv & (AT_BK - 1));
         v16f s0, s1;
@@ -323,9 +331,17 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a
             acc_o[c % NDT] = mfma32_16bit<T>(rv[4 * (c % NDT) + 2 + c / NDT], pop[2 + c / NDT], acc_o[c % NDT]);
             rk[2 * c] = *(const v4i *)(sn + ((2 * c) / NC) * (32 * G::KROW) + koff[(2 * c) % NC]);
             rk[2 * c + 1] = *(const v4i *)(sn + ((2 * c + 1) / NC) * (32 * G::KROW) + koff[(2 * c + 1) % NC]);
-            if (c & 1) issue_k(nxt, blk & 1, c >> 1); else issue_v(nxt, blk & 1, c >> 1);
+            if (c & 1) issue_k(nxt, st, c >> 1); else issue_v(nxt, st, c >> 1);
             __builtin_amdgcn_sched_barrier(0);
         }
+    };
+    {
+        int blk = 0;
+        for (; blk + 1 < nblk; blk += 2) {
+            tile(std::integral_constant<int, 0>{}, blk);
+            tile(std::integral_constant<int, 1>{}, blk + 1);
+        }
+        if (blk < nblk) tile(std::integral_constant<int, 0>{}, blk);
     }
 
     // ---- O = O^T / l, staged through LDS so that rows leave as 256-byte segments -------------------------------------
@@ -340,7 +356,7 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a
             uint2 w;
             w.x = pack2<T>(acc_o[dt][4 * j] * inv, acc_o[dt][4 * j + 1] * inv);
             w.y = pack2<T>(acc_o[dt][4 * j + 2] * inv, acc_o[dt][4 * j + 3] * inv);
-            *(uint2 *)(smem + (wave * 32 + l32) * G::OPITCH + (32 * dt + 8 * j + 4 * half) * 2) = w;
+            *(uint2 *)((wave < 2 ? smem0 : smem1) + ((wave & 1) * 32 + l32) * G::OPITCH + (32 * dt + 8 * j + 4 * half) * 2) = w;
         }
     __syncthreads();
     uint16_t *op = (uint16_t *)a.o + (long)b * a.sob + (long)h * D;
@@ -349,7 +365,7 @@ __global__ __launch_bounds__(256, 2) void attention_kernel(svdq_attention_args a
 #pragma unroll
     for (int pass = 0; pass < AT_BQ / OROWS; pass++) {
         const int row = pass * OROWS + tid / OCH, q = q0 + row;
-        if (q < a.Tq) *(v4i *)(op + (long)q * a.som + 8 * c) = *(const v4i *)(smem + row * G::OPITCH + c * 16);
+        if (q < a.Tq) *(v4i *)(op + (long)q * a.som + 8 * c) = *(const v4i *)((row < 64 ? smem0 : smem1) + (row & 63) * G::OPITCH + c * 16);
     }
 }
 
