@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define SVDQ_ABI_VERSION 5
+#define SVDQ_ABI_VERSION 6
 
 enum { SVDQ_BF16 = 0, SVDQ_FP16 = 1 };
 enum { SVDQ_PRE_NONE = 0, SVDQ_PRE_GLU = 1, SVDQ_PRE_GELU = 2 }; /* svdq_quantize_args.prologue */

@@ -14,7 +14,7 @@ import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libsvdq_mi355x.so")
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 BF16, FP16 = 0, 1
 EPI_PLAIN, EPI_QK_NORM_ROPE, EPI_GELU_QUANT, EPI_SWIGLU_QUANT = 0, 1, 2, 3
