@@ -110,6 +110,20 @@ __device__ inline void f6_pack(const v4i lo16, const v4i hi16, int odd, uint32_t
     }
 }
 
+// Register loads of the fp8 loop go through raw buffers: address = descriptor base + scalar offset (the group or stage)
+// + 32-bit lane offset, so no vector instruction computes an address.  The range covers everything (offsets are clamped
+// where rows or columns run out).
+typedef unsigned int g_v4u __attribute__((ext_vector_type(4)));
+__device__ inline __amdgpu_buffer_rsrc_t g_buffer(const void *base) {
+    return __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, (int)0xFFFFFFFFu, 0x00020000);  // raw buffer, 32-bit data format
+}
+__device__ inline uint16_t g_load16(__amdgpu_buffer_rsrc_t r, uint32_t lane_off, uint32_t uniform_off) {
+    return __builtin_amdgcn_raw_buffer_load_b16(r, (int)lane_off, (int)uniform_off, 0);
+}
+__device__ inline v4i g_load128(__amdgpu_buffer_rsrc_t r, uint32_t lane_off, uint32_t uniform_off) {
+    return __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(r, (int)lane_off, (int)uniform_off, 0));
+}
+
 __device__ inline v16i magic_acc() {
     v16i c;
 #pragma unroll
@@ -253,26 +267,28 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
     // straight into registers: the activation scale of row wm * 32 + l32 and the weight scales of columns lane and
     // 64 + lane, for both groups of the stage.  Groups past the end (odd K / 64) are staged as zero.
     uint16_t qa[2], qw[4];
-    const uint16_t *pA = (const uint16_t *)a.ascales + min(m0 + wm * 32 + l32, a.M - 1);
-    const uint16_t *pW0 = (const uint16_t *)a.wscales + min(n0 + lane, a.N - 1);
-    const uint16_t *pW1 = (const uint16_t *)a.wscales + min(n0 + 64 + lane, a.N - 1);
+    const __amdgpu_buffer_rsrc_t rAS = g_buffer(a.ascales), rWS = g_buffer(a.wscales);
+    const uint32_t oA = 2u * (uint32_t)min(m0 + wm * 32 + l32, a.M - 1);
+    const uint32_t oW0 = 2u * (uint32_t)min(n0 + lane, a.N - 1), oW1 = 2u * (uint32_t)min(n0 + 64 + lane, a.N - 1);
     // ... and the 16 packed bytes of its activation row (row wm * 32 + l32, K half lane / 32) for both groups: exactly
     // what the lane holds as MFMA operand after the unpack.
     v4i araw[2];
-    const uint8_t *pAct = (const uint8_t *)a.act + (size_t)min(m0 + wm * 32 + l32, a.M - 1) * a.ld_act + half * 16;
+    const __amdgpu_buffer_rsrc_t rAct = g_buffer((const uint8_t *)a.act + (size_t)m0 * a.ld_act);
+    const uint32_t oAct = (uint32_t)(min(m0 + wm * 32 + l32, a.M - 1) - m0) * (uint32_t)a.ld_act + half * 16;
     auto load_act = [&](int s) {
 #pragma unroll
         for (int gg = 0; gg < 2; gg++) {
             const int gi = ODDG ? min(2 * s + gg, G - 1) : 2 * s + gg;  // a group past the end re-reads the last one (scales zero)
-            araw[gg] = *(const v4i *)(pAct + (size_t)gi * 32);
+            araw[gg] = g_load128(rAct, oAct, (uint32_t)gi * 32);
         }
     };
     auto load_scales8 = [&](int s) {
 #pragma unroll
         for (int gg = 0; gg < 2; gg++) {
             const int gi = ODDG ? min(2 * s + gg, G - 1) : 2 * s + gg;
-            const uint16_t va = pA[(size_t)gi * a.ld_ascales];
-            const uint16_t v0 = pW0[(size_t)gi * a.ld_wscales], v1 = pW1[(size_t)gi * a.ld_wscales];
+            const uint32_t ga = (uint32_t)gi * (uint32_t)a.ld_ascales * 2u, gw = (uint32_t)gi * (uint32_t)a.ld_wscales * 2u;  // uniform
+            const uint16_t va = g_load16(rAS, oA, ga);
+            const uint16_t v0 = g_load16(rWS, oW0, gw), v1 = g_load16(rWS, oW1, gw);
             const bool on = !ODDG || 2 * s + gg < G;
             qa[gg] = on ? va : (uint16_t)0;
             qw[2 * gg] = on ? v0 : (uint16_t)0;
