@@ -1203,6 +1203,15 @@ static int gemm_w4a4_checked(const svdq_gemm_args &a, void *stream) {
         set_error("svdq_gemm_w4a4: scale rows shorter than M / N");
         return SVDQ_E_INVALID;
     }
+    {   // the kernel addresses operands with 32-bit offsets from a tile's base
+        const size_t lim = (size_t)1 << 32, G = (size_t)(a.K / GROUP);
+        if (G * a.ld_ascales * 2 >= lim || G * a.ld_wscales * 2 >= lim || (size_t)(BM + 1) * a.ld_act >= lim ||
+            (size_t)(BN + 1) * a.ld_wgt >= lim) {
+            set_error("svdq_gemm_w4a4: K=%d with row strides %d / %d / %d / %d: operands too large for 32-bit offsets", a.K,
+                      a.ld_act, a.ld_wgt, a.ld_ascales, a.ld_wscales);
+            return SVDQ_E_UNSUPPORTED;
+        }
+    }
     if (a.R < 0 || a.R % 16 || (a.R > 0 && (!a.lora_act || !a.lora_up))) {
         set_error("svdq_gemm_w4a4: R=%d must be a multiple of 16 with lora_act and lora_up given", a.R);
         return SVDQ_E_INVALID;
