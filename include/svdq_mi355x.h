@@ -109,7 +109,7 @@ int svdq_transpose_lora_down(const void *lora_down, void *lora_down_t, int32_t K
 
 /*
  * W4A4 GEMM: out[m, n] = sum_g as[g, m] * ws[g, n] * (sum_{k in g} a[m, k] w[n, k])  (exact integer per group: int8 MFMA
- *                        on packed weights, fp8 MFMA on int4-valued codes with pre-split weights)
+ *                        on packed weights, fp8 x fp6 MFMA on int4-valued codes with pre-split weights)
  *                        + T(lora_act[m, :]) . lora_up[n, :] + bias[n],  then the epilogue.
  * Reference arithmetic: ops/triton/gemm_w4a4.py:447-488 (main loop), 156-209 (epilogue), 499-521 (QK), 730-778
  * (GELU + requantization), 998-1000 (SwiGLU semantics).
@@ -187,7 +187,7 @@ size_t svdq_gemm_w4a4_static_scratch_capacity(void);
 /*
  * Debug: exact int32 accumulators of one scale group, p[m, n] = sum_{k in group g} a[m, k] * w[n, k], computed by
  * the instruction sequence of one of the GEMM's two main loops: path 0 = nibble unpack + v_mfma_i32_32x32x32_i8 (packed
- * weights), path 1 = fp8 codes + v_mfma_scale_f32_32x32x64_f8f6f4 with the +8 offset of signed activations taken out
+ * weights), path 1 = fp8 / fp6 codes + v_mfma_scale_f32_32x32x64_f8f6f4 with the +8 offset of signed activations taken out
  * (pre-split weights).  out (M, N) int32 row-major.
  */
 int svdq_group_acc_i32(const void *act, const void *wgt, int32_t *out, int32_t M, int32_t N, int32_t K,
