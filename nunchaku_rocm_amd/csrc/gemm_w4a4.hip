@@ -4,37 +4,44 @@
 //   out[m, n] = sum_g as[g, m] * ws[g, n] * p_g[m, n]  +  T(lora_act[m, :]) . lora_up[n, :]  +  bias[n]
 // with p_g the exact int32 dot product of the group's 64 int4 pairs.
 //
-// How it maps to CDNA4:
-//  * 256 threads = four wavefronts, each 32 activation rows x all 128 weight rows of a 128x128 tile; two workgroups per
-//    CU = two wavefronts per SIMD.  The MFMA's A operand is the activation tile and its B operand the weight tile, so
-//    in the main loop a lane owns one weight row n and its registers walk the wavefront's 32 activation rows.
-//  * Packed weights (int8 loop): a 16-byte LDS read holds 32 nibbles; the even and the odd nibbles are split into two
-//    int8 planes with shift/mask only (signed values land in the high nibble of each byte, i.e. times 16; unsigned
-//    activations in the low nibble, times 1).  Both operands use the same split, so the K order inside a group is a
-//    shared permutation and the dot product is unchanged; the power-of-two factor is folded exactly into the weight
-//    scale.  p_g comes from two v_mfma_i32_32x32x32_i8 whose accumulator starts at the bit pattern of 1.5*2^23, so
-//    the int32 result read as fp32 is (1.5*2^23 + p) exactly and  fma(bits, ws', -1.5*2^23*ws')  gives p*ws' with one
+// Two kernels share one epilogue.  In both, 256 threads = four wavefronts, each 32 activation rows x all 128 weight rows
+// of a 128x128 tile; the MFMA's A operand is the activation tile and its B operand the weight tile, so in the main loop a
+// lane owns one weight row n and its registers walk the wavefront's 32 activation rows.  K is staged through LDS 128 at
+// a time (two scale groups), two stages; operands that several wavefronts read go global -> LDS directly
+// (global_load_lds, no registers), one stage ahead, into a lane-linear layout (LDS slot l of a 1 KB block = the 16 bytes
+// MFMA lane l needs), so the operand reads are bank-conflict free by construction; one raw s_barrier per stage with
+// explicit s_waitcnt.
+//
+//  * gemm_w4a4_f8_kernel (pre-split weights, svdq_split_weight_planes; the default for module weights): an activation
+//    is carried as the fp8 (e4m3) code of value * 2^-9, a weight as the fp6 (e2m3) code of value / 8, 24 bytes per lane
+//    and group.  One v_mfma_scale_f32_32x32x64_f8f6f4 with block scales 2^9 and 2^3 gives the exact p_g of a whole
+//    group as fp32; as[g, m] * ws[g, n] of the block comes from a 16-bit matrix instruction on the scales themselves
+//    (exact: one non-zero product); one FMA per output and group is left for the VALU.  Signed activations become
+//    sign | magnitude codes by one bit operation per plane: even k carry a + 8, odd k carry a - 7, so that the offset
+//    term 8 * (sum of even weights) - 7 * (sum of odd weights) has no systematic part whatever the mean of the
+//    weight codes; it is taken out again every four stages with a 16-bit matrix instruction on (as, -ws * offset),
+//    whose operands travel with the weights.  Only the weights go through LDS (with their scales and offset terms);
+//    a wavefront's own 32 activation rows and activation scales go to registers, one stage ahead.  The kernel is held
+//    to 168 vector registers and 50.25 KB of LDS so that three workgroups share a CU (three wavefronts per SIMD): a
+//    wavefront issues scale product, group product and the sixteen FMAs of a step in program order (single result
+//    buffers) and the other two wavefronts of the SIMD fill the matrix pipe and the vector ALU meanwhile.
+//  * gemm_w4a4_i8_kernel (packed weights): a 16-byte LDS read holds 32 nibbles; the even and the odd nibbles are split
+//    into two int8 planes with shift/mask only (signed values land in the high nibble of each byte, i.e. times 16;
+//    unsigned activations in the low nibble, times 1).  Both operands use the same split, so the K order inside a group
+//    is a shared permutation and the dot product is unchanged; the power-of-two factor is folded exactly into the weight
+//    scale.  p_g comes from two v_mfma_i32_32x32x32_i8 whose accumulator starts at the bit pattern of 1.5*2^23, so the
+//    int32 result read as fp32 is (1.5*2^23 + p) exactly and  fma(bits, ws', -1.5*2^23*ws')  gives p*ws' with one
 //    rounding and no int->float convert; a second fma applies as[g, m] and accumulates: two VALU ops per output and
-//    group.
-//  * Pre-split weights (fp8 loop, svdq_split_weight_planes): an activation is carried as the fp8 (e4m3) code of
-//    value * 2^-9, a signed one as value + 8 (one three-input bit operation per plane; the offset is taken out after
-//    the loop with the weights' group sums); a weight as the fp6 (e2m3) code of value / 8, 24 bytes per lane and group
-//    instead of 32.  One v_mfma_scale_f32_32x32x64_f8f6f4 with block scales 2^9 and 2^3 gives the exact p_g of a
-//    whole group as fp32; as[g, m] * ws[g, n] of the block comes from a 16-bit matrix instruction
-//    on the scales themselves (exact: one non-zero product); one FMA per output and group is left for the VALU.
-//  * K is staged through LDS 128 at a time (two scale groups), two stages.  Operands that several wavefronts read (the
-//    weights; with packed weights also the activations) go global -> LDS directly (global_load_lds_dwordx4, no
-//    registers), one stage ahead, into a lane-linear layout (LDS slot l of a 1 KB block = the 16 bytes MFMA lane l
-//    needs), so the operand reads are bank-conflict free by construction; one raw s_barrier per stage with explicit
-//    s_waitcnt.  A wavefront issues its block loads one per step of the stage.  In the fp8 loop a wavefront's own 32
-//    activation rows and its scales go to registers, one stage ahead.
-//  * The epilogue's operands (bias, the first 32 ranks of lora_up and lora_act of the tile: 24.25 KB) are fetched into
-//    LDS together with stage 0, in MFMA lane order, so that the LoRA-up section does not wait for memory; with them
-//    a workgroup holds 78.25 KB of LDS, two workgroups still share a CU's 160 KB.
+//    group.  Needs no copy of the weight.
+//
+//  * The bias and the first 32 ranks of lora_up of the tile are fetched into LDS together with stage 0, in MFMA lane
+//    order, so that the LoRA-up section does not wait for them.
 //  * After LoRA-up and bias each wavefront turns its four 32x32 blocks through a private LDS tile into "lane =
 //    activation row": row-wise epilogue work (RMSNorm sum of squares, RoPE pairs, group absmax, nibble packing, the
 //    next layer's LoRA-down operand) is then in-lane plus one exchange with lane ^ 32.
-//  * The 16-bit output tile leaves through LDS as 256-byte row segments, stored non-temporally.
+//  * The 16-bit output leaves through a wavefront-private, XOR-swizzled LDS tile as 256-byte row segments, stored
+//    non-temporally.  Everything after the main loop is private to a wavefront: one barrier follows the loop, none
+//    after it.
 //  * Workgroup ids are first regrouped so that each XCD (ids are dealt round-robin over 8 XCDs) works on a
 //    contiguous range of tiles, then swizzled in bands of m-tiles for L2 reuse of the weight tile.
 #include <atomic>
@@ -46,36 +53,57 @@ namespace svdq {
 
 constexpr int BM = 128, BN = 128;     // workgroup tile (activation rows x weight rows)
 constexpr int KSTAGE = 128;           // K per LDS stage = two scale groups
-constexpr int NSTAGE = 2;             // LDS stages: one being computed on, one being filled
 constexpr int BLK_BYTES = 64 * 16;    // one MFMA operand block (32 rows x 16 bytes per lane) of one group, lane-linear
-// stage layout: activation blocks [4 blocks of 32 rows][2 groups] packed (1 KB each), weight blocks
-// [4 blocks][group 0 low, group 1 low, both high] (pre-split weights) or [4 blocks][2 groups] (packed), then the scales
-constexpr int W_OFF = 4 * 2 * BLK_BYTES;                  // 8192
-constexpr int AS_OFF = W_OFF + 4 * 2 * 2 * BLK_BYTES;     // 24576: float as[2][BM]
-constexpr int WS_OFF = AS_OFF + 2 * BM * 4;               // 25600: float2 (ws', -magic * ws')[2][BN]
-constexpr int BUF_BYTES = WS_OFF + 2 * BN * 8;            // 27648
-constexpr int SMEM_BYTES = NSTAGE * BUF_BYTES;            // 55296
-// the first 32 ranks of the tile's LoRA operands, fetched next to stage 0: lora_up [2 c][4 blocks] and lora_act
-// [2 c][4 blocks][2 halves of 8 floats] 1 KB blocks in MFMA lane order
-constexpr int LORA_BYTES = (8 + 16) * BLK_BYTES;          // 24576
-constexpr int BIAS_BYTES = BN * 2;                        // the tile's 128 bias values
 constexpr int NWAVES = 4, NTHREADS = NWAVES * 64;  // one wavefront per 32 activation rows
 constexpr int NBN = BN / 32;                        // 32-row weight blocks per wavefront: it owns 32 x 128 outputs
+// the first 32 ranks of the tile's lora_up, fetched next to stage 0: [2 c][4 blocks] 1 KB blocks in MFMA lane order,
+// then the tile's 128 bias values
+constexpr int LORA_UP_BYTES = 8 * BLK_BYTES;
+constexpr int EPI_LDS_BYTES = LORA_UP_BYTES + BN * 2;
 constexpr int TP_PITCH = 36;                        // floats per row of the accumulator transposition tile
-constexpr int TP_WAVE_BYTES = 2 * 32 * TP_PITCH * 4;  // two 32x32 blocks at a time
-static_assert(2 * TP_WAVE_BYTES <= BUF_BYTES, "transposition tiles do not fit");
+constexpr int PRIV_BYTES = 32 * BN * 2;             // a wavefront's private epilogue memory: its 32 output rows of 256 bytes
+static_assert(32 * TP_PITCH * 4 <= PRIV_BYTES, "the transposition tile of one block does not fit");
+constexpr int GROUP_M_TILES = 8;      // m-tiles per raster band
+constexpr int NUM_XCD = 8;
+
+// ---- int8 kernel: stage layout: activation blocks [4 blocks of 32 rows][2 groups] packed (1 KB each), weight blocks
+// [4 blocks][2 groups], then the scales
+constexpr int I8_W_OFF = 4 * 2 * BLK_BYTES;                  // 8192
+constexpr int I8_AS_OFF = I8_W_OFF + 4 * 2 * BLK_BYTES;      // 16384: float as[2][BM]
+constexpr int I8_WS_OFF = I8_AS_OFF + 2 * BM * 4;            // 17408: float2 (ws', -magic * ws')[2][BN]
+constexpr int I8_BUF_BYTES = I8_WS_OFF + 2 * BN * 8;         // 19456
+static_assert(2 * PRIV_BYTES <= I8_BUF_BYTES, "two wavefronts' private epilogue memory must fit one staging buffer");
+
+// ---- fp8 kernel
 constexpr int F8_SCALE = (int)0x88888888;  // e8m0 block scale 2^9 in every byte: an fp8 code c (value c * 2^-9) counts as c
 constexpr int F6_SCALE = (int)0x82828282;  // e8m0 block scale 2^3: an fp6 (e2m3) code c <= 15 (value c / 8) counts as c
 // Pre-split weights, per (block of 32 rows, stage of two groups): three 1 KB blocks in MFMA lane order.  A lane's 32
 // weights of a group are 32 six-bit codes = six registers: blocks 0 and 1 hold registers 0-3 of the stage's first and
 // second group (16 bytes per lane), block 2 registers 4-5 of both (8 + 8 bytes per lane).
 constexpr int WPL_BLOCKS = 3;
-constexpr int CORR_PER_WAVE = 6;       // staged group-sum blocks fetched per wavefront
-constexpr int NPIECE = 2;              // 16-bit pieces per group sum behind the weight planes (hi + lo: 16 / 22 significant bits)
-constexpr int CORR_LDS_G = 48;         // groups whose sums one staging buffer holds for the offset correction (24 blocks of 1 KB)
-constexpr int GROUP_M_TILES = 8;      // m-tiles per raster band
-constexpr int NUM_XCD = 8;
+constexpr int F8_STAGE_BYTES = NBN * WPL_BLOCKS * BLK_BYTES;  // 12288
+// ... and, per (block of 32 rows, stage), 32 rows of six 16-bit values: the two pieces (hi + lo) of
+// D = -ws * (8 * sum of the group's even weights - 7 * sum of its odd weights) for the stage's two groups, then the two
+// weight scales.  A 12-byte-per-lane global -> LDS load puts lane l's bytes at 16 l, so in LDS a row takes 16 bytes; they
+// sit in a ring of eight stages per block; one load brings a stage and the one after it (64 lanes = two stages' rows), so
+// a ninth slot takes what runs past slot 7.
+constexpr int AUX_ROW = 12;                                  // bytes per row and stage in memory
+constexpr int AUX_BLK = 32 * AUX_ROW;                        // 384
+constexpr int AUX_LROW = 16;                                 // ... and in LDS
+constexpr int AUX_LBLK = 32 * AUX_LROW;                      // 512
+constexpr int AUX_SLOTS = 8;
+constexpr int AUX_NBLK_BYTES = (AUX_SLOTS + 1) * AUX_LBLK;   // 4608
+constexpr int F8_RING_BYTES = NBN * AUX_NBLK_BYTES;          // 18432: after the loop two wavefronts' private memory
+static_assert(2 * PRIV_BYTES <= F8_RING_BYTES, "two wavefronts' private epilogue memory must fit the ring");
+static_assert(PRIV_BYTES <= F8_STAGE_BYTES, "a wavefront's private epilogue memory must fit a staging buffer");
+constexpr int PLANES_STATUS_BYTES = 16;  // trailing status word of a pre-split weight
 
+__host__ __device__ inline size_t planes_code_bytes(int N, int K) {
+    return (size_t)((N + 31) / 32) * (size_t)((K / GROUP + 1) / 2) * (WPL_BLOCKS * BLK_BYTES);
+}
+__host__ __device__ inline size_t planes_aux_bytes(int N, int K) {  // one stage of padding per block of rows
+    return (size_t)((N + 31) / 32) * (size_t)((K / GROUP + 1) / 2 + 1) * AUX_BLK;
+}
 
 __device__ inline void unpack_signed(v4i p, v4i &even, v4i &odd) {
     even = (p << 4) & (int)0xF0F0F0F0;  // 16 * value in each byte
@@ -88,9 +116,6 @@ __device__ inline void unpack_unsigned(v4i p, v4i &even, v4i &odd) {
     odd = __builtin_bit_cast(v4i, (u >> 4) & 0x0F0F0F0Fu);
 }
 
-// fp8 (e4m3) code of a signed int4 value: sign bit | magnitude in the low four bits.  A code c <= 15 stands for
-// c * 2^-9 (subnormals and the first binade form one linear run).
-__device__ inline uint32_t f8_code(int v) { return (uint32_t)((v < 0 ? 0x80 : 0) | (v < 0 ? -v : v)); }
 // fp6 (e2m3) code of a signed int4 value: sign bit | magnitude in the low four bits; a code c <= 15 stands for c / 8.
 __device__ inline uint32_t f6_code(int v) { return (uint32_t)((v < 0 ? 0x20 : 0) | (v < 0 ? -v : v)); }
 // The six registers of a lane's fp6 operand: 32 six-bit codes, code p in bits 6 p .. 6 p + 5.  The matrix instruction
@@ -109,11 +134,27 @@ __device__ inline void f6_pack(const v4i lo16, const v4i hi16, int odd, uint32_t
         if ((bit & 31) > 26) d[(bit >> 5) + 1] |= c >> (32 - (bit & 31));
     }
 }
+// 8 * (sum of the even-k weights) - 7 * (sum of the odd-k weights) of one group (32 packed bytes): what the fp8 path's
+// offset activation codes (a + 8 for even k, a - 7 for odd k) add to the group's dot product.
+__device__ inline int group_offset_term(const v4i lo16, const v4i hi16) {
+    int we = 0, wo = 0;
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        const v4i p = h ? hi16 : lo16;
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+#pragma unroll
+            for (int j = 0; j < 8; j += 2) {
+                we += (((p[e] >> (4 * j)) & 0xF) ^ 8) - 8;
+                wo += (((p[e] >> (4 * j + 4)) & 0xF) ^ 8) - 8;
+            }
+    }
+    return 8 * we - 7 * wo;
+}
 
 // Register loads of the fp8 loop go through raw buffers: address = descriptor base + scalar offset (the group or stage)
 // + 32-bit lane offset, so no vector instruction computes an address.  The range covers everything (offsets are clamped
 // where rows or columns run out).
-typedef unsigned int g_v4u __attribute__((ext_vector_type(4)));
 __device__ inline __amdgpu_buffer_rsrc_t g_buffer(const void *base) {
     return __builtin_amdgcn_make_buffer_rsrc((void *)base, 0, (int)0xFFFFFFFFu, 0x00020000);  // raw buffer, 32-bit data format
 }
@@ -146,456 +187,41 @@ __device__ inline void tile_ids(int tiles_m, int tiles_n, int &pid_m, int &pid_n
     pid_n = (id % band) / gm;
 }
 
-template <typename T, bool ACT_UNSIGNED, int EPI, bool WPL, bool ODDG>  // ODDG: K / 64 is odd
-__global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a) {
-    // Three separate LDS objects: the compiler then knows that a block load into one staging buffer cannot touch what
-    // is being read from the other (one object would make every LDS read wait for the loads in flight).
-    __shared__ __align__(16) uint8_t sbuf0[BUF_BYTES];
-    __shared__ __align__(16) uint8_t sbuf1[BUF_BYTES];
-    __shared__ __align__(16) uint8_t sepi[LORA_BYTES + BIAS_BYTES];
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wm = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: the wavefront's 32-row block of the tile
+// Epilogue operands every wavefront of the tile needs, fetched global -> LDS next to stage 0: the tile's 128 bias
+// values and the first 32 ranks of lora_up.
+__device__ inline void fetch_epilogue_operands(const svdq_gemm_args &a, uint8_t *sepi, int n0, int wm, int lane) {
     const int l32 = lane & 31, half = lane >> 5;
-
-    int pid_m, pid_n;
-    tile_ids((a.M + BM - 1) / BM, (a.N + BN - 1) / BN, pid_m, pid_n);
-    const int m0 = pid_m * BM, n0 = pid_n * BN;
-
-    // ---- operand staging: global -> LDS directly (global_load_lds_dwordx4), one stage ahead ----------------------
-    // A stage holds 1 KB operand blocks (operand, 32-row block, group[, plane]).  Lane l of a block load fetches the
-    // 16 bytes MFMA lane l will read and the hardware writes them to LDS slot l of the block: the layout the operand
-    // read wants, free of bank conflicts by construction.  Packed operands: lane l = (row l % 32, half l / 32) of a
-    // row-major tile.  Pre-split weights are already stored block by block in that order (1 KB contiguous per load).
-    // Packed weights: the 8 activation + 8 weight block loads of a stage are dealt in runs to the four wavefronts.
-    // Pre-split weights: only the 12 weight blocks go through LDS; a wavefront's 32 activation rows are read by nobody
-    // else, so it fetches them straight into registers (see load_act below).
-    constexpr int NLOADS = WPL ? 4 * WPL_BLOCKS : 16, PER_WAVE = NLOADS / NWAVES, NABLK = WPL ? 0 : 8;
-    // each load's address = wave-uniform base (SGPRs) + a 32-bit offset (lane part + stage * step; operands < 4 GiB)
-    const uint8_t *gbase[PER_WAVE];
-    uint32_t goff[PER_WAVE];
-    int ldst[PER_WAVE], gstep[PER_WAVE];
-    uint32_t gcap[PER_WAVE];
-    const int G = a.K / GROUP;
-    // K / 64 odd: the last stage has one group only.  The loads of its second group stop one stage earlier (they re-read
-    // valid memory) and its scales are staged as zero, so it adds nothing.  A load's stage offset is min(s * step, cap).
-    auto cap_of = [&](int gg, int step, const uint8_t *&base, int back) -> uint32_t {
-        if (gg == 0) return (uint32_t)(G / 2) * (uint32_t)step;  // G is odd: stages 0 .. G / 2
-        if (G == 1) {  // no earlier stage: read the first group's bytes instead
-            base -= back;
-            return 0u;
-        }
-        return (uint32_t)(G / 2 - 1) * (uint32_t)step;
-    };
-#pragma unroll
-    for (int i = 0; i < PER_WAVE; i++) {
-        const int q = wm * PER_WAVE + i;  // wave-uniform
-        if (q < NABLK) {                  // activation block q: (blk = q / 2, group q % 2)
-            const int blk = q >> 1, gg = q & 1;
-            gbase[i] = (const uint8_t *)a.act + (size_t)m0 * a.ld_act + gg * 32;
-            goff[i] = (uint32_t)(min(m0 + blk * 32 + l32, a.M - 1) - m0) * (uint32_t)a.ld_act + half * 16;
-            ldst[i] = (blk * 2 + gg) * BLK_BYTES;
-            gstep[i] = KSTAGE / 2;
-            if constexpr (ODDG) gcap[i] = cap_of(gg, gstep[i], gbase[i], 32);
-        } else if (WPL) {                 // pre-split weight block j: (blk = j / 3, part j % 3)
-            const int j = q, blk = j / WPL_BLOCKS, part = j % WPL_BLOCKS;
-            const int nblk = min(n0 / 32 + blk, (a.N + 31) / 32 - 1);
-            gbase[i] = (const uint8_t *)a.wgt_planes + ((size_t)nblk * ((G + 1) / 2) * WPL_BLOCKS + part) * BLK_BYTES;
-            goff[i] = lane * 16;
-            ldst[i] = W_OFF + (blk * WPL_BLOCKS + part) * BLK_BYTES;
-            gstep[i] = WPL_BLOCKS * BLK_BYTES;
-            if constexpr (ODDG) gcap[i] = 0xFFFFFFFFu;  // a last stage of one group is stored with zeros for the other
-        } else {                          // packed weight block j: (blk = j / 2, group j % 2)
-            const int j = q - NABLK, blk = j >> 1, gg = j & 1;
-            gbase[i] = (const uint8_t *)a.wgt + (size_t)n0 * a.ld_wgt + gg * 32;
-            goff[i] = (uint32_t)(min(n0 + blk * 32 + l32, a.N - 1) - n0) * (uint32_t)a.ld_wgt + half * 16;
-            ldst[i] = W_OFF + (blk * 2 + gg) * BLK_BYTES;
-            gstep[i] = KSTAGE / 2;
-            if constexpr (ODDG) gcap[i] = cap_of(gg, gstep[i], gbase[i], 32);
-        }
-    }
-    auto dma_one = [&](int s, uint8_t *dstbuf, int i) {  // block load i of stage s into a staging buffer
-        const uint8_t *src;
-        if constexpr (ODDG)
-            src = gbase[i] + (goff[i] + min((uint32_t)s * (uint32_t)gstep[i], gcap[i]));  // stage part wave-uniform
-        else
-            src = gbase[i] + (goff[i] + (uint32_t)s * (uint32_t)gstep[i]);
-        __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)src, (SVDQ_AS3 void *)(dstbuf + ldst[i]), 16, 0, 0);
-    };
-    // Scales go through registers (converted to fp32 and pre-multiplied on the way), one stage ahead: thread
-    // (group sg of the stage, row sr of the tile) fetches one activation scale and one weight scale.
-    const int sg = tid >> 7, sr = tid & 127;
-    const int sgu = __builtin_amdgcn_readfirstlane(sg);
-    const uint16_t *gAS = (const uint16_t *)a.ascales + (size_t)sgu * a.ld_ascales + m0;  // wave-uniform
-    const uint16_t *gWS = (const uint16_t *)a.wscales + (size_t)sgu * a.ld_wscales + n0;
-    const uint32_t as_off = 2 * (uint32_t)(min(m0 + sr, a.M - 1) - m0), ws_off = 2 * (uint32_t)(min(n0 + sr, a.N - 1) - n0);
-    const uint32_t as_step = 4 * (uint32_t)a.ld_ascales, ws_step = 4 * (uint32_t)a.ld_wscales;  // bytes per stage
-    const float fold = ACT_UNSIGNED ? (1.0f / 16.0f) : (1.0f / 256.0f);
-    uint16_t ras, rws;
-    uint32_t as_cap = 0, ws_cap = 0;
-    if constexpr (ODDG) {
-        as_cap = (uint32_t)(G / 2) * as_step;
-        ws_cap = (uint32_t)(G / 2) * ws_step;
-        if (sgu == 1) {  // this wavefront's group of the last stage does not exist
-            if (G == 1) {
-                gAS -= a.ld_ascales;
-                gWS -= a.ld_wscales;
-            }
-            as_cap = G == 1 ? 0u : (uint32_t)(G / 2 - 1) * as_step;
-            ws_cap = G == 1 ? 0u : (uint32_t)(G / 2 - 1) * ws_step;
-        }
-    }
-    auto load_scales = [&](int s) {
-        if (ODDG) {
-            const uint16_t va = *(const uint16_t *)((const uint8_t *)gAS + (as_off + min((uint32_t)s * as_step, as_cap)));
-            const uint16_t vw = *(const uint16_t *)((const uint8_t *)gWS + (ws_off + min((uint32_t)s * ws_step, ws_cap)));
-            const bool off = s == G / 2 && sgu == 1;
-            ras = off ? (uint16_t)0 : va;  // +0 in both 16-bit types
-            rws = off ? (uint16_t)0 : vw;
-        } else {
-            ras = *(const uint16_t *)((const uint8_t *)gAS + (as_off + (uint32_t)s * as_step));
-            rws = *(const uint16_t *)((const uint8_t *)gWS + (ws_off + (uint32_t)s * ws_step));
-        }
-    };
-    auto store_scales = [&](uint8_t *base) {
-        ((float *)(base + AS_OFF))[sg * BM + sr] = T::to_f32(ras);
-        const float w = T::to_f32(rws) * fold;
-        ((float2 *)(base + WS_OFF))[sg * BN + sr] = make_float2(w, -RNE_MAGIC * w);
-    };
-    // Pre-split weights (fp8 path): every lane fetches the scales its scale-product MFMA operands need, one stage ahead,
-    // straight into registers: the activation scale of row wm * 32 + l32 and the weight scales of columns lane and
-    // 64 + lane, for both groups of the stage.  Groups past the end (odd K / 64) are staged as zero.
-    uint16_t qa[2], qw[4];
-    const __amdgpu_buffer_rsrc_t rAS = g_buffer(a.ascales), rWS = g_buffer(a.wscales);
-    const uint32_t oA = 2u * (uint32_t)min(m0 + wm * 32 + l32, a.M - 1);
-    const uint32_t oW0 = 2u * (uint32_t)min(n0 + lane, a.N - 1), oW1 = 2u * (uint32_t)min(n0 + 64 + lane, a.N - 1);
-    // ... and the 16 packed bytes of its activation row (row wm * 32 + l32, K half lane / 32) for both groups: exactly
-    // what the lane holds as MFMA operand after the unpack.
-    v4i araw[2];
-    const __amdgpu_buffer_rsrc_t rAct = g_buffer((const uint8_t *)a.act + (size_t)m0 * a.ld_act);
-    const uint32_t oAct = (uint32_t)(min(m0 + wm * 32 + l32, a.M - 1) - m0) * (uint32_t)a.ld_act + half * 16;
-    auto load_act = [&](int s) {
-#pragma unroll
-        for (int gg = 0; gg < 2; gg++) {
-            const int gi = ODDG ? min(2 * s + gg, G - 1) : 2 * s + gg;  // a group past the end re-reads the last one (scales zero)
-            araw[gg] = g_load128(rAct, oAct, (uint32_t)gi * 32);
-        }
-    };
-    auto load_scales8 = [&](int s) {
-#pragma unroll
-        for (int gg = 0; gg < 2; gg++) {
-            const int gi = ODDG ? min(2 * s + gg, G - 1) : 2 * s + gg;
-            const uint32_t ga = (uint32_t)gi * (uint32_t)a.ld_ascales * 2u, gw = (uint32_t)gi * (uint32_t)a.ld_wscales * 2u;  // uniform
-            const uint16_t va = g_load16(rAS, oA, ga);
-            const uint16_t v0 = g_load16(rWS, oW0, gw), v1 = g_load16(rWS, oW1, gw);
-            const bool on = !ODDG || 2 * s + gg < G;
-            qa[gg] = on ? va : (uint16_t)0;
-            qw[2 * gg] = on ? v0 : (uint16_t)0;
-            qw[2 * gg + 1] = on ? v1 : (uint16_t)0;
-        }
-    };
-
-    // Operands of the offset correction that follows the main loop on the fp8 path with signed activations (see there).
-    // The group sums of the first CORR_LDS_G groups are fetched by the tile's last stage into the staging buffer that
-    // stage leaves idle, in MFMA lane order (block (weight block, piece, sixteen groups) = 1 KB, lane l's 16 bytes in
-    // slot l), one copy for the four wavefronts; the activation scales of those groups go to registers in the same
-    // stage.  Groups beyond that are read from global memory after the loop, sixteen at a time, two sets in flight.
-    const int G16 = (G + 15) / 16 * 16;
-    const int GL = min(G16, CORR_LDS_G);  // groups whose sums are staged in LDS
-    uint16_t cav[CORR_LDS_G / 16][8];
-    uint16_t cav2[2][8];
-    v4i cdb[2][NPIECE][NBN];
-    const uint16_t *cdp = nullptr, *cap = nullptr;
-    uint32_t cdrow[NBN];
-    const int cnpad = (a.N + 31) / 32 * 32;
-    static_assert(NBN * NPIECE * (CORR_LDS_G / 16) == NWAVES * CORR_PER_WAVE && NBN * NPIECE * (CORR_LDS_G / 16) * BLK_BYTES <= BUF_BYTES,
-                  "the staged group sums are dealt six blocks to a wavefront and must fit one staging buffer");
-    if constexpr (WPL && !ACT_UNSIGNED) {
-        const int npad = cnpad;
-        cdp = (const uint16_t *)((const uint8_t *)a.wgt_planes + (size_t)(npad / 32) * ((G + 1) / 2) * (WPL_BLOCKS * BLK_BYTES)) + 8 * half;
-        cap = (const uint16_t *)a.ascales + min(m0 + wm * 32 + l32, a.M - 1);
-#pragma unroll
-        for (int bn = 0; bn < NBN; bn++) cdrow[bn] = (uint32_t)min(n0 + bn * 32 + l32, npad - 1) * (uint32_t)(NPIECE * G16);
-    }
-    auto corr_stage_lds = [&](uint8_t *dstbuf) {  // this wavefront's share of the (NBN x NPIECE x GL / 16) blocks
-#pragma unroll
-        for (int i = 0; i < CORR_PER_WAVE; i++) {
-            const int q = wm * CORR_PER_WAVE + i;  // wave-uniform: (sixteen groups gc, piece, weight block)
-            const int bn = q % NBN, pc = (q / NBN) % NPIECE, gc = q / (NBN * NPIECE);
-            const uint32_t row = (uint32_t)min(n0 + bn * 32 + l32, cnpad - 1) * (uint32_t)(NPIECE * G16);
-            if (gc * 16 < GL)
-                __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)(cdp + row + pc * G16 + gc * 16),
-                                                 (SVDQ_AS3 void *)(dstbuf + q * BLK_BYTES), 16, 0, 0);
-        }
-#pragma unroll
-        for (int gc = 0; gc < CORR_LDS_G / 16; gc++)
-            if (gc * 16 < GL) {
-#pragma unroll
-                for (int j = 0; j < 8; j++) cav[gc][j] = cap[(size_t)min(gc * 16 + 8 * half + j, G - 1) * a.ld_ascales];
-            }
-    };
-    auto corr_fetch = [&](int buf, int g0) {  // all loads issued before their first use
-#pragma unroll
-        for (int j = 0; j < 8; j++) cav2[buf][j] = cap[(size_t)min(g0 + 8 * half + j, G - 1) * a.ld_ascales];
-#pragma unroll
-        for (int pc = 0; pc < NPIECE; pc++)
-#pragma unroll
-            for (int bn = 0; bn < NBN; bn++) cdb[buf][pc][bn] = *(const v4i *)(cdp + cdrow[bn] + pc * G16 + g0);
-    };
-    // Main-loop accumulators: MFMA A operand = activations, B operand = weights, so a lane owns one weight row n and its
-    // registers walk the wavefront's 32 activation rows: the weight scale is a per-lane scalar and the 16 activation
-    // scales a lane needs per group are shared by the wavefront's four weight blocks.
-    v16f acc[NBN];
-#pragma unroll
-    for (int bn = 0; bn < NBN; bn++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) acc[bn][i] = 0.0f;
-
-    auto pack8 = [&](const uint16_t (&v)[8]) -> v4i {
-        v4i ub;
-#pragma unroll
-        for (int e = 0; e < 4; e++) ub[e] = (int)((uint32_t)v[2 * e] | ((uint32_t)v[2 * e + 1] << 16));
-        return ub;
-    };
-    auto corr_apply = [&](int buf) {
-        const v4i ub = pack8(cav2[buf]);
-#pragma unroll
-        for (int pc = 0; pc < NPIECE; pc++)
-#pragma unroll
-            for (int bn = 0; bn < NBN; bn++) acc[bn] = mfma32_16bit<T>(ub, cdb[buf][pc][bn], acc[bn]);
-    };
-    const v16i cmagic = magic_acc();
-    const int nstages = ODDG ? a.K / KSTAGE + 1 : a.K / KSTAGE;
-    const int offW = W_OFF + lane * 16;
-    const int offA = wm * 2 * BLK_BYTES + lane * 16;
-
-    if constexpr (WPL) {
-        load_scales8(0);
-        load_act(0);
-    } else {
-        load_scales(0);
-    }
-#pragma unroll
-    for (int i = 0; i < PER_WAVE; i++) dma_one(0, sbuf0, i);
-    // epilogue operands, fetched now so that the epilogue does not wait for memory
     if (a.bias != nullptr && wm == 3) {  // 64 lanes x 4 bytes = the tile's 128 bias values
         const uint8_t *src = (const uint8_t *)a.bias + (size_t)min(n0 + 2 * lane, a.N - 2) * 2;
-        __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)src, (SVDQ_AS3 void *)(sepi + LORA_BYTES), 4, 0, 0);
+        __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)src, (SVDQ_AS3 void *)(sepi + LORA_UP_BYTES), 4, 0, 0);
     }
     if (a.R > 0) {
 #pragma unroll
-        for (int i = 0; i < 6; i++) {
-            const int q = wm * 6 + i;  // wave-uniform
-            const uint8_t *src;
-            bool on = true;
-            if (q < 8) {
-                const int c = q >> 2, blk = q & 3;
-                on = 16 * c < a.R;
-                src = (const uint8_t *)a.lora_up + ((size_t)min(n0 + blk * 32 + l32, a.N - 1) * a.ld_lora_up + 16 * c + 8 * half) * 2;
-            } else {
-                const int j = q - 8, c = j >> 3, blk = (j >> 1) & 3, part = j & 1;
-                on = 16 * c < a.R;
-                src = (const uint8_t *)a.lora_act + ((size_t)min(m0 + blk * 32 + l32, a.M - 1) * a.ld_lora_act + 16 * c + 8 * half + 4 * part) * 4;
-            }
-            if (on)
+        for (int i = 0; i < 2; i++) {
+            const int q = wm * 2 + i, c = q >> 2, blk = q & 3;  // wave-uniform
+            const uint8_t *src = (const uint8_t *)a.lora_up + ((size_t)min(n0 + blk * 32 + l32, a.N - 1) * a.ld_lora_up + 16 * c + 8 * half) * 2;
+            if (16 * c < a.R)
                 __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)src, (SVDQ_AS3 void *)(sepi + q * BLK_BYTES), 16, 0, 0);
         }
     }
-    // One stage = eight (group, weight block) steps, software-pipelined inside the wavefront: the MFMAs of step b + 1
-    // are issued before the dequantisation FMAs of step b, and the operands of step b + 2 are read from LDS behind
-    // them, so the VALU work of a step runs while the matrix pipe works on the next one.
-    auto stage = [&](auto par_tag, auto last_tag, int s) {
-        constexpr int P = decltype(par_tag)::value;
-        constexpr bool LAST = decltype(last_tag)::value;  // the tile's last stage: the offset correction's first operands are fetched
-        uint8_t *base = P ? sbuf1 : sbuf0;   // this stage's operands
-        uint8_t *other = P ? sbuf0 : sbuf1;  // being refilled for the next stage
-        // everything issued for stage s (scale registers, then operand blocks) has landed
-        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
-        // Operands of the scale products as[m] * ws[n] (see the loop below) for a 32x32x8 matrix instruction on 16-bit values:
-        // lanes 0-31 hold K 0-3 and lanes 32-63 hold K 4-7, two K slots to a register.  The first slot of a lane carries
-        // the stage's first group, the second slot its second group: the activation operand holds both activation scales,
-        // the weight operand one weight scale in the slot of its group and zero in the other.  A lane loaded the weight
-        // scales of column lane and column 64 + lane, so the even weight blocks find theirs in lanes 0-31 and the odd ones
-        // in lanes 32-63: sa[0] is zero in lanes 32-63, sa[1] in lanes 0-31.  Seven of the eight products are zero.
-        v2i sa[2], sw[2][2];
-        v8i a8[2];  // fp8 path: the wavefront's activation operands of the stage's two groups
-        if constexpr (WPL) {
-            // two's complement nibble -> value + 8 is a flip of the nibble's top bit; written per plane so that mask and
-            // flip are one three-input bit operation
-#pragma unroll
-            for (int gg = 0; gg < 2; gg++) {
-                typedef unsigned v4u __attribute__((ext_vector_type(4)));
-                const v4u u = __builtin_bit_cast(v4u, araw[gg]);
-                const unsigned flip = ACT_UNSIGNED ? 0u : 0x08080808u;
-                const v4u e = (u & 0x0F0F0F0Fu) ^ flip, o = ((u >> 4) & 0x0F0F0F0Fu) ^ flip;
-                a8[gg] = (v8i){(int)e[0], (int)e[1], (int)e[2], (int)e[3], (int)o[0], (int)o[1], (int)o[2], (int)o[3]};
-            }
-            const int both = (int)((uint32_t)qa[0] | ((uint32_t)qa[1] << 16));
-            sa[0] = (v2i){half ? 0 : both, 0};
-            sa[1] = (v2i){half ? both : 0, 0};
-#pragma unroll
-            for (int j = 0; j < 2; j++) {
-                sw[0][j] = (v2i){(int)qw[j], 0};
-                sw[1][j] = (v2i){(int)((uint32_t)qw[2 + j] << 16), 0};
-            }
-        } else {
-            store_scales(base);
-            __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));  // scale writes visible before the barrier
-        }
-        __builtin_amdgcn_s_barrier();
-        if constexpr (LAST && WPL && !ACT_UNSIGNED) corr_stage_lds(other);  // behind the wait above: lands while this stage computes
-        // The other buffer was last read in the previous stage, before the barrier: refill it during this stage.  The last
-        // stage re-fetches itself into the idle buffer (harmless, and keeps the stage one basic block).
-        const int sn = min(s + 1, nstages - 1);
-        if constexpr (WPL) {
-            load_scales8(sn);
-            load_act(sn);
-        } else {
-            load_scales(sn);
-        }
-        if constexpr (WPL) {
-            // One stage = eight (group, weight block) steps.  The two matrix instructions of step b + 1 (scale product and
-            // group dot product) are issued ahead of the sixteen FMAs of step b.
-            auto read_w8 = [&](int b) -> v8i {  // six registers of fp6 codes (the matrix instruction ignores the last two)
-                const int gg = b >> 2, bn = b & 3;
-                const v4i lo = *(const v4i *)(base + offW + (bn * WPL_BLOCKS + gg) * BLK_BYTES);
-                const v2i hi = *(const v2i *)(base + offW + (bn * WPL_BLOCKS + 2) * BLK_BYTES + gg * 8);
-                return (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], 0, 0};
-            };
-            const v16f z16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-            // as[m] * ws[n] of step b, exact (two 16-bit values, one non-zero product): a 16-bit matrix instruction, which
-            // runs beside the vector FMAs; the fp32 rank-1 matrix instruction shares the vector ALUs and does not
-            auto scales = [&](int b) -> v16f { return mfma32_16bit_k8<T>(sa[b & 1], sw[b >> 2][(b >> 1) & 1], z16); };
-            v8i w8[3];
-            v16f S[2], P[2];
-            w8[0] = read_w8(0);
-            w8[1] = read_w8(1);
-            S[0] = scales(0);
-            P[0] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8[0], w8[0], z16, 0, 2, 0, F8_SCALE, 0, F6_SCALE);
-#pragma unroll
-            for (int b = 0; b < 8; b++) {
-                const int cur = b & 1, nxt = cur ^ 1;
-                if (b + 1 < 8) {
-                    S[nxt] = scales(b + 1);
-                    P[nxt] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8[(b + 1) >> 2], w8[(b + 1) % 3], z16, 0, 2, 0,
-                                                                             F8_SCALE, 0, F6_SCALE);
-                }
-                // the operand reads of step b + 2 stay behind the matrix instructions: hoisted above them, the wait for step
-                // b + 1's operands would also wait for these
-                __builtin_amdgcn_sched_barrier(0);
-                if (b + 2 < 8) w8[(b + 2) % 3] = read_w8(b + 2);
-                if (!(LAST && !ACT_UNSIGNED) && b < PER_WAVE) dma_one(sn, other, b);
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int i = 0; i < 16; i++) acc[b & 3][i] = __builtin_fmaf(P[cur][i], S[cur][i], acc[b & 3][i]);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        } else {
-            auto read_w = [&](int b, v4i &we, v4i &wo, float2 &wsp) {
-                const int gg = b >> 2, bn = b & 3;
-                const v4i wp = *(const v4i *)(base + offW + (bn * 2 + gg) * BLK_BYTES);
-                unpack_signed(wp, we, wo);
-                wsp = ((const float2 *)(base + WS_OFF))[gg * BN + bn * 32 + l32];
-            };
-            auto read_a = [&](int gg, v4i &ae, v4i &ao) {
-                const v4i ap = *(const v4i *)(base + offA + gg * BLK_BYTES);
-                if (ACT_UNSIGNED)
-                    unpack_unsigned(ap, ae, ao);
-                else
-                    unpack_signed(ap, ae, ao);
-            };
-            auto read_as = [&](int gg, v4f (&asv)[4]) {
-    #pragma unroll
-                for (int j = 0; j < 4; j++)
-                    asv[j] = *(const v4f *)((const float *)(base + AS_OFF) + gg * BM + wm * 32 + 8 * j + 4 * half);
-            };
-            v4i ae[2], ao[2], we[2], wo[2];
-            float2 wsp[2];
-            v4f asv[2][4];
-            v16i t[2];
-            read_a(0, ae[0], ao[0]);
-            read_w(0, we[0], wo[0], wsp[0]);
-            read_as(0, asv[0]);
-            read_w(1, we[1], wo[1], wsp[1]);
-            t[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ae[0], we[0], cmagic, 0, 0, 0);
-            t[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ao[0], wo[0], t[0], 0, 0, 0);
-            read_a(1, ae[1], ao[1]);
-            read_as(1, asv[1]);
-    #pragma unroll
-            for (int b = 0; b < 8; b++) {
-                const int cur = b & 1, nxt = cur ^ 1;
-                float2 wcur = wsp[cur];
-                if (b + 1 < 8) {
-                    const int g1 = (b + 1) >> 2;
-                    t[nxt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ae[g1], we[nxt], cmagic, 0, 0, 0);
-                    t[nxt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ao[g1], wo[nxt], t[nxt], 0, 0, 0);
-                }
-                if (b + 2 < 8) read_w(b + 2, we[cur], wo[cur], wsp[cur]);
-                if (b < PER_WAVE) dma_one(sn, other, b);
-                __builtin_amdgcn_sched_barrier(0);
-    #pragma unroll
-                for (int i = 0; i < 16; i++) {
-                    const float u = __builtin_fmaf(__int_as_float(t[cur][i]), wcur.x, wcur.y);
-                    acc[b & 3][i] = __builtin_fmaf(u, asv[b >> 2][i >> 2][i & 3], acc[b & 3][i]);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
-    };
-    {
-        const int last = nstages - 1;
-        int s = 0;
-        for (; s + 1 < last; s += 2) {
-            stage(std::integral_constant<int, 0>{}, std::false_type{}, s);
-            stage(std::integral_constant<int, 1>{}, std::false_type{}, s + 1);
-        }
-        if (s < last) {
-            stage(std::integral_constant<int, 0>{}, std::false_type{}, s);
-            s++;
-        }
-        if (s & 1)
-            stage(std::integral_constant<int, 1>{}, std::true_type{}, s);
-        else
-            stage(std::integral_constant<int, 0>{}, std::true_type{}, s);
-    }
-    // The last stage's (redundant) block loads of this wavefront have landed.
-    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
+}
 
-    // ---- fp8 path, signed activations: take the +8 offset out again -------------------------------------------------
-    // sum_g as[g, m] ws[g, n] sum_k (a + 8) w  =  wanted  +  sum_g as[g, m] * (8 ws[g, n] W[g, n]),  W = the weights' group
-    // sums.  svdq_split_weight_planes stored D[g, n] = -8 ws[g, n] W[g, n] behind the planes as two 16-bit pieces
-    // (hi + lo: 16 significant bits in bf16, 22 in fp16), K-contiguous per weight row like a LoRA-up matrix of rank 2 * G16; the
-    // activation scales are the other operand.  Products of two 16-bit values are exact, the sum is fp32.
-    if constexpr (WPL && !ACT_UNSIGNED) {
-        if (GL < G16) corr_fetch(0, GL);
-        __syncthreads();  // every wavefront's share of the staged blocks has landed (each waited for its own above)
-        const uint8_t *cl = (((nstages - 1) & 1) ? sbuf0 : sbuf1) + lane * 16;  // the buffer the last stage left idle
-#pragma unroll
-        for (int gc = 0; gc < CORR_LDS_G / 16; gc++)
-            if (gc * 16 < GL) {
-                const v4i ub = pack8(cav[gc]);
-#pragma unroll
-                for (int pc = 0; pc < NPIECE; pc++)
-#pragma unroll
-                    for (int bn = 0; bn < NBN; bn++)
-                        acc[bn] = mfma32_16bit<T>(ub, *(const v4i *)(cl + ((gc * NPIECE + pc) * NBN + bn) * BLK_BYTES), acc[bn]);
-            }
-        for (int g0 = GL; g0 < G16; g0 += 32) {  // two sets of operand registers, the next sixteen groups in flight
-            if (g0 + 16 < G16) corr_fetch(1, g0 + 16);
-            corr_apply(0);
-            if (g0 + 32 < G16) corr_fetch(0, g0 + 32);
-            if (g0 + 16 < G16) corr_apply(1);
-        }
-    }
+// Everything after the main loop, for one wavefront: acc[bn][i] holds out[m = mw0 + 8 (i >> 2) + 4 half + (i & 3)]
+// [n = n0 + 32 bn + lane % 32] without LoRA-up and bias.  `priv` is PRIV_BYTES of LDS nobody else touches from here on;
+// `sepi` holds what fetch_epilogue_operands brought.  No workgroup barrier inside.
+template <typename T, int EPI>
+__device__ __forceinline__ void tile_epilogue(const svdq_gemm_args &a, v16f (&acc)[NBN], uint8_t *priv, const uint8_t *sepi,
+                                              int m0, int n0, int pid_n, int wm, int lane) {
+    const int l32 = lane & 31, half = lane >> 5;
+    const int mw0 = m0 + wm * 32;
 
     // ---- LoRA-up and bias, still in the main loop's orientation (lane = weight row, registers = activation rows) ----
-    // The bias and the first 32 ranks of both LoRA operands were fetched into LDS next to stage 0 and arrived long ago;
-    // ranks beyond 32 come from global memory, all loads of a 32-rank pass issued before their first use.  Rows past
-    // N / M hold copies of the last row: they only reach outputs that are never stored.
-    const int mw0 = m0 + wm * 32;
+    // The bias and the first 32 ranks of lora_up were fetched into LDS next to stage 0 and arrived long ago; the
+    // wavefront's own rows of lora_act and ranks beyond 32 come from global memory, all loads of a 32-rank pass issued
+    // before their first use.  Rows past N / M hold copies of the last row: they only reach outputs that are never stored.
     if (a.R > 0) {
         const uint16_t *lu = (const uint16_t *)a.lora_up;
+        const float *la = a.lora_act + (size_t)min(mw0 + l32, a.M - 1) * a.ld_lora_act + half * 8;
         for (int r0 = 0; r0 < a.R; r0 += 32) {
             const bool two = r0 + 16 < a.R;  // uniform: the second 16 ranks of this pass exist
             v4i ua[2][NBN];
@@ -603,25 +229,14 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
 #pragma unroll
             for (int c = 0; c < 2; c++) {
                 if (c == 1 && !two) break;
+                uf[c][0] = *(const v4f *)(la + r0 + 16 * c);
+                uf[c][1] = *(const v4f *)(la + r0 + 16 * c + 4);
 #pragma unroll
                 for (int blk = 0; blk < NBN; blk++) {
-                    const int n = n0 + blk * 32 + l32;
-                    ua[c][blk] = (v4i){0, 0, 0, 0};
                     if (r0 == 0)
                         ua[c][blk] = *(const v4i *)(sepi + (c * 4 + blk) * BLK_BYTES + lane * 16);
-                    else if (n < a.N)
-                        ua[c][blk] = *(const v4i *)(lu + (size_t)n * a.ld_lora_up + r0 + 16 * c + half * 8);
-                }
-                const int m = mw0 + l32;
-                uf[c][0] = uf[c][1] = (v4f){0.f, 0.f, 0.f, 0.f};
-                if (r0 == 0) {
-                    const uint8_t *lp = sepi + 8 * BLK_BYTES + ((c * 4 + wm) * 2) * BLK_BYTES + lane * 16;
-                    uf[c][0] = *(const v4f *)lp;
-                    uf[c][1] = *(const v4f *)(lp + BLK_BYTES);
-                } else if (m < a.M) {
-                    const float *lp = a.lora_act + (size_t)m * a.ld_lora_act + r0 + 16 * c + half * 8;
-                    uf[c][0] = *(const v4f *)lp;
-                    uf[c][1] = *(const v4f *)(lp + 4);
+                    else
+                        ua[c][blk] = *(const v4i *)(lu + (size_t)min(n0 + blk * 32 + l32, a.N - 1) * a.ld_lora_up + r0 + 16 * c + half * 8);
                 }
             }
 #pragma unroll
@@ -641,51 +256,38 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
     if (a.bias != nullptr) {
 #pragma unroll
         for (int bn = 0; bn < NBN; bn++) {
-            const float b = T::to_f32(*(const uint16_t *)(sepi + LORA_BYTES + (bn * 32 + l32) * 2));
+            const float b = T::to_f32(*(const uint16_t *)(sepi + LORA_UP_BYTES + (bn * 32 + l32) * 2));
 #pragma unroll
             for (int i = 0; i < 16; i++) acc[bn][i] += b;
         }
     }
 
     // ---- transposition: lane = weight row -> lane = activation row ---------------------------------------------
-    // Each wavefront turns its four 32x32 blocks through a private LDS tile (the staging memory is free once every
-    // wavefront has left the main loop and read its LoRA operands).  Afterwards lane (m = lane % 32, half) holds
-    // columns 32 bn + 8 j + 4 half + e of row m in acc[bn][4 j + e]: row-wise epilogue work (RMSNorm sum of squares,
-    // RoPE pairs, group absmax, nibble packing, the next layer's LoRA-down B operand) is in-lane plus one exchange
-    // with lane ^ 32, and no epilogue needs another wavefront's data.
-    __syncthreads();
+    // One 32x32 block at a time through the private tile (the LDS operations of one wavefront complete in order).
+    // Afterwards lane (m = lane % 32, half) holds columns 32 bn + 8 j + 4 half + e of row m in acc[bn][4 j + e]: row-wise
+    // epilogue work is in-lane plus one exchange with lane ^ 32, and no epilogue needs another wavefront's data.
     {
-        // wavefronts 0, 1 use the first staging buffer, 2, 3 the second; two blocks per round
-        float *tp = (float *)((wm < 2 ? sbuf0 : sbuf1) + (wm & 1) * TP_WAVE_BYTES);
+        float *tp = (float *)priv;
 #pragma unroll
-        for (int rnd = 0; rnd < NBN / 2; rnd++) {
+        for (int bn = 0; bn < NBN; bn++) {
 #pragma unroll
-            for (int b2 = 0; b2 < 2; b2++)
+            for (int i = 0; i < 16; i++) tp[(8 * (i >> 2) + 4 * half + (i & 3)) * TP_PITCH + l32] = acc[bn][i];
 #pragma unroll
-                for (int i = 0; i < 16; i++)
-                    tp[(b2 * 32 + 8 * (i >> 2) + 4 * half + (i & 3)) * TP_PITCH + l32] = acc[2 * rnd + b2][i];
-            // the same wavefront writes and reads: the LDS operations of one wavefront complete in order
-#pragma unroll
-            for (int b2 = 0; b2 < 2; b2++)
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    const v4f v = *(const v4f *)(tp + (b2 * 32 + l32) * TP_PITCH + 8 * j + 4 * half);
-                    acc[2 * rnd + b2][4 * j + 0] = v[0];
-                    acc[2 * rnd + b2][4 * j + 1] = v[1];
-                    acc[2 * rnd + b2][4 * j + 2] = v[2];
-                    acc[2 * rnd + b2][4 * j + 3] = v[3];
-                }
+            for (int j = 0; j < 4; j++) {
+                const v4f v = *(const v4f *)(tp + l32 * TP_PITCH + 8 * j + 4 * half);
+                acc[bn][4 * j + 0] = v[0];
+                acc[bn][4 * j + 1] = v[1];
+                acc[bn][4 * j + 2] = v[2];
+                acc[bn][4 * j + 3] = v[3];
+            }
         }
     }
 
     // Output rows go out through LDS: in registers a lane holds 4 consecutive columns of one row, which stored directly
-    // is an 8-byte piece per row and lane; staged as a [row][column] tile, each store instruction writes four
-    // contiguous 256-byte row segments instead.
+    // is an 8-byte piece per row and lane; staged as the wavefront's [32 rows][256 bytes] tile, each store instruction
+    // writes four contiguous 256-byte row segments instead.  16-byte chunk c of row r sits at chunk c ^ (r & 15), its two
+    // 8-byte halves swapped for rows 16-31: writes and reads are free of bank conflicts.
     auto store_out = [&]() {
-        constexpr int PITCH = BN * 2 + 16;  // bytes per staged row (16-byte aligned, off the power of two)
-        static_assert(BM / 2 * PITCH <= BUF_BYTES, "half an output tile does not fit a staging buffer");
-        __syncthreads();  // earlier users of the staging memory are done
-        uint8_t *mine = (wm < 2 ? sbuf0 : sbuf1) + ((wm & 1) * 32 + l32) * PITCH;  // rows 0-63 | rows 64-127
 #pragma unroll
         for (int bn = 0; bn < NBN; bn++)
 #pragma unroll
@@ -693,20 +295,19 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
                 uint2 v;
                 v.x = pack2<T>(acc[bn][4 * j], acc[bn][4 * j + 1]);
                 v.y = pack2<T>(acc[bn][4 * j + 2], acc[bn][4 * j + 3]);
-                *(uint2 *)(mine + (bn * 32 + 8 * j + 4 * half) * 2) = v;
+                *(uint2 *)(priv + l32 * (BN * 2) + (((4 * bn + j) ^ (l32 & 15)) << 4) + 8 * (half ^ (l32 >> 4))) = v;
             }
-        __syncthreads();
         uint16_t *out = (uint16_t *)a.out;
-        const int c = tid & 15, n = n0 + c * 8;
-        constexpr int PASSES = BM * 16 / NTHREADS;
+        const int c = lane & 15, n = n0 + c * 8;
 #pragma unroll
-        for (int pass = 0; pass < PASSES; pass++) {
-            const int row = pass * (NTHREADS / 16) + (tid >> 4), m = m0 + row;
-            const uint8_t *src = (pass < PASSES / 2 ? sbuf0 : sbuf1) + (row & 63) * PITCH + c * 16;
+        for (int pass = 0; pass < 8; pass++) {
+            const int r = 4 * pass + (lane >> 4), m = mw0 + r;  // rows 16-31 are passes 4-7
+            v4i q = *(const v4i *)(priv + r * (BN * 2) + ((c ^ (r & 15)) << 4));
+            if (pass >= 4) q = (v4i){q[2], q[3], q[0], q[1]};
             if (m < a.actual_m && n < a.N)
                 // streamed: the 85 MB of a QKV output do not fit any cache level of the CU, and lines left dirty in L2 have
                 // to be written back before the next kernel on the stream starts (measured: 1 % of the launch)
-                __builtin_nontemporal_store(*(const v4i *)src, (v4i *)(out + (size_t)m * a.ld_out + n));
+                __builtin_nontemporal_store(q, (v4i *)(out + (size_t)m * a.ld_out + n));
         }
     };
 
@@ -719,17 +320,17 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
         // the 128-wide tile is one head, all of it in this wavefront; part 0 = Q, 1 = K, 2 = V (untouched)
         const int part = n0 / (a.N / 3);
         if (part < 2) {
+            const uint16_t *nw = (const uint16_t *)(part == 0 ? a.norm_q : a.norm_k);
+            const int m = mw0 + l32;
+            const bool rok = m < a.actual_m;
+            const float *rot = a.rotary + (size_t)(rok ? m : 0) * a.ld_rotary;
             float ss = 0.0f;
 #pragma unroll
             for (int bn = 0; bn < NBN; bn++)
 #pragma unroll
                 for (int i = 0; i < 16; i++) ss += acc[bn][i] * acc[bn][i];
             ss += __shfl_xor(ss, 32);
-            const uint16_t *nw = (const uint16_t *)(part == 0 ? a.norm_q : a.norm_k);
-            const int m = mw0 + l32;
             const float rstd = 1.0f / sqrtf(ss / 128.0f + a.eps);
-            const bool rok = m < a.actual_m;
-            const float *rot = a.rotary + (size_t)(rok ? m : 0) * a.ld_rotary;
 #pragma unroll
             for (int bn = 0; bn < NBN; bn++)
 #pragma unroll
@@ -754,10 +355,13 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
     if (EPI == SVDQ_EPI_GELU_QUANT) {
         const uint16_t *ldt = (const uint16_t *)a.lora_down_t;
         // loads whose values are needed further down, issued before the GELU arithmetic: the next layer's smoothing
-        // factor of this thread's column and the first 32 ranks of its LoRA-down weight
-        uint16_t smv = 0;
-        const bool has_sm = a.smooth_next != nullptr && tid < BN && n0 + tid < a.N;
-        if (has_sm) smv = ((const uint16_t *)a.smooth_next)[n0 + tid];
+        // factors of columns lane and 64 + lane and the first 32 ranks of its LoRA-down weight
+        uint16_t smv[2] = {0, 0};
+        const bool has_sm = a.smooth_next != nullptr;
+        if (has_sm) {
+#pragma unroll
+            for (int t = 0; t < 2; t++) smv[t] = ((const uint16_t *)a.smooth_next)[min(n0 + 64 * t + lane, a.N - 1)];
+        }
         uint2 lq[NBN][2][2];
         if (a.R2 > 0) {
 #pragma unroll
@@ -813,10 +417,9 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
         }
 
         // +shift, * 1/smooth, unsigned per-64 quantization: the wavefront's 128 columns are two groups
-        float *lds_rs = (float *)sbuf0;  // [BN]
-        __syncthreads();                // transposition tiles / staged output are no longer read
-        if (tid < BN) lds_rs[tid] = has_sm ? 1.0f / T::to_f32(smv) : 1.0f;
-        __syncthreads();
+        float *lds_rs = (float *)priv;  // [BN], this wavefront's own copy
+#pragma unroll
+        for (int t = 0; t < 2; t++) lds_rs[64 * t + lane] = has_sm ? 1.0f / T::to_f32(smv[t]) : 1.0f;
         const int m = mw0 + l32;
 #pragma unroll
         for (int gi = 0; gi < 2; gi++) {
@@ -879,12 +482,15 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
         // y columns = one quantization group, all of it in this wavefront.
         const int H = a.N / 2;
         const uint16_t *ldt = (const uint16_t *)a.lora_down_t;
+        const int yt0 = n0 / 2;  // first y column of the tile
+        uint16_t smv = 0;
+        const bool has_sm = a.smooth_next != nullptr;
+        if (has_sm) smv = ((const uint16_t *)a.smooth_next)[min(yt0 + lane, H - 1)];
         float y[NBN][8];  // [bn][4 j + e]: y column 16 bn + 8 j + 4 half + e of the tile's 64
 #pragma unroll
         for (int bn = 0; bn < NBN; bn++)
 #pragma unroll
             for (int i = 0; i < 8; i++) y[bn][i] = silu(acc[bn][i]) * acc[bn][8 + i];
-        const int yt0 = n0 / 2;  // first y column of the tile
         const int m = mw0 + l32;
         for (int rc = 0; rc < a.R2; rc += 32) {
             v16f d;
@@ -913,14 +519,8 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
         }
 
         // * 1/smooth, signed per-64 quantization over the tile's 64 y columns
-        float *lds_rs = (float *)sbuf0;  // [64]
-        __syncthreads();                // transposition tiles are no longer read
-        if (tid < 64) {
-            float rs = 1.0f;
-            if (a.smooth_next != nullptr) rs = 1.0f / T::to_f32(((const uint16_t *)a.smooth_next)[yt0 + tid]);
-            lds_rs[tid] = rs;
-        }
-        __syncthreads();
+        float *lds_rs = (float *)priv;  // [64], this wavefront's own copy
+        lds_rs[lane] = has_sm ? 1.0f / T::to_f32(smv) : 1.0f;
         float gmax = 0.0f;
 #pragma unroll
         for (int bn = 0; bn < NBN; bn++)
@@ -965,6 +565,406 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_kernel(svdq_gemm_args a
     }
 }
 
+// ---- packed weights: int8 main loop -------------------------------------------------------------------------------------
+template <typename T, bool ACT_UNSIGNED, int EPI, bool ODDG>  // ODDG: K / 64 is odd
+__global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_i8_kernel(svdq_gemm_args a) {
+    // Three separate LDS objects: the compiler then knows that a block load into one staging buffer cannot touch what
+    // is being read from the other (one object would make every LDS read wait for the loads in flight).
+    __shared__ __align__(16) uint8_t sbuf0[I8_BUF_BYTES];
+    __shared__ __align__(16) uint8_t sbuf1[I8_BUF_BYTES];
+    __shared__ __align__(16) uint8_t sepi[EPI_LDS_BYTES];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wm = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: the wavefront's 32-row block of the tile
+    const int l32 = lane & 31, half = lane >> 5;
+
+    int pid_m, pid_n;
+    tile_ids((a.M + BM - 1) / BM, (a.N + BN - 1) / BN, pid_m, pid_n);
+    const int m0 = pid_m * BM, n0 = pid_n * BN;
+
+    // ---- operand staging: global -> LDS directly (global_load_lds_dwordx4), one stage ahead ----------------------
+    // A stage holds 1 KB operand blocks (operand, 32-row block, group).  Lane l of a block load fetches the 16 bytes MFMA
+    // lane l will read and the hardware writes them to LDS slot l of the block: lane l = (row l % 32, half l / 32) of a
+    // row-major tile.  The 8 activation + 8 weight block loads of a stage are dealt in runs to the four wavefronts.
+    constexpr int NLOADS = 16, PER_WAVE = NLOADS / NWAVES, NABLK = 8;
+    // each load's address = wave-uniform base (SGPRs) + a 32-bit offset (lane part + stage * step; operands < 4 GiB)
+    const uint8_t *gbase[PER_WAVE];
+    uint32_t goff[PER_WAVE];
+    int ldst[PER_WAVE];
+    uint32_t gcap[PER_WAVE];
+    const int G = a.K / GROUP;
+    // K / 64 odd: the last stage has one group only.  The loads of its second group stop one stage earlier (they re-read
+    // valid memory) and its scales are staged as zero, so it adds nothing.  A load's stage offset is min(s * step, cap).
+    auto cap_of = [&](int gg, const uint8_t *&base) -> uint32_t {
+        if (gg == 0) return (uint32_t)(G / 2) * (uint32_t)(KSTAGE / 2);  // G is odd: stages 0 .. G / 2
+        if (G == 1) {  // no earlier stage: read the first group's bytes instead
+            base -= 32;
+            return 0u;
+        }
+        return (uint32_t)(G / 2 - 1) * (uint32_t)(KSTAGE / 2);
+    };
+#pragma unroll
+    for (int i = 0; i < PER_WAVE; i++) {
+        const int q = wm * PER_WAVE + i;  // wave-uniform
+        if (q < NABLK) {                  // activation block q: (blk = q / 2, group q % 2)
+            const int blk = q >> 1, gg = q & 1;
+            gbase[i] = (const uint8_t *)a.act + (size_t)m0 * a.ld_act + gg * 32;
+            goff[i] = (uint32_t)(min(m0 + blk * 32 + l32, a.M - 1) - m0) * (uint32_t)a.ld_act + half * 16;
+            ldst[i] = (blk * 2 + gg) * BLK_BYTES;
+            if constexpr (ODDG) gcap[i] = cap_of(gg, gbase[i]);
+        } else {                          // packed weight block j: (blk = j / 2, group j % 2)
+            const int j = q - NABLK, blk = j >> 1, gg = j & 1;
+            gbase[i] = (const uint8_t *)a.wgt + (size_t)n0 * a.ld_wgt + gg * 32;
+            goff[i] = (uint32_t)(min(n0 + blk * 32 + l32, a.N - 1) - n0) * (uint32_t)a.ld_wgt + half * 16;
+            ldst[i] = I8_W_OFF + (blk * 2 + gg) * BLK_BYTES;
+            if constexpr (ODDG) gcap[i] = cap_of(gg, gbase[i]);
+        }
+    }
+    auto dma_one = [&](int s, uint8_t *dstbuf, int i) {  // block load i of stage s into a staging buffer
+        const uint8_t *src;
+        if constexpr (ODDG)
+            src = gbase[i] + (goff[i] + min((uint32_t)s * (uint32_t)(KSTAGE / 2), gcap[i]));  // stage part wave-uniform
+        else
+            src = gbase[i] + (goff[i] + (uint32_t)s * (uint32_t)(KSTAGE / 2));
+        __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)src, (SVDQ_AS3 void *)(dstbuf + ldst[i]), 16, 0, 0);
+    };
+    // Scales go through registers (converted to fp32 and pre-multiplied on the way), one stage ahead: thread
+    // (group sg of the stage, row sr of the tile) fetches one activation scale and one weight scale.
+    const int sg = tid >> 7, sr = tid & 127;
+    const int sgu = __builtin_amdgcn_readfirstlane(sg);
+    const uint16_t *gAS = (const uint16_t *)a.ascales + (size_t)sgu * a.ld_ascales + m0;  // wave-uniform
+    const uint16_t *gWS = (const uint16_t *)a.wscales + (size_t)sgu * a.ld_wscales + n0;
+    const uint32_t as_off = 2 * (uint32_t)(min(m0 + sr, a.M - 1) - m0), ws_off = 2 * (uint32_t)(min(n0 + sr, a.N - 1) - n0);
+    const uint32_t as_step = 4 * (uint32_t)a.ld_ascales, ws_step = 4 * (uint32_t)a.ld_wscales;  // bytes per stage
+    const float fold = ACT_UNSIGNED ? (1.0f / 16.0f) : (1.0f / 256.0f);
+    uint16_t ras, rws;
+    uint32_t as_cap = 0, ws_cap = 0;
+    if constexpr (ODDG) {
+        as_cap = (uint32_t)(G / 2) * as_step;
+        ws_cap = (uint32_t)(G / 2) * ws_step;
+        if (sgu == 1) {  // this wavefront's group of the last stage does not exist
+            if (G == 1) {
+                gAS -= a.ld_ascales;
+                gWS -= a.ld_wscales;
+            }
+            as_cap = G == 1 ? 0u : (uint32_t)(G / 2 - 1) * as_step;
+            ws_cap = G == 1 ? 0u : (uint32_t)(G / 2 - 1) * ws_step;
+        }
+    }
+    auto load_scales = [&](int s) {
+        if (ODDG) {
+            const uint16_t va = *(const uint16_t *)((const uint8_t *)gAS + (as_off + min((uint32_t)s * as_step, as_cap)));
+            const uint16_t vw = *(const uint16_t *)((const uint8_t *)gWS + (ws_off + min((uint32_t)s * ws_step, ws_cap)));
+            const bool off = s == G / 2 && sgu == 1;
+            ras = off ? (uint16_t)0 : va;  // +0 in both 16-bit types
+            rws = off ? (uint16_t)0 : vw;
+        } else {
+            ras = *(const uint16_t *)((const uint8_t *)gAS + (as_off + (uint32_t)s * as_step));
+            rws = *(const uint16_t *)((const uint8_t *)gWS + (ws_off + (uint32_t)s * ws_step));
+        }
+    };
+    auto store_scales = [&](uint8_t *base) {
+        ((float *)(base + I8_AS_OFF))[sg * BM + sr] = T::to_f32(ras);
+        const float w = T::to_f32(rws) * fold;
+        ((float2 *)(base + I8_WS_OFF))[sg * BN + sr] = make_float2(w, -RNE_MAGIC * w);
+    };
+
+    // Main-loop accumulators: MFMA A operand = activations, B operand = weights, so a lane owns one weight row n and its
+    // registers walk the wavefront's 32 activation rows: the weight scale is a per-lane scalar and the 16 activation
+    // scales a lane needs per group are shared by the wavefront's four weight blocks.
+    v16f acc[NBN];
+#pragma unroll
+    for (int bn = 0; bn < NBN; bn++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) acc[bn][i] = 0.0f;
+
+    const v16i cmagic = magic_acc();
+    const int nstages = ODDG ? a.K / KSTAGE + 1 : a.K / KSTAGE;
+    const int offW = I8_W_OFF + lane * 16;
+    const int offA = wm * 2 * BLK_BYTES + lane * 16;
+
+    load_scales(0);
+#pragma unroll
+    for (int i = 0; i < PER_WAVE; i++) dma_one(0, sbuf0, i);
+    fetch_epilogue_operands(a, sepi, n0, wm, lane);
+    // One stage = eight (group, weight block) steps, software-pipelined inside the wavefront: the MFMAs of step b + 1
+    // are issued before the dequantisation FMAs of step b, and the operands of step b + 2 are read from LDS behind
+    // them, so the VALU work of a step runs while the matrix pipe works on the next one.
+    auto stage = [&](auto par_tag, int s) {
+        constexpr int P = decltype(par_tag)::value;
+        uint8_t *base = P ? sbuf1 : sbuf0;   // this stage's operands
+        uint8_t *other = P ? sbuf0 : sbuf1;  // being refilled for the next stage
+        // everything issued for stage s (scale registers, then operand blocks) has landed
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
+        store_scales(base);
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));  // scale writes visible before the barrier
+        __builtin_amdgcn_s_barrier();
+        // The other buffer was last read in the previous stage, before the barrier: refill it during this stage.  The last
+        // stage re-fetches itself into the idle buffer (harmless, and keeps the stage one basic block).
+        const int sn = min(s + 1, nstages - 1);
+        load_scales(sn);
+        auto read_w = [&](int b, v4i &we, v4i &wo, float2 &wsp) {
+            const int gg = b >> 2, bn = b & 3;
+            const v4i wp = *(const v4i *)(base + offW + (bn * 2 + gg) * BLK_BYTES);
+            unpack_signed(wp, we, wo);
+            wsp = ((const float2 *)(base + I8_WS_OFF))[gg * BN + bn * 32 + l32];
+        };
+        auto read_a = [&](int gg, v4i &ae, v4i &ao) {
+            const v4i ap = *(const v4i *)(base + offA + gg * BLK_BYTES);
+            if (ACT_UNSIGNED)
+                unpack_unsigned(ap, ae, ao);
+            else
+                unpack_signed(ap, ae, ao);
+        };
+        auto read_as = [&](int gg, v4f (&asv)[4]) {
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                asv[j] = *(const v4f *)((const float *)(base + I8_AS_OFF) + gg * BM + wm * 32 + 8 * j + 4 * half);
+        };
+        v4i ae[2], ao[2], we[2], wo[2];
+        float2 wsp[2];
+        v4f asv[2][4];
+        v16i t[2];
+        read_a(0, ae[0], ao[0]);
+        read_w(0, we[0], wo[0], wsp[0]);
+        read_as(0, asv[0]);
+        read_w(1, we[1], wo[1], wsp[1]);
+        t[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ae[0], we[0], cmagic, 0, 0, 0);
+        t[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ao[0], wo[0], t[0], 0, 0, 0);
+        read_a(1, ae[1], ao[1]);
+        read_as(1, asv[1]);
+#pragma unroll
+        for (int b = 0; b < 8; b++) {
+            const int cur = b & 1, nxt = cur ^ 1;
+            float2 wcur = wsp[cur];
+            if (b + 1 < 8) {
+                const int g1 = (b + 1) >> 2;
+                t[nxt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ae[g1], we[nxt], cmagic, 0, 0, 0);
+                t[nxt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ao[g1], wo[nxt], t[nxt], 0, 0, 0);
+            }
+            if (b + 2 < 8) read_w(b + 2, we[cur], wo[cur], wsp[cur]);
+            if (b < PER_WAVE) dma_one(sn, other, b);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const float u = __builtin_fmaf(__int_as_float(t[cur][i]), wcur.x, wcur.y);
+                acc[b & 3][i] = __builtin_fmaf(u, asv[b >> 2][i >> 2][i & 3], acc[b & 3][i]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    {
+        int s = 0;
+        for (; s + 1 < nstages; s += 2) {
+            stage(std::integral_constant<int, 0>{}, s);
+            stage(std::integral_constant<int, 1>{}, s + 1);
+        }
+        if (s < nstages) stage(std::integral_constant<int, 0>{}, s);
+    }
+    // The last stage's (redundant) block loads of this wavefront have landed; then every wavefront has left the main loop:
+    // the staging memory becomes the wavefronts' private epilogue memory.
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
+    __syncthreads();
+    tile_epilogue<T, EPI>(a, acc, (wm < 2 ? sbuf0 : sbuf1) + (wm & 1) * PRIV_BYTES, sepi, m0, n0, pid_n, wm, lane);
+}
+
+// ---- pre-split weights: fp8 x fp6 main loop --------------------------------------------------------------------------------
+template <typename T, bool ACT_UNSIGNED, int EPI>
+__global__ __launch_bounds__(NTHREADS, 3) void gemm_w4a4_f8_kernel(svdq_gemm_args a) {
+    // Separate LDS objects: the compiler then knows that a block load into one staging buffer cannot touch what is being
+    // read from the other (one object would make every LDS read wait for the loads in flight).
+    __shared__ __align__(16) uint8_t sbuf0[F8_STAGE_BYTES];
+    __shared__ __align__(16) uint8_t sbuf1[F8_STAGE_BYTES];
+    __shared__ __align__(16) uint8_t sring[F8_RING_BYTES];
+    __shared__ __align__(16) uint8_t sepi[EPI_LDS_BYTES];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wm = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: the wavefront's 32-row block of the tile
+    const int l32 = lane & 31, half = lane >> 5;
+
+    int pid_m, pid_n;
+    tile_ids((a.M + BM - 1) / BM, (a.N + BN - 1) / BN, pid_m, pid_n);
+    const int m0 = pid_m * BM, n0 = pid_n * BN;
+    const int G = a.K / GROUP, nstages = (G + 1) / 2;
+
+    // ---- what a wavefront fetches per stage, one stage ahead ------------------------------------------------------
+    // global -> LDS: the three 1 KB code blocks of weight block wm of the tile and its 12-byte rows of scales and offset
+    // terms (address = wave-uniform base in SGPRs + a 32-bit offset: lane part + stage * step).  A block of rows past N
+    // re-reads the last block (its outputs are never stored).
+    const int nblk = min(n0 / 32 + wm, (a.N + 31) / 32 - 1);
+    const uint8_t *wbase = (const uint8_t *)a.wgt_planes + (size_t)nblk * nstages * (WPL_BLOCKS * BLK_BYTES);
+    const uint8_t *xbase = (const uint8_t *)a.wgt_planes + planes_code_bytes(a.N, a.K) + (size_t)nblk * (nstages + 1) * AUX_BLK;
+    auto dma = [&](int s, uint8_t *dstbuf, int slot, int i) {  // i = 0, 1, 2: code blocks of stage s; i = 3: its scales and offset terms
+        if (i < WPL_BLOCKS) {
+            const uint8_t *src = wbase + i * BLK_BYTES + ((uint32_t)lane * 16u + (uint32_t)s * (uint32_t)(WPL_BLOCKS * BLK_BYTES));
+            __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)src, (SVDQ_AS3 void *)(dstbuf + (wm * WPL_BLOCKS + i) * BLK_BYTES), 16, 0, 0);
+        } else {
+            // 64 lanes x 12 bytes = the rows of stage s and of stage s + 1 (the copy has one stage of padding), into the given
+            // ring slot and the one after it, which the next stage's load fills with the same bytes again
+            const uint8_t *src = xbase + ((uint32_t)lane * (uint32_t)AUX_ROW + (uint32_t)s * (uint32_t)AUX_BLK);
+            __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)src,
+                                             (SVDQ_AS3 void *)(sring + wm * AUX_NBLK_BYTES + slot * AUX_LBLK), 12, 0, 0);
+        }
+    };
+    // registers: the 16 packed bytes of the lane's activation row (row wm * 32 + l32, K half lane / 32) of both groups,
+    // exactly what the lane holds as MFMA operand after the unpack, and the row's two activation scales.  A group past
+    // the end (K / 64 odd) re-reads the last one: its weight codes, scale and offset term are stored as zero.
+    v4i araw[2];
+    uint16_t qa[2];
+    const int mrow = min(m0 + wm * 32 + l32, a.M - 1);
+    const __amdgpu_buffer_rsrc_t rAct = g_buffer((const uint8_t *)a.act + (size_t)m0 * a.ld_act);
+    const __amdgpu_buffer_rsrc_t rAS = g_buffer(a.ascales);
+    const uint32_t oAct = (uint32_t)(mrow - m0) * (uint32_t)a.ld_act + half * 16;
+    const uint32_t oA = 2u * (uint32_t)mrow;
+    auto load_regs = [&](int s) {
+#pragma unroll
+        for (int gg = 0; gg < 2; gg++) {
+            const int gi = min(2 * s + gg, G - 1);
+            qa[gg] = g_load16(rAS, oA, (uint32_t)gi * (uint32_t)a.ld_ascales * 2u);
+            araw[gg] = g_load128(rAct, oAct, (uint32_t)gi * 32);
+        }
+    };
+
+    v16f acc[NBN];
+#pragma unroll
+    for (int bn = 0; bn < NBN; bn++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) acc[bn][i] = 0.0f;
+
+    // ---- the offset of signed activations, taken out every four stages ------------------------------------------------
+    // The fp8 operand holds a + 8 for even k and a - 7 for odd k, so a group's product comes out
+    // as p_g + (8 We - 7 Wo) with We / Wo the sums of the group's even / odd weights.  D[g, n] = -ws[g, n] (8 We - 7 Wo)
+    // travels with the weights as two 16-bit pieces; acc += sum_g as[g, m] * D[g, n] over the eight groups of four stages is
+    // one 32x32x16 matrix instruction per weight block: K slot 4 * (stage of the four) + 2 * (group of the stage) + piece.
+    // The activation-side operand collects the activation scales stage by stage (lanes of half h own stages 2 h and
+    // 2 h + 1); the weight-side operand is read from the ring.  It is applied at the start of the following stage, when none
+    // of this wavefront's loads is in flight.
+    int ub[4] = {0, 0, 0, 0};
+    auto corr = [&](uint32_t off0, uint32_t off1) {  // byte offsets in a block's ring of the lane's two stages
+        const v4i ubv = {ub[0], ub[1], ub[2], ub[3]};
+#pragma unroll
+        for (int bn = 0; bn < NBN; bn++) {
+            const uint32_t *p0 = (const uint32_t *)(sring + bn * AUX_NBLK_BYTES + off0);
+            const uint32_t *p1 = (const uint32_t *)(sring + bn * AUX_NBLK_BYTES + off1);
+            acc[bn] = mfma32_16bit<T>(ubv, (v4i){(int)p0[0], (int)p0[1], (int)p1[0], (int)p1[1]}, acc[bn]);
+        }
+    };
+    int par = 0;                                         // parity of the group of four stages: ring slots 0-3 or 4-7
+    uint32_t rcur = (uint32_t)l32 * AUX_LROW;            // this lane's row in slot 0 / 4 of the current four stages
+    uint32_t rprev = rcur + (uint32_t)(4 + 2 * half) * AUX_LBLK;  // ... in its first stage of the previous four
+    if constexpr (!ACT_UNSIGNED) {
+        // the first stage applies a correction for four stages that never ran: its weight-side operand must be finite
+        v4i *z = (v4i *)(sring + wm * AUX_NBLK_BYTES + 4 * AUX_LBLK) + lane;
+        z[0] = z[64] = (v4i){0, 0, 0, 0};
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
+    }
+
+    load_regs(0);
+#pragma unroll
+    for (int i = 0; i < 4; i++) dma(0, sbuf0, 0, i);
+    fetch_epilogue_operands(a, sepi, n0, wm, lane);
+
+    // One stage = eight (group, weight block) steps: scale product, group product, sixteen FMAs, in program order.  The
+    // operands of the next step are read from LDS behind the matrix instructions.
+    auto stage = [&](auto st_tag, int s) {
+        constexpr int ST = decltype(st_tag)::value;   // stage within its group of four
+        uint8_t *base = (ST & 1) ? sbuf1 : sbuf0;     // this stage's operands
+        uint8_t *other = (ST & 1) ? sbuf0 : sbuf1;    // being refilled for the next stage
+        // everything this wavefront issued for stage s (registers, then blocks) has landed
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 15));
+        // two's complement nibble -> a + 8 is a flip of the nibble's top bit; -> a - 7 = -(7 - a) is a flip of the other
+        // three plus the fp8 sign bit: written per plane so that mask and flip are one three-input bit operation
+        v8i a8[2];
+#pragma unroll
+        for (int gg = 0; gg < 2; gg++) {
+            typedef unsigned v4u __attribute__((ext_vector_type(4)));
+            const v4u u = __builtin_bit_cast(v4u, araw[gg]);
+            const unsigned fe = ACT_UNSIGNED ? 0u : 0x08080808u, fo = ACT_UNSIGNED ? 0u : 0x87878787u;
+            const v4u e = (u & 0x0F0F0F0Fu) ^ fe, o = ((u >> 4) & 0x0F0F0F0Fu) ^ fo;
+            a8[gg] = (v8i){(int)e[0], (int)e[1], (int)e[2], (int)e[3], (int)o[0], (int)o[1], (int)o[2], (int)o[3]};
+        }
+        // Operands of the scale products as[m] * ws[n] for a 32x32x8 matrix instruction on 16-bit values: lanes 0-31 hold K
+        // slots 0-3, two to a register.  The weight side is the dword (ws of the first group, ws of the second group) as it
+        // lies in the ring; the activation side carries as of the step's group in that group's slot and zero elsewhere
+        // (also in lanes 32-63, whose weight-side values therefore do not matter).
+        const int qa0 = (int)qa[0], qa1 = (int)((uint32_t)qa[1] << 16);
+        const v2i sa[2] = {(v2i){half ? 0 : qa0, 0}, (v2i){half ? 0 : qa1, 0}};
+        __builtin_amdgcn_s_barrier();
+        if constexpr (!ACT_UNSIGNED) {
+            if constexpr (ST == 0) {
+                corr(rprev, rprev + AUX_LBLK);
+#pragma unroll
+                for (int e = 0; e < 4; e++) ub[e] = 0;
+            }
+            const bool mine = half == (ST >> 1);
+            ub[2 * (ST & 1)] = mine ? (qa0 | (qa0 << 16)) : ub[2 * (ST & 1)];
+            ub[2 * (ST & 1) + 1] = mine ? (qa1 | (int)((uint32_t)qa1 >> 16)) : ub[2 * (ST & 1) + 1];
+        }
+        uint32_t wsd[NBN];
+#pragma unroll
+        for (int bn = 0; bn < NBN; bn++) wsd[bn] = *(const uint32_t *)(sring + bn * AUX_NBLK_BYTES + ST * AUX_LBLK + 8 + rcur);
+        // The other buffer was last read in the previous stage, before the barrier: refill it during this stage.  The last
+        // stage re-fetches itself (harmless, and keeps the stage one basic block); its rows go to the next ring slot all
+        // the same, which nobody reads.
+        const int sn = min(s + 1, nstages - 1), slotn = (s + 1) & (AUX_SLOTS - 1);
+        load_regs(sn);
+        auto read_w8 = [&](int b) -> v8i {  // six registers of fp6 codes (the matrix instruction ignores the last two)
+            const int gg = b >> 2, bn = b & 3;
+            const v4i lo = *(const v4i *)(base + lane * 16 + (bn * WPL_BLOCKS + gg) * BLK_BYTES);
+            const v2i hi = *(const v2i *)(base + lane * 16 + (bn * WPL_BLOCKS + 2) * BLK_BYTES + gg * 8);
+            return (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], 0, 0};
+        };
+        const v16f z16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        v8i w8[2];
+        w8[0] = read_w8(0);
+#pragma unroll
+        for (int b = 0; b < 8; b++) {
+            // as[m] * ws[n] of the step, exact (two 16-bit values, one non-zero product): a 16-bit matrix instruction, which
+            // runs beside the vector FMAs; the fp32 rank-1 matrix instruction shares the vector ALUs and does not
+            const v16f S = mfma32_16bit_k8<T>(sa[b >> 2], (v2i){(int)wsd[b & 3], 0}, z16);
+            const v16f P = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8[b >> 2], w8[b & 1], z16, 0, 2, 0, F8_SCALE, 0, F6_SCALE);
+            __builtin_amdgcn_sched_barrier(0);
+            if (b + 1 < 8) w8[(b + 1) & 1] = read_w8(b + 1);
+            if (b < 4) dma(sn, other, slotn, b);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < 16; i++) acc[b & 3][i] = __builtin_fmaf(P[i], S[i], acc[b & 3][i]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    int s = 0;
+    for (; s + 4 <= nstages; s += 4) {
+        stage(std::integral_constant<int, 0>{}, s);
+        stage(std::integral_constant<int, 1>{}, s + 1);
+        stage(std::integral_constant<int, 2>{}, s + 2);
+        stage(std::integral_constant<int, 3>{}, s + 3);
+        par ^= 1;
+        rcur = (uint32_t)l32 * AUX_LROW + (uint32_t)(4 * par) * AUX_LBLK;
+        rprev = (uint32_t)l32 * AUX_LROW + (uint32_t)(4 * (par ^ 1) + 2 * half) * AUX_LBLK;
+    }
+    const int rem = nstages - s;  // 0 .. 3 stages of a last, partial group of four
+    if (rem >= 1) stage(std::integral_constant<int, 0>{}, s);
+    if (rem >= 2) stage(std::integral_constant<int, 1>{}, s + 1);
+    if (rem >= 3) stage(std::integral_constant<int, 2>{}, s + 2);
+    // The last stage's (redundant) loads of this wavefront have landed.
+    __builtin_amdgcn_s_waitcnt(waitcnt_imm(0, 0));
+    if constexpr (!ACT_UNSIGNED) {
+        if (rem == 0) {
+            corr(rprev, rprev + AUX_LBLK);
+        } else {
+            // a stage past the end reads the rows of the last real one: its activation-side entries are zero
+            const uint32_t r0 = (uint32_t)l32 * AUX_LROW + (uint32_t)(4 * par) * AUX_LBLK;
+            corr(r0 + (uint32_t)min(2 * half, rem - 1) * AUX_LBLK, r0 + (uint32_t)min(2 * half + 1, rem - 1) * AUX_LBLK);
+        }
+    }
+    // Every wavefront has left the main loop: the staging memory becomes the wavefronts' private epilogue memory.
+    __syncthreads();
+    uint8_t *priv = wm == 0 ? sbuf0 : wm == 1 ? sbuf1 : sring + (wm - 2) * PRIV_BYTES;
+    tile_epilogue<T, EPI>(a, acc, priv, sepi, m0, n0, pid_n, wm, lane);
+}
+
 // lora_act_out[m, r] = sum over n-tiles of the partial LoRA-down products, in tile order (deterministic)
 __global__ __launch_bounds__(64) void lora_part_reduce_kernel(const float *part, float *out, int tiles, int M, int R2,
                                                               int ld_out) {
@@ -1003,32 +1003,25 @@ __global__ __launch_bounds__(64) void group_acc_kernel(const uint8_t *act, const
     }
 }
 
-// The same read-out through the instruction sequence of the pre-split (fp8) path: activation nibbles as fp8 codes,
-// offset by 8 when signed, weights as fp6 codes, v_mfma_scale_f32_32x32x64_f8f6f4 with block scales 2^9 and 2^3, offset
-// taken out with the weights' group sum.  Every value involved is an integer below 2^24, so the fp32 result is exact.
+// The same read-out through the instruction sequence of the pre-split (fp8) path: activation nibbles as fp8 codes
+// (signed ones as a + 8 for even k and a - 7 for odd k), weights as fp6 codes,
+// v_mfma_scale_f32_32x32x64_f8f6f4 with block scales 2^9 and 2^3, offset term 8 We - 7 Wo taken out.  Every value involved
+// is an integer below 2^24, so the fp32 result is exact.
 template <bool ACT_UNSIGNED>
 __global__ __launch_bounds__(64) void group_acc_f8_kernel(const uint8_t *act, const uint8_t *wgt, int32_t *out, int M,
                                                           int N, int ld_act, int ld_wgt, int group) {
     typedef unsigned v4u __attribute__((ext_vector_type(4)));
     const int lane = threadIdx.x, l32 = lane & 31, half = lane >> 5;
     const int nb = blockIdx.x * 32, mb = blockIdx.y * 32;
-    const v4i wp = *(const v4i *)(wgt + (size_t)min(nb + l32, N - 1) * ld_wgt + group * 32 + half * 16);
-    v4u u = __builtin_bit_cast(v4u, *(const v4i *)(act + (size_t)min(mb + l32, M - 1) * ld_act + group * 32 + half * 16));
-    if (!ACT_UNSIGNED) u ^= 0x88888888u;
-    const v4u e = u & 0x0F0F0F0Fu, o = (u >> 4) & 0x0F0F0F0Fu;
+    const v4u u = __builtin_bit_cast(v4u, *(const v4i *)(act + (size_t)min(mb + l32, M - 1) * ld_act + group * 32 + half * 16));
+    const unsigned fe = ACT_UNSIGNED ? 0u : 0x08080808u, fo = ACT_UNSIGNED ? 0u : 0x87878787u;
+    const v4u e = (u & 0x0F0F0F0Fu) ^ fe, o = ((u >> 4) & 0x0F0F0F0Fu) ^ fo;
     const v8i a8 = {(int)e[0], (int)e[1], (int)e[2], (int)e[3], (int)o[0], (int)o[1], (int)o[2], (int)o[3]};
     uint32_t w6[6];
-    {
-        const uint8_t *wrow = wgt + (size_t)min(nb + l32, N - 1) * ld_wgt + group * 32;
-        f6_pack(*(const v4i *)wrow, *(const v4i *)(wrow + 16), half, w6);
-    }
+    const uint8_t *wrow = wgt + (size_t)min(nb + l32, N - 1) * ld_wgt + group * 32;
+    f6_pack(*(const v4i *)wrow, *(const v4i *)(wrow + 16), half, w6);
     const v8i w8 = {(int)w6[0], (int)w6[1], (int)w6[2], (int)w6[3], (int)w6[4], (int)w6[5], 0, 0};
-    int wsum = 0;
-#pragma unroll
-    for (int d = 0; d < 4; d++)
-#pragma unroll
-        for (int j = 0; j < 8; j++) wsum += (((wp[d] >> (4 * j)) & 0xF) ^ 8) - 8;
-    wsum += __shfl_xor(wsum, 32);  // the other half of the group
+    const int offs = ACT_UNSIGNED ? 0 : group_offset_term(*(const v4i *)wrow, *(const v4i *)(wrow + 16));
     const v16f z16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
     v16f t = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8, w8, z16, 0, 2, 0, F8_SCALE, 0, F6_SCALE);
     // The matrix instruction reads the operands of all 64 lanes: pin it here, ahead of the lane-dependent stores below
@@ -1038,49 +1031,63 @@ __global__ __launch_bounds__(64) void group_acc_f8_kernel(const uint8_t *act, co
 #pragma unroll
     for (int i = 0; i < 16; i++) {
         const int m = mb + 8 * (i >> 2) + 4 * half + (i & 3);
-        if (m < M && n < N) out[(size_t)m * N + n] = (int)t[i] - (ACT_UNSIGNED ? 0 : 8 * wsum);
+        if (m < M && n < N) out[(size_t)m * N + n] = (int)t[i] - offs;
     }
 }
 
-template <typename T, bool U, bool WPL, bool ODDG>
-static void launch_gemm_epi3(const svdq_gemm_args &a, hipStream_t s) {
+template <typename T, bool U, bool ODDG>
+static void launch_gemm_i8(const svdq_gemm_args &a, hipStream_t s) {
     const dim3 grid(((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN)), block(NTHREADS);
     switch (a.epilogue) {
         case SVDQ_EPI_PLAIN:
-            hipLaunchKernelGGL((gemm_w4a4_kernel<T, U, SVDQ_EPI_PLAIN, WPL, ODDG>), grid, block, 0, s, a);
+            hipLaunchKernelGGL((gemm_w4a4_i8_kernel<T, U, SVDQ_EPI_PLAIN, ODDG>), grid, block, 0, s, a);
             break;
         case SVDQ_EPI_QK_NORM_ROPE:
-            hipLaunchKernelGGL((gemm_w4a4_kernel<T, U, SVDQ_EPI_QK_NORM_ROPE, WPL, ODDG>), grid, block, 0, s, a);
+            hipLaunchKernelGGL((gemm_w4a4_i8_kernel<T, U, SVDQ_EPI_QK_NORM_ROPE, ODDG>), grid, block, 0, s, a);
             break;
         case SVDQ_EPI_GELU_QUANT:
-            hipLaunchKernelGGL((gemm_w4a4_kernel<T, U, SVDQ_EPI_GELU_QUANT, WPL, ODDG>), grid, block, 0, s, a);
+            hipLaunchKernelGGL((gemm_w4a4_i8_kernel<T, U, SVDQ_EPI_GELU_QUANT, ODDG>), grid, block, 0, s, a);
             break;
         case SVDQ_EPI_SWIGLU_QUANT:
-            hipLaunchKernelGGL((gemm_w4a4_kernel<T, U, SVDQ_EPI_SWIGLU_QUANT, WPL, ODDG>), grid, block, 0, s, a);
+            hipLaunchKernelGGL((gemm_w4a4_i8_kernel<T, U, SVDQ_EPI_SWIGLU_QUANT, ODDG>), grid, block, 0, s, a);
             break;
     }
 }
 
-template <typename T, bool U, bool WPL>
-static void launch_gemm_epi2(const svdq_gemm_args &a, hipStream_t s) {
-    if ((a.K / GROUP) & 1)
-        launch_gemm_epi3<T, U, WPL, true>(a, s);
-    else
-        launch_gemm_epi3<T, U, WPL, false>(a, s);
+template <typename T, bool U>
+static void launch_gemm_f8(const svdq_gemm_args &a, hipStream_t s) {
+    const dim3 grid(((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN)), block(NTHREADS);
+    switch (a.epilogue) {
+        case SVDQ_EPI_PLAIN:
+            hipLaunchKernelGGL((gemm_w4a4_f8_kernel<T, U, SVDQ_EPI_PLAIN>), grid, block, 0, s, a);
+            break;
+        case SVDQ_EPI_QK_NORM_ROPE:
+            hipLaunchKernelGGL((gemm_w4a4_f8_kernel<T, U, SVDQ_EPI_QK_NORM_ROPE>), grid, block, 0, s, a);
+            break;
+        case SVDQ_EPI_GELU_QUANT:
+            hipLaunchKernelGGL((gemm_w4a4_f8_kernel<T, U, SVDQ_EPI_GELU_QUANT>), grid, block, 0, s, a);
+            break;
+        case SVDQ_EPI_SWIGLU_QUANT:
+            hipLaunchKernelGGL((gemm_w4a4_f8_kernel<T, U, SVDQ_EPI_SWIGLU_QUANT>), grid, block, 0, s, a);
+            break;
+    }
 }
 
 template <typename T, bool U>
 static void launch_gemm_epi(const svdq_gemm_args &a, hipStream_t s) {
     if (a.wgt_planes != nullptr)
-        launch_gemm_epi2<T, U, true>(a, s);
+        launch_gemm_f8<T, U>(a, s);
+    else if ((a.K / GROUP) & 1)
+        launch_gemm_i8<T, U, true>(a, s);
     else
-        launch_gemm_epi2<T, U, false>(a, s);
+        launch_gemm_i8<T, U, false>(a, s);
 }
 
-// weight re-layout: thread (block of 32 rows, stage of two groups, lane) turns the nibbles of its parity of each group's
-// 32 packed bytes into six registers of fp6 codes; a group past the end (K / 64 odd) is stored as zeros
-__global__ void split_weight_planes_kernel(const uint8_t *wgt, uint8_t *planes, int N, int G, int ld_wgt) {
+// Weight re-layout, codes: thread (block of 32 rows, stage of two groups, lane) turns the nibbles of its parity of each
+// group's 32 packed bytes into six registers of fp6 codes; a group past the end (K / 64 odd) is stored as zeros.  Thread 0 clears the status word.
+__global__ void split_weight_planes_kernel(const uint8_t *wgt, uint8_t *planes, int32_t *status, int N, int G, int ld_wgt) {
     const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx == 0) *status = 0;  // the kernel that may raise it runs after this one
     const int lane = idx & 63;
     const size_t bs = idx >> 6;  // nblk * nst + s
     const int nst = (G + 1) / 2;
@@ -1101,37 +1108,45 @@ __global__ void split_weight_planes_kernel(const uint8_t *wgt, uint8_t *planes, 
     }
 }
 
-// D[g, n] = -8 * ws[g, n] * (sum of the 64 weights of group g in row n), exact in fp32, written as NPIECE T values whose
-// sum is D to 16 (bf16) or 22 (fp16) significant bits, exactly when D is an integer below 2^16 (a third piece was
-// measured: it changes no requantized code at the FLUX fc1 shape and costs 4 % of the launch):
-// dpieces[n][piece * G16 + g]; rows >= N and groups >= G are zero.
+// Weight re-layout, scales and offset terms: thread (block of 32 rows, stage, row of the block) writes the row's six
+// 16-bit values of the stage: for each of the two groups the pieces hi, lo of
+// D = -ws * (8 * sum of the even-k weights - 7 * sum of the odd-k weights)  (the product is exact in fp32; hi + lo carry it
+// to 16 significant bits in bf16, 22 in fp16), then the two weight scales.  Rows past N repeat row N - 1; a group past the
+// end and the stage of padding behind each block's last stage are zeros.  `status` is set to 1 when a piece is not finite
+// (fp16 scales of about 17 and more), in which case the copy must not be used.
 template <typename T>
-__global__ void weight_group_sums_kernel(const uint8_t *wgt, const uint16_t *wscales, uint16_t *dpieces, int N, int npad,
-                                         int G, int G16, int ld_wgt, int ld_wscales) {
+__global__ void weight_aux_kernel(const uint8_t *wgt, const uint16_t *wscales, uint16_t *aux, int32_t *status, int N, int G,
+                                  int ld_wgt, int ld_wscales) {
     const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    const int g = (int)(idx % G16), n = (int)(idx / G16);
-    if (n >= npad) return;
-    float d = 0.0f;
-    if (n < N && g < G) {
-        int w = 0;
-        const v4i *src = (const v4i *)(wgt + (size_t)n * ld_wgt + g * 32);
+    const int r = idx & 31;
+    const size_t bs = idx >> 5;  // nblk * (nst + 1) + s
+    const int nst = (G + 1) / 2;
+    const int s = (int)(bs % (nst + 1)), nblk = (int)(bs / (nst + 1));
+    if (nblk >= (N + 31) / 32) return;
+    const int row = min(nblk * 32 + r, N - 1);
+    uint16_t v[6] = {0, 0, 0, 0, 0, 0};
+    bool bad = false;
 #pragma unroll
-        for (int h = 0; h < 2; h++) {
-            const v4i p = src[h];
-#pragma unroll
-            for (int e = 0; e < 4; e++)
-#pragma unroll
-                for (int j = 0; j < 8; j++) w += (((p[e] >> (4 * j)) & 0xF) ^ 8) - 8;
+    for (int gg = 0; gg < 2; gg++) {
+        const int g = 2 * s + gg;
+        if (s < nst && g < G) {
+            const uint8_t *src = wgt + (size_t)row * ld_wgt + g * 32;
+            const uint16_t ws = wscales[(size_t)g * ld_wscales + row];
+            float d = -(T::to_f32(ws) * (float)group_offset_term(*(const v4i *)src, *(const v4i *)(src + 16)));
+            const uint16_t hi = T::from_f32(d);
+            d -= T::to_f32(hi);
+            const uint16_t lo = T::from_f32(d);
+            bad = bad || !isfinite(T::to_f32(hi)) || !isfinite(T::to_f32(lo)) || !isfinite(T::to_f32(ws));
+            v[2 * gg] = hi;
+            v[2 * gg + 1] = lo;
+            v[4 + gg] = ws;
         }
-        d = -8.0f * (T::to_f32(wscales[(size_t)g * ld_wscales + n]) * (float)w);
     }
-    uint16_t *dst = dpieces + (size_t)n * NPIECE * G16 + g;
-#pragma unroll
-    for (int pc = 0; pc < NPIECE; pc++) {
-        const uint16_t h = T::from_f32(d);
-        dst[pc * G16] = h;
-        d -= T::to_f32(h);
-    }
+    uint32_t *dst = (uint32_t *)(aux + idx * 6);
+    dst[0] = (uint32_t)v[0] | ((uint32_t)v[1] << 16);
+    dst[1] = (uint32_t)v[2] | ((uint32_t)v[3] << 16);
+    dst[2] = (uint32_t)v[4] | ((uint32_t)v[5] << 16);
+    if (bad) *status = 1;
 }
 
 }  // namespace svdq
@@ -1142,9 +1157,7 @@ static bool al16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
 extern "C" size_t svdq_weight_planes_bytes(int32_t N, int32_t K) {
     if (N <= 0 || K <= 0) return 0;
-    const size_t npad = (size_t)((N + 31) / 32) * 32, g16 = (size_t)((K / GROUP + 15) / 16) * 16;
-    const size_t nst = (size_t)(K / GROUP + 1) / 2;
-    return npad / 32 * nst * (WPL_BLOCKS * BLK_BYTES) + npad * NPIECE * g16 * 2;  // fp6 codes, then the 16-bit pieces of D[g, n]
+    return planes_code_bytes(N, K) + planes_aux_bytes(N, K) + PLANES_STATUS_BYTES;  // fp6 codes, scales and offset terms, status word
 }
 
 extern "C" int svdq_split_weight_planes(const void *wgt, const void *wscales, void *planes, int32_t N, int32_t K,
@@ -1155,21 +1168,23 @@ extern "C" int svdq_split_weight_planes(const void *wgt, const void *wscales, vo
                   N, K, ld_wgt, ld_wscales, dtype);
         return SVDQ_E_INVALID;
     }
-    const int G = K / GROUP, G16 = (G + 15) / 16 * 16, npad = (N + 31) / 32 * 32;
-    const size_t n = (size_t)(npad / 32) * ((G + 1) / 2) * 64;
-    hipLaunchKernelGGL(split_weight_planes_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
-                       (const uint8_t *)wgt, (uint8_t *)planes, N, G, ld_wgt);
+    const int G = K / GROUP, nblk = (N + 31) / 32, nst = (G + 1) / 2;
+    hipStream_t st = (hipStream_t)stream;
+    uint8_t *aux = (uint8_t *)planes + planes_code_bytes(N, K);
+    int32_t *status = (int32_t *)(aux + planes_aux_bytes(N, K));
+    const size_t n = (size_t)nblk * nst * 64;
+    hipLaunchKernelGGL(split_weight_planes_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st,
+                       (const uint8_t *)wgt, (uint8_t *)planes, status, N, G, ld_wgt);
     int rc = check_launch("svdq_split_weight_planes");
     if (rc) return rc;
-    uint16_t *dpieces = (uint16_t *)((uint8_t *)planes + (size_t)(npad / 32) * ((G + 1) / 2) * (WPL_BLOCKS * BLK_BYTES));
-    const size_t nd = (size_t)npad * G16;
+    const size_t nd = (size_t)nblk * (nst + 1) * 32;
     if (dtype == SVDQ_BF16)
-        hipLaunchKernelGGL(weight_group_sums_kernel<BF16>, dim3((unsigned)((nd + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
-                           (const uint8_t *)wgt, (const uint16_t *)wscales, dpieces, N, npad, G, G16, ld_wgt, ld_wscales);
+        hipLaunchKernelGGL(weight_aux_kernel<BF16>, dim3((unsigned)((nd + 255) / 256)), dim3(256), 0, st,
+                           (const uint8_t *)wgt, (const uint16_t *)wscales, (uint16_t *)aux, status, N, G, ld_wgt, ld_wscales);
     else
-        hipLaunchKernelGGL(weight_group_sums_kernel<FP16>, dim3((unsigned)((nd + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
-                           (const uint8_t *)wgt, (const uint16_t *)wscales, dpieces, N, npad, G, G16, ld_wgt, ld_wscales);
-    return check_launch("svdq_split_weight_planes (group sums)");
+        hipLaunchKernelGGL(weight_aux_kernel<FP16>, dim3((unsigned)((nd + 255) / 256)), dim3(256), 0, st,
+                           (const uint8_t *)wgt, (const uint16_t *)wscales, (uint16_t *)aux, status, N, G, ld_wgt, ld_wscales);
+    return check_launch("svdq_split_weight_planes (scales and offset terms)");
 }
 
 extern "C" size_t svdq_gemm_w4a4_scratch_bytes(int32_t M, int32_t N, int32_t R2, int32_t epilogue) {

@@ -89,17 +89,20 @@ def lora_down_t(lora_down: torch.Tensor) -> torch.Tensor:
 _planes_cache: dict[int, tuple] = {}
 
 
-def weight_planes(qweight: torch.Tensor, wscales: torch.Tensor) -> torch.Tensor:
+def weight_planes(qweight: torch.Tensor, wscales: torch.Tensor) -> torch.Tensor | None:
     """The GEMM's working copy of a packed ``(N, K/2)`` weight (``svdq_split_weight_planes``): six-bit fp6 codes in
-    MFMA lane order, followed by the per-group weight sums times ``-8 * wscales`` that take the offset of signed
-    activations out again.  Made on first use and kept while both tensors live unmodified.  Costs ``0.75 * N * K``
-    bytes (one and a half times the packed weight) plus ``4 * N * K / 64`` bytes."""
+    MFMA lane order, followed by the weight scales and the per-group terms that take the offset of signed activations
+    out again.  Made on first use and kept while both tensors live unmodified.  Costs ``0.75 * N * K`` bytes (one and a
+    half times the packed weight) plus ``6 * N * K / 64`` bytes.  ``None`` when the offset terms do not fit the 16-bit
+    type (fp16 scales of about 17 and more): the caller then uses the packed weight.  Reading that status word waits for
+    the re-layout once, when the copy is made."""
     key = id(qweight)
     hit = _planes_cache.get(key)
     if hit is not None:
         ref, src, src_s, t, ready = hit
         if ref() is qweight and _same_source(src, qweight) and _same_source(src_s, wscales):
-            ready.wait(t.device)
+            if t is not None:
+                ready.wait(t.device)
             return t
     N, K = qweight.shape[0], qweight.shape[1] * 2
     lib = _lib.load()
@@ -108,6 +111,8 @@ def weight_planes(qweight: torch.Tensor, wscales: torch.Tensor) -> torch.Tensor:
         _lib.check(lib.svdq_split_weight_planes(qweight.data_ptr(), wscales.data_ptr(), t.data_ptr(), N, K, qweight.stride(0),
                                                 wscales.stride(0), _lib.dtype_code(wscales.dtype), _lib.stream_of(qweight)))  # fmt: skip
         ready = _Ready(t.device)
+        if int(t[-16:-12].view(torch.int32).item()) != 0:  # a piece of an offset term is not finite
+            t = None
     try:
         ref = weakref.ref(qweight, lambda _r, k=key: _planes_cache.pop(k, None))
         _planes_cache[key] = (ref, _source_of(qweight), _source_of(wscales), t, ready)

@@ -142,7 +142,7 @@ def test_strided_row_views(dev):
 
 
 @pytest.mark.parametrize("M", [1024, 4608, 8192])
-def test_flux_qkv_shapes_quantizer_then_gemm(dev, M):
+def test_flux_qkv_shapes_quantizer_then_gemm(dev, M, main_loop):
     """The benchmark linear (K=3072, N=9216, R=32): quantizer -> GEMM on the GPU; oracle on the same seeded inputs.
     The oracle runs on a row sample (rows are independent), all groups of which are also checked bit-exactly."""
     from nunchaku_rocm_amd import ops
@@ -167,7 +167,7 @@ def test_flux_qkv_shapes_quantizer_then_gemm(dev, M):
     print(f"M={M}: max rel err {err:.3e}", flush=True)
     assert err <= TOL
     for g in (0, 17, 47):
-        got = group_acc_i32(qx[rows].contiguous(), dl["qweight"], g).cpu()
+        got = group_acc_i32(qx[rows].contiguous(), dl["qweight"], g, fp8_path=main_loop == "all").cpu()
         assert torch.equal(got, O.group_acc_i32(rp, lin["qweight"], False, groups=[g])[0])
 
 
@@ -237,9 +237,10 @@ def test_linear_module_matches_dequantised_reference(dev):
 def _planes_expected(wgt, wsc, N, K):
     """Host restatement of the pre-split weight layout.  Per (block of 32 rows, stage of two groups) three 1 KB blocks:
     a lane (= parity * 32 + row) holds, per group, 32 six-bit codes sign | magnitude (position p = the nibble of its parity
-    of the row's packed byte p of the group; code p in bits 6 p .. 6 p + 5 of 24 little-endian bytes); blocks 0 and 1 = bytes
-    0-15 of the stage's two groups, block 2 = bytes 16-23 of both.  A group past the end is zeros.  Then per row two 16-bit
-    pieces (hi, lo) per group (piece-major, groups padded to 16) of -8 * wscale * (sum of the group's weights)."""
+    of the row's packed byte p of the group; code p in bits 6 p .. 6 p + 5 of 24 little-endian bytes); blocks 0 and 1 = bytes 0-15 of the stage's two groups, block 2 = bytes 16-23 of both.  A group past the end is
+    zeros.  Then per (block of rows, stage; one stage of zero padding behind the last) 32 rows of six 16-bit values: for
+    each of the stage's two groups the pieces (hi, lo) of -wscale * (8 * sum of the even-k weights - 7 * sum of the odd-k
+    weights), then the two weight scales.  Last, a 16-byte status word (0 = usable)."""
     import numpy as np
 
     nb, G = (N + 31) // 32, K // 64
@@ -247,6 +248,7 @@ def _planes_expected(wgt, wsc, N, K):
     q = O.unpack_int4(wgt, signed=True).to(torch.int16)  # (N, K) in [-8, 7]
     rows = torch.arange(nb * 32).clamp(max=N - 1)
     qb = q[rows].view(nb, 32, G, 32, 2)  # (nblk, row in block, g, packed byte, even/odd nibble)
+    offs = 8 * qb[..., 0].sum(-1) - 7 * qb[..., 1].sum(-1)  # (nblk, row, g)
     code = (qb.abs() | ((qb < 0).to(torch.int16) << 5)).to(torch.uint8)
     code = code.permute(0, 2, 4, 1, 3).reshape(nb, G, 64, 32)  # (nblk, g, lane = parity * 32 + row, position = byte)
     full = torch.zeros(nb, nst * 2, 64, 32, dtype=torch.uint8)
@@ -258,14 +260,16 @@ def _planes_expected(wgt, wsc, N, K):
     planes[:, :, 1] = by[:, :, 1, :, :16]
     planes[:, :, 2, :, :8] = by[:, :, 0, :, 16:]
     planes[:, :, 2, :, 8:] = by[:, :, 1, :, 16:]
-    G16 = (G + 15) // 16 * 16
-    d = torch.zeros(nb * 32, G16, dtype=torch.float32)
-    d[:N, :G] = -8.0 * (wsc.float().t()[:N] * q.view(N, G, 64).sum(-1).float())
-    pieces = torch.zeros(nb * 32, 2, G16, dtype=wsc.dtype)
-    for pc in range(2):
-        pieces[:, pc] = d.to(wsc.dtype)
-        d = d - pieces[:, pc].float()
-    return planes, pieces
+    ws = wsc.t()[rows].reshape(nb, 32, G)  # (nblk, row, g)
+    d = -(ws.float() * offs.float())
+    aux = torch.zeros(nb, nst + 1, 32, 6, dtype=wsc.dtype)
+    for g in range(G):
+        s, gg = divmod(g, 2)
+        hi = d[:, :, g].to(wsc.dtype)
+        aux[:, s, :, 2 * gg] = hi
+        aux[:, s, :, 2 * gg + 1] = (d[:, :, g] - hi.float()).to(wsc.dtype)
+        aux[:, s, :, 4 + gg] = ws[:, :, g]
+    return planes, aux
 
 
 @pytest.mark.parametrize("N,K", [(32, 64), (264, 256), (100, 128), (64, 2048), (72, 320)])
@@ -276,30 +280,55 @@ def test_weight_planes_layout(dev, N, K):
     wgt = torch.randint(0, 256, (N, K // 2), generator=g, dtype=torch.uint8)
     wsc = (torch.rand(K // 64, N, generator=g) * 0.02 + 0.005).to(torch.bfloat16)
     got = weight_planes(wgt.to(dev), wsc.to(dev)).cpu()
-    planes, pieces = _planes_expected(wgt, wsc, N, K)
-    assert got.numel() == planes.numel() + pieces.numel() * 2
+    planes, aux = _planes_expected(wgt, wsc, N, K)
+    assert got.numel() == planes.numel() + aux.numel() * 2 + 16
     assert torch.equal(got[: planes.numel()], planes.view(-1))
-    assert torch.equal(got[planes.numel() :].view(torch.int16), pieces.view(torch.int16).view(-1))
+    assert torch.equal(got[planes.numel() : -16].view(torch.int16), aux.view(torch.int16).view(-1))
+    assert int(got[-16:-12].view(torch.int32)) == 0
+
+
+def test_weight_planes_refuse_scales_beyond_fp16(dev):
+    """fp16 weight scales so large that -ws * (8 We - 7 Wo) overflows a 16-bit piece: the re-layout raises its status word and
+    the operator falls back to the packed weight (int8 main loop) instead of producing NaN."""
+    from nunchaku_rocm_amd.ops import gemm as gemm_mod
+    from nunchaku_rocm_amd.ops._prep import weight_planes
+
+    p = _rand_problem(64, 128, 256, 0, torch.float16, seed=3)
+    p["wsc"] = (p["wsc"].float() * 4000).to(torch.float16)  # about 20 .. 80
+    assert weight_planes(p["wgt"].to(dev), p["wsc"].to(dev)) is None
+    old = gemm_mod.USE_WEIGHT_PLANES
+    try:
+        gemm_mod.USE_WEIGHT_PLANES = "all"
+        out = _gpu_gemm(p, dev, dtype=torch.float16)
+    finally:
+        gemm_mod.USE_WEIGHT_PLANES = old
+    assert torch.isfinite(out.float()).all()
+    ref = O.gemm_w4a4(p["act"], p["wgt"], p["asc"], p["wsc"], bias=p["bias"], lora_act=p["la"], lora_up=p["lu"])
+    assert O.max_rel_err(out.float(), ref) <= TOL
 
 
 @pytest.mark.parametrize("unsigned", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M,N,K,R", [(136, 264, 256, 16), (256, 512, 1024, 32), (64, 72, 128, 0), (300, 3072, 3072, 32),
-                                     (100, 136, 64, 16), (257, 264, 320, 0)])  # the last two: K / 64 odd
-def test_presplit_weights_against_packed(dev, M, N, K, R, unsigned):
+                                     (100, 136, 64, 16), (257, 264, 320, 0),  # K / 64 odd
+                                     # long K: the offset of signed activations is taken out every four stages (512 of K); these
+                                     # end on 1, 0, 0, 3 and 2 stages of a last partial set
+                                     (100, 136, 4160, 16), (64, 264, 5120, 0), (64, 128, 6144, 32), (96, 128, 896, 0), (40, 136, 768, 16)])
+def test_presplit_weights_against_packed(dev, M, N, K, R, unsigned, dtype):
     """The two main loops (int8 MFMA on packed weights, fp8 MFMA on pre-split weights) compute the same integer group sums
     and differ only in the order of fp32 roundings: outputs agree to one 16-bit ulp of the largest value."""
-    print(f"case M={M} N={N} K={K} R={R} unsigned={unsigned}", flush=True)
-    p = _rand_problem(M, N, K, R, torch.bfloat16, seed=7 + M)
+    print(f"case M={M} N={N} K={K} R={R} unsigned={unsigned} {dtype}", flush=True)
+    p = _rand_problem(M, N, K, R, dtype, seed=7 + M)
     from nunchaku_rocm_amd.ops import gemm as gemm_mod
 
     old = gemm_mod.USE_WEIGHT_PLANES
     try:
         gemm_mod.USE_WEIGHT_PLANES = "none"
-        packed = _gpu_gemm(p, dev, unsigned=unsigned)
+        packed = _gpu_gemm(p, dev, unsigned=unsigned, dtype=dtype)
         gemm_mod.USE_WEIGHT_PLANES = "all"
-        split = _gpu_gemm(p, dev, unsigned=unsigned)
+        split = _gpu_gemm(p, dev, unsigned=unsigned, dtype=dtype)
     finally:
         gemm_mod.USE_WEIGHT_PLANES = old
-    assert O.max_rel_err(split.float(), packed.float()) <= 2.0**-7
+    assert O.max_rel_err(split.float(), packed.float()) <= (2.0**-7 if dtype == torch.bfloat16 else 2.0**-10)
     ref = O.gemm_w4a4(p["act"], p["wgt"], p["asc"], p["wsc"], bias=p["bias"], lora_act=p["la"], lora_up=p["lu"], act_unsigned=unsigned)
     assert O.max_rel_err(split.float(), ref) <= TOL
