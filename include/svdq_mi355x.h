@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define SVDQ_ABI_VERSION 6
+#define SVDQ_ABI_VERSION 7
 
 enum { SVDQ_BF16 = 0, SVDQ_FP16 = 1 };
 enum { SVDQ_PRE_NONE = 0, SVDQ_PRE_GLU = 1, SVDQ_PRE_GELU = 2 }; /* svdq_quantize_args.prologue */
@@ -151,6 +151,12 @@ typedef struct {
 } svdq_gemm_args;
 
 int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream);
+
+/* The fp8 main loop exists in two builds: three workgroups per CU (fills a loaded CU best) and two per CU with
+ * software-pipelined steps (a workgroup on its own runs faster); svdq_gemm_w4a4 picks by the number of 128x128 tiles and
+ * CUs.  This overrides the choice for the whole process: -1 = by tile count (default), 0 = three per CU, 1 = two per CU.
+ * For tuning and tests; results of the two are bit-identical.  No counterpart in the reference. */
+int svdq_gemm_w4a4_set_variant(int32_t variant);
 
 /*
  * One-time re-layout of a weight for the GEMM.  Every (32-row block, pair of scale groups) becomes three 1 KB blocks of

@@ -14,7 +14,7 @@ import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libsvdq_mi355x.so")
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 BF16, FP16 = 0, 1
 EPI_PLAIN, EPI_QK_NORM_ROPE, EPI_GELU_QUANT, EPI_SWIGLU_QUANT = 0, 1, 2, 3
@@ -27,6 +27,7 @@ EXPORTS = (
     "svdq_gated_residual",
     "svdq_transpose_lora_down",
     "svdq_gemm_w4a4",
+    "svdq_gemm_w4a4_set_variant",
     "svdq_gemm_w4a4_scratch_bytes",
     "svdq_gemm_w4a4_static_scratch",
     "svdq_gemm_w4a4_static_scratch_capacity",
@@ -124,6 +125,7 @@ def load() -> ctypes.CDLL:
     lib.svdq_row_stats.argtypes = [_vp, _vp, _i32, _i32, _i32, _i32, _f32, _vp]
     lib.svdq_quantize_act.argtypes = [ctypes.POINTER(QuantizeArgs), _vp]
     lib.svdq_gemm_w4a4.argtypes = [ctypes.POINTER(GemmArgs), _vp]
+    lib.svdq_gemm_w4a4_set_variant.argtypes = [_i32]
     lib.svdq_gemm_w4a4_static_scratch.argtypes = [ctypes.POINTER(GemmArgs), _vp]
     lib.svdq_gemm_w4a4_static_scratch_capacity.restype = ctypes.c_size_t
     lib.svdq_gemm_w4a4_static_scratch_capacity.argtypes = []

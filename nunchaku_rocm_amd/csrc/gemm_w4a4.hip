@@ -44,6 +44,7 @@
 //    after it.
 //  * Workgroup ids are first regrouped so that each XCD (ids are dealt round-robin over 8 XCDs) works on a
 //    contiguous range of tiles, then swizzled in bands of m-tiles for L2 reuse of the weight tile.
+#include <algorithm>
 #include <atomic>
 #include <type_traits>
 
@@ -354,27 +355,13 @@ __device__ __forceinline__ void tile_epilogue(const svdq_gemm_args &a, v16f (&ac
 
     if (EPI == SVDQ_EPI_GELU_QUANT) {
         const uint16_t *ldt = (const uint16_t *)a.lora_down_t;
-        // loads whose values are needed further down, issued before the GELU arithmetic: the next layer's smoothing
-        // factors of columns lane and 64 + lane and the first 32 ranks of its LoRA-down weight
+        // needed further down, issued before the GELU arithmetic: the next layer's smoothing factors of columns lane and
+        // 64 + lane
         uint16_t smv[2] = {0, 0};
         const bool has_sm = a.smooth_next != nullptr;
         if (has_sm) {
 #pragma unroll
             for (int t = 0; t < 2; t++) smv[t] = ((const uint16_t *)a.smooth_next)[min(n0 + 64 * t + lane, a.N - 1)];
-        }
-        uint2 lq[NBN][2][2];
-        if (a.R2 > 0) {
-#pragma unroll
-            for (int bn = 0; bn < NBN; bn++)
-#pragma unroll
-                for (int s = 0; s < 2; s++) {
-                    lq[bn][s][0] = lq[bn][s][1] = make_uint2(0u, 0u);
-                    if (l32 < a.R2) {
-                        const uint16_t *lp = ldt + (size_t)l32 * a.N + n0 + bn * 32 + 16 * s + 4 * half;
-                        lq[bn][s][0] = *(const uint2 *)lp;
-                        lq[bn][s][1] = *(const uint2 *)(lp + 8);
-                    }
-                }
         }
         if (a.out != nullptr) store_out();  // pre-GELU output, when asked for
 #pragma unroll
@@ -395,9 +382,7 @@ __device__ __forceinline__ void tile_epilogue(const svdq_gemm_args &a, v16f (&ac
 #pragma unroll
                 for (int s = 0; s < 2; s++) {
                     v4i la = (v4i){0, 0, 0, 0};
-                    if (rc == 0) {
-                        la = (v4i){(int)lq[bn][s][0].x, (int)lq[bn][s][0].y, (int)lq[bn][s][1].x, (int)lq[bn][s][1].y};
-                    } else if (r < a.R2) {
+                    if (r < a.R2) {
                         const uint16_t *lp = ldt + (size_t)r * a.N + n0 + bn * 32 + 16 * s + 4 * half;
                         const uint2 q0 = *(const uint2 *)lp, q1 = *(const uint2 *)(lp + 8);
                         la = (v4i){(int)q0.x, (int)q0.y, (int)q1.x, (int)q1.y};
@@ -770,8 +755,11 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_i8_kernel(svdq_gemm_arg
 }
 
 // ---- pre-split weights: fp8 x fp6 main loop --------------------------------------------------------------------------------
-template <typename T, bool ACT_UNSIGNED, int EPI>
-__global__ __launch_bounds__(NTHREADS, 3) void gemm_w4a4_f8_kernel(svdq_gemm_args a) {
+// PIPE = false: held to 168 registers, three workgroups per CU, a step's matrix instructions and FMAs in program order.
+// PIPE = true: two workgroups per CU, the matrix instructions of step b + 1 issued ahead of the FMAs of step b (two sets
+// of result registers): a workgroup on its own runs faster, which pays when few, long tiles leave CUs half empty.
+template <typename T, bool ACT_UNSIGNED, int EPI, bool PIPE>
+__global__ __launch_bounds__(NTHREADS, PIPE ? 2 : 3) void gemm_w4a4_f8_kernel(svdq_gemm_args a) {
     // Separate LDS objects: the compiler then knows that a block load into one staging buffer cannot touch what is being
     // read from the other (one object would make every LDS read wait for the loads in flight).
     __shared__ __align__(16) uint8_t sbuf0[F8_STAGE_BYTES];
@@ -866,8 +854,8 @@ __global__ __launch_bounds__(NTHREADS, 3) void gemm_w4a4_f8_kernel(svdq_gemm_arg
     for (int i = 0; i < 4; i++) dma(0, sbuf0, 0, i);
     fetch_epilogue_operands(a, sepi, n0, wm, lane);
 
-    // One stage = eight (group, weight block) steps: scale product, group product, sixteen FMAs, in program order.  The
-    // operands of the next step are read from LDS behind the matrix instructions.
+    // One stage = eight (group, weight block) steps: scale product, group product, sixteen FMAs.  The operands of the next
+    // step (the step after next when PIPE) are read from LDS behind the matrix instructions.
     auto stage = [&](auto st_tag, int s) {
         constexpr int ST = decltype(st_tag)::value;   // stage within its group of four
         uint8_t *base = (ST & 1) ? sbuf1 : sbuf0;     // this stage's operands
@@ -917,21 +905,51 @@ __global__ __launch_bounds__(NTHREADS, 3) void gemm_w4a4_f8_kernel(svdq_gemm_arg
             return (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], 0, 0};
         };
         const v16f z16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-        v8i w8[2];
-        w8[0] = read_w8(0);
+        // as[m] * ws[n] of a step, exact (two 16-bit values, one non-zero product): a 16-bit matrix instruction, which runs
+        // beside the vector FMAs; the fp32 rank-1 matrix instruction shares the vector ALUs and does not
+        auto scales = [&](int b) -> v16f { return mfma32_16bit_k8<T>(sa[b >> 2], (v2i){(int)wsd[b & 3], 0}, z16); };
+        auto group = [&](int b, const v8i &w) -> v16f {
+            return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8[b >> 2], w, z16, 0, 2, 0, F8_SCALE, 0, F6_SCALE);
+        };
+        if constexpr (!PIPE) {
+            v8i w8[2];
+            w8[0] = read_w8(0);
 #pragma unroll
-        for (int b = 0; b < 8; b++) {
-            // as[m] * ws[n] of the step, exact (two 16-bit values, one non-zero product): a 16-bit matrix instruction, which
-            // runs beside the vector FMAs; the fp32 rank-1 matrix instruction shares the vector ALUs and does not
-            const v16f S = mfma32_16bit_k8<T>(sa[b >> 2], (v2i){(int)wsd[b & 3], 0}, z16);
-            const v16f P = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8[b >> 2], w8[b & 1], z16, 0, 2, 0, F8_SCALE, 0, F6_SCALE);
-            __builtin_amdgcn_sched_barrier(0);
-            if (b + 1 < 8) w8[(b + 1) & 1] = read_w8(b + 1);
-            if (b < 4) dma(sn, other, slotn, b);
-            __builtin_amdgcn_sched_barrier(0);
+            for (int b = 0; b < 8; b++) {
+                const v16f S = scales(b);
+                const v16f P = group(b, w8[b & 1]);
+                __builtin_amdgcn_sched_barrier(0);
+                if (b + 1 < 8) w8[(b + 1) & 1] = read_w8(b + 1);
+                if (b < 4) dma(sn, other, slotn, b);
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int i = 0; i < 16; i++) acc[b & 3][i] = __builtin_fmaf(P[i], S[i], acc[b & 3][i]);
-            __builtin_amdgcn_sched_barrier(0);
+                for (int i = 0; i < 16; i++) acc[b & 3][i] = __builtin_fmaf(P[i], S[i], acc[b & 3][i]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        } else {
+            v8i w8[3];
+            v16f S[2], P[2];
+            w8[0] = read_w8(0);
+            w8[1] = read_w8(1);
+            S[0] = scales(0);
+            P[0] = group(0, w8[0]);
+#pragma unroll
+            for (int b = 0; b < 8; b++) {
+                const int cur = b & 1, nxt = cur ^ 1;
+                if (b + 1 < 8) {
+                    S[nxt] = scales(b + 1);
+                    P[nxt] = group(b + 1, w8[(b + 1) % 3]);
+                }
+                // the operand reads of step b + 2 stay behind the matrix instructions: hoisted above them, the wait for step
+                // b + 1's operands would also wait for these
+                __builtin_amdgcn_sched_barrier(0);
+                if (b + 2 < 8) w8[(b + 2) % 3] = read_w8(b + 2);
+                if (b < 4) dma(sn, other, slotn, b);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int i = 0; i < 16; i++) acc[b & 3][i] = __builtin_fmaf(P[cur][i], S[cur][i], acc[b & 3][i]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         }
     };
     int s = 0;
@@ -1054,23 +1072,61 @@ static void launch_gemm_i8(const svdq_gemm_args &a, hipStream_t s) {
     }
 }
 
-template <typename T, bool U>
-static void launch_gemm_f8(const svdq_gemm_args &a, hipStream_t s) {
+// Workgroups per CU for the fp8 kernel.  Three (PIPE = false) keep a full CU about 8 % busier than two (PIPE = true), but a
+// workgroup of the two-per-CU kernel runs faster, which decides when the last round of tiles leaves most CUs with one or
+// two workgroups.  Cost model, in units of a tile's share of a fully loaded three-per-CU CU: whole rounds cost 3 (three per
+// CU) or 2 * 1.08 (two per CU); a last round whose fullest CU holds k tiles costs 1.75 / 2.15 / 3 (k = 1 / 2 / 3) or
+// 1.4 / 2 (k = 1 / 2).  The constants are measured (K = 3072, N = 9216: M = 512 -> 288 tiles, M = 1024 -> 576, M = 4608 -> 2592;
+// K = 12288, N = 3072, M = 4608 -> 864), and the model picks as the measurements do: 2592, 3456, 4608 and 576 tiles -> three per
+// CU; 864 and 288 tiles -> two.
+static int cu_count() {
+    static std::atomic<int> cached{0};
+    int n = cached.load(std::memory_order_relaxed);
+    if (n > 0) return n;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+        n = 256;
+    cached.store(n, std::memory_order_relaxed);
+    return n;
+}
+static std::atomic<int> g_f8_variant{-1};  // svdq_gemm_w4a4_set_variant
+static bool two_workgroups_per_cu(long tiles) {
+    const int forced = g_f8_variant.load(std::memory_order_relaxed);
+    if (forced >= 0) return forced == 1;
+    const long cus = cu_count();
+    auto cost = [&](long occ, double round, const double (&last)[3]) {
+        const long full = tiles / (cus * occ), rem = tiles - full * cus * occ;
+        return (double)full * round + (rem == 0 ? 0.0 : last[(rem + cus - 1) / cus - 1]);
+    };
+    const double last3[3] = {1.75, 2.15, 3.0}, last2[3] = {1.4, 2.0, 2.0};
+    return cost(2, 2.16, last2) < cost(3, 3.0, last3);
+}
+
+template <typename T, bool U, bool PIPE>
+static void launch_gemm_f8p(const svdq_gemm_args &a, hipStream_t s) {
     const dim3 grid(((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN)), block(NTHREADS);
     switch (a.epilogue) {
         case SVDQ_EPI_PLAIN:
-            hipLaunchKernelGGL((gemm_w4a4_f8_kernel<T, U, SVDQ_EPI_PLAIN>), grid, block, 0, s, a);
+            hipLaunchKernelGGL((gemm_w4a4_f8_kernel<T, U, SVDQ_EPI_PLAIN, PIPE>), grid, block, 0, s, a);
             break;
         case SVDQ_EPI_QK_NORM_ROPE:
-            hipLaunchKernelGGL((gemm_w4a4_f8_kernel<T, U, SVDQ_EPI_QK_NORM_ROPE>), grid, block, 0, s, a);
+            hipLaunchKernelGGL((gemm_w4a4_f8_kernel<T, U, SVDQ_EPI_QK_NORM_ROPE, PIPE>), grid, block, 0, s, a);
             break;
         case SVDQ_EPI_GELU_QUANT:
-            hipLaunchKernelGGL((gemm_w4a4_f8_kernel<T, U, SVDQ_EPI_GELU_QUANT>), grid, block, 0, s, a);
+            hipLaunchKernelGGL((gemm_w4a4_f8_kernel<T, U, SVDQ_EPI_GELU_QUANT, PIPE>), grid, block, 0, s, a);
             break;
         case SVDQ_EPI_SWIGLU_QUANT:
-            hipLaunchKernelGGL((gemm_w4a4_f8_kernel<T, U, SVDQ_EPI_SWIGLU_QUANT>), grid, block, 0, s, a);
+            hipLaunchKernelGGL((gemm_w4a4_f8_kernel<T, U, SVDQ_EPI_SWIGLU_QUANT, PIPE>), grid, block, 0, s, a);
             break;
     }
+}
+
+template <typename T, bool U>
+static void launch_gemm_f8(const svdq_gemm_args &a, hipStream_t s) {
+    if (two_workgroups_per_cu((long)((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN)))
+        launch_gemm_f8p<T, U, true>(a, s);
+    else
+        launch_gemm_f8p<T, U, false>(a, s);
 }
 
 template <typename T, bool U>
@@ -1309,6 +1365,15 @@ static int gemm_w4a4_checked(const svdq_gemm_args &a, void *stream) {
         rc = check_launch("svdq_gemm_w4a4 (LoRA-down partial sum)");
     }
     return rc;
+}
+
+extern "C" int svdq_gemm_w4a4_set_variant(int32_t variant) {
+    if (variant < -1 || variant > 1) {
+        set_error("svdq_gemm_w4a4_set_variant: %d is not -1 (by tile count), 0 (three workgroups per CU) or 1 (two)", variant);
+        return SVDQ_E_INVALID;
+    }
+    g_f8_variant.store(variant, std::memory_order_relaxed);
+    return SVDQ_OK;
 }
 
 extern "C" int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream) {

@@ -20,6 +20,15 @@ USE_WEIGHT_PLANES = "parameters"
 # by every call on the GPU, so calls on two streams must not overlap.
 STATIC_SCRATCH = False
 
+
+
+def set_fp8_loop_variant(variant: int) -> None:
+    """Which build of the fp8 main loop every following GEMM on pre-split weights uses: -1 = chosen by the number of tiles
+    (default), 0 = three workgroups per CU, 1 = two per CU with software-pipelined steps.  The two give identical bits; the
+    switch exists for tuning and for tests (``svdq_gemm_w4a4_set_variant``)."""
+    _lib.check(_lib.load().svdq_gemm_w4a4_set_variant(int(variant)))
+
+
 HEAD_DIM = 128
 GELU_SHIFT = 0.171875
 

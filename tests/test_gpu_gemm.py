@@ -287,6 +287,31 @@ def test_weight_planes_layout(dev, N, K):
     assert int(got[-16:-12].view(torch.int32)) == 0
 
 
+@pytest.mark.parametrize("unsigned", [False, True])
+@pytest.mark.parametrize("M,N,K,R", [(300, 520, 1152, 32), (129, 136, 320, 16), (2048, 1280, 512, 0)])
+def test_fp8_loop_builds_agree_bit_for_bit(dev, M, N, K, R, unsigned):
+    """The fp8 main loop is built twice (three workgroups per CU, steps in program order; two per CU, steps software
+    pipelined) and the library picks by tile count: both issue the same arithmetic in the same order, so every output bit
+    agrees, whichever one a shape gets."""
+    from nunchaku_rocm_amd.ops import gemm as gemm_mod
+
+    print(f"case M={M} N={N} K={K} R={R} unsigned={unsigned}", flush=True)
+    p = _rand_problem(M, N, K, R, torch.bfloat16, seed=11 + M)
+    old = gemm_mod.USE_WEIGHT_PLANES
+    try:
+        gemm_mod.USE_WEIGHT_PLANES = "all"
+        gemm_mod.set_fp8_loop_variant(0)
+        three = _gpu_gemm(p, dev, unsigned=unsigned)
+        gemm_mod.set_fp8_loop_variant(1)
+        two = _gpu_gemm(p, dev, unsigned=unsigned)
+    finally:
+        gemm_mod.set_fp8_loop_variant(-1)
+        gemm_mod.USE_WEIGHT_PLANES = old
+    assert torch.equal(three.view(torch.int16), two.view(torch.int16))
+    ref = O.gemm_w4a4(p["act"], p["wgt"], p["asc"], p["wsc"], bias=p["bias"], lora_act=p["la"], lora_up=p["lu"], act_unsigned=unsigned)
+    assert O.max_rel_err(three.float(), ref) <= TOL
+
+
 def test_weight_planes_refuse_scales_beyond_fp16(dev):
     """fp16 weight scales so large that -ws * (8 We - 7 Wo) overflows a 16-bit piece: the re-layout raises its status word and
     the operator falls back to the packed weight (int8 main loop) instead of producing NaN."""
