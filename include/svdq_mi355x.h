@@ -116,7 +116,8 @@ int svdq_transpose_lora_down(const void *lora_down, void *lora_down_t, int32_t K
  */
 typedef struct {
     const void *act;        /* (M, K/2) packed int4, row stride ld_act bytes (multiple of 16, base 16-B aligned) */
-    const void *wgt;        /* (N, K/2) packed signed int4, row stride ld_wgt bytes (same alignment)            */
+    const void *wgt;        /* (N, K/2) packed signed int4, row stride ld_wgt bytes (same alignment); not read,  */
+                            /* and may be NULL, when wgt_planes is given                                         */
     const void *wgt_planes; /* optional: the same weights and `wscales` re-laid-out by svdq_split_weight_planes  */
                             /* (then `wgt` is not read, fp8 main loop); NULL = unpack `wgt` inside the GEMM      */
                             /* (int8 main loop)                                                                  */

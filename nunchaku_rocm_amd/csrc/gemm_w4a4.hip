@@ -1257,15 +1257,16 @@ static int gemm_w4a4_checked(const svdq_gemm_args &a, void *stream) {
         set_error("svdq_gemm_w4a4: M=%d N=%d K=%d needs K %% 64 == 0 and N %% 8 == 0", a.M, a.N, a.K);
         return SVDQ_E_INVALID;
     }
-    if (!a.act || !a.wgt || !a.ascales || !a.wscales) {
-        set_error("svdq_gemm_w4a4: act, wgt, ascales and wscales are required");
+    if (!a.act || (!a.wgt && !a.wgt_planes) || !a.ascales || !a.wscales) {
+        set_error("svdq_gemm_w4a4: act, wgt (or wgt_planes), ascales and wscales are required");
         return SVDQ_E_INVALID;
     }
     if (a.wgt_planes && !al16(a.wgt_planes)) {
         set_error("svdq_gemm_w4a4: wgt_planes must be 16-byte aligned");
         return SVDQ_E_INVALID;
     }
-    if (!al16(a.act) || !al16(a.wgt) || a.ld_act % 16 || a.ld_wgt % 16 || a.ld_act < a.K / 2 || a.ld_wgt < a.K / 2) {
+    if (!al16(a.act) || a.ld_act % 16 || a.ld_act < a.K / 2 ||
+        (!a.wgt_planes && (!al16(a.wgt) || a.ld_wgt % 16 || a.ld_wgt < a.K / 2))) {  // wgt is not read next to wgt_planes
         set_error("svdq_gemm_w4a4: act/wgt rows must be 16-byte aligned and at least K/2 bytes (ld_act=%d ld_wgt=%d)",
                   a.ld_act, a.ld_wgt);
         return SVDQ_E_INVALID;
@@ -1277,7 +1278,8 @@ static int gemm_w4a4_checked(const svdq_gemm_args &a, void *stream) {
     {   // the kernel addresses operands with 32-bit offsets from a tile's base
         const size_t lim = (size_t)1 << 32, G = (size_t)(a.K / GROUP);
         if (G * a.ld_ascales * 2 >= lim || G * a.ld_wscales * 2 >= lim || (size_t)(BM + 1) * a.ld_act >= lim ||
-            (size_t)(BN + 1) * a.ld_wgt >= lim) {
+            (!a.wgt_planes && (size_t)(BN + 1) * a.ld_wgt >= lim) ||
+            (a.wgt_planes && (size_t)(G / 2 + 2) * (WPL_BLOCKS * BLK_BYTES) >= lim)) {
             set_error("svdq_gemm_w4a4: K=%d with row strides %d / %d / %d / %d: operands too large for 32-bit offsets", a.K,
                       a.ld_act, a.ld_wgt, a.ld_ascales, a.ld_wscales);
             return SVDQ_E_UNSUPPORTED;

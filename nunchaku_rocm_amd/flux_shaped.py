@@ -349,6 +349,19 @@ class FluxShapedTransformer(nn.Module):
         (r"^norm_out\.linear\.", "norm_out_linear."),
     )
     # tensors a checkpoint may carry that the int4 path does not use (NVFP4 scales, the un-fused smoothing factors)
+    def release_packed_weights(self) -> int:
+        """Let every ``SVDQW4A4Linear`` keep only the GEMM's working copy of its weight (``release_packed_weight``): a
+        FLUX.1-sized model then holds about 9 GB of 4-bit weights instead of 15 GB.  Returns the bytes released."""
+        from .linear import SVDQW4A4Linear
+
+        freed = 0
+        for m in self.modules():
+            if isinstance(m, SVDQW4A4Linear):
+                n = m.out_features * (m.in_features // 2)
+                if m.qweight.untyped_storage().nbytes() >= n and m.release_packed_weight():
+                    freed += n
+        return freed
+
     _CHECKPOINT_IGNORED = (".smooth_factor_orig", ".wtscale", ".wcscales")
 
     @torch.no_grad()

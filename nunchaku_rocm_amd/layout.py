@@ -22,6 +22,7 @@ __all__ = [
     "convert_svdq_linear_to_natural_layout",
     "convert_flux_state_dict",
     "load_checkpoint",
+    "join_weight_planes",
 ]
 
 
@@ -169,3 +170,29 @@ def load_checkpoint(path, device: str | torch.device = "cpu") -> tuple[dict[str,
             state_dict[key] = f.get_tensor(key)
     config = json.loads(metadata["config"]) if "config" in metadata else {}
     return state_dict, metadata, config
+
+
+def join_weight_planes(planes: torch.Tensor, n: int, k: int) -> torch.Tensor:
+    """Packed ``(n, k // 2)`` int8 weight back from the GEMM's working copy (``svdq_split_weight_planes``): the inverse of
+    the code part of that re-layout, for modules that released their packed weight and are asked for it again
+    (``state_dict``).  Per (block of 32 rows, stage of two scale groups) the copy holds three 1 KB blocks: lane
+    ``parity * 32 + row`` owns, per group, 32 six-bit codes ``sign | magnitude`` (code ``p`` = the nibble of its parity of
+    the row's packed byte ``p`` of the group) as 24 little-endian bytes; blocks 0 and 1 = bytes 0-15 of the stage's two
+    groups, block 2 = bytes 16-23 of both.  Plain torch operations on the tensor's device; one-off, not fast."""
+    nb, G = (n + 31) // 32, k // 64
+    nst = (G + 1) // 2
+    codes = planes[: nb * nst * 3072].view(nb, nst, 3, 64, 16)
+    by = torch.empty(nb, nst, 2, 64, 24, dtype=torch.uint8, device=planes.device)  # (.., group of the stage, lane, byte)
+    by[:, :, 0, :, :16] = codes[:, :, 0]
+    by[:, :, 1, :, :16] = codes[:, :, 1]
+    by[:, :, 0, :, 16:] = codes[:, :, 2, :, :8]
+    by[:, :, 1, :, 16:] = codes[:, :, 2, :, 8:]
+    shifts = torch.arange(8, dtype=torch.uint8, device=planes.device)
+    bits = ((by[..., None] >> shifts) & 1).reshape(nb, nst, 2, 64, 32, 6)  # little-endian bit stream -> 32 codes of 6 bits
+    weights = (1 << torch.arange(6, device=planes.device)).to(torch.int16)
+    code = (bits.to(torch.int16) * weights).sum(-1)  # (nb, nst, 2, lane, position)
+    value = torch.where(code >= 32, -(code - 32), code)  # sign | magnitude -> [-8, 8)
+    nib = (value & 0xF).to(torch.uint8).view(nb, nst * 2, 2, 32, 32)  # (nb, group, parity, row, packed byte)
+    packed = nib[:, :, 0] | (nib[:, :, 1] << 4)  # (nb, group, row, packed byte)
+    packed = packed[:, :G].permute(0, 2, 1, 3).reshape(nb * 32, G * 32)
+    return packed[:n].contiguous().view(torch.int8)

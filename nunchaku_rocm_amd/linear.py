@@ -51,6 +51,57 @@ class SVDQW4A4Linear(nn.Module):
         return cls(in_features=in_features, out_features=linear.out_features, bias=linear.bias is not None,
                    torch_dtype=torch_dtype, device=linear.weight.device, **kwargs)  # fmt: skip
 
+    # ---- memory: the GEMM's working copy can stand in for the packed weight ------------------------------------------
+    def release_packed_weight(self) -> bool:
+        """Drop the bytes of ``qweight`` and keep only the GEMM's working copy of it (1.5 x as large; made now if it does not
+        exist yet).  The fp8 main loop never reads the packed weight, so a model that would otherwise hold both (2.5 x the
+        packed bytes) holds 1.5 x.  ``qweight`` keeps its shape (every row a view of one spare row); ``state_dict()`` still
+        returns the packed weight, rebuilt from the copy; :meth:`restore_packed_weight` puts it back in place.  Returns
+        ``False`` (and changes nothing) when the weight has no usable working copy (rows not 16-byte aligned, or fp16
+        scales too large for its 16-bit offset terms)."""
+        from .ops import _prep
+
+        if _prep.pinned_weight_planes(self.qweight) is not None:
+            return True
+        if not self.qweight.is_cuda or self.qweight.stride(0) % 16:
+            return False
+        planes = _prep.weight_planes(self.qweight, self.wscales)
+        if planes is None:
+            return False
+        _prep.pin_weight_planes(self.qweight, planes)
+        self.qweight.data = torch.empty(self.in_features // 2, dtype=self.qweight.dtype, device=self.qweight.device).expand(self.out_features, -1)
+        return True
+
+    def restore_packed_weight(self) -> None:
+        """Undo :meth:`release_packed_weight`: ``qweight`` holds its packed bytes again."""
+        from .layout import join_weight_planes
+        from .ops import _prep
+
+        planes = _prep.pinned_weight_planes(self.qweight)
+        if planes is None:
+            return
+        packed = join_weight_planes(planes, self.out_features, self.in_features).view(self.qweight.dtype)
+        _prep.unpin_weight_planes(self.qweight)
+        self.qweight.data = packed
+
+    def _save_to_state_dict(self, destination, prefix, keep_vars):
+        super()._save_to_state_dict(destination, prefix, keep_vars)
+        from .ops import _prep
+
+        planes = _prep.pinned_weight_planes(self.qweight)
+        if planes is not None:  # released: hand out the packed form, rebuilt from the working copy
+            from .layout import join_weight_planes
+
+            destination[prefix + "qweight"] = join_weight_planes(planes, self.out_features, self.in_features).view(self.qweight.dtype)
+
+    def _load_from_state_dict(self, state_dict, prefix, *args, **kwargs):
+        from .ops import _prep
+
+        if _prep.pinned_weight_planes(self.qweight) is not None:  # a new weight is coming: give it storage to land in
+            _prep.unpin_weight_planes(self.qweight)
+            self.qweight.data = torch.empty(self.out_features, self.in_features // 2, dtype=self.qweight.dtype, device=self.qweight.device)
+        super()._load_from_state_dict(state_dict, prefix, *args, **kwargs)
+
     def forward(self, x: torch.Tensor, output: torch.Tensor | None = None, norm: tuple | None = None) -> torch.Tensor:
         """``norm=(scale, shift[, stats])``: apply ``layer_norm(x) * scale + shift`` inside the quantizer (an addition
         to the reference's signature; see ``ops.quantize``)."""

@@ -61,6 +61,7 @@ def invalidate(t: torch.Tensor) -> None:
     """Drop the derived copies of ``t`` (for callers that rewrite a weight through a path the version counter misses)."""
     _cache.pop(id(t), None)
     _planes_cache.pop(id(t), None)
+    _pinned.pop(id(t), None)
 
 
 def lora_down_t(lora_down: torch.Tensor) -> torch.Tensor:
@@ -87,6 +88,24 @@ def lora_down_t(lora_down: torch.Tensor) -> torch.Tensor:
 
 
 _planes_cache: dict[int, tuple] = {}
+_pinned: dict[int, tuple] = {}  # id(weight parameter) -> (weakref, planes): a weight whose packed bytes were released
+
+
+def pin_weight_planes(qweight: torch.Tensor, planes: torch.Tensor) -> None:
+    """Make ``planes`` the working copy of ``qweight`` for good, whatever storage ``qweight`` points at from now on (its
+    packed bytes are about to be released: the fp8 main loop never reads them).  Undone by :func:`unpin_weight_planes`."""
+    key = id(qweight)
+    _pinned[key] = (weakref.ref(qweight, lambda _r, k=key: _pinned.pop(k, None)), planes)
+    _planes_cache.pop(key, None)
+
+
+def unpin_weight_planes(qweight: torch.Tensor) -> None:
+    _pinned.pop(id(qweight), None)
+
+
+def pinned_weight_planes(qweight: torch.Tensor) -> torch.Tensor | None:
+    hit = _pinned.get(id(qweight))
+    return hit[1] if hit is not None and hit[0]() is qweight else None
 
 
 def weight_planes(qweight: torch.Tensor, wscales: torch.Tensor) -> torch.Tensor | None:
@@ -96,6 +115,9 @@ def weight_planes(qweight: torch.Tensor, wscales: torch.Tensor) -> torch.Tensor 
     half times the packed weight) plus ``6 * N * K / 64`` bytes.  ``None`` when the offset terms do not fit the 16-bit
     type (fp16 scales of about 17 and more): the caller then uses the packed weight.  Reading that status word waits for
     the re-layout once, when the copy is made."""
+    pinned = pinned_weight_planes(qweight)
+    if pinned is not None:
+        return pinned
     key = id(qweight)
     hit = _planes_cache.get(key)
     if hit is not None:

@@ -6,6 +6,7 @@ import torch
 
 from .. import _lib
 from ._prep import lora_down_t as _lora_down_t
+from ._prep import pinned_weight_planes as _pinned_weight_planes
 from ._prep import weight_planes as _weight_planes
 
 # Which weights get the GEMM's working copy (fp6 codes in MFMA lane order + group sums, cached per tensor, see
@@ -162,8 +163,10 @@ def svdq_gemm_w4a4_cuda(
     if out2d is not None and out2d.stride(1) != 1:
         raise ValueError("out not row-major")
 
-    want_planes = USE_WEIGHT_PLANES == "all" or (USE_WEIGHT_PLANES == "parameters" and isinstance(wgt, torch.nn.Parameter))
-    planes = _weight_planes(wgt, wscales) if want_planes and wgt.stride(0) % 16 == 0 else None
+    planes = _pinned_weight_planes(wgt)  # a module whose packed weight was released: this copy is all there is
+    if planes is None:
+        want_planes = USE_WEIGHT_PLANES == "all" or (USE_WEIGHT_PLANES == "parameters" and isinstance(wgt, torch.nn.Parameter))
+        planes = _weight_planes(wgt, wscales) if want_planes and wgt.stride(0) % 16 == 0 else None
     args = _lib.GemmArgs(
         act=act.data_ptr(),
         wgt=wgt.data_ptr(),

@@ -234,6 +234,46 @@ def test_linear_module_matches_dequantised_reference(dev):
     assert O.cosine(y.view(-1, N), truth) > 0.98
 
 
+@pytest.mark.parametrize("N,K", [(384, 512), (200, 320)])
+def test_release_packed_weight(dev, N, K, main_loop):
+    """A module can drop its packed weight and keep only the GEMM's working copy: the forward pass gives the same bits,
+    the device holds the packed bytes less, ``state_dict()`` still hands out the packed weight (rebuilt from the copy) and
+    ``restore_packed_weight`` puts it back."""
+    from nunchaku_rocm_amd.linear import SVDQW4A4Linear
+    from nunchaku_rocm_amd.ops import gemm as gemm_mod
+
+    lin = O.make_svdq_linear(K, N, seed=9)
+    mod = SVDQW4A4Linear(K, N, rank=32, device=dev)
+    with torch.no_grad():
+        for name in ("qweight", "wscales", "smooth_factor", "proj_down", "proj_up", "bias"):
+            getattr(mod, name).copy_(lin[name])
+    x = O.make_activations(150, K, seed=6).view(1, 150, K).to(dev)
+    gemm_mod.USE_WEIGHT_PLANES = "all"  # the autouse fixture puts the switch back
+    before = mod(x).clone()
+    torch.cuda.synchronize()
+    held = torch.cuda.memory_allocated(dev)
+    assert mod.release_packed_weight()
+    torch.cuda.synchronize()
+    assert held - torch.cuda.memory_allocated(dev) >= N * K // 2 - 4096
+    assert mod.qweight.shape == (N, K // 2) and mod.qweight.untyped_storage().nbytes() <= K // 2
+    for switch in ("all", "parameters", "none"):  # the working copy is all there is: the switch no longer matters
+        gemm_mod.USE_WEIGHT_PLANES = switch
+        assert torch.equal(mod(x).view(torch.int16), before.view(torch.int16))
+    sd = mod.state_dict()
+    assert torch.equal(sd["qweight"].cpu().view(torch.uint8), lin["qweight"].view(torch.uint8))
+    mod.restore_packed_weight()
+    assert torch.equal(mod.qweight.cpu().view(torch.uint8), lin["qweight"].view(torch.uint8))
+    gemm_mod.USE_WEIGHT_PLANES = main_loop
+    ref = mod(x)
+    rp, rs, rl, _ = O.quantize_act(x.cpu().view(-1, K), lin["proj_down"], lin["smooth_factor"])
+    assert O.max_rel_err(ref.cpu().view(-1, N), O.gemm_w4a4(rp, lin["qweight"], rs, lin["wscales"], lin["bias"], rl, lin["proj_up"])) <= TOL
+    # a released module takes a new weight through load_state_dict
+    assert mod.release_packed_weight()
+    mod.load_state_dict(sd)
+    assert torch.equal(mod.qweight.cpu().view(torch.uint8), lin["qweight"].view(torch.uint8))
+    assert torch.equal(mod(x).view(torch.int16), before.view(torch.int16)) or main_loop == "none"
+
+
 def _planes_expected(wgt, wsc, N, K):
     """Host restatement of the pre-split weight layout.  Per (block of 32 rows, stage of two groups) three 1 KB blocks:
     a lane (= parity * 32 + row) holds, per group, 32 six-bit codes sign | magnitude (position p = the nibble of its parity
