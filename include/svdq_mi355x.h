@@ -190,6 +190,11 @@ size_t svdq_gemm_w4a4_scratch_bytes(int32_t M, int32_t N, int32_t R2, int32_t ep
 #define SVDQ_STATIC_SCRATCH_BYTES (16u << 20)
 int svdq_gemm_w4a4_static_scratch(const svdq_gemm_args *args, void *stream);
 size_t svdq_gemm_w4a4_static_scratch_capacity(void);
+/* Looks up the buffer's address on the current device now instead of in the first svdq_gemm_w4a4_static_scratch call
+ * there: call it once per device before capturing that entry point into a HIP graph (the look-up is not a stream
+ * operation).  16 MiB hold M * ceil(N / 128) * R2 * 4 bytes: at R2 = 32, M * N up to 16.8 M (M = 4608: N <= 3584); the
+ * FLUX.1 fc1 shape (M = 4608, N = 12288: 56.6 MB) needs svdq_gemm_w4a4 with a caller's buffer. */
+int svdq_gemm_w4a4_static_scratch_prepare(void);
 
 /*
  * Debug: exact int32 accumulators of one scale group, p[m, n] = sum_{k in group g} a[m, k] * w[n, k], computed by

@@ -31,6 +31,7 @@ EXPORTS = (
     "svdq_gemm_w4a4_scratch_bytes",
     "svdq_gemm_w4a4_static_scratch",
     "svdq_gemm_w4a4_static_scratch_capacity",
+    "svdq_gemm_w4a4_static_scratch_prepare",
     "svdq_split_weight_planes",
     "svdq_weight_planes_bytes",
     "svdq_group_acc_i32",
@@ -129,6 +130,7 @@ def load() -> ctypes.CDLL:
     lib.svdq_gemm_w4a4_static_scratch.argtypes = [ctypes.POINTER(GemmArgs), _vp]
     lib.svdq_gemm_w4a4_static_scratch_capacity.restype = ctypes.c_size_t
     lib.svdq_gemm_w4a4_static_scratch_capacity.argtypes = []
+    lib.svdq_gemm_w4a4_static_scratch_prepare.argtypes = []
     lib.svdq_awq_gemv_w4a16.argtypes = [ctypes.POINTER(AwqGemvArgs), _vp]
     lib.svdq_awq_dequantize.argtypes = [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _vp]
     lib.svdq_attention_fp16.argtypes = [ctypes.POINTER(AttentionArgs), _vp]

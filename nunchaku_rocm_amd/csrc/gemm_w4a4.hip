@@ -1397,6 +1397,31 @@ static std::atomic<void *> g_scratch_ptr[MAX_DEVICES];
 
 extern "C" size_t svdq_gemm_w4a4_static_scratch_capacity(void) { return STATIC_SCRATCH_BYTES; }
 
+// Device address of the array on the current device, looked up on first use there (every device holds its own copy).
+static int static_scratch_ptr(void **out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
+        set_error("svdq_gemm_w4a4_static_scratch: no current device (or device index above %d)", MAX_DEVICES - 1);
+        return SVDQ_E_LAUNCH;
+    }
+    void *ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (ptr == nullptr) {
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || ptr == nullptr) {
+            set_error("svdq_gemm_w4a4_static_scratch: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+            return SVDQ_E_LAUNCH;
+        }
+        g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+    }
+    *out = ptr;
+    return SVDQ_OK;
+}
+
+extern "C" int svdq_gemm_w4a4_static_scratch_prepare(void) {
+    void *ptr = nullptr;
+    return static_scratch_ptr(&ptr);
+}
+
 extern "C" int svdq_gemm_w4a4_static_scratch(const svdq_gemm_args *args, void *stream) {
     if (!args) {
         set_error("svdq_gemm_w4a4_static_scratch: null args");
@@ -1412,20 +1437,9 @@ extern "C" int svdq_gemm_w4a4_static_scratch(const svdq_gemm_args *args, void *s
     }
     a.scratch = nullptr;
     if (need > 0) {
-        int dev = -1;
-        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
-            set_error("svdq_gemm_w4a4_static_scratch: no current device (or device index above %d)", MAX_DEVICES - 1);
-            return SVDQ_E_LAUNCH;
-        }
-        void *ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
-        if (ptr == nullptr) {  // first call on this device: every device holds its own copy of the array
-            const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
-            if (e != hipSuccess || ptr == nullptr) {
-                set_error("svdq_gemm_w4a4_static_scratch: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
-                return SVDQ_E_LAUNCH;
-            }
-            g_scratch_ptr[dev].store(ptr, std::memory_order_release);
-        }
+        void *ptr = nullptr;
+        const int rc = static_scratch_ptr(&ptr);
+        if (rc) return rc;
         a.scratch = (float *)ptr;  // every (tile, row, rank) entry the reduction reads is written first: nothing to clear
     }
     return gemm_w4a4_checked(a, stream);

@@ -22,6 +22,13 @@ USE_WEIGHT_PLANES = "parameters"
 STATIC_SCRATCH = False
 
 
+def prepare_static_scratch(device=None) -> None:
+    """Look up the built-in buffer on ``device`` (default: the current one) now, outside any graph capture; the first
+    ``STATIC_SCRATCH`` call on a device would otherwise do it (``svdq_gemm_w4a4_static_scratch_prepare``)."""
+    with torch.cuda.device(device):
+        _lib.check(_lib.load().svdq_gemm_w4a4_static_scratch_prepare())
+
+
 
 def set_fp8_loop_variant(variant: int) -> None:
     """Which build of the fp8 main loop every following GEMM on pre-split weights uses: -1 = chosen by the number of tiles

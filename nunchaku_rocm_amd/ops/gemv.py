@@ -23,8 +23,12 @@ def awq_gemv_w4a16_cuda(
     """
     ``out = in_feats @ (q * scaling_factors + zeros).T`` with ``q`` the TinyChat-packed uint4 weight
     (``kernel`` ``(n // 4, k // 2)`` int32).  Group size 64 runs the fused GEMV kernel (weights read once for all ``m``
-    rows); other group sizes decode the weight and multiply, as the reference does.  Returns
-    ``in_feats.shape[:-1] + (n,)`` in the input dtype.
+    rows).  Two cases take the reference's own route for everything but group size 64 (ops/triton/awq.py:226-228), still
+    on the GPU: :func:`awq_dequantize` to a dense ``(n, k)`` 16-bit weight (``2 n k`` bytes, allocated per call), then a
+    library matmul -- other group sizes or ``n % 32 != 0``, and shapes whose per-group tables do not fit the kernel's
+    64 KB of LDS (``k = 12288`` with more than 16 rows; no FLUX shape).  Weights of 4 GiB and more are refused
+    (``RuntimeError``): the kernels address them with 32-bit offsets.  Returns ``in_feats.shape[:-1] + (n,)`` in the
+    input dtype.
     """
     _lib.require_cuda(in_feats, kernel, scaling_factors, zeros)
     x = in_feats.reshape(m, k)
@@ -40,6 +44,8 @@ def awq_gemv_w4a16_cuda(
         raise ValueError("scaling_factors and zeros must share a row-major (k // 64, n) layout")
     if scaling_factors.dtype != x.dtype or zeros.dtype != x.dtype:
         raise ValueError("scaling_factors / zeros must have the input dtype")
+    if n * k // 2 >= 1 << 32:
+        raise RuntimeError(f"AWQ weight of {n * k // 2} bytes: 4 GiB and more are not supported (32-bit offsets)")
     out = torch.empty(m, n, dtype=x.dtype, device=x.device)
     lib = _lib.load()
     with torch.cuda.device(x.device):
@@ -62,7 +68,8 @@ def awq_gemv_w4a16_cuda(
             rc = lib.svdq_awq_gemv_w4a16(args, _lib.stream_of(x))
             if rc == _lib.E_UNSUPPORTED:
                 # the kernel's per-group tables do not fit LDS (K = 12288 with more than 16 rows, longer K with fewer):
-                # decode the weight and multiply, the reference's route for everything but group size 64
+                # decode the weight and multiply on the GPU, the reference's route for everything but group size 64 (the
+                # other refusal, a weight of 4 GiB and more, was raised above)
                 w = awq_dequantize(kernel, scaling_factors, zeros, n, k, group_size, x.dtype)
                 return torch.matmul(x, w.t()).reshape(*in_feats.shape[:-1], n)
             _lib.check(rc)

@@ -52,6 +52,49 @@ def test_static_scratch_matches_caller_scratch_twice(dev, swiglu):
         assert ref[2].abs().max() > 0  # the LoRA-down branch did run
 
 
+def test_static_scratch_under_graph_capture(dev):
+    """The use the entry point is for: a GELU-epilogue GEMM captured into a HIP graph (the buffer's address looked up
+    beforehand, as the header asks) and replayed, the program's own eager work between the replays; every replay gives
+    the eager call's bits."""
+    from nunchaku_rocm_amd import ops
+    from nunchaku_rocm_amd.ops import gemm as G
+
+    M, N, K, R2, dtype = 272, 512, 256, 48, torch.bfloat16
+    lin = O.make_svdq_linear(K, N, seed=7, dtype=dtype)
+    g = torch.Generator().manual_seed(8)
+    t = {"act": torch.randint(0, 256, (M, K // 2), generator=g, dtype=torch.uint8), "asc": (torch.rand(K // 64, M, generator=g) * 0.2 + 0.05).to(dtype),
+         "smooth": (torch.rand(N, generator=g) + 0.5).to(dtype), "ld": (torch.randn(N, R2, generator=g) * 0.1).to(dtype)}  # fmt: skip
+    t = {k: v.to(dev) for k, v in t.items()}
+    w = {k: v.to(dev) for k, v in lin.items()}
+    qout = torch.zeros(M, N // 2, dtype=torch.uint8, device=dev)
+    osc = torch.zeros(N // 64, M, dtype=dtype, device=dev)
+    lao = torch.zeros(M, R2, dtype=torch.float32, device=dev)
+    out = torch.zeros(M, N, dtype=dtype, device=dev)
+
+    def call():
+        ops.svdq_gemm_w4a4_cuda(act=t["act"], wgt=w["qweight"], out=out, qout=qout, ascales=t["asc"], wscales=w["wscales"],
+                                oscales=osc, lora_down=t["ld"], lora_act_out=lao, bias=w["bias"], smooth_factor=t["smooth"])  # fmt: skip
+
+    call()  # eager, caller-provided scratch; also makes the cached re-layouts of the weights
+    torch.cuda.synchronize()
+    want = [x.clone() for x in (qout, osc, lao, out)]
+    G.prepare_static_scratch(dev)
+    G.STATIC_SCRATCH = True
+    try:
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            call()
+        for rep in range(3):
+            for x in (qout, osc, lao, out):
+                x.fill_(0)  # a fill kernel, eager, between the replays
+            graph.replay()
+            torch.cuda.synchronize()
+            for got, ref in zip((qout, osc, lao, out), want):
+                assert torch.equal(got.view(torch.uint8), ref.view(torch.uint8)), f"replay {rep}"
+    finally:
+        G.STATIC_SCRATCH = False
+
+
 def test_static_scratch_refuses_what_does_not_fit(dev):
     from nunchaku_rocm_amd import _lib
 
