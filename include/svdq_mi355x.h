@@ -223,6 +223,19 @@ typedef struct {
 int svdq_awq_gemv_w4a16(const svdq_awq_gemv_args *args, void *stream);
 
 /*
+ * The same GEMV for `count` weights of one shape in a single launch (M <= 8).  The adaLN projections of a diffusion
+ * transformer all take the same vector (models/normalization.py: silu(temb)) and do not depend on the blocks before them,
+ * so they can run together; one 32 MB weight is too short a read to reach the HBM rate (launch ramp and tail), many
+ * behind each other stream like one long read.  `first` (host memory) is problem 0: M, N, K, the leading dimensions and
+ * the dtype hold for all problems.  `problems` is a DEVICE array of `count` svdq_awq_gemv_args (8-byte aligned), of which
+ * only the five pointers x, qweight, scales, zeros, out are read; entry 0 must equal `first`'s.  Every problem's tensors
+ * must meet the alignment rules of svdq_awq_gemv_w4a16: only problem 0 can be checked here, the others are the caller's to
+ * check.  Results are bit-identical to count single calls.  No counterpart in the reference.
+ */
+int svdq_awq_gemv_w4a16_batched(const svdq_awq_gemv_args *first, const svdq_awq_gemv_args *problems, int32_t count,
+                                void *stream);
+
+/*
  * Dense decode of a TinyChat-packed AWQ weight (nunchaku/ops/triton/awq.py:48-118 awq_dequantize, the first half of
  * awq_gemm_w4a16 :232-251 and of the group_size != 64 branch of awq_gemv_w4a16 :226-228; the matmul that follows is
  * the caller's): out[n, k] = T(q[n, k] * s[k / group_size, n] + z[k / group_size, n]) in fp32.

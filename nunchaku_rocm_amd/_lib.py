@@ -36,6 +36,7 @@ EXPORTS = (
     "svdq_weight_planes_bytes",
     "svdq_group_acc_i32",
     "svdq_awq_gemv_w4a16",
+    "svdq_awq_gemv_w4a16_batched",
     "svdq_awq_dequantize",
     "svdq_attention_fp16",
     "svdq_unpack_mma_weight",
@@ -132,6 +133,7 @@ def load() -> ctypes.CDLL:
     lib.svdq_gemm_w4a4_static_scratch_capacity.argtypes = []
     lib.svdq_gemm_w4a4_static_scratch_prepare.argtypes = []
     lib.svdq_awq_gemv_w4a16.argtypes = [ctypes.POINTER(AwqGemvArgs), _vp]
+    lib.svdq_awq_gemv_w4a16_batched.argtypes = [ctypes.POINTER(AwqGemvArgs), _vp, _i32, _vp]
     lib.svdq_awq_dequantize.argtypes = [_vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _vp]
     lib.svdq_attention_fp16.argtypes = [ctypes.POINTER(AttentionArgs), _vp]
     lib.svdq_unpack_mma_weight.argtypes = [_vp, _vp, _i32, _i32, _i32, _vp]

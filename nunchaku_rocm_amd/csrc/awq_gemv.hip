@@ -89,15 +89,30 @@ __device__ inline float dpp_f32(float x) {
 template <int RP>
 constexpr int awq_wave_bytes() { return AWQ_PF * RP * 128 + 2 * AWQ_PF * 64; }
 
-template <typename T, int RP>
-__global__ __launch_bounds__(AWQ_WAVES * 64) __attribute__((amdgpu_waves_per_eu(RP <= 4 ? 6 : 4))) void awq_gemv_rows_kernel(svdq_awq_gemv_args a) {
+//
+// BATCH: one launch serves `count` weights of one shape (the adaLN projections of a model all take the same vector and
+// differ only in their tensors): workgroup b works on problem b / (N / 32), whose five pointers it reads from `table`;
+// everything else comes from `a`.  A 32 MB weight by itself is read at 60 % of the HBM peak at best (launch ramp and
+// tail of a 6 us kernel); several in one launch stream like one long read.
+template <typename T, int RP, bool BATCH>
+__global__ __launch_bounds__(AWQ_WAVES * 64) __attribute__((amdgpu_waves_per_eu(RP <= 4 ? 6 : 4))) void awq_gemv_rows_kernel(svdq_awq_gemv_args a, const svdq_awq_gemv_args *table) {
     extern __shared__ __align__(16) uint8_t lds8[];
+    int blk = blockIdx.x;
+    if constexpr (BATCH) {
+        const int nblk = a.N / AWQ_NB, pi = blk / nblk;  // uniform: scalar loads
+        blk -= pi * nblk;
+        a.x = table[pi].x;
+        a.qweight = table[pi].qweight;
+        a.scales = table[pi].scales;
+        a.zeros = table[pi].zeros;
+        a.out = table[pi].out;
+    }
     constexpr bool SMALL = RP <= 4;
     constexpr int WB = awq_wave_bytes<RP>(), XPIECES = AWQ_PF * 8 * RP, XPASSES = (XPIECES + 63) / 64;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int ngroups = a.K / GROUP;
-    const int nb0 = blockIdx.x * AWQ_NB;
+    const int nb0 = blk * AWQ_NB;
     uint8_t *xw = lds8 + wave * WB, *szw = xw + AWQ_PF * RP * 128;
     float *xsw = (float *)(lds8 + AWQ_WAVES * WB) + wave * (AWQ_PF * 8);
 
@@ -390,20 +405,29 @@ static size_t awq_lds_bytes(int K, int M) {
     return b;
 }
 
+template <typename T, bool BATCH>
+static void launch_awq_rows(const svdq_awq_gemv_args &a, const svdq_awq_gemv_args *table, int count, hipStream_t s) {
+    const dim3 grid((unsigned)(a.N / AWQ_NB) * (unsigned)count), block(AWQ_WAVES * 64);
+    constexpr size_t XS_BYTES = (size_t)AWQ_WAVES * AWQ_PF * 8 * sizeof(float);
+    if (a.M <= 1)
+        hipLaunchKernelGGL((awq_gemv_rows_kernel<T, 1, BATCH>), grid, block, AWQ_WAVES * awq_wave_bytes<1>() + XS_BYTES, s, a, table);
+    else if (a.M <= 2)
+        hipLaunchKernelGGL((awq_gemv_rows_kernel<T, 2, BATCH>), grid, block, AWQ_WAVES * awq_wave_bytes<2>() + XS_BYTES, s, a, table);
+    else if (a.M <= 4)
+        hipLaunchKernelGGL((awq_gemv_rows_kernel<T, 4, BATCH>), grid, block, AWQ_WAVES * awq_wave_bytes<4>() + XS_BYTES, s, a, table);
+    else
+        hipLaunchKernelGGL((awq_gemv_rows_kernel<T, 8, BATCH>), grid, block, AWQ_WAVES * awq_wave_bytes<8>() + XS_BYTES, s, a, table);
+}
+
 template <typename T>
 static void launch_awq(const svdq_awq_gemv_args &a, hipStream_t s) {
+    if (a.M <= 8) {
+        launch_awq_rows<T, false>(a, nullptr, 1, s);
+        return;
+    }
     const dim3 grid(a.N / AWQ_NB), block(AWQ_WAVES * 64);
-    constexpr size_t XS_BYTES = (size_t)AWQ_WAVES * AWQ_PF * 8 * sizeof(float);
     const size_t sh = awq_lds_bytes(a.K, a.M);
-    if (a.M <= 1)
-        hipLaunchKernelGGL((awq_gemv_rows_kernel<T, 1>), grid, block, AWQ_WAVES * awq_wave_bytes<1>() + XS_BYTES, s, a);
-    else if (a.M <= 2)
-        hipLaunchKernelGGL((awq_gemv_rows_kernel<T, 2>), grid, block, AWQ_WAVES * awq_wave_bytes<2>() + XS_BYTES, s, a);
-    else if (a.M <= 4)
-        hipLaunchKernelGGL((awq_gemv_rows_kernel<T, 4>), grid, block, AWQ_WAVES * awq_wave_bytes<4>() + XS_BYTES, s, a);
-    else if (a.M <= 8)
-        hipLaunchKernelGGL((awq_gemv_rows_kernel<T, 8>), grid, block, AWQ_WAVES * awq_wave_bytes<8>() + XS_BYTES, s, a);
-    else if (a.M <= 16)
+    if (a.M <= 16)
         hipLaunchKernelGGL((awq_gemv_kernel<T, 2>), grid, block, sh, s, a);
     else if (a.M <= 24)
         hipLaunchKernelGGL((awq_gemv_kernel<T, 3>), grid, block, sh, s, a);
@@ -415,45 +439,72 @@ static void launch_awq(const svdq_awq_gemv_args &a, hipStream_t s) {
 
 using namespace svdq;
 
+// shape and the tensors of one problem; `what` names the entry point in messages
+static int awq_check(const svdq_awq_gemv_args &a, const char *what, int max_rows) {
+    if (a.dtype != SVDQ_BF16 && a.dtype != SVDQ_FP16) {
+        set_error("%s: dtype %d", what, a.dtype);
+        return SVDQ_E_INVALID;
+    }
+    if (a.M < 0 || a.M > max_rows || a.N <= 0 || a.N % AWQ_NB || a.K <= 0 || a.K % GROUP) {
+        set_error("%s: M=%d N=%d K=%d needs M <= %d, N %% 32 == 0, K %% 64 == 0", what, a.M, a.N, a.K, max_rows);
+        return SVDQ_E_INVALID;
+    }
+    if (!a.x || !a.qweight || !a.scales || !a.zeros || !a.out) {
+        set_error("%s: null tensor", what);
+        return SVDQ_E_INVALID;
+    }
+    if (((uintptr_t)a.x & 15) || a.ld_x % 8 || a.ld_x < a.K || ((uintptr_t)a.qweight & 15) || a.ld_scales < a.N ||
+        a.ld_out < a.N || ((uintptr_t)a.scales & 15) || ((uintptr_t)a.zeros & 15) || a.ld_scales % 8) {
+        set_error("%s: x rows, qweight and scale / zero rows must be 16-byte aligned; leading dimensions >= row length", what);
+        return SVDQ_E_INVALID;
+    }
+    if (awq_lds_bytes(a.K, a.M) > AWQ_LDS_MAX) {  // K = 12288 with M > 16, K > 16384 with M > 8
+        set_error("%s: K=%d with M=%d needs %zu bytes of LDS tables (limit %zu)", what, a.K, a.M, awq_lds_bytes(a.K, a.M), AWQ_LDS_MAX);
+        return SVDQ_E_UNSUPPORTED;
+    }
+    if (a.M <= 8 && ((size_t)a.N * a.K / 2 >= ((size_t)1 << 32) || (size_t)(a.K / GROUP) * a.ld_scales * 2 >= ((size_t)1 << 32) ||
+                     (size_t)a.M * a.ld_x * 2 >= ((size_t)1 << 32))) {  // the kernel for up to eight rows addresses with 32-bit byte offsets
+        set_error("%s: N=%d K=%d ld_scales=%d ld_x=%d: a tensor of 4 GiB or more", what, a.N, a.K, a.ld_scales, a.ld_x);
+        return SVDQ_E_UNSUPPORTED;
+    }
+    return SVDQ_OK;
+}
+
 extern "C" int svdq_awq_gemv_w4a16(const svdq_awq_gemv_args *args, void *stream) {
     if (!args) {
         set_error("svdq_awq_gemv_w4a16: null args");
         return SVDQ_E_INVALID;
     }
     const svdq_awq_gemv_args &a = *args;
-    if (a.dtype != SVDQ_BF16 && a.dtype != SVDQ_FP16) {
-        set_error("svdq_awq_gemv_w4a16: dtype %d", a.dtype);
-        return SVDQ_E_INVALID;
-    }
-    if (a.M < 0 || a.M > 32 || a.N <= 0 || a.N % AWQ_NB || a.K <= 0 || a.K % GROUP) {
-        set_error("svdq_awq_gemv_w4a16: M=%d N=%d K=%d needs M <= 32, N %% 32 == 0, K %% 64 == 0", a.M, a.N, a.K);
-        return SVDQ_E_INVALID;
-    }
-    if (!a.x || !a.qweight || !a.scales || !a.zeros || !a.out) {
-        set_error("svdq_awq_gemv_w4a16: null tensor");
-        return SVDQ_E_INVALID;
-    }
-    if (((uintptr_t)a.x & 15) || a.ld_x % 8 || a.ld_x < a.K || ((uintptr_t)a.qweight & 15) || a.ld_scales < a.N ||
-        a.ld_out < a.N || ((uintptr_t)a.scales & 15) || ((uintptr_t)a.zeros & 15) || a.ld_scales % 8) {
-        set_error("svdq_awq_gemv_w4a16: x rows, qweight and scale / zero rows must be 16-byte aligned; leading dimensions >= row length");
-        return SVDQ_E_INVALID;
-    }
-    if (awq_lds_bytes(a.K, a.M) > AWQ_LDS_MAX) {  // K = 12288 with M > 16, K > 16384 with M > 8
-        set_error("svdq_awq_gemv_w4a16: K=%d with M=%d needs %zu bytes of LDS tables (limit %zu)", a.K, a.M,
-                  awq_lds_bytes(a.K, a.M), AWQ_LDS_MAX);
-        return SVDQ_E_UNSUPPORTED;
-    }
+    const int rc = awq_check(a, "svdq_awq_gemv_w4a16", 32);
+    if (rc) return rc;
     if (a.M == 0) return SVDQ_OK;
-    if (a.M <= 8 && ((size_t)a.N * a.K / 2 >= ((size_t)1 << 32) || (size_t)(a.K / GROUP) * a.ld_scales * 2 >= ((size_t)1 << 32) ||
-                     (size_t)a.M * a.ld_x * 2 >= ((size_t)1 << 32))) {  // the kernel for up to eight rows addresses with 32-bit byte offsets
-        set_error("svdq_awq_gemv_w4a16: N=%d K=%d ld_scales=%d ld_x=%d: a tensor of 4 GiB or more", a.N, a.K, a.ld_scales, a.ld_x);
-        return SVDQ_E_UNSUPPORTED;
-    }
     if (a.dtype == SVDQ_BF16)
         launch_awq<BF16>(a, (hipStream_t)stream);
     else
         launch_awq<FP16>(a, (hipStream_t)stream);
     return check_launch("svdq_awq_gemv_w4a16");
+}
+
+extern "C" int svdq_awq_gemv_w4a16_batched(const svdq_awq_gemv_args *first, const svdq_awq_gemv_args *problems, int32_t count,
+                                           void *stream) {
+    if (!first || !problems || count <= 0 || ((uintptr_t)problems & 7)) {
+        set_error("svdq_awq_gemv_w4a16_batched: needs the first problem (host), the table of all problems (device) and count > 0");
+        return SVDQ_E_INVALID;
+    }
+    const svdq_awq_gemv_args &a = *first;
+    const int rc = awq_check(a, "svdq_awq_gemv_w4a16_batched", 8);
+    if (rc) return rc;
+    if ((size_t)(a.N / AWQ_NB) * (size_t)count >= ((size_t)1 << 31)) {
+        set_error("svdq_awq_gemv_w4a16_batched: %d problems of N=%d are too many workgroups for one launch", count, a.N);
+        return SVDQ_E_UNSUPPORTED;
+    }
+    if (a.M == 0) return SVDQ_OK;
+    if (a.dtype == SVDQ_BF16)
+        launch_awq_rows<BF16, true>(a, problems, count, (hipStream_t)stream);
+    else
+        launch_awq_rows<FP16, true>(a, problems, count, (hipStream_t)stream);
+    return check_launch("svdq_awq_gemv_w4a16_batched");
 }
 
 extern "C" int svdq_awq_dequantize(const void *qweight, const void *scales, const void *zeros, void *out, int32_t N,

@@ -4,7 +4,7 @@ from .attention import attention_fp16, scaled_dot_product_attention
 from .elementwise import gated_residual
 from .fused import fused_gelu_mlp, fused_qkv_norm_rottary, fused_swiglu_mlp, interleave_swiglu_linear_
 from .gemm import svdq_gemm_w4a4_cuda
-from .gemv import awq_dequantize, awq_gemm_w4a16, awq_gemv_w4a16_cuda, gemm_awq, gemv_awq
+from .gemv import AwqGemvBatch, awq_dequantize, awq_gemm_w4a16, awq_gemv_w4a16_cuda, gemm_awq, gemv_awq
 from .quantize import (
     layer_norm_stats,
     quantize_w4a4_act,
@@ -20,6 +20,7 @@ __all__ = [
     "quantize_w4a4_wgt",
     "svdq_gemm_w4a4_cuda",
     "awq_gemv_w4a16_cuda",
+    "AwqGemvBatch",
     "awq_dequantize",
     "awq_gemm_w4a16",
     "gemv_awq",

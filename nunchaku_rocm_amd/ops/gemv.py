@@ -76,6 +76,53 @@ def awq_gemv_w4a16_cuda(
     return out.reshape(*in_feats.shape[:-1], n)
 
 
+class AwqGemvBatch:
+    """Several AWQ W4A16 GEMVs of one shape, all on the same input, in one launch (``svdq_awq_gemv_w4a16_batched``).
+
+    The adaLN projections of a diffusion transformer all take ``silu(temb)`` and depend on nothing else in the model
+    (nunchaku/models/normalization.py), so the model can compute them together; one 32 MB weight is too short a read to
+    reach the HBM rate, many behind each other are not.  Built once from the layers' tensors (``kernels[i]``
+    ``(n // 4, k // 2)`` int32, ``scales[i]`` / ``zeros[i]`` ``(k // 64, n)``); ``__call__`` copies the input into the
+    batch's own buffer and returns ``(count, m, n)``, a buffer the next call overwrites.  Results are bit-identical to
+    :func:`awq_gemv_w4a16_cuda` layer by layer.  Up to eight rows, group size 64.  No counterpart in the reference.
+    """
+
+    def __init__(self, kernels, scales, zeros, m: int, n: int, k: int):
+        import ctypes
+
+        if not 1 <= m <= 8:
+            raise ValueError(f"m={m}: a batched launch takes up to eight rows")
+        _lib.require_cuda(*kernels, *scales, *zeros)
+        count, dev, dtype = len(kernels), kernels[0].device, scales[0].dtype
+        if count == 0 or len(scales) != count or len(zeros) != count:
+            raise ValueError("kernels, scales and zeros must be equally long, non-empty lists")
+        if n * k // 2 >= 1 << 32:
+            raise RuntimeError(f"AWQ weight of {n * k // 2} bytes: 4 GiB and more are not supported (32-bit offsets)")
+        self.m, self.n, self.k, self.count = m, n, k, count
+        self.x = torch.zeros(m, k, dtype=dtype, device=dev)
+        self.out = torch.empty(count, m, n, dtype=dtype, device=dev)
+        self._keep = (list(kernels), list(scales), list(zeros))
+        table = (_lib.AwqGemvArgs * count)()
+        for i, (q, sc, z) in enumerate(zip(kernels, scales, zeros)):
+            if q.element_size() * q.numel() != n * k // 2 or not q.is_contiguous() or q.data_ptr() % 16:
+                raise ValueError(f"problem {i}: unexpected packed AWQ weight {tuple(q.shape)} for n={n}, k={k}")
+            for name, t in (("scales", sc), ("zeros", z)):
+                if t.shape != (k // 64, n) or t.dtype != dtype or t.stride() != (n, 1) or t.data_ptr() % 16 or t.device != dev:
+                    raise ValueError(f"problem {i}: {name} must be a contiguous ({k // 64}, {n}) {dtype} tensor on {dev}")
+            table[i] = _lib.AwqGemvArgs(x=self.x.data_ptr(), qweight=q.data_ptr(), scales=sc.data_ptr(), zeros=z.data_ptr(),
+                                        out=self.out[i].data_ptr(), M=m, N=n, K=k, ld_x=k, ld_scales=n, ld_out=n,
+                                        dtype=_lib.dtype_code(dtype))  # fmt: skip
+        self._first = table[0]
+        raw = torch.frombuffer(bytearray(bytes(table)), dtype=torch.uint8)
+        self._table = raw.to(dev)  # the device copy the kernel reads its pointers from
+
+    def __call__(self, in_feats: torch.Tensor) -> torch.Tensor:
+        self.x.copy_(in_feats.reshape(self.m, self.k))
+        with torch.cuda.device(self.x.device):
+            _lib.check(_lib.load().svdq_awq_gemv_w4a16_batched(self._first, self._table.data_ptr(), self.count, _lib.stream_of(self.x)))
+        return self.out
+
+
 def awq_dequantize(
     kernel: torch.Tensor,
     scaling_factors: torch.Tensor,

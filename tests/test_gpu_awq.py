@@ -41,6 +41,29 @@ def test_flux_adaln_shape(dev, m):
     assert ((out.float() - ref).abs() <= ref.abs() * 2**-7 + 2e-2).all()
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("m,N,K,count", [(1, 18432, 3072, 3), (2, 96, 576, 5), (8, 256, 1088, 2), (3, 64, 64, 7), (5, 9216, 3072, 1)])
+def test_batched_launch_matches_single_launches(dev, m, N, K, count, dtype):
+    """``count`` weights of one shape on the same input in one launch (the adaLN projections of a model): every output
+    bit as from the single launches, and the oracle's result."""
+    from nunchaku_rocm_amd import ops
+
+    print(f"case m={m} N={N} K={K} count={count} {dtype}", flush=True)
+    lins = [O.make_awq_linear(K, N, seed=40 + i, dtype=dtype) for i in range(count)]
+    d = [{k: v.to(dev) for k, v in lin.items() if k != "codes"} for lin in lins]
+    x = torch.randn(m, K, generator=torch.Generator().manual_seed(3)).to(dtype)
+    batch = ops.AwqGemvBatch([t["qweight"] for t in d], [t["wscales"] for t in d], [t["wzeros"] for t in d], m, N, K)
+    for rep in range(2):  # the batch object is reused: its output buffer is overwritten
+        xr = (x * (rep + 1)).to(dtype)
+        got = batch(xr.to(dev)).cpu()
+        assert got.shape == (count, m, N)
+        for i, (lin, t) in enumerate(zip(lins, d)):
+            single = ops.awq_gemv_w4a16_cuda(xr.to(dev), t["qweight"], t["wscales"], t["wzeros"], m, N, K).cpu()
+            assert torch.equal(got[i].view(torch.int16), single.view(torch.int16)), f"problem {i}"
+            ref = O.awq_gemv(xr, lin["qweight"].view(torch.int16).reshape(N // 4, K), lin["wscales"], lin["wzeros"])
+            assert O.max_rel_err(got[i], ref) <= 1e-2
+
+
 @pytest.mark.parametrize("m", [1, 3, 4, 7, 12])
 @pytest.mark.parametrize("K", [64, 192, 576, 1088, 3136, 3520, 6208])
 def test_ragged_k(dev, m, K):
