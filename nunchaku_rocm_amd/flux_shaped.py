@@ -62,6 +62,7 @@ class HipBackend:
         # stream's launches leave empty instead of queueing behind them.
         self.two_streams = two_streams
         self._side = {}
+        self._awq_plans = {}
 
     def __deepcopy__(self, memo):
         return HipBackend(self.two_streams)  # streams are per process, not part of a model copy
@@ -97,6 +98,34 @@ class HipBackend:
     @staticmethod
     def awq(x, lin: AWQW4A16Linear):
         return lin(x)
+
+    def awq_many(self, x, lins):
+        """``[lin(x) for lin in lins]`` with the layers of equal width in one launch each (``ops.AwqGemvBatch``): the
+        adaLN projections of all blocks take the same vector and nothing else, so a forward pass runs them first, all
+        together; a 32 MB weight by itself is too short a read for the HBM rate.  The results live in buffers the next
+        call overwrites."""
+        if x.shape[0] > 8 or any(lin.group_size != 64 or lin.out_features % 32 for lin in lins):
+            return [lin(x) for lin in lins]
+        key = tuple(id(lin) for lin in lins) + (x.shape[0], x.dtype)
+        plan = self._awq_plans.get(key)
+        if plan is None:
+            plan = []
+            for n in sorted({lin.out_features for lin in lins}):
+                idx = [i for i, lin in enumerate(lins) if lin.out_features == n]
+                batch = _ops.AwqGemvBatch([lins[i].qweight for i in idx], [lins[i].wscales for i in idx],
+                                          [lins[i].wzeros for i in idx], x.shape[0], n, lins[0].in_features)  # fmt: skip
+                bias = torch.stack([lins[i].bias for i in idx])[:, None] if all(lins[i].bias is not None for i in idx) else None
+                assert bias is not None or all(lins[i].bias is None for i in idx)
+                plan.append((idx, batch, bias))
+            self._awq_plans = {key: plan}  # one model at a time: a new set of layers replaces the old plan
+        out = [None] * len(lins)
+        for idx, batch, bias in plan:
+            y = batch(x)
+            if bias is not None:
+                y += bias
+            for j, i in enumerate(idx):
+                out[i] = y[j]
+        return out
 
     @staticmethod
     def attention(q, k, v):
@@ -216,8 +245,9 @@ class _DoubleBlock(nn.Module):
         self.C = C
 
     @staticmethod
-    def _mod6(be, lin, temb):
-        emb = be.awq(F.silu(temb), lin)
+    def _mod6(be, lin, temb, emb=None):
+        if emb is None:
+            emb = be.awq(F.silu(temb), lin)
         return emb.view(emb.shape[0], -1, 6).permute(2, 0, 1)  # interleaved split: channel c -> (c // 6, c % 6)
 
     def _forward_two_streams(self, be, side, x, ctx, mods_x, mods_ctx, rot_img, rot_txt):
@@ -248,10 +278,11 @@ class _DoubleBlock(nn.Module):
         ctx.record_stream(main)  # read next on either stream
         return ctx, x
 
-    def forward(self, be, x, ctx, temb, rot_img, rot_txt):
+    def forward(self, be, x, ctx, temb, rot_img, rot_txt, embs=(None, None)):
+        """``embs``: the outputs of ``norm1`` / ``norm1_context`` where the caller has already computed them."""
         # layer_norm(x) * scale + shift in front of each quantized linear runs inside its quantizer (mod=)
-        sh_a, sc_a, g_a, sh_m, sc_m, g_m = self._mod6(be, self.norm1, temb)
-        csh_a, csc_a, cg_a, csh_m, csc_m, cg_m = self._mod6(be, self.norm1_context, temb)
+        sh_a, sc_a, g_a, sh_m, sc_m, g_m = self._mod6(be, self.norm1, temb, embs[0])
+        csh_a, csc_a, cg_a, csh_m, csc_m, cg_m = self._mod6(be, self.norm1_context, temb, embs[1])
         side = be.side_stream(x.device) if x.shape[0] == 1 and hasattr(be, "side_stream") else None
         if side is not None:
             return self._forward_two_streams(be, side, x, ctx, (sh_a, sc_a, g_a, sh_m, sc_m, g_m),
@@ -275,9 +306,11 @@ class _SingleBlock(nn.Module):
         self.attn = _Attention(cfg, joint=False, single=True, device=device, dtype=dtype)
         self.C = C
 
-    def forward(self, be, x, temb, rot, stats=None):
-        """``stats``: row statistics of x if the producer of x already has them.  Returns (x, statistics of it)."""
-        emb = be.awq(F.silu(temb), self.norm)
+    def forward(self, be, x, temb, rot, stats=None, emb=None):
+        """``stats``: row statistics of x if the producer of x already has them; ``emb``: the output of ``norm`` if the
+        caller has already computed it.  Returns (x, statistics of it)."""
+        if emb is None:
+            emb = be.awq(F.silu(temb), self.norm)
         shift, scale, gate = emb.view(emb.shape[0], -1, 3).permute(2, 0, 1)
         mod = (scale, shift, stats if stats is not None else be.norm_stats(x))  # one set for both consumers
         side = be.side_stream(x.device) if hasattr(be, "side_stream") else None
@@ -419,14 +452,21 @@ class FluxShapedTransformer(nn.Module):
         temb = self.time_in(_timestep_embedding(timestep).to(x.dtype)) + self.pooled_in(pooled)
         t_txt = ctx.shape[1]
         rot_txt, rot_img = rot[:t_txt].contiguous(), rot[t_txt:].contiguous()
-        for blk in self.double_blocks:
-            ctx, x = blk(be, x, ctx, temb, rot_img, rot_txt)
+        # every adaLN projection takes silu(temb) and nothing else: all of them first, layers of equal width in one launch
+        nd = len(self.double_blocks)
+        if hasattr(be, "awq_many"):
+            embs = be.awq_many(F.silu(temb), [lin for blk in self.double_blocks for lin in (blk.norm1, blk.norm1_context)]
+                               + [blk.norm for blk in self.single_blocks])  # fmt: skip
+        else:
+            embs = [None] * (2 * nd + len(self.single_blocks))
+        for i, blk in enumerate(self.double_blocks):
+            ctx, x = blk(be, x, ctx, temb, rot_img, rot_txt, embs=(embs[2 * i], embs[2 * i + 1]))
         if hasattr(be, "join"):
             be.join(x.device)  # the last block's text stream was produced on the side stream
         x = torch.cat([ctx, x], dim=1)
         stats = None
-        for blk in self.single_blocks:
-            x, stats = blk(be, x, temb, rot, stats)
+        for i, blk in enumerate(self.single_blocks):
+            x, stats = blk(be, x, temb, rot, stats, emb=embs[2 * nd + i])
         x = x[:, t_txt:]
         scale, shift = self.norm_out_linear(F.silu(temb)).chunk(2, dim=1)
         x = F.layer_norm(x, (self.cfg.hidden,), eps=1e-6) * (1 + scale)[:, None] + shift[:, None]
