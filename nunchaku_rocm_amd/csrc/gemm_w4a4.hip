@@ -58,9 +58,10 @@ constexpr int BLK_BYTES = 64 * 16;    // one MFMA operand block (32 rows x 16 by
 constexpr int NWAVES = 4, NTHREADS = NWAVES * 64;  // one wavefront per 32 activation rows
 constexpr int NBN = BN / 32;                        // 32-row weight blocks per wavefront: it owns 32 x 128 outputs
 // the first 32 ranks of the tile's lora_up, fetched next to stage 0: [2 c][4 blocks] 1 KB blocks in MFMA lane order,
-// then the tile's 128 bias values
+// then the tile's 128 bias values, then the 128 RMSNorm weights of the tile's head (Q/K norm + RoPE epilogue)
 constexpr int LORA_UP_BYTES = 8 * BLK_BYTES;
-constexpr int EPI_LDS_BYTES = LORA_UP_BYTES + BN * 2;
+constexpr int EPI_NORM_OFF = LORA_UP_BYTES + BN * 2;
+constexpr int EPI_LDS_BYTES = EPI_NORM_OFF + 128 * 2;
 constexpr int TP_PITCH = 36;                        // floats per row of the accumulator transposition tile
 constexpr int PRIV_BYTES = 32 * BN * 2;             // a wavefront's private epilogue memory: its 32 output rows of 256 bytes
 static_assert(32 * TP_PITCH * 4 <= PRIV_BYTES, "the transposition tile of one block does not fit");
@@ -189,9 +190,17 @@ __device__ inline void tile_ids(int tiles_m, int tiles_n, int &pid_m, int &pid_n
 }
 
 // Epilogue operands every wavefront of the tile needs, fetched global -> LDS next to stage 0: the tile's 128 bias
-// values and the first 32 ranks of lora_up.
+// values, the first 32 ranks of lora_up and (Q/K norm + RoPE epilogue, Q and K tiles) the head's 128 norm weights.
+template <int EPI>
 __device__ inline void fetch_epilogue_operands(const svdq_gemm_args &a, uint8_t *sepi, int n0, int wm, int lane) {
     const int l32 = lane & 31, half = lane >> 5;
+    if constexpr (EPI == SVDQ_EPI_QK_NORM_ROPE) {
+        const int part = n0 / (a.N / 3);
+        if (part < 2 && wm == 2) {  // 64 lanes x 4 bytes
+            const uint8_t *src = (const uint8_t *)(part == 0 ? a.norm_q : a.norm_k) + 4 * lane;
+            __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)src, (SVDQ_AS3 void *)(sepi + EPI_NORM_OFF), 4, 0, 0);
+        }
+    }
     if (a.bias != nullptr && wm == 3) {  // 64 lanes x 4 bytes = the tile's 128 bias values
         const uint8_t *src = (const uint8_t *)a.bias + (size_t)min(n0 + 2 * lane, a.N - 2) * 2;
         __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)src, (SVDQ_AS3 void *)(sepi + LORA_UP_BYTES), 4, 0, 0);
@@ -215,6 +224,23 @@ __device__ __forceinline__ void tile_epilogue(const svdq_gemm_args &a, v16f (&ac
                                               int m0, int n0, int pid_n, int wm, int lane) {
     const int l32 = lane & 31, half = lane >> 5;
     const int mw0 = m0 + wm * 32;
+
+    // Q/K RMSNorm + RoPE: the lane's rotary entries of a 32-column block are fetched two blocks ahead of their use, the
+    // first two blocks' before the transposition (issued one load at a time next to the arithmetic, as the compiler orders
+    // them under this register pressure, the sixteen dependent L2 round trips took 6 % of the launch); the head's norm
+    // weights came into LDS next to stage 0.
+    const int qk_part = EPI == SVDQ_EPI_QK_NORM_ROPE ? n0 / (a.N / 3) : 2;  // 0 = Q, 1 = K, 2 = V or no such epilogue
+    v4f qk_sc[2][4];
+    auto qk_fetch = [&](int bn, int buf) {
+        const int m = mw0 + l32;
+        const float *rot = a.rotary + (size_t)(m < a.actual_m ? m : 0) * a.ld_rotary;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int d = bn * 32 + 8 * j + 4 * half;  // channel within the head
+            qk_sc[buf][j] = *(const v4f *)(rot + d);  // (sin, cos, sin, cos)
+        }
+    };
+
 
     // ---- LoRA-up and bias, still in the main loop's orientation (lane = weight row, registers = activation rows) ----
     // The bias and the first 32 ranks of lora_up were fetched into LDS next to stage 0 and arrived long ago; the
@@ -260,6 +286,13 @@ __device__ __forceinline__ void tile_epilogue(const svdq_gemm_args &a, v16f (&ac
             const float b = T::to_f32(*(const uint16_t *)(sepi + LORA_UP_BYTES + (bn * 32 + l32) * 2));
 #pragma unroll
             for (int i = 0; i < 16; i++) acc[bn][i] += b;
+        }
+    }
+
+    if constexpr (EPI == SVDQ_EPI_QK_NORM_ROPE) {
+        if (qk_part < 2) {  // measured: issued ahead of LoRA-up as well, the launch takes 0.6 % longer
+            qk_fetch(0, 0);
+            qk_fetch(1, 1);
         }
     }
 
@@ -319,12 +352,7 @@ __device__ __forceinline__ void tile_epilogue(const svdq_gemm_args &a, v16f (&ac
 
     if (EPI == SVDQ_EPI_QK_NORM_ROPE) {
         // the 128-wide tile is one head, all of it in this wavefront; part 0 = Q, 1 = K, 2 = V (untouched)
-        const int part = n0 / (a.N / 3);
-        if (part < 2) {
-            const uint16_t *nw = (const uint16_t *)(part == 0 ? a.norm_q : a.norm_k);
-            const int m = mw0 + l32;
-            const bool rok = m < a.actual_m;
-            const float *rot = a.rotary + (size_t)(rok ? m : 0) * a.ld_rotary;
+        if (qk_part < 2) {
             float ss = 0.0f;
 #pragma unroll
             for (int bn = 0; bn < NBN; bn++)
@@ -333,12 +361,12 @@ __device__ __forceinline__ void tile_epilogue(const svdq_gemm_args &a, v16f (&ac
             ss += __shfl_xor(ss, 32);
             const float rstd = 1.0f / sqrtf(ss / 128.0f + a.eps);
 #pragma unroll
-            for (int bn = 0; bn < NBN; bn++)
+            for (int bn = 0; bn < NBN; bn++) {
+                const int buf = bn & 1;
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
-                    const int d = bn * 32 + 8 * j + 4 * half;  // channel within the head
-                    const uint2 wb = *(const uint2 *)(nw + d);
-                    const v4f sc = *(const v4f *)(rot + d);  // (sin, cos, sin, cos)
+                    const uint2 wb = *(const uint2 *)(sepi + EPI_NORM_OFF + (bn * 32 + 8 * j + 4 * half) * 2);
+                    const v4f sc = qk_sc[buf][j];
                     const float x0 = acc[bn][4 * j + 0] * rstd * T::lo_f32(wb.x);
                     const float x1 = acc[bn][4 * j + 1] * rstd * T::hi_f32(wb.x);
                     const float x2 = acc[bn][4 * j + 2] * rstd * T::lo_f32(wb.y);
@@ -348,6 +376,8 @@ __device__ __forceinline__ void tile_epilogue(const svdq_gemm_args &a, v16f (&ac
                     acc[bn][4 * j + 2] = x2 * sc[3] - x3 * sc[2];
                     acc[bn][4 * j + 3] = x2 * sc[2] + x3 * sc[3];
                 }
+                if (bn + 2 < NBN) qk_fetch(bn + 2, buf);  // behind the block's last use of this buffer
+            }
         }
         store_out();
         return;
@@ -672,7 +702,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_i8_kernel(svdq_gemm_arg
     load_scales(0);
 #pragma unroll
     for (int i = 0; i < PER_WAVE; i++) dma_one(0, sbuf0, i);
-    fetch_epilogue_operands(a, sepi, n0, wm, lane);
+    fetch_epilogue_operands<EPI>(a, sepi, n0, wm, lane);
     // One stage = eight (group, weight block) steps, software-pipelined inside the wavefront: the MFMAs of step b + 1
     // are issued before the dequantisation FMAs of step b, and the operands of step b + 2 are read from LDS behind
     // them, so the VALU work of a step runs while the matrix pipe works on the next one.
@@ -852,7 +882,7 @@ __global__ __launch_bounds__(NTHREADS, PIPE ? 2 : 3) void gemm_w4a4_f8_kernel(sv
     load_regs(0);
 #pragma unroll
     for (int i = 0; i < 4; i++) dma(0, sbuf0, 0, i);
-    fetch_epilogue_operands(a, sepi, n0, wm, lane);
+    fetch_epilogue_operands<EPI>(a, sepi, n0, wm, lane);
 
     // One stage = eight (group, weight block) steps: scale product, group product, sixteen FMAs.  The operands of the next
     // step (the step after next when PIPE) are read from LDS behind the matrix instructions.
