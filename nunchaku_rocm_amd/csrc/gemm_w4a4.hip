@@ -408,9 +408,11 @@ __device__ __forceinline__ void tile_epilogue(const svdq_gemm_args &a, v16f (&ac
             for (int i = 0; i < 16; i++) d[i] = 0.0f;
             const int r = rc + l32;
 #pragma unroll
-            for (int bn = 0; bn < NBN; bn++)
+            for (int bn = 0; bn < NBN; bn++) {
 #pragma unroll
                 for (int s = 0; s < 2; s++) {
+                    // (fetched ahead of the GELU arithmetic, all at once or two column blocks ahead, these loads spill
+                    // registers and the launch is no faster: the other workgroups of the CU cover their latency)
                     v4i la = (v4i){0, 0, 0, 0};
                     if (r < a.R2) {
                         const uint16_t *lp = ldt + (size_t)r * a.N + n0 + bn * 32 + 16 * s + 4 * half;
@@ -422,6 +424,7 @@ __device__ __forceinline__ void tile_epilogue(const svdq_gemm_args &a, v16f (&ac
                     for (int e = 0; e < 4; e++) xb[e] = (int)pack2<T>(acc[bn][8 * s + 2 * e], acc[bn][8 * s + 2 * e + 1]);
                     d = mfma32_16bit<T>(la, xb, d);
                 }
+            }
             const int m = mw0 + l32;
 #pragma unroll
             for (int j = 0; j < 4; j++) {

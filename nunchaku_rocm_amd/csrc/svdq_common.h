@@ -133,11 +133,13 @@ __device__ inline float max_with_lane_xor16(float v) {
 
 __device__ inline float gelu_tanh(float x) {
     // 0.5 x (1 + tanh(u)), u = 0.79788456 (x + 0.044715 x^3), which the reference spells 0.5 x (1 + 2 / (1 + exp(-2 u)) - 1)
-    // (nunchaku/ops/triton/_common.py:71-78).  That is x / (1 + exp(-2 u)); with the hardware reciprocal (1 ulp) it is 9
-    // instructions instead of 22 (an IEEE divide is ten of them) and agrees with the spelled-out form to a few ulp of
-    // fp32, which is also how far exp() implementations differ from each other.
-    float inner = 0.79788456f * (x + 0.044715f * x * x * x);
-    return x * __builtin_amdgcn_rcpf(1.0f + __expf(-2.0f * inner));
+    // (nunchaku/ops/triton/_common.py:71-78).  That is x / (1 + exp(-2 u)) = x / (1 + 2^(x (c0 + c1 x^2))) with
+    // c0 = -2 * 0.79788456 * log2(e), c1 = 0.044715 c0: seven instructions with the hardware exp2 and reciprocal (1 ulp
+    // each) instead of 22 for the spelled-out form (an IEEE divide alone is ten), and within a few ulp of fp32 of it, which
+    // is also how far exp() implementations differ from each other.
+    constexpr float c0 = -2.0f * 0.79788456f * 1.4426950408889634f, c1 = 0.044715f * c0;
+    const float p = __builtin_fmaf(x * x, c1, c0);
+    return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * p));
 }
 
 __device__ inline float silu(float x) { return x / (1.0f + __expf(-x)); }
