@@ -160,17 +160,24 @@ int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream);
 int svdq_gemm_w4a4_set_variant(int32_t variant);
 
 /*
- * One-time re-layout of a weight for the GEMM.  Every (32-row block, pair of scale groups) becomes three 1 KB blocks of
- * fp6 (e2m3) codes in the order the MFMA lanes read them: a signed int4 value v is stored as the six bits
- * sign | |v|, which the matrix instruction reads as v / 8 exactly; a lane's 32 weights of a group are six registers
- * (blocks 0 and 1: registers 0-3 of the pair's first and second group, block 2: registers 4-5 of both; a missing second
- * group is zeros).  v_mfma_scale_f32_32x32x64_f8f6f4 takes them next to fp8 activation codes at the int8 rate, a whole
- * 64-deep group per instruction, and returns the integer dot product as fp32, which saves the GEMM one of its two
- * scaling multiplies per output and group.  Behind the codes sit, per weight row, two T
- * pieces per group (hi + lo) of -8 * ws[g, n] * (sum of the group's 64 weights): the GEMM offsets signed activations by
- * +8 for the fp8 operand and takes that term out again.  `planes` needs svdq_weight_planes_bytes(N, K) bytes
- * (= ceil(N/32) * (ceil(K/128) * 3072 + 32 * 4 * ceil(K/1024)*16): three quarters of a byte per weight).  The copy depends on `wgt` AND `wscales` (dtype = their type).  No
- * counterpart in the reference (its SwiGLU path re-orders weight rows at load in the same spirit, ops/fused.py:83-105).
+ * One-time re-layout of a weight for the GEMM.  Every (32-row block, pair of scale groups = one stage of the main
+ * loop) becomes three 1 KB blocks of fp6 (e2m3) codes in the order the MFMA lanes read them: a signed int4 value v is
+ * stored as the six bits sign | |v|, which the matrix instruction reads as v / 8 exactly; a lane's 32 weights of a
+ * group are six registers (blocks 0 and 1: registers 0-3 of the pair's first and second group, block 2: registers 4-5
+ * of both; a missing second group is zeros).  v_mfma_scale_f32_32x32x64_f8f6f4 takes them next to fp8 activation codes
+ * at the int8 rate, a whole 64-deep group per instruction, and returns the integer dot product as fp32, which saves
+ * the GEMM one of its two scaling multiplies per output and group.  Behind the codes sit, per (32-row block, stage),
+ * 32 rows of six T values: the two pieces (hi + lo) of D = -ws[g, n] * (8 * sum of the group's even-k weights
+ * - 7 * sum of its odd-k weights) for the stage's two groups, then the two weight scales themselves; each block of
+ * rows has one more (zero) stage than the loop runs.  The GEMM carries a signed activation a as a + 8 for even k and
+ * a - 7 for odd k (sign | magnitude fp8 codes, one bit operation per plane) and adds as[g, m] * D[g, n] back with a
+ * 16-bit matrix instruction; with the two signs the offset term has no systematic part whatever the mean of the
+ * weights.  The last 16 bytes are a status word: non-zero when a D piece or a scale is not finite in T (fp16 weight
+ * scales above about 17: |8 We - 7 Wo| reaches 3840); such a copy must not be used (the Python cache then keeps the packed weight and the int8 loop).
+ * `planes` needs svdq_weight_planes_bytes(N, K) bytes = ceil(N/32) * (ceil(K/128) * 3072 + (ceil(K/128) + 1) * 384)
+ * + 16: 0.84 bytes per weight.  The copy depends on `wgt` AND `wscales` (dtype = their type); once it exists the
+ * GEMM reads neither (`wgt` may then be NULL, and a caller may free the packed weight).  No counterpart in the
+ * reference (its SwiGLU path re-orders weight rows at load in the same spirit, ops/fused.py:83-105).
  */
 int svdq_split_weight_planes(const void *wgt, const void *wscales, void *planes, int32_t N, int32_t K, int32_t ld_wgt,
                              int32_t ld_wscales, int32_t dtype, void *stream);

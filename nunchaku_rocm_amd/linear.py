@@ -53,9 +53,9 @@ class SVDQW4A4Linear(nn.Module):
 
     # ---- memory: the GEMM's working copy can stand in for the packed weight ------------------------------------------
     def release_packed_weight(self) -> bool:
-        """Drop the bytes of ``qweight`` and keep only the GEMM's working copy of it (1.5 x as large; made now if it does not
-        exist yet).  The fp8 main loop never reads the packed weight, so a model that would otherwise hold both (2.5 x the
-        packed bytes) holds 1.5 x.  ``qweight`` keeps its shape (every row a view of one spare row); ``state_dict()`` still
+        """Drop the bytes of ``qweight`` and keep only the GEMM's working copy of it (1.7 x as large; made now if it does not
+        exist yet).  The fp8 main loop never reads the packed weight, so a model that would otherwise hold both (2.7 x the
+        packed bytes) holds 1.7 x.  ``qweight`` keeps its shape (every row a view of one spare row); ``state_dict()`` still
         returns the packed weight, rebuilt from the copy; :meth:`restore_packed_weight` puts it back in place.  Returns
         ``False`` (and changes nothing) when the weight has no usable working copy (rows not 16-byte aligned, or fp16
         scales too large for its 16-bit offset terms)."""
