@@ -34,7 +34,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # in profiles/bench_all_kernels_hbm_traffic.txt, the factors being what the same counters read on plain copy kernels of
 # known size in the same run (FETCH_SIZE reads half the bytes of 16-byte-per-lane loads); counters cannot be read from
 # inside this process
-GEMM_QKV_HBM_BYTES = (2.0 * 77861.3 + 82944.5) * 1024
+GEMM_QKV_HBM_BYTES = (2.0 * 78804.4 + 82944.0) * 1024
 
 
 def _events(n):
@@ -371,7 +371,7 @@ def main():
                    "M": M, "K": K, "N": N, "rank": R, "group": 64},  # fmt: skip
         "roofline": {
             "bound": "mfma",
-            "kernel": "gemm_w4a4_kernel<BF16, signed, plain, pre-split weights>",
+            "kernel": "gemm_w4a4_f8_kernel<BF16, signed activations, plain epilogue, three workgroups per CU>",
             "achieved": round(achieved, 2),
             "peak": INT8_MFMA_PEAK_TOPS,
             "unit": "TOP/s",
