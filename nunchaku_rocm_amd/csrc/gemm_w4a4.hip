@@ -87,15 +87,15 @@ constexpr int F8_STAGE_BYTES = NBN * WPL_BLOCKS * BLK_BYTES;  // 12288
 // ... and, per (block of 32 rows, stage), 32 rows of six 16-bit values: the two pieces (hi + lo) of
 // D = -ws * (8 * sum of the group's even weights - 7 * sum of its odd weights) for the stage's two groups, then the two
 // weight scales.  A 12-byte-per-lane global -> LDS load puts lane l's bytes at 16 l, so in LDS a row takes 16 bytes; they
-// sit in a ring of eight stages per block; one load brings a stage and the one after it (64 lanes = two stages' rows), so
-// a ninth slot takes what runs past slot 7.
+// sit in a ring of eight stages per block; one load brings a stage and the one after it (64 lanes = two stages' rows)
+// into an even slot and its neighbour.
 constexpr int AUX_ROW = 12;                                  // bytes per row and stage in memory
 constexpr int AUX_BLK = 32 * AUX_ROW;                        // 384
 constexpr int AUX_LROW = 16;                                 // ... and in LDS
 constexpr int AUX_LBLK = 32 * AUX_LROW;                      // 512
 constexpr int AUX_SLOTS = 8;
-constexpr int AUX_NBLK_BYTES = (AUX_SLOTS + 1) * AUX_LBLK;   // 4608
-constexpr int F8_RING_BYTES = NBN * AUX_NBLK_BYTES;          // 18432: after the loop two wavefronts' private memory
+constexpr int AUX_NBLK_BYTES = AUX_SLOTS * AUX_LBLK;         // 4096
+constexpr int F8_RING_BYTES = NBN * AUX_NBLK_BYTES;          // 16384: after the loop two wavefronts' private memory
 static_assert(2 * PRIV_BYTES <= F8_RING_BYTES, "two wavefronts' private epilogue memory must fit the ring");
 static_assert(PRIV_BYTES <= F8_STAGE_BYTES, "a wavefront's private epilogue memory must fit a staging buffer");
 constexpr int PLANES_STATUS_BYTES = 16;  // trailing status word of a pre-split weight
@@ -823,7 +823,8 @@ __global__ __launch_bounds__(NTHREADS, PIPE ? 2 : 3) void gemm_w4a4_f8_kernel(sv
             __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)src, (SVDQ_AS3 void *)(dstbuf + (wm * WPL_BLOCKS + i) * BLK_BYTES), 16, 0, 0);
         } else {
             // 64 lanes x 12 bytes = the rows of stage s and of stage s + 1 (the copy has one stage of padding), into the given
-            // ring slot and the one after it, which the next stage's load fills with the same bytes again
+            // ring slot and the one after it: issued before the loop for stages 0 and 1 and then by every odd stage for the two
+            // stages after it (an even slot and its neighbour)
             const uint8_t *src = xbase + ((uint32_t)lane * (uint32_t)AUX_ROW + (uint32_t)s * (uint32_t)AUX_BLK);
             __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)src,
                                              (SVDQ_AS3 void *)(sring + wm * AUX_NBLK_BYTES + slot * AUX_LBLK), 12, 0, 0);
@@ -953,7 +954,7 @@ __global__ __launch_bounds__(NTHREADS, PIPE ? 2 : 3) void gemm_w4a4_f8_kernel(sv
                 const v16f P = group(b, w8[b & 1]);
                 __builtin_amdgcn_sched_barrier(0);
                 if (b + 1 < 8) w8[(b + 1) & 1] = read_w8(b + 1);
-                if (b < 4) dma(sn, other, slotn, b);
+                if (b < WPL_BLOCKS || (b == WPL_BLOCKS && (ST & 1))) dma(sn, other, slotn, b);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int i = 0; i < 16; i++) acc[b & 3][i] = __builtin_fmaf(P[i], S[i], acc[b & 3][i]);
@@ -977,7 +978,7 @@ __global__ __launch_bounds__(NTHREADS, PIPE ? 2 : 3) void gemm_w4a4_f8_kernel(sv
                 // b + 1's operands would also wait for these
                 __builtin_amdgcn_sched_barrier(0);
                 if (b + 2 < 8) w8[(b + 2) % 3] = read_w8(b + 2);
-                if (b < 4) dma(sn, other, slotn, b);
+                if (b < WPL_BLOCKS || (b == WPL_BLOCKS && (ST & 1))) dma(sn, other, slotn, b);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int i = 0; i < 16; i++) acc[b & 3][i] = __builtin_fmaf(P[cur][i], S[cur][i], acc[b & 3][i]);
