@@ -22,7 +22,7 @@
 //    weight codes; it is taken out again every four stages with a 16-bit matrix instruction on (as, -ws * offset),
 //    whose operands travel with the weights.  Only the weights go through LDS (with their scales and offset terms);
 //    a wavefront's own 32 activation rows and activation scales go to registers, one stage ahead.  The kernel is held
-//    to 168 vector registers and 50.25 KB of LDS so that three workgroups share a CU (three wavefronts per SIMD): a
+//    to 168 vector registers and 48.5 KB of LDS so that three workgroups share a CU (three wavefronts per SIMD): a
 //    wavefront issues scale product, group product and the sixteen FMAs of a step in program order (single result
 //    buffers) and the other two wavefronts of the SIMD fill the matrix pipe and the vector ALU meanwhile.
 //  * gemm_w4a4_i8_kernel (packed weights): a 16-byte LDS read holds 32 nibbles; the even and the odd nibbles are split
