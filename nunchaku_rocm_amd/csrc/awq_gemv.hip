@@ -163,9 +163,9 @@ __global__ __launch_bounds__(AWQ_WAVES * 64) __attribute__((amdgpu_waves_per_eu(
         for (int i = 0; i < XPASSES; i++) {
             const int q = min(lane + 64 * i, XPIECES - 1), u = q / (8 * RP), r = (q >> 3) & (RP - 1), slot = q & 7;
             const v4i v = *(const v4i *)(xw + 16 * q);
-            float s = 0.0f;
+            float s = 0.0f;  // one dot-product instruction per pair of values (against (1, 1)) instead of two unpacks and two adds
 #pragma unroll
-            for (int e = 0; e < 4; e++) s += T::lo_f32((uint32_t)v[e]) + T::hi_f32((uint32_t)v[e]);
+            for (int e = 0; e < 4; e++) s = T::sum2((uint32_t)v[e], s);
             s += dpp_f32<0xB1>(s);  // quad_perm [1, 0, 3, 2]
             s += dpp_f32<0x4E>(s);  // quad_perm [2, 3, 0, 1]
             if (SMALL) {            // slots 4 h .. 4 h + 3 hold the pieces of half h (r < 4 permutes within them)
