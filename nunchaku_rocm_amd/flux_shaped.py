@@ -106,7 +106,10 @@ class HipBackend:
         call overwrites."""
         if x.shape[0] > 8 or any(lin.group_size != 64 or lin.out_features % 32 for lin in lins):
             return [lin(x) for lin in lins]
-        key = tuple(id(lin) for lin in lins) + (x.shape[0], x.dtype)
+        # the plan holds device addresses and a stacked copy of the biases: it is only good while the layers' tensors stay
+        # where they are (a model moved, reloaded or given other parameters gets a new plan)
+        key = tuple((lin.qweight.data_ptr(), lin.wscales.data_ptr(), lin.wzeros.data_ptr(),
+                     None if lin.bias is None else (lin.bias.data_ptr(), lin.bias._version)) for lin in lins) + (x.shape[0], x.dtype)  # fmt: skip
         plan = self._awq_plans.get(key)
         if plan is None:
             plan = []

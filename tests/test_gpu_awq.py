@@ -105,6 +105,42 @@ def test_linear_module_adds_bias_after_kernel(dev):
     assert O.max_rel_err(y, ref) <= 1e-2
 
 
+def test_model_side_batching_follows_the_layers_tensors(dev):
+    """The harness batches its adaLN layers through a cached plan of device addresses; a layer whose tensors were replaced
+    or whose bias changed in place must not be served from the old plan."""
+    from nunchaku_rocm_amd.flux_shaped import HipBackend
+    from nunchaku_rocm_amd.linear import AWQW4A16Linear
+
+    K, N = 256, 128
+    mods = []
+    for i in range(3):
+        lin = O.make_awq_linear(K, N, seed=50 + i)
+        mod = AWQW4A16Linear(K, N, bias=True, device=dev)
+        with torch.no_grad():
+            mod.qweight.copy_(lin["qweight"])
+            mod.wscales.copy_(lin["wscales"])
+            mod.wzeros.copy_(lin["wzeros"])
+            mod.bias.copy_(torch.full((N,), 0.25 * i).to(torch.bfloat16))
+        mods.append(mod)
+    x = torch.randn(1, K, generator=torch.Generator().manual_seed(7)).to(torch.bfloat16).to(dev)
+    be = HipBackend(two_streams=False)
+
+    def check():
+        got = be.awq_many(x, mods)
+        for g, mod in zip(got, mods):
+            assert torch.equal(g.cpu().view(torch.int16), mod(x).cpu().view(torch.int16))
+
+    check()
+    check()  # from the cached plan
+    other = O.make_awq_linear(K, N, seed=99)
+    mods[1].qweight.data = other["qweight"].to(dev)  # new storage
+    mods[1].wscales.data = other["wscales"].to(dev)
+    check()
+    with torch.no_grad():
+        mods[2].bias.add_(1.0)  # same storage, new values
+    check()
+
+
 @pytest.mark.parametrize("group_size", [32, 64, 128])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_dequantize_bit_exact(dev, group_size, dtype):
