@@ -5,8 +5,10 @@
 // with p_g the exact int32 dot product of the group's 64 int4 pairs.
 //
 // Two kernels share one epilogue.  In both, 256 threads = four wavefronts, each 32 activation rows x all 128 weight rows
-// of a 128x128 tile; the MFMA's A operand is the activation tile and its B operand the weight tile, so in the main loop a
-// lane owns one weight row n and its registers walk the wavefront's 32 activation rows.  K is staged through LDS 128 at
+// of a 128x128 tile.  The fp8 kernel passes the weight tile as the MFMA's first operand and the activation tile as its
+// second, so a lane of the result owns one activation row m and its registers walk the block's weight rows: the
+// orientation every row-wise epilogue wants; the int8 kernel has them the other way round (its scale FMAs want the weight
+// scale per lane) and turns its results through LDS after the loop.  K is staged through LDS 128 at
 // a time (two scale groups), two stages; operands that several wavefronts read go global -> LDS directly
 // (global_load_lds, no registers), one stage ahead, into a lane-linear layout (LDS slot l of a 1 KB block = the 16 bytes
 // MFMA lane l needs), so the operand reads are bank-conflict free by construction; one raw s_barrier per stage with
@@ -36,9 +38,9 @@
 //
 //  * The bias and the first 32 ranks of lora_up of the tile are fetched into LDS together with stage 0, in MFMA lane
 //    order, so that the LoRA-up section does not wait for them.
-//  * After LoRA-up and bias each wavefront turns its four 32x32 blocks through a private LDS tile into "lane =
-//    activation row": row-wise epilogue work (RMSNorm sum of squares, RoPE pairs, group absmax, nibble packing, the
-//    next layer's LoRA-down operand) is then in-lane plus one exchange with lane ^ 32.
+//  * With "lane = activation row" (the fp8 kernel's native orientation; the int8 kernel turns its four 32x32 blocks
+//    through a private LDS tile after LoRA-up and bias) row-wise epilogue work (RMSNorm sum of squares, RoPE pairs,
+//    group absmax, nibble packing, the next layer's LoRA-down operand) is in-lane plus one exchange with lane ^ 32.
 //  * The 16-bit output leaves through a wavefront-private, XOR-swizzled LDS tile as 256-byte row segments, stored
 //    non-temporally.  Everything after the main loop is private to a wavefront: one barrier follows the loop, none
 //    after it.
@@ -217,9 +219,11 @@ __device__ inline void fetch_epilogue_operands(const svdq_gemm_args &a, uint8_t 
 }
 
 // Everything after the main loop, for one wavefront: acc[bn][i] holds out[m = mw0 + 8 (i >> 2) + 4 half + (i & 3)]
-// [n = n0 + 32 bn + lane % 32] without LoRA-up and bias.  `priv` is PRIV_BYTES of LDS nobody else touches from here on;
+// [n = n0 + 32 bn + lane % 32] without LoRA-up and bias -- or, with ROWS_IN_LANES (a main loop that passes the weights as
+// the matrix instruction's first operand), out[m = mw0 + lane % 32][n = n0 + 32 bn + 8 (i >> 2) + 4 half + (i & 3)],
+// which is the orientation every row-wise epilogue wants: the turn through LDS below is then not needed.  `priv` is PRIV_BYTES of LDS nobody else touches from here on;
 // `sepi` holds what fetch_epilogue_operands brought.  No workgroup barrier inside.
-template <typename T, int EPI>
+template <typename T, int EPI, bool ROWS_IN_LANES = false>
 __device__ __forceinline__ void tile_epilogue(const svdq_gemm_args &a, v16f (&acc)[NBN], uint8_t *priv, const uint8_t *sepi,
                                               int m0, int n0, int pid_n, int wm, int lane) {
     const int l32 = lane & 31, half = lane >> 5;
@@ -276,16 +280,28 @@ __device__ __forceinline__ void tile_epilogue(const svdq_gemm_args &a, v16f (&ac
                 ub[2] = (int)pack2<T>(f1[0], f1[1]);
                 ub[3] = (int)pack2<T>(f1[2], f1[3]);
 #pragma unroll
-                for (int bn = 0; bn < NBN; bn++) acc[bn] = mfma32_16bit<T>(ub, ua[c][bn], acc[bn]);
+                for (int bn = 0; bn < NBN; bn++)
+                    acc[bn] = ROWS_IN_LANES ? mfma32_16bit<T>(ua[c][bn], ub, acc[bn]) : mfma32_16bit<T>(ub, ua[c][bn], acc[bn]);
             }
         }
     }
     if (a.bias != nullptr) {
 #pragma unroll
         for (int bn = 0; bn < NBN; bn++) {
-            const float b = T::to_f32(*(const uint16_t *)(sepi + LORA_UP_BYTES + (bn * 32 + l32) * 2));
+            if constexpr (ROWS_IN_LANES) {
 #pragma unroll
-            for (int i = 0; i < 16; i++) acc[bn][i] += b;
+                for (int j = 0; j < 4; j++) {
+                    const uint2 b4 = *(const uint2 *)(sepi + LORA_UP_BYTES + (bn * 32 + 8 * j + 4 * half) * 2);
+                    acc[bn][4 * j + 0] += T::lo_f32(b4.x);
+                    acc[bn][4 * j + 1] += T::hi_f32(b4.x);
+                    acc[bn][4 * j + 2] += T::lo_f32(b4.y);
+                    acc[bn][4 * j + 3] += T::hi_f32(b4.y);
+                }
+            } else {
+                const float b = T::to_f32(*(const uint16_t *)(sepi + LORA_UP_BYTES + (bn * 32 + l32) * 2));
+#pragma unroll
+                for (int i = 0; i < 16; i++) acc[bn][i] += b;
+            }
         }
     }
 
@@ -300,7 +316,7 @@ __device__ __forceinline__ void tile_epilogue(const svdq_gemm_args &a, v16f (&ac
     // One 32x32 block at a time through the private tile (the LDS operations of one wavefront complete in order).
     // Afterwards lane (m = lane % 32, half) holds columns 32 bn + 8 j + 4 half + e of row m in acc[bn][4 j + e]: row-wise
     // epilogue work is in-lane plus one exchange with lane ^ 32, and no epilogue needs another wavefront's data.
-    {
+    if constexpr (!ROWS_IN_LANES) {
         float *tp = (float *)priv;
 #pragma unroll
         for (int bn = 0; bn < NBN; bn++) {
@@ -870,7 +886,7 @@ __global__ __launch_bounds__(NTHREADS, PIPE ? 2 : 3) void gemm_w4a4_f8_kernel(sv
         for (int bn = 0; bn < NBN; bn++) {
             const uint32_t *p0 = (const uint32_t *)(sring + bn * AUX_NBLK_BYTES + off0);
             const uint32_t *p1 = (const uint32_t *)(sring + bn * AUX_NBLK_BYTES + off1);
-            acc[bn] = mfma32_16bit<T>(ubv, (v4i){(int)p0[0], (int)p0[1], (int)p1[0], (int)p1[1]}, acc[bn]);
+            acc[bn] = mfma32_16bit<T>((v4i){(int)p0[0], (int)p0[1], (int)p1[0], (int)p1[1]}, ubv, acc[bn]);
         }
     };
     int par = 0;                                         // parity of the group of four stages: ring slots 0-3 or 4-7
@@ -941,9 +957,9 @@ __global__ __launch_bounds__(NTHREADS, PIPE ? 2 : 3) void gemm_w4a4_f8_kernel(sv
         const v16f z16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
         // as[m] * ws[n] of a step, exact (two 16-bit values, one non-zero product): a 16-bit matrix instruction, which runs
         // beside the vector FMAs; the fp32 rank-1 matrix instruction shares the vector ALUs and does not
-        auto scales = [&](int b) -> v16f { return mfma32_16bit_k8<T>(sa[b >> 2], (v2i){(int)wsd[b & 3], 0}, z16); };
+        auto scales = [&](int b) -> v16f { return mfma32_16bit_k8<T>((v2i){(int)wsd[b & 3], 0}, sa[b >> 2], z16); };
         auto group = [&](int b, const v8i &w) -> v16f {
-            return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8[b >> 2], w, z16, 0, 2, 0, F8_SCALE, 0, F6_SCALE);
+            return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(w, a8[b >> 2], z16, 2, 0, 0, F6_SCALE, 0, F8_SCALE);
         };
         if constexpr (!PIPE) {
             v8i w8[2];
@@ -1014,7 +1030,7 @@ __global__ __launch_bounds__(NTHREADS, PIPE ? 2 : 3) void gemm_w4a4_f8_kernel(sv
     // Every wavefront has left the main loop: the staging memory becomes the wavefronts' private epilogue memory.
     __syncthreads();
     uint8_t *priv = wm == 0 ? sbuf0 : wm == 1 ? sbuf1 : sring + (wm - 2) * PRIV_BYTES;
-    tile_epilogue<T, EPI>(a, acc, priv, sepi, m0, n0, pid_n, wm, lane);
+    tile_epilogue<T, EPI, true>(a, acc, priv, sepi, m0, n0, pid_n, wm, lane);
 }
 
 // lora_act_out[m, r] = sum over n-tiles of the partial LoRA-down products, in tile order (deterministic)
@@ -1055,7 +1071,7 @@ __global__ __launch_bounds__(64) void group_acc_kernel(const uint8_t *act, const
     }
 }
 
-// The same read-out through the instruction sequence of the pre-split (fp8) path: activation nibbles as fp8 codes
+// The same read-out through the instructions of the pre-split (fp8) path (operands in the other order): activation nibbles as fp8 codes
 // (signed ones as a + 8 for even k and a - 7 for odd k), weights as fp6 codes,
 // v_mfma_scale_f32_32x32x64_f8f6f4 with block scales 2^9 and 2^3, offset term 8 We - 7 Wo taken out.  Every value involved
 // is an integer below 2^24, so the fp32 result is exact.
