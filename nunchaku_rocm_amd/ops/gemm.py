@@ -10,8 +10,8 @@ from ._prep import pinned_weight_planes as _pinned_weight_planes
 from ._prep import weight_planes as _weight_planes
 
 # Which weights get the GEMM's working copy (fp6 codes in MFMA lane order with their scales and offset terms, cached per
-# tensor, see _prep.weight_planes; 0.84 bytes per weight next to the packed weight's 0.5; without it the GEMM is 35 %
-# slower, 236 against 175 us at the FLUX QKV shape): "parameters" = weights that are nn.Parameter (module weights, which
+# tensor, see _prep.weight_planes; 0.84 bytes per weight next to the packed weight's 0.5; without it the GEMM is 36 %
+# slower, 240 against 176 us at the FLUX QKV shape): "parameters" = weights that are nn.Parameter (module weights, which
 # live long), "all" = any weight tensor (a temporary pays the re-layout on every call), "none" = the GEMM unpacks the
 # packed weight itself (int8 main loop, no extra memory).
 USE_WEIGHT_PLANES = "parameters"
