@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define SVDQ_ABI_VERSION 7
+#define SVDQ_ABI_VERSION 8
 
 enum { SVDQ_BF16 = 0, SVDQ_FP16 = 1 };
 enum { SVDQ_PRE_NONE = 0, SVDQ_PRE_GLU = 1, SVDQ_PRE_GELU = 2 }; /* svdq_quantize_args.prologue */
@@ -149,9 +149,24 @@ typedef struct {
     float *scratch;           /* svdq_gemm_w4a4_scratch_bytes() bytes of fp32 LoRA-down partial sums, or NULL    */
     int32_t R2, ld_qout, ld_oscales, ld_lora_act_out;
     float shift;              /* 0.171875 for GELU (ops/triton/gemm_w4a4.py:918), 0 for SwiGLU                  */
+    /* SVDQ_EPI_QK_NORM_ROPE, optional: the same table as `rotary`, re-laid-out by svdq_block_rotary (the fp8 main    */
+    /* loop's epilogue then reads 1 KB per load instruction instead of 32-byte pieces of 32 rows); NULL = not given  */
+    const float *rotary_blocked;
 } svdq_gemm_args;
 
 int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream);
+
+/*
+ * One-time re-layout of a rotary table for the Q/K RMSNorm + RoPE epilogue: (rows, 128) fp32 rows of (sin, cos) pairs,
+ * row stride ld_rotary elements -> ceil(rows / 32) blocks of 32 rows, each as sixteen 1 KB pieces in the order the
+ * epilogue's lanes read them: piece (column block bn, j) holds, for lane (row r = lane % 32, h = lane / 32), the four
+ * floats of columns 32 bn + 8 j + 4 h .. + 3 of row r (rows past the end repeat row 0, as the epilogue does for rows it
+ * never stores).  `blocked` needs svdq_rotary_blocked_bytes(rows) = ceil(rows / 32) * 16 KB, 16-byte aligned.  The
+ * table of a diffusion transformer is the same for every block and step, so callers make this once per table.  No
+ * counterpart in the reference.
+ */
+int svdq_block_rotary(const float *rotary, float *blocked, int32_t rows, int32_t ld_rotary, void *stream);
+size_t svdq_rotary_blocked_bytes(int32_t rows);
 
 /* The fp8 main loop exists in two builds: three workgroups per CU (fills a loaded CU best) and two per CU with
  * software-pipelined steps (a workgroup on its own runs faster); svdq_gemm_w4a4 picks by the number of 128x128 tiles and

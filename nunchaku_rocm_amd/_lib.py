@@ -14,7 +14,7 @@ import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libsvdq_mi355x.so")
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 BF16, FP16 = 0, 1
 EPI_PLAIN, EPI_QK_NORM_ROPE, EPI_GELU_QUANT, EPI_SWIGLU_QUANT = 0, 1, 2, 3
@@ -28,6 +28,8 @@ EXPORTS = (
     "svdq_transpose_lora_down",
     "svdq_gemm_w4a4",
     "svdq_gemm_w4a4_set_variant",
+    "svdq_block_rotary",
+    "svdq_rotary_blocked_bytes",
     "svdq_gemm_w4a4_scratch_bytes",
     "svdq_gemm_w4a4_static_scratch",
     "svdq_gemm_w4a4_static_scratch_capacity",
@@ -72,7 +74,7 @@ class GemmArgs(ctypes.Structure):
         + [("ld_rotary", _i32), ("eps", _f32)]
         + [(n, _vp) for n in ("qout", "oscales", "smooth_next", "lora_down_t", "lora_act_out", "scratch")]
         + [(n, _i32) for n in ("R2", "ld_qout", "ld_oscales", "ld_lora_act_out")]
-        + [("shift", _f32)]
+        + [("shift", _f32), ("rotary_blocked", _vp)]
     )  # fmt: skip
 
 
@@ -128,6 +130,9 @@ def load() -> ctypes.CDLL:
     lib.svdq_quantize_act.argtypes = [ctypes.POINTER(QuantizeArgs), _vp]
     lib.svdq_gemm_w4a4.argtypes = [ctypes.POINTER(GemmArgs), _vp]
     lib.svdq_gemm_w4a4_set_variant.argtypes = [_i32]
+    lib.svdq_block_rotary.argtypes = [_vp, _vp, _i32, _i32, _vp]
+    lib.svdq_rotary_blocked_bytes.restype = ctypes.c_size_t
+    lib.svdq_rotary_blocked_bytes.argtypes = [_i32]
     lib.svdq_gemm_w4a4_static_scratch.argtypes = [ctypes.POINTER(GemmArgs), _vp]
     lib.svdq_gemm_w4a4_static_scratch_capacity.restype = ctypes.c_size_t
     lib.svdq_gemm_w4a4_static_scratch_capacity.argtypes = []

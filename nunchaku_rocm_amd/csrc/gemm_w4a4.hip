@@ -236,6 +236,15 @@ __device__ __forceinline__ void tile_epilogue(const svdq_gemm_args &a, v16f (&ac
     const int qk_part = EPI == SVDQ_EPI_QK_NORM_ROPE ? n0 / (a.N / 3) : 2;  // 0 = Q, 1 = K, 2 = V or no such epilogue
     v4f qk_sc[2][4];
     auto qk_fetch = [&](int bn, int buf) {
+        if (a.rotary_blocked != nullptr) {
+            // re-laid-out table: the 64 lanes of a load read 1 KB in a row.  (From the (rows, 128) table a load fetches
+            // 32-byte pieces of 32 different rows; at the QKV shape that was 8 of the epilogue's 11 us.)
+            const int rb = min(mw0 >> 5, (a.actual_m + 31) / 32 - 1);
+            const v4f *p = (const v4f *)a.rotary_blocked + ((size_t)rb * 16 + bn * 4) * 64 + lane;
+#pragma unroll
+            for (int j = 0; j < 4; j++) qk_sc[buf][j] = p[j * 64];
+            return;
+        }
         const int m = mw0 + l32;
         const float *rot = a.rotary + (size_t)(m < a.actual_m ? m : 0) * a.ld_rotary;
 #pragma unroll
@@ -1103,6 +1112,16 @@ __global__ __launch_bounds__(64) void group_acc_f8_kernel(const uint8_t *act, co
     }
 }
 
+
+// rotary table -> the order the Q/K epilogue's lanes read it (svdq_block_rotary): one thread per 16-byte piece
+__global__ __launch_bounds__(256) void block_rotary_kernel(const float *rot, v4f *out, int rows, int ld, int pieces) {
+    const int o = blockIdx.x * 256 + threadIdx.x;
+    if (o >= pieces) return;
+    const int lane = o & 63, j = (o >> 6) & 3, bn = (o >> 8) & 3, rb = o >> 10;
+    const int row = rb * 32 + (lane & 31), d = bn * 32 + 8 * j + 4 * (lane >> 5);
+    out[o] = *(const v4f *)(rot + (size_t)(row < rows ? row : 0) * ld + d);
+}
+
 template <typename T, bool U, bool ODDG>
 static void launch_gemm_i8(const svdq_gemm_args &a, hipStream_t s) {
     const dim3 grid(((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN)), block(NTHREADS);
@@ -1371,6 +1390,10 @@ static int gemm_w4a4_checked(const svdq_gemm_args &a, void *stream) {
             set_error("svdq_gemm_w4a4: norm_q, norm_k (128,) and rotary (actual_m, 128) fp32 16-byte aligned rows are required");
             return SVDQ_E_INVALID;
         }
+        if (a.rotary_blocked && !al16(a.rotary_blocked)) {
+            set_error("svdq_gemm_w4a4: rotary_blocked must be 16-byte aligned");
+            return SVDQ_E_INVALID;
+        }
     } else if (quant) {
         const int NQ = a.epilogue == SVDQ_EPI_SWIGLU_QUANT ? a.N / 2 : a.N;
         if (a.N % 128 || a.M % 16) {
@@ -1417,6 +1440,18 @@ static int gemm_w4a4_checked(const svdq_gemm_args &a, void *stream) {
         rc = check_launch("svdq_gemm_w4a4 (LoRA-down partial sum)");
     }
     return rc;
+}
+
+extern "C" size_t svdq_rotary_blocked_bytes(int32_t rows) { return rows <= 0 ? 0 : (size_t)((rows + 31) / 32) * 16 * 1024; }
+
+extern "C" int svdq_block_rotary(const float *rotary, float *blocked, int32_t rows, int32_t ld_rotary, void *stream) {
+    if (!rotary || !blocked || rows <= 0 || ld_rotary < 128 || ld_rotary % 4 || ((uintptr_t)rotary & 15) || ((uintptr_t)blocked & 15)) {
+        set_error("svdq_block_rotary: rows=%d ld_rotary=%d; needs rows > 0, rows of 128 fp32 with ld_rotary %% 4 == 0, 16-byte aligned tensors", rows, ld_rotary);
+        return SVDQ_E_INVALID;
+    }
+    const int pieces = (rows + 31) / 32 * 1024;
+    hipLaunchKernelGGL(block_rotary_kernel, dim3((pieces + 255) / 256), dim3(256), 0, (hipStream_t)stream, rotary, (v4f *)blocked, rows, ld_rotary, pieces);
+    return check_launch("svdq_block_rotary");
 }
 
 extern "C" int svdq_gemm_w4a4_set_variant(int32_t variant) {

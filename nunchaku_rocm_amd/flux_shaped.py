@@ -446,6 +446,19 @@ class FluxShapedTransformer(nn.Module):
                 convert_svdq_linear_to_natural_layout(m)
 
     @torch.no_grad()
+    def _rot_parts(self, rot: torch.Tensor, t_txt: int):
+        """The text and image rows of the rotary table as tensors of their own, the same two objects for as long as the
+        table is the same tensor with the same contents: the operators keep a re-laid-out copy per table tensor, and a
+        forward pass recorded into a graph must not make new ones."""
+        hit = getattr(self, "_rot_split", None)
+        if hit is not None and hit[0]() is rot and hit[1] == (rot.data_ptr(), rot._version, t_txt):
+            return hit[2], hit[3]
+        import weakref
+
+        parts = (rot[:t_txt].contiguous(), rot[t_txt:].contiguous())
+        self._rot_split = (weakref.ref(rot), (rot.data_ptr(), rot._version, t_txt), parts[0], parts[1])
+        return parts
+
     def forward(self, latents, text, pooled, timestep, rot, backend=None):
         """latents (B, T_img, 64), text (B, T_txt, 4096), pooled (B, 768), timestep (B,) in [0, 1], rot the
         (T_txt + T_img, 64, 1, 2) rotary table (text rows first).  Returns the (B, T_img, 64) velocity."""
@@ -454,7 +467,7 @@ class FluxShapedTransformer(nn.Module):
         ctx = self.context_embedder(text)
         temb = self.time_in(_timestep_embedding(timestep).to(x.dtype)) + self.pooled_in(pooled)
         t_txt = ctx.shape[1]
-        rot_txt, rot_img = rot[:t_txt].contiguous(), rot[t_txt:].contiguous()
+        rot_txt, rot_img = self._rot_parts(rot, t_txt)
         # every adaLN projection takes silu(temb) and nothing else: all of them first, layers of equal width in one launch
         nd = len(self.double_blocks)
         if hasattr(be, "awq_many"):

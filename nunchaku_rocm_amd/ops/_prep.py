@@ -87,6 +87,36 @@ def lora_down_t(lora_down: torch.Tensor) -> torch.Tensor:
     return t
 
 
+_rotary_cache: dict[int, tuple] = {}
+
+
+def rotary_blocked(rotary_emb: torch.Tensor, rot2d: torch.Tensor) -> torch.Tensor | None:
+    """The rotary table in the order the Q/K RMSNorm + RoPE epilogue reads it (``svdq_block_rotary``).  ``rotary_emb`` is
+    the tensor the caller passed (the cache key: a model passes the same table to every block and step), ``rot2d`` its
+    ``(rows, 128)`` fp32 view with unit inner stride."""
+    key = id(rotary_emb)
+    hit = _rotary_cache.get(key)
+    if hit is not None:
+        ref, src, t, ready, rows = hit
+        if ref() is rotary_emb and _same_source(src, rotary_emb) and rows == rot2d.shape[0]:
+            ready.wait(t.device)
+            return t
+    if torch.cuda.is_current_stream_capturing():
+        return None  # no new copies while a graph is being recorded: the epilogue reads the table itself
+    lib = _lib.load()
+    rows = rot2d.shape[0]
+    t = torch.empty(lib.svdq_rotary_blocked_bytes(rows) // 4, dtype=torch.float32, device=rot2d.device)
+    with torch.cuda.device(t.device):
+        _lib.check(lib.svdq_block_rotary(rot2d.data_ptr(), t.data_ptr(), rows, rot2d.stride(0), _lib.stream_of(rot2d)))
+        ready = _Ready(t.device)
+    try:
+        ref = weakref.ref(rotary_emb, lambda _r, k=key: _rotary_cache.pop(k, None))
+        _rotary_cache[key] = (ref, _source_of(rotary_emb), t, ready, rows)
+    except TypeError:
+        pass
+    return t
+
+
 _planes_cache: dict[int, tuple] = {}
 _pinned: dict[int, tuple] = {}  # id(weight parameter) -> (weakref, planes): a weight whose packed bytes were released
 

@@ -7,6 +7,7 @@ import torch
 from .. import _lib
 from ._prep import lora_down_t as _lora_down_t
 from ._prep import pinned_weight_planes as _pinned_weight_planes
+from ._prep import rotary_blocked as _rotary_blocked
 from ._prep import weight_planes as _weight_planes
 
 # Which weights get the GEMM's working copy (fp6 codes in MFMA lane order with their scales and offset terms, cached per
@@ -15,6 +16,11 @@ from ._prep import weight_planes as _weight_planes
 # live long), "all" = any weight tensor (a temporary pays the re-layout on every call), "none" = the GEMM unpacks the
 # packed weight itself (int8 main loop, no extra memory).
 USE_WEIGHT_PLANES = "parameters"
+
+# The Q/K RMSNorm + RoPE epilogue reads the rotary table through a copy in the order its lanes want it (made once per
+# table tensor and cached, 16 KB per 32 rows): 1 KB per load instruction instead of 32-byte pieces of 32 rows, which was
+# most of that epilogue's cost.  False = read the (rows, 128) table itself (same results).
+USE_BLOCKED_ROTARY = True
 
 # True sends the requantizing epilogues' LoRA-down partial sums to the buffer built into the library
 # (svdq_gemm_w4a4_static_scratch) instead of a torch allocation per call: for callers that may not allocate, e.g. while
@@ -204,6 +210,7 @@ def svdq_gemm_w4a4_cuda(
     keep = [planes]  # tensors that must outlive the launch call
     lib = _lib.load()
     if want_qk:
+        rot_key = rotary_emb  # the caller's tensor: what the re-laid-out copy is cached under
         if rotary_emb.dtype != torch.float32:
             rotary_emb = rotary_emb.float()  # the reference's unfused kernel reads any dtype and computes in fp32
         rot = rotary_emb.reshape(actual_m, HEAD_DIM)
@@ -216,6 +223,12 @@ def svdq_gemm_w4a4_cuda(
         args.epilogue = _lib.EPI_QK_NORM_ROPE
         args.norm_q, args.norm_k, args.rotary = norm_q.data_ptr(), norm_k.data_ptr(), rot.data_ptr()
         args.ld_rotary = rot.stride(0)
+        if USE_BLOCKED_ROTARY and rot.data_ptr() % 16 == 0 and rot.stride(0) % 4 == 0:
+            # the epilogue reads the table re-laid-out for its lanes (made once per table, see _prep)
+            rb = _rotary_blocked(rot_key, rot)
+            if rb is not None:
+                keep.append(rb)
+                args.rotary_blocked = rb.data_ptr()
     elif want_quant:
         NQ = N // 2 if fuse_swiglu else N
         qout2d = qout.reshape(-1, qout.shape[-1])

@@ -55,8 +55,18 @@ def test_qk_norm_rope(dev, M, H, actual_m, unsigned, dtype):
     ops.svdq_gemm_w4a4_cuda(out=buf[:actual_m], norm_q=d(nq), norm_k=d(nk), rotary_emb=d(rot), **kw)
     plain = torch.empty(actual_m, N, dtype=dtype, device=dev)
     ops.svdq_gemm_w4a4_cuda(out=plain, **kw)
+    # the same from the (rows, 128) table itself instead of its re-laid-out copy: the same bits
+    from nunchaku_rocm_amd.ops import gemm as gemm_mod
+
+    natural = torch.empty(actual_m, N, dtype=dtype, device=dev)
+    gemm_mod.USE_BLOCKED_ROTARY = False
+    try:
+        ops.svdq_gemm_w4a4_cuda(out=natural, norm_q=d(nq), norm_k=d(nk), rotary_emb=d(rot), **kw)
+    finally:
+        gemm_mod.USE_BLOCKED_ROTARY = True
     torch.cuda.synchronize()
     assert bool(buf[actual_m:].isnan().all())
+    assert torch.equal(buf[:actual_m].view(torch.int16), natural.view(torch.int16))
     out = buf[:actual_m].cpu()
     lin = O.gemm_w4a4(p["act"], p["wgt"], p["asc"], p["wsc"], p["bias"], p["la"], p["lu"], unsigned)[:actual_m]
     ref = O.qk_norm_rope(lin, nq, nk, rot.reshape(actual_m, 128))
