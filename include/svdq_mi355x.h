@@ -152,6 +152,9 @@ typedef struct {
     /* SVDQ_EPI_QK_NORM_ROPE, optional: the same table as `rotary`, re-laid-out by svdq_block_rotary (the fp8 main    */
     /* loop's epilogue then reads 1 KB per load instruction instead of 32-byte pieces of 32 rows); NULL = not given  */
     const float *rotary_blocked;
+    /* SVDQ_EPI_GELU_QUANT, optional: `lora_down_t` re-laid-out by svdq_block_lora_down (the epilogue then reads each of */
+    /* its LoRA-down operands as 1 KB in a row instead of 8-byte pieces of 32 rows); NULL = not given                   */
+    const void *lora_down_blocked;
 } svdq_gemm_args;
 
 int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream);
@@ -167,6 +170,17 @@ int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream);
  */
 int svdq_block_rotary(const float *rotary, float *blocked, int32_t rows, int32_t ld_rotary, void *stream);
 size_t svdq_rotary_blocked_bytes(int32_t rows);
+
+/*
+ * One-time re-layout of the next layer's transposed LoRA-down weight (R2, N) T for the GELU + requantization epilogue:
+ * per (128-column tile, chunk of 32 ranks) eight 1 KB pieces, one per matrix instruction of the tile's partial product
+ * (column block bn, half s of it), in lane order: lane (rank r = lane % 32, h = lane / 32) finds the eight values
+ * lora_down_t[32 c + r][128 t + 32 bn + 16 s + 4 h + {0..3, 8..11}] as 16 contiguous bytes (ranks past R2: zeros).
+ * `blocked` needs svdq_lora_down_blocked_bytes(N, R2) = (N / 128) * ceil(R2 / 32) * 8 KB, 16-byte aligned; N % 128 == 0.
+ * Made once per weight like the transposed copy itself.  No counterpart in the reference.
+ */
+int svdq_block_lora_down(const void *lora_down_t, void *blocked, int32_t N, int32_t R2, int32_t dtype, void *stream);
+size_t svdq_lora_down_blocked_bytes(int32_t N, int32_t R2);
 
 /* The fp8 main loop exists in two builds: three workgroups per CU (fills a loaded CU best) and two per CU with
  * software-pipelined steps (a workgroup on its own runs faster); svdq_gemm_w4a4 picks by the number of 128x128 tiles and

@@ -30,6 +30,8 @@ EXPORTS = (
     "svdq_gemm_w4a4_set_variant",
     "svdq_block_rotary",
     "svdq_rotary_blocked_bytes",
+    "svdq_block_lora_down",
+    "svdq_lora_down_blocked_bytes",
     "svdq_gemm_w4a4_scratch_bytes",
     "svdq_gemm_w4a4_static_scratch",
     "svdq_gemm_w4a4_static_scratch_capacity",
@@ -74,7 +76,7 @@ class GemmArgs(ctypes.Structure):
         + [("ld_rotary", _i32), ("eps", _f32)]
         + [(n, _vp) for n in ("qout", "oscales", "smooth_next", "lora_down_t", "lora_act_out", "scratch")]
         + [(n, _i32) for n in ("R2", "ld_qout", "ld_oscales", "ld_lora_act_out")]
-        + [("shift", _f32), ("rotary_blocked", _vp)]
+        + [("shift", _f32), ("rotary_blocked", _vp), ("lora_down_blocked", _vp)]
     )  # fmt: skip
 
 
@@ -133,6 +135,9 @@ def load() -> ctypes.CDLL:
     lib.svdq_block_rotary.argtypes = [_vp, _vp, _i32, _i32, _vp]
     lib.svdq_rotary_blocked_bytes.restype = ctypes.c_size_t
     lib.svdq_rotary_blocked_bytes.argtypes = [_i32]
+    lib.svdq_block_lora_down.argtypes = [_vp, _vp, _i32, _i32, _i32, _vp]
+    lib.svdq_lora_down_blocked_bytes.restype = ctypes.c_size_t
+    lib.svdq_lora_down_blocked_bytes.argtypes = [_i32, _i32]
     lib.svdq_gemm_w4a4_static_scratch.argtypes = [ctypes.POINTER(GemmArgs), _vp]
     lib.svdq_gemm_w4a4_static_scratch_capacity.restype = ctypes.c_size_t
     lib.svdq_gemm_w4a4_static_scratch_capacity.argtypes = []

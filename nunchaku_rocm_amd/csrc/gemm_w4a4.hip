@@ -439,7 +439,11 @@ __device__ __forceinline__ void tile_epilogue(const svdq_gemm_args &a, v16f (&ac
                     // (fetched ahead of the GELU arithmetic, all at once or two column blocks ahead, these loads spill
                     // registers and the launch is no faster: the other workgroups of the CU cover their latency)
                     v4i la = (v4i){0, 0, 0, 0};
-                    if (r < a.R2) {
+                    if (a.lora_down_blocked != nullptr) {
+                        // re-laid-out copy: the operand of this instruction is 1 KB in lane order (from the (R2, N) copy a
+                        // lane fetches two 8-byte pieces of its rank's row, 32 rows to a load instruction)
+                        la = ((const v4i *)a.lora_down_blocked)[(((size_t)pid_n * ((a.R2 + 31) / 32) + rc / 32) * 8 + bn * 2 + s) * 64 + lane];
+                    } else if (r < a.R2) {
                         const uint16_t *lp = ldt + (size_t)r * a.N + n0 + bn * 32 + 16 * s + 4 * half;
                         const uint2 q0 = *(const uint2 *)lp, q1 = *(const uint2 *)(lp + 8);
                         la = (v4i){(int)q0.x, (int)q0.y, (int)q1.x, (int)q1.y};
@@ -1113,6 +1117,21 @@ __global__ __launch_bounds__(64) void group_acc_f8_kernel(const uint8_t *act, co
 }
 
 
+// transposed LoRA-down weight -> the order the GELU epilogue's lanes read it (svdq_block_lora_down): one thread per lane
+// and matrix-instruction operand
+__global__ __launch_bounds__(256) void block_lora_down_kernel(const uint16_t *ldt, v4i *out, int N, int R2, int pieces) {
+    const int o = blockIdx.x * 256 + threadIdx.x;
+    if (o >= pieces) return;
+    const int lane = o & 63, blk = (o >> 6) & 7, nrc = (R2 + 31) / 32, chunk = (o >> 9) % nrc, tile = (o >> 9) / nrc;
+    const int r = chunk * 32 + (lane & 31), col = tile * 128 + (blk >> 1) * 32 + 16 * (blk & 1) + 4 * (lane >> 5);
+    v4i v = {0, 0, 0, 0};
+    if (r < R2) {
+        const uint2 q0 = *(const uint2 *)(ldt + (size_t)r * N + col), q1 = *(const uint2 *)(ldt + (size_t)r * N + col + 8);
+        v = (v4i){(int)q0.x, (int)q0.y, (int)q1.x, (int)q1.y};
+    }
+    out[o] = v;
+}
+
 // rotary table -> the order the Q/K epilogue's lanes read it (svdq_block_rotary): one thread per 16-byte piece
 __global__ __launch_bounds__(256) void block_rotary_kernel(const float *rot, v4f *out, int rows, int ld, int pieces) {
     const int o = blockIdx.x * 256 + threadIdx.x;
@@ -1440,6 +1459,22 @@ static int gemm_w4a4_checked(const svdq_gemm_args &a, void *stream) {
         rc = check_launch("svdq_gemm_w4a4 (LoRA-down partial sum)");
     }
     return rc;
+}
+
+extern "C" size_t svdq_lora_down_blocked_bytes(int32_t N, int32_t R2) {
+    return N <= 0 || R2 <= 0 ? 0 : (size_t)(N / 128) * ((R2 + 31) / 32) * 8 * 1024;
+}
+
+extern "C" int svdq_block_lora_down(const void *lora_down_t, void *blocked, int32_t N, int32_t R2, int32_t dtype, void *stream) {
+    if (!lora_down_t || !blocked || N <= 0 || N % 128 || R2 <= 0 || R2 % 16 || ((uintptr_t)lora_down_t & 7) || ((uintptr_t)blocked & 15) ||
+        (dtype != SVDQ_BF16 && dtype != SVDQ_FP16)) {
+        set_error("svdq_block_lora_down: N=%d R2=%d dtype=%d; needs N %% 128 == 0, R2 %% 16 == 0, aligned tensors", N, R2, dtype);
+        return SVDQ_E_INVALID;
+    }
+    const int pieces = (N / 128) * ((R2 + 31) / 32) * 512;
+    hipLaunchKernelGGL(block_lora_down_kernel, dim3((pieces + 255) / 256), dim3(256), 0, (hipStream_t)stream, (const uint16_t *)lora_down_t,
+                       (v4i *)blocked, N, R2, pieces);
+    return check_launch("svdq_block_lora_down");
 }
 
 extern "C" size_t svdq_rotary_blocked_bytes(int32_t rows) { return rows <= 0 ? 0 : (size_t)((rows + 31) / 32) * 16 * 1024; }

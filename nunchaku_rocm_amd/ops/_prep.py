@@ -60,6 +60,8 @@ def _same_source(src: tuple, t: torch.Tensor) -> bool:
 def invalidate(t: torch.Tensor) -> None:
     """Drop the derived copies of ``t`` (for callers that rewrite a weight through a path the version counter misses)."""
     _cache.pop(id(t), None)
+    _ldb_cache.pop(id(t), None)
+    _rotary_cache.pop(id(t), None)
     _planes_cache.pop(id(t), None)
     _pinned.pop(id(t), None)
 
@@ -82,6 +84,35 @@ def lora_down_t(lora_down: torch.Tensor) -> torch.Tensor:
     try:
         ref = weakref.ref(lora_down, lambda _r, k=key: _cache.pop(k, None))
         _cache[key] = (ref, _source_of(lora_down), t, ready)
+    except TypeError:
+        pass
+    return t
+
+
+_ldb_cache: dict[int, tuple] = {}
+
+
+def lora_down_blocked(lora_down: torch.Tensor, ldt: torch.Tensor) -> torch.Tensor | None:
+    """The transposed LoRA-down weight ``ldt`` ``(R2, N)`` in the order the GELU + requantization epilogue reads it
+    (``svdq_block_lora_down``), cached under the weight ``lora_down`` like the transposed copy itself."""
+    key = id(lora_down)
+    hit = _ldb_cache.get(key)
+    if hit is not None:
+        ref, src, t, ready = hit
+        if ref() is lora_down and _same_source(src, lora_down):
+            ready.wait(t.device)
+            return t
+    if torch.cuda.is_current_stream_capturing():
+        return None  # no new copies while a graph is being recorded
+    R2, N = ldt.shape
+    lib = _lib.load()
+    t = torch.empty(lib.svdq_lora_down_blocked_bytes(N, R2) // 2, dtype=ldt.dtype, device=ldt.device)
+    with torch.cuda.device(t.device):
+        _lib.check(lib.svdq_block_lora_down(ldt.data_ptr(), t.data_ptr(), N, R2, _lib.dtype_code(ldt.dtype), _lib.stream_of(ldt)))
+        ready = _Ready(t.device)
+    try:
+        ref = weakref.ref(lora_down, lambda _r, k=key: _ldb_cache.pop(k, None))
+        _ldb_cache[key] = (ref, _source_of(lora_down), t, ready)
     except TypeError:
         pass
     return t

@@ -5,6 +5,7 @@ from __future__ import annotations
 import torch
 
 from .. import _lib
+from ._prep import lora_down_blocked as _lora_down_blocked
 from ._prep import lora_down_t as _lora_down_t
 from ._prep import pinned_weight_planes as _pinned_weight_planes
 from ._prep import rotary_blocked as _rotary_blocked
@@ -21,6 +22,11 @@ USE_WEIGHT_PLANES = "parameters"
 # table tensor and cached, 16 KB per 32 rows): 1 KB per load instruction instead of 32-byte pieces of 32 rows, which was
 # most of that epilogue's cost.  False = read the (rows, 128) table itself (same results).
 USE_BLOCKED_ROTARY = True
+
+# The GELU + requantization epilogue reads the next layer's LoRA-down weight through a copy in the order its matrix
+# instructions want it (made once per weight and cached, as large as the weight): 1 KB per load instruction instead of
+# 8-byte pieces of 32 rows.  False = read the transposed (R2, N) copy (same results).
+USE_BLOCKED_LORA_DOWN = True
 
 # True sends the requantizing epilogues' LoRA-down partial sums to the buffer built into the library
 # (svdq_gemm_w4a4_static_scratch) instead of a torch allocation per call: for callers that may not allocate, e.g. while
@@ -248,6 +254,11 @@ def svdq_gemm_w4a4_cuda(
             epi = _lib.EPI_SWIGLU_QUANT if fuse_swiglu else _lib.EPI_GELU_QUANT
             keep.append(ldt)
             args.lora_down_t, args.lora_act_out = ldt.data_ptr(), lora_act_out.data_ptr()
+            if USE_BLOCKED_LORA_DOWN and not fuse_swiglu and N % 128 == 0:
+                ldb = _lora_down_blocked(lora_down, ldt)  # the GELU epilogue's own order (made once per weight, see _prep)
+                if ldb is not None:
+                    keep.append(ldb)
+                    args.lora_down_blocked = ldb.data_ptr()
             if not STATIC_SCRATCH:
                 nbytes = lib.svdq_gemm_w4a4_scratch_bytes(M, N, R2, epi)
                 scratch = torch.empty(nbytes // 4, dtype=torch.float32, device=dev)

@@ -103,6 +103,22 @@ def test_gelu_quant_epilogue(dev, M, N, R2, store_out, unsigned, dtype):
     assert torch.equal(first[0], qout) and torch.equal(first[1].view(torch.int16), osc.view(torch.int16))
     assert R2 == 0 or torch.equal(first[2], lao)
     assert (qout[M:] == 0).all()  # rows past M untouched
+    if R2:
+        # the LoRA-down weight read from its transposed copy instead of the copy in the epilogue's own order: the same bits
+        from nunchaku_rocm_amd.ops import gemm as gemm_mod
+
+        gemm_mod.USE_BLOCKED_LORA_DOWN = False
+        try:
+            lao2 = torch.empty_like(lao)
+            ops.svdq_gemm_w4a4_cuda(
+                act=d(p["act"]), wgt=d(p["wgt"]), out=out, qout=qout, ascales=d(p["asc"]), wscales=d(p["wsc"]), oscales=osc,
+                lora_act_in=d(p["la"]), lora_up=d(p["lu"]), lora_down=d(ld), lora_act_out=lao2, bias=d(p["bias"]),
+                smooth_factor=d(smooth), act_unsigned=unsigned,
+            )  # fmt: skip
+            torch.cuda.synchronize()
+        finally:
+            gemm_mod.USE_BLOCKED_LORA_DOWN = True
+        assert torch.equal(first[0], qout) and torch.equal(first[2], lao2)
 
     lin = O.gemm_w4a4(p["act"], p["wgt"], p["asc"], p["wsc"], p["bias"], p["la"], p["lu"], unsigned)
     rp, rs, rl, rc = O.gelu_quant(lin, smooth, ld, dtype)
