@@ -81,6 +81,12 @@ typedef struct {
     const void *norm_shift;        /* (batches, K) T, same strides                                           */
     int32_t norm_rows_per_batch;   /* rows m sharing one scale / shift vector (multiple of 16); 0 = all rows */
     int32_t norm_ld, norm_stride;  /* in elements (the adaLN projection interleaves its six vectors: stride 6) */
+    /* non-zero: `out` is written in the lane order of the GEMM's fp8 main loop instead of as the (M, K / 2) matrix:  */
+    /* the 32 packed bytes of (row m, group g) go to out + ((m / 32) * (K / 64) + g) * 1024 + (32 * h + m % 32) * 16,  */
+    /* h = 0 / 1 for bytes 0-15 / 16-31 (ld_out is not used; `out` must hold ceil(M / 32) * 32 rows' worth).  The GEMM */
+    /* then takes it with svdq_gemm_args.act_blocked: each of its load instructions reads 1 KB in a row instead of     */
+    /* 16-byte pieces of 32 rows (about 3 % of a launch).  No counterpart in the reference.                            */
+    int32_t out_blocked;
 } svdq_quantize_args;
 
 int svdq_quantize_act(const svdq_quantize_args *args, void *stream);
@@ -155,6 +161,12 @@ typedef struct {
     /* SVDQ_EPI_GELU_QUANT, optional: `lora_down_t` re-laid-out by svdq_block_lora_down (the epilogue then reads each of */
     /* its LoRA-down operands as 1 KB in a row instead of 8-byte pieces of 32 rows); NULL = not given                   */
     const void *lora_down_blocked;
+    /* non-zero: `act` is not the (M, K / 2) matrix but the same bytes in the fp8 main loop's lane order, as the        */
+    /* quantizer writes them with out_blocked (pre-split weights only)                                                  */
+    int32_t act_blocked;    /* (`act` must then hold ceil(M / 32) * 32 rows' worth, 16-byte aligned; ld_act unused) */
+    /* non-zero: the requantizing epilogues write `qout` in that same lane order, for the GEMM that consumes it        */
+    /* (ld_qout unused; `qout` must hold ceil(M / 32) * 32 rows' worth)                                                 */
+    int32_t qout_blocked;
 } svdq_gemm_args;
 
 int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream);

@@ -515,9 +515,13 @@ __device__ __forceinline__ void tile_epilogue(const svdq_gemm_args &a, v16f (&ac
                     const uint32_t theirs = __shfl_xor(send, 32);
                     dw[t] = half ? (theirs | (keep << 16)) : (keep | (theirs << 16));
                 }
-                if (m < a.M)
-                    *(uint2 *)((uint8_t *)a.qout + (size_t)m * a.ld_qout + (n0 + bn * 32) / 2 + 8 * half) =
-                        make_uint2(dw[0], dw[1]);
+                if (m < a.M) {
+                    // (qout_blocked: where lane (m % 32, bn % 2) of the consuming GEMM's row block and group reads its 16 bytes)
+                    uint8_t *dst = a.qout_blocked
+                                       ? (uint8_t *)a.qout + ((size_t)(m >> 5) * (a.N / GROUP) + g) * 1024 + (((bn & 1) * 32 + (m & 31)) * 16 + 8 * half)
+                                       : (uint8_t *)a.qout + (size_t)m * a.ld_qout + (n0 + bn * 32) / 2 + 8 * half;
+                    *(uint2 *)dst = make_uint2(dw[0], dw[1]);
+                }
             }
         }
         return;
@@ -605,8 +609,13 @@ __device__ __forceinline__ void tile_epilogue(const svdq_gemm_args &a, v16f (&ac
             const uint32_t send = half ? mine[0] : mine[1];
             const uint32_t theirs = __shfl_xor(send, 32);
             const uint32_t dw = half ? (theirs | (keep << 16)) : (keep | (theirs << 16));
-            if (m < a.M)
-                *(uint32_t *)((uint8_t *)a.qout + (size_t)m * a.ld_qout + (yt0 + 16 * bn) / 2 + 4 * half) = dw;
+            if (m < a.M) {
+                // (qout_blocked: the tile's 64 y columns are one group of the consuming GEMM; byte 8 bn + 4 half of its 32)
+                uint8_t *dst = a.qout_blocked
+                                   ? (uint8_t *)a.qout + ((size_t)(m >> 5) * (H / GROUP) + yt0 / GROUP) * 1024 + (((bn >> 1) * 32 + (m & 31)) * 16 + 8 * (bn & 1) + 4 * half)
+                                   : (uint8_t *)a.qout + (size_t)m * a.ld_qout + (yt0 + 16 * bn) / 2 + 4 * half;
+                *(uint32_t *)dst = dw;
+            }
         }
         return;
     }
@@ -865,16 +874,22 @@ __global__ __launch_bounds__(NTHREADS, PIPE ? 2 : 3) void gemm_w4a4_f8_kernel(sv
     v4i araw[2];
     uint16_t qa[2];
     const int mrow = min(m0 + wm * 32 + l32, a.M - 1);
-    const __amdgpu_buffer_rsrc_t rAct = g_buffer((const uint8_t *)a.act + (size_t)m0 * a.ld_act);
+    // Activations either as the (M, K / 2) matrix (a lane fetches the 16 bytes of its own row: 32 rows to a load
+    // instruction) or in lane order (act_blocked: per 32 rows and group 1 KB = lane l's 16 bytes at 16 l, groups in a
+    // row): the same two loads per stage, base + lane offset + group * step, with other constants.
+    const bool ablk = a.act_blocked != 0;
+    const __amdgpu_buffer_rsrc_t rAct =
+        g_buffer((const uint8_t *)a.act + (ablk ? (size_t)((m0 >> 5) + wm) * G * 1024 : (size_t)m0 * a.ld_act));
     const __amdgpu_buffer_rsrc_t rAS = g_buffer(a.ascales);
-    const uint32_t oAct = (uint32_t)(mrow - m0) * (uint32_t)a.ld_act + half * 16;
+    const uint32_t oAct = ablk ? (uint32_t)lane * 16u : (uint32_t)(mrow - m0) * (uint32_t)a.ld_act + half * 16;
+    const uint32_t sAct = ablk ? 1024u : 32u;
     const uint32_t oA = 2u * (uint32_t)mrow;
     auto load_regs = [&](int s) {
 #pragma unroll
         for (int gg = 0; gg < 2; gg++) {
             const int gi = min(2 * s + gg, G - 1);
             qa[gg] = g_load16(rAS, oA, (uint32_t)gi * (uint32_t)a.ld_ascales * 2u);
-            araw[gg] = g_load128(rAct, oAct, (uint32_t)gi * 32);
+            araw[gg] = g_load128(rAct, oAct, (uint32_t)gi * sAct);
         }
     };
 
@@ -1353,7 +1368,11 @@ static int gemm_w4a4_checked(const svdq_gemm_args &a, void *stream) {
         set_error("svdq_gemm_w4a4: wgt_planes must be 16-byte aligned");
         return SVDQ_E_INVALID;
     }
-    if (!al16(a.act) || a.ld_act % 16 || a.ld_act < a.K / 2 ||
+    if (a.act_blocked && !a.wgt_planes) {
+        set_error("svdq_gemm_w4a4: act_blocked needs wgt_planes (the int8 main loop reads the (M, K / 2) matrix only)");
+        return SVDQ_E_UNSUPPORTED;
+    }
+    if (!al16(a.act) || (!a.act_blocked && (a.ld_act % 16 || a.ld_act < a.K / 2)) ||
         (!a.wgt_planes && (!al16(a.wgt) || a.ld_wgt % 16 || a.ld_wgt < a.K / 2))) {  // wgt is not read next to wgt_planes
         set_error("svdq_gemm_w4a4: act/wgt rows must be 16-byte aligned and at least K/2 bytes (ld_act=%d ld_wgt=%d)",
                   a.ld_act, a.ld_wgt);
@@ -1423,7 +1442,8 @@ static int gemm_w4a4_checked(const svdq_gemm_args &a, void *stream) {
             set_error("svdq_gemm_w4a4: the SwiGLU epilogue writes qout/oscales only; out must be NULL");
             return SVDQ_E_INVALID;
         }
-        if (!a.qout || !a.oscales || ((uintptr_t)a.qout & 7) || a.ld_qout % 8 || a.ld_qout < NQ / 2 || a.ld_oscales < a.M) {
+        if (!a.qout || !a.oscales || ((uintptr_t)a.qout & (a.qout_blocked ? 15 : 7)) ||
+            (!a.qout_blocked && (a.ld_qout % 8 || a.ld_qout < NQ / 2)) || a.ld_oscales < a.M) {
             set_error("svdq_gemm_w4a4: qout (8-byte aligned rows) and oscales are required");
             return SVDQ_E_INVALID;
         }

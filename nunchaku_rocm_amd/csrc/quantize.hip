@@ -78,6 +78,14 @@ __global__ __launch_bounds__(Q_WAVES * 64, QR == 32 ? 1 : (NORM ? 4 : 2)) void q
     uint8_t *__restrict__ outbase = (uint8_t *)a.out + (size_t)m0 * a.ld_out + wave * (GROUP / 2);
     const uint32_t outoff = (uint32_t)ml * a.ld_out + kq * 8;
     uint16_t *__restrict__ scales = (uint16_t *)a.scales + (size_t)wave * a.ld_scales + m0;
+    // out_blocked: the 32 packed bytes of (row, group) go where the GEMM's lane (row % 32, half) of that 32-row block and
+    // group finds them, [32-row block][group][64 lanes x 16 bytes]: this lane's 8 bytes are half kq / 2, offset 8 (kq % 2)
+    uint8_t *__restrict__ bout[NH];
+#pragma unroll
+    for (int h = 0; h < NH; h++) {
+        const int m = m0 + Q_ROWS * h + ml;
+        bout[h] = (uint8_t *)a.out + (size_t)(m >> 5) * ngroups * 1024 + (((kq >> 1) * 32 + (m & 31)) * 16 + (kq & 1) * 8);
+    }
     constexpr int GSTEP = Q_WAVES * GROUP;  // elements between consecutive groups of one wavefront
     const float qmax = UNSIGNED ? 15.0f : 7.0f;
     const float rmagic = UNSIGNED ? RNE_MAGIC : RNE_MAGIC + 8.0f;  // signed codes are packed as c + 8, then ^ 8
@@ -296,7 +304,9 @@ __global__ __launch_bounds__(Q_WAVES * 64, QR == 32 ? 1 : (NORM ? 4 : 2)) void q
             }
             if (row_ok) {
                 if (kq == 0) (scales + (size_t)i * Q_WAVES * a.ld_scales)[Q_ROWS * h + ml] = T::from_f32(scale);
-                *(uint2 *)(outbase + (size_t)i * (GSTEP / 2) + (uint32_t)(Q_ROWS * h) * a.ld_out + outoff) = make_uint2(w0, w1);
+                uint8_t *dst = a.out_blocked ? bout[h] + (size_t)(wave + Q_WAVES * i) * 1024
+                                             : outbase + (size_t)i * (GSTEP / 2) + (uint32_t)(Q_ROWS * h) * a.ld_out + outoff;
+                *(uint2 *)dst = make_uint2(w0, w1);
             }
             }  // halves
             __builtin_amdgcn_wave_barrier();  // the shared vectors are rewritten by the next group
@@ -632,7 +642,7 @@ extern "C" int svdq_quantize_act(const svdq_quantize_args *args, void *stream) {
         set_error("svdq_quantize_act: x rows and lora_down_t must be 16-byte aligned (ld_x=%d)", a.ld_x);
         return SVDQ_E_INVALID;
     }
-    if (a.ld_out % 8 || ((uintptr_t)a.out & 7)) {
+    if ((!a.out_blocked && a.ld_out % 8) || ((uintptr_t)a.out & (a.out_blocked ? 15 : 7))) {
         set_error("svdq_quantize_act: out rows must be 8-byte aligned (ld_out=%d)", a.ld_out);
         return SVDQ_E_INVALID;
     }
@@ -640,7 +650,7 @@ extern "C" int svdq_quantize_act(const svdq_quantize_args *args, void *stream) {
         set_error("svdq_quantize_act: unknown prologue %d", a.prologue);
         return SVDQ_E_INVALID;
     }
-    if (a.ld_x < (a.prologue == SVDQ_PRE_GLU ? 2 : 1) * a.K || a.ld_out < a.K / 2 || a.ld_scales < a.M ||
+    if (a.ld_x < (a.prologue == SVDQ_PRE_GLU ? 2 : 1) * a.K || (!a.out_blocked && a.ld_out < a.K / 2) || a.ld_scales < a.M ||
         (a.R > 0 && a.ld_lora_act < a.R)) {
         set_error("svdq_quantize_act: a leading dimension is smaller than its row");
         return SVDQ_E_INVALID;

@@ -196,3 +196,19 @@ def join_weight_planes(planes: torch.Tensor, n: int, k: int) -> torch.Tensor:
     packed = nib[:, :, 0] | (nib[:, :, 1] << 4)  # (nb, group, row, packed byte)
     packed = packed[:, :G].permute(0, 2, 1, 3).reshape(nb * 32, G * 32)
     return packed[:n].contiguous().view(torch.int8)
+
+
+def block_activations(act: torch.Tensor) -> torch.Tensor:
+    """Packed activations ``(rows, K/2)`` (rows a multiple of 32, K of 64) -> the same bytes in the order the GEMM's fp8
+    main loop reads them (what the quantizer writes with ``out_blocked=True``): per 32 rows and group of 64 values 1 KB,
+    lane ``32 h + r`` holding bytes ``16 h .. 16 h + 15`` of row ``r``'s 32.  Same shape; pure torch."""
+    rows, kb = act.shape
+    assert rows % 32 == 0 and kb % 32 == 0, "rows must be a multiple of 32 and K of 64"
+    return act.reshape(rows // 32, 32, kb // 32, 2, 16).permute(0, 2, 3, 1, 4).contiguous().reshape(rows, kb)
+
+
+def unblock_activations(blocked: torch.Tensor) -> torch.Tensor:
+    """Inverse of :func:`block_activations`."""
+    rows, kb = blocked.shape
+    assert rows % 32 == 0 and kb % 32 == 0, "rows must be a multiple of 32 and K of 64"
+    return blocked.reshape(rows // 32, kb // 32, 2, 32, 16).permute(0, 3, 1, 2, 4).contiguous().reshape(rows, kb)

@@ -109,16 +109,26 @@ class SVDQW4A4Linear(nn.Module):
         x = x.reshape(batch_size * seq_len, channels)
         if output is None:
             output = torch.empty(batch_size * seq_len, self.out_features, dtype=x.dtype, device=x.device)
-        quantized_x, ascales, lora_act_out = self.quantize(x, norm=norm)
-        output = self.forward_quant(quantized_x, ascales, lora_act_out, output)
+        blocked = self.takes_blocked(batch_size * seq_len)
+        quantized_x, ascales, lora_act_out = self.quantize(x, norm=norm, blocked=blocked)
+        output = self.forward_quant(quantized_x, ascales, lora_act_out, output, act_blocked=blocked)
         return output.reshape(batch_size, seq_len, -1)
 
-    def quantize(self, x: torch.Tensor, pad_size: int = 256, norm: tuple | None = None):
+    def takes_blocked(self, rows: int, pad_size: int = 256) -> bool:
+        """Whether this layer's GEMM wants its quantized input in the fp8 main loop's own order (``blocked=True`` in
+        :meth:`quantize`, ``act_blocked=True`` in :meth:`forward_quant`) for ``rows`` rows padded to ``pad_size``."""
+        from .ops.gemm import takes_blocked_activations
+
+        return takes_blocked_activations(self.qweight, self.wscales, -(-rows // pad_size) * pad_size)
+
+    def quantize(self, x: torch.Tensor, pad_size: int = 256, norm: tuple | None = None, blocked: bool = False):
+        """``blocked`` (an addition to the reference's signature): the codes in the order the GEMM's fp8 main loop reads
+        them, for :meth:`forward_quant` with ``act_blocked=True``; ``False`` = the reference's ``(M_pad, K/2)`` matrix."""
         return svdq_quantize_w4a4_act_fuse_lora_cuda(
-            x, lora_down=self.proj_down, smooth=self.smooth_factor, fp4=False, pad_size=pad_size, norm=norm
+            x, lora_down=self.proj_down, smooth=self.smooth_factor, fp4=False, pad_size=pad_size, norm=norm, out_blocked=blocked
         )
 
-    def forward_quant(self, quantized_x, ascales, lora_act, output: torch.Tensor | None = None) -> torch.Tensor:
+    def forward_quant(self, quantized_x, ascales, lora_act, output: torch.Tensor | None = None, act_blocked: bool = False) -> torch.Tensor:
         if output is None:
             output = torch.empty(quantized_x.shape[0], self.out_features, dtype=self.proj_up.dtype, device=quantized_x.device)
         svdq_gemm_w4a4_cuda(
@@ -134,6 +144,7 @@ class SVDQW4A4Linear(nn.Module):
             alpha=self.wtscale,
             wcscales=self.wcscales,
             act_unsigned=self.act_unsigned,
+            act_blocked=act_blocked,
         )
         return output
 

@@ -23,6 +23,13 @@ USE_WEIGHT_PLANES = "parameters"
 # most of that epilogue's cost.  False = read the (rows, 128) table itself (same results).
 USE_BLOCKED_ROTARY = True
 
+# The modules and composite operators (SVDQW4A4Linear.forward, fused_gelu_mlp, fused_qkv_norm_rottary, fused_swiglu_mlp)
+# pass quantized activations from the quantizer, or from a requantizing epilogue, to the GEMM in the order the fp8 main
+# loop's lanes read them (out_blocked / act_blocked / qout_blocked): 1 KB per load instruction instead of 16-byte pieces
+# of 32 rows, about 3 % of a GEMM launch.  The operators themselves (svdq_quantize_w4a4_act_fuse_lora_cuda,
+# svdq_gemm_w4a4_cuda) keep the reference's (M, K/2) matrix unless asked.  False = the matrix everywhere (same results).
+USE_BLOCKED_ACTIVATIONS = True
+
 # The GELU + requantization epilogue reads the next layer's LoRA-down weight through a copy in the order its matrix
 # instructions want it (made once per weight and cached, as large as the weight): 1 KB per load instruction instead of
 # 8-byte pieces of 32 rows.  False = read the transposed (R2, N) copy (same results).
@@ -47,6 +54,23 @@ def set_fp8_loop_variant(variant: int) -> None:
     (default), 0 = three workgroups per CU, 1 = two per CU with software-pipelined steps.  The two give identical bits; the
     switch exists for tuning and for tests (``svdq_gemm_w4a4_set_variant``)."""
     _lib.check(_lib.load().svdq_gemm_w4a4_set_variant(int(variant)))
+
+
+def working_copy(wgt: torch.Tensor, wscales: torch.Tensor) -> torch.Tensor | None:
+    """The re-laid-out copy of ``wgt`` the fp8 main loop reads (made and cached on first use), or ``None`` when this
+    weight runs through the int8 main loop: not a parameter (see ``USE_WEIGHT_PLANES``), rows not 16-byte aligned, or
+    fp16 scales too large for the copy's 16-bit offset terms."""
+    planes = _pinned_weight_planes(wgt)  # a module whose packed weight was released: this copy is all there is
+    if planes is None:
+        want_planes = USE_WEIGHT_PLANES == "all" or (USE_WEIGHT_PLANES == "parameters" and isinstance(wgt, torch.nn.Parameter))
+        planes = _weight_planes(wgt, wscales) if want_planes and wgt.stride(0) % 16 == 0 else None
+    return planes
+
+
+def takes_blocked_activations(wgt: torch.Tensor, wscales: torch.Tensor, rows: int) -> bool:
+    """Whether a GEMM on this weight should be fed activations in the fp8 main loop's own order (``act_blocked``): the
+    switch is on, the weight has a working copy, and the (padded) row count is a multiple of 32."""
+    return USE_BLOCKED_ACTIVATIONS and rows % 32 == 0 and working_copy(wgt, wscales) is not None
 
 
 HEAD_DIM = 128
@@ -84,6 +108,8 @@ def svdq_gemm_w4a4_cuda(
     out_v: torch.Tensor | None = None,
     attn_tokens: int = 0,
     fuse_swiglu: bool = False,
+    act_blocked: bool = False,
+    qout_blocked: bool = False,
 ):
     """
     ``out = deq(act) @ deq(wgt).T + lora_act_in @ lora_up.T + bias`` on packed int4 operands with per-group-64 scales,
@@ -94,6 +120,9 @@ def svdq_gemm_w4a4_cuda(
     * ``qout``/``oscales`` (+ ``smooth_factor``, ``lora_down``, ``lora_act_out``): fused GELU, next layer's LoRA-down
       and unsigned int4 requantization; ``out`` may then be ``None``.
     * ``act`` may have more (padded) rows than ``out``; only ``out.shape[0]`` rows are written.
+    * ``act_blocked`` / ``qout_blocked`` (no counterpart in the reference): ``act`` holds its codes in the order the fp8
+      main loop reads them, as the quantizer writes them with ``out_blocked=True`` / the requantizing epilogue writes
+      ``qout`` that way for the GEMM that consumes it.  Needs a weight with a working copy (see ``USE_WEIGHT_PLANES``).
 
     Raises ``NotImplementedError`` for the arguments the reference's ROCm backend rejects as well (``poolout``,
     ``out_vk``, ``out_linearattn``, ``out_q/k/v``) and for the NVFP4-only ones (``fp4``, ``wcscales``, ``alpha != 1``,
@@ -141,17 +170,17 @@ def svdq_gemm_w4a4_cuda(
         T = oscales.dtype
         x = out.reshape(-1, N) if out is not None else torch.empty(M, N, dtype=T, device=dev)
         svdq_gemm_w4a4_cuda(act, wgt, out=x, ascales=ascales, wscales=wscales, lora_act_in=lora_act_in, lora_up=lora_up,
-                            bias=bias, act_unsigned=act_unsigned)  # fmt: skip
+                            bias=bias, act_unsigned=act_unsigned, act_blocked=act_blocked)  # fmt: skip
         rows = x.shape[0]
         qout2d = qout.reshape(-1, qout.shape[-1])
         la_out = lora_act_out if lora_down is not None else None
         if fuse_swiglu:
             x = x.view(rows, N // 32, 2, 16)
             y = (torch.nn.functional.silu(x[:, :, 0]) * x[:, :, 1]).reshape(rows, N // 2)
-            quantize_w4a4_act_fuse_lora(y, qout2d, oscales, lora_down, la_out, smooth_factor)
+            quantize_w4a4_act_fuse_lora(y, qout2d, oscales, lora_down, la_out, smooth_factor, out_blocked=qout_blocked)
         else:
             quantize_w4a4_act_fuse_lora(x, qout2d, oscales, lora_down, la_out, smooth_factor, fuse_gelu=True,
-                                        shift_value=GELU_SHIFT, unsigned=True)  # fmt: skip
+                                        shift_value=GELU_SHIFT, unsigned=True, out_blocked=qout_blocked)  # fmt: skip
         return None
 
     T = out.dtype if out is not None else (oscales.dtype if oscales is not None else ascales.dtype)
@@ -182,10 +211,12 @@ def svdq_gemm_w4a4_cuda(
     if out2d is not None and out2d.stride(1) != 1:
         raise ValueError("out not row-major")
 
-    planes = _pinned_weight_planes(wgt)  # a module whose packed weight was released: this copy is all there is
-    if planes is None:
-        want_planes = USE_WEIGHT_PLANES == "all" or (USE_WEIGHT_PLANES == "parameters" and isinstance(wgt, torch.nn.Parameter))
-        planes = _weight_planes(wgt, wscales) if want_planes and wgt.stride(0) % 16 == 0 else None
+    planes = working_copy(wgt, wscales)
+    if act_blocked:
+        if planes is None:
+            raise ValueError("act_blocked needs a weight with a working copy (the int8 main loop reads the (M, K/2) matrix)")
+        if not act.is_contiguous() or M % 32 or act.data_ptr() % 16:
+            raise ValueError("act_blocked needs a contiguous act with a multiple of 32 rows")
     args = _lib.GemmArgs(
         act=act.data_ptr(),
         wgt=wgt.data_ptr(),
@@ -212,6 +243,7 @@ def svdq_gemm_w4a4_cuda(
         act_unsigned=int(act_unsigned),
         epilogue=_lib.EPI_PLAIN,
         eps=1e-6,
+        act_blocked=int(act_blocked),
     )
     keep = [planes]  # tensors that must outlive the launch call
     lib = _lib.load()
@@ -268,6 +300,10 @@ def svdq_gemm_w4a4_cuda(
         args.epilogue = _lib.EPI_SWIGLU_QUANT if fuse_swiglu else _lib.EPI_GELU_QUANT
         args.qout, args.oscales, args.smooth_next = qout2d.data_ptr(), oscales.data_ptr(), _lib.ptr(smooth_factor)
         args.R2, args.ld_qout, args.ld_oscales = R2, qout2d.stride(0), oscales.stride(0)
+        if qout_blocked:
+            if not qout2d.is_contiguous() or qout2d.shape[0] % 32 or qout2d.data_ptr() % 16:
+                raise ValueError("qout_blocked needs a contiguous qout with a multiple of 32 rows")
+            args.qout_blocked = 1
         args.shift = 0.0 if fuse_swiglu else GELU_SHIFT
 
     with torch.cuda.device(dev):

@@ -60,6 +60,7 @@ def quantize_w4a4_act_fuse_lora(
     unsigned: bool = False,
     norm: tuple | None = None,
     norm_eps: float = 1e-6,
+    out_blocked: bool = False,
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """
     Backend-level quantizer with the reference's full option set (reference:
@@ -71,6 +72,10 @@ def quantize_w4a4_act_fuse_lora(
     torch kernels): what is quantized and LoRA-projected is ``layer_norm(input) * scale + shift`` (no affine,
     ``eps=norm_eps``, every step rounded to the input dtype), with ``scale`` / ``shift`` of shape ``(K,)`` or
     ``(batches, K)`` (rows split evenly over the batches) and ``stats`` from :func:`layer_norm_stats`.
+
+    ``out_blocked=True`` (no counterpart in the reference): ``output`` keeps its shape but holds the codes in the order
+    the GEMM's fp8 main loop reads them (``svdq_quantize_args.out_blocked``; pass it on with ``act_blocked=True``); it
+    must be contiguous with a multiple of 32 rows.  :func:`nunchaku_rocm_amd.layout.unblock_activations` undoes it.
     """
     if fp4:
         raise NotImplementedError("NVFP4 quantization is not implemented (int4 only)")
@@ -94,6 +99,8 @@ def quantize_w4a4_act_fuse_lora(
         inp = inp.contiguous()
     if output.element_size() != 1 or output.stride(1) != 1 or output.shape[0] < M:
         raise ValueError("output must be a (>= M, K/2) byte tensor with unit inner stride")
+    if out_blocked and (not output.is_contiguous() or output.shape[0] % 32 or output.shape[1] != K // 2 or output.data_ptr() % 16):
+        raise ValueError("out_blocked needs a contiguous (rows, K/2) output with rows a multiple of 32")
     if oscales.dtype != inp.dtype or oscales.stride(1) != 1 or oscales.shape[1] < M or oscales.shape[0] < K // 64:
         raise ValueError("oscales must be (K/64, >= M) of the input dtype with unit inner stride")
     if rank and (lora_act_out.dtype != torch.float32 or lora_act_out.stride(1) != 1 or lora_act_out.shape[0] < M):
@@ -133,6 +140,7 @@ def quantize_w4a4_act_fuse_lora(
         is_unsigned=int(unsigned),
         prologue=_lib.PRE_GLU if fuse_glu else (_lib.PRE_GELU if fuse_gelu else _lib.PRE_NONE),
         shift=float(shift_value),
+        out_blocked=int(out_blocked),
     )
     with torch.cuda.device(inp.device):
         _lib.check(_lib.load().svdq_quantize_act(args, _lib.stream_of(inp)))
@@ -175,6 +183,7 @@ def svdq_quantize_w4a4_act_fuse_lora_cuda(
     pad_size: int = 256,
     norm: tuple | None = None,
     norm_eps: float = 1e-6,
+    out_blocked: bool = False,
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """
     Quantize activations to int4 (per-group-64 absmax, after dividing by ``smooth``) and compute the LoRA
@@ -188,6 +197,7 @@ def svdq_quantize_w4a4_act_fuse_lora_cuda(
     Unlike the reference wrapper (which dereferences ``lora_down.shape`` unconditionally), ``lora_down=None`` is
     accepted and returns ``lora_act_out`` with zero columns.  ``norm`` / ``norm_eps``: the LayerNorm + modulate
     prologue described in :func:`quantize_w4a4_act_fuse_lora` (an addition; ``None`` = the reference's behaviour).
+    ``out_blocked``: see there as well (an addition; ``False`` = the reference's ``(M_pad, C/2)`` matrix).
     """
     if fp4:
         raise NotImplementedError("NVFP4 quantization is not implemented (int4 only)")
@@ -204,5 +214,5 @@ def svdq_quantize_w4a4_act_fuse_lora_cuda(
     if lora_act_out is None:
         lora_act_out = torch.empty(batch_size_pad, rank, dtype=torch.float32, device=input.device)
     quantize_w4a4_act_fuse_lora(input, output, oscales, lora_down, lora_act_out if rank else None, smooth, fuse_glu, fp4,
-                                norm=norm, norm_eps=norm_eps)
+                                norm=norm, norm_eps=norm_eps, out_blocked=out_blocked)
     return output, oscales, lora_act_out

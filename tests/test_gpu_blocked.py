@@ -1,0 +1,148 @@
+"""Quantized activations in the GEMM's own order (``out_blocked`` / ``act_blocked`` / ``qout_blocked``): the same codes
+as the (M, K/2) matrix, bit for bit, moved; the same GEMM outputs, bit for bit; and modules / composite operators that
+compute the same bits whichever way they pass activations along."""
+
+import pytest
+import torch
+
+from oracle import svdq_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _module(dev, K, N, seed, dtype=torch.bfloat16, act_unsigned=False):
+    from nunchaku_rocm_amd.linear import SVDQW4A4Linear
+
+    lin = O.make_svdq_linear(K, N, seed=seed, dtype=dtype)
+    mod = SVDQW4A4Linear(K, N, rank=32, act_unsigned=act_unsigned, torch_dtype=dtype, device=dev)
+    with torch.no_grad():
+        for name in ("qweight", "wscales", "smooth_factor", "proj_down", "proj_up", "bias"):
+            getattr(mod, name).copy_(lin[name])
+    return mod
+
+
+def test_layout_helpers_invert_each_other():
+    from nunchaku_rocm_amd.layout import block_activations, unblock_activations
+
+    a = torch.randint(0, 256, (96, 160), dtype=torch.uint8, generator=torch.Generator().manual_seed(0))
+    b = block_activations(a)
+    assert b.shape == a.shape and not torch.equal(a, b)
+    assert torch.equal(unblock_activations(b), a)
+    # lane 32 h + r of (row block rb, group g) = bytes 16 h .. of row 32 rb + r
+    rb, g, h, r = 2, 3, 1, 7
+    piece = b.reshape(-1)[((rb * 5 + g) * 64 + 32 * h + r) * 16 :][:16]
+    assert torch.equal(piece, a[32 * rb + r, 32 * g + 16 * h :][:16])
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,K,R,norm", [(300, 256, 16, False), (4608, 3072, 32, False), (272, 320, 32, True), (100, 64, 0, False)])
+def test_quantizer_writes_the_same_codes_elsewhere(dev, M, K, R, norm, dtype):
+    from nunchaku_rocm_amd import ops
+    from nunchaku_rocm_amd.layout import unblock_activations
+
+    print(f"case M={M} K={K} R={R} norm={norm} {dtype}", flush=True)
+    g = torch.Generator().manual_seed(M + K)
+    x = torch.randn(M, K, generator=g).to(dtype).to(dev)
+    smooth = (torch.rand(K, generator=g) + 0.5).to(dtype).to(dev)
+    ld = (torch.randn(K, R, generator=g) * 0.1).to(dtype).to(dev) if R else None
+    nm = ((torch.randn(K, generator=g) * 0.1 + 1).to(dtype).to(dev), (torch.randn(K, generator=g) * 0.1).to(dtype).to(dev)) if norm else None
+    nat = ops.svdq_quantize_w4a4_act_fuse_lora_cuda(x, lora_down=ld, smooth=smooth, norm=nm)
+    out_b = torch.full_like(nat[0], 0xEE)
+    blk = ops.svdq_quantize_w4a4_act_fuse_lora_cuda(x, output=out_b, lora_down=ld, smooth=smooth, norm=nm, out_blocked=True)
+    torch.cuda.synchronize()
+    assert torch.equal(unblock_activations(blk[0].cpu())[:M], nat[0].cpu()[:M])
+    assert (unblock_activations(blk[0].cpu())[M:] == 0xEE).all()  # pad rows untouched
+    assert torch.equal(blk[1].cpu()[:, :M].view(torch.int16), nat[1].cpu()[:, :M].view(torch.int16))
+    if R:
+        assert torch.equal(blk[2].cpu()[:M], nat[2].cpu()[:M])
+
+
+@pytest.mark.parametrize("unsigned", [False, True])
+@pytest.mark.parametrize("M,N,K,R", [(256, 264, 256, 16), (96, 128, 320, 0), (4608, 3072, 3072, 32)])
+def test_gemm_reads_either_order(dev, M, N, K, R, unsigned):
+    from nunchaku_rocm_amd import ops
+    from nunchaku_rocm_amd.layout import block_activations
+    from nunchaku_rocm_amd.ops import gemm as gemm_mod
+
+    print(f"case M={M} N={N} K={K} R={R} unsigned={unsigned}", flush=True)
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(M + N)
+    act = torch.randint(0, 256, (M, K // 2), generator=g, dtype=torch.uint8)
+    t = dict(wgt=torch.randint(0, 256, (N, K // 2), generator=g, dtype=torch.uint8),
+             ascales=(torch.rand(K // 64, M, generator=g) * 0.02 + 0.01).to(dtype),
+             wscales=(torch.rand(K // 64, N, generator=g) * 0.02 + 0.01).to(dtype), bias=torch.randn(N, generator=g).to(dtype))  # fmt: skip
+    if R:
+        t.update(lora_act_in=torch.randn(M, R, generator=g), lora_up=(torch.randn(N, R, generator=g) * 0.1).to(dtype))
+    t = {k: v.to(dev) for k, v in t.items()}
+    old = gemm_mod.USE_WEIGHT_PLANES
+    gemm_mod.USE_WEIGHT_PLANES = "all"
+    try:
+        nat = torch.empty(M - 5, N, dtype=dtype, device=dev)
+        ops.svdq_gemm_w4a4_cuda(act=act.to(dev), out=nat, act_unsigned=unsigned, **t)
+        blk = torch.empty(M - 5, N, dtype=dtype, device=dev)
+        ops.svdq_gemm_w4a4_cuda(act=block_activations(act).to(dev), out=blk, act_unsigned=unsigned, act_blocked=True, **t)
+        torch.cuda.synchronize()
+        assert torch.equal(nat.view(torch.int16), blk.view(torch.int16))
+        gemm_mod.USE_WEIGHT_PLANES = "none"  # the int8 main loop reads the matrix only
+        with pytest.raises(ValueError):
+            ops.svdq_gemm_w4a4_cuda(act=block_activations(act).to(dev), out=blk, act_unsigned=unsigned, act_blocked=True, **t)
+    finally:
+        gemm_mod.USE_WEIGHT_PLANES = old
+
+
+@pytest.mark.parametrize("swiglu", [False, True])
+def test_requantizing_epilogues_write_either_order(dev, swiglu):
+    from nunchaku_rocm_amd import ops
+    from nunchaku_rocm_amd.layout import unblock_activations
+    from nunchaku_rocm_amd.ops import gemm as gemm_mod
+
+    M, N, K, R2, dtype = 288, 512, 256, 32, torch.bfloat16
+    NQ = N // 2 if swiglu else N
+    g = torch.Generator().manual_seed(11)
+    t = dict(act=torch.randint(0, 256, (M, K // 2), generator=g, dtype=torch.uint8), wgt=torch.randint(0, 256, (N, K // 2), generator=g, dtype=torch.uint8),
+             ascales=(torch.rand(K // 64, M, generator=g) * 0.2 + 0.05).to(dtype), wscales=(torch.rand(K // 64, N, generator=g) * 0.02 + 0.01).to(dtype),
+             bias=torch.randn(N, generator=g).to(dtype), smooth_factor=(torch.rand(NQ, generator=g) + 0.5).to(dtype),
+             lora_down=(torch.randn(NQ, R2, generator=g) * 0.1).to(dtype))  # fmt: skip
+    t = {k: v.to(dev) for k, v in t.items()}
+    res = []
+    for blocked in (False, True):
+        qout = torch.full((M, NQ // 2), 0xEE, dtype=torch.uint8, device=dev)
+        osc = torch.zeros(NQ // 64, M, dtype=dtype, device=dev)
+        lao = torch.zeros(M, R2, dtype=torch.float32, device=dev)
+        ops.svdq_gemm_w4a4_cuda(qout=qout, oscales=osc, lora_act_out=lao, fuse_swiglu=swiglu, qout_blocked=blocked, **t)
+        torch.cuda.synchronize()
+        res.append((unblock_activations(qout.cpu()) if blocked else qout.cpu(), osc.cpu().view(torch.int16), lao.cpu()))
+    for a, b in zip(*res):
+        assert torch.equal(a, b)
+    assert (res[0][0] != 0xEE).any()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_modules_compute_the_same_bits_either_way(dev, dtype):
+    """SVDQW4A4Linear.forward, fused_gelu_mlp, fused_qkv_norm_rottary and fused_swiglu_mlp with and without the blocked
+    hand-over (row counts that are and are not multiples of 256)."""
+    from nunchaku_rocm_amd import ops
+    from nunchaku_rocm_amd.ops import gemm as gemm_mod
+
+    C, H4 = 256, 1024
+    fc1, fc2 = _module(dev, C, H4, 1, dtype), _module(dev, H4, C, 2, dtype, act_unsigned=True)
+    qkv = _module(dev, C, 3 * 128, 3, dtype)
+    g1, g2 = _module(dev, C, 2 * 512, 4, dtype), _module(dev, 512, C, 5, dtype)
+    ops.interleave_swiglu_linear_(g1)
+    nq = torch.nn.RMSNorm(128, eps=1e-6, device=dev, dtype=dtype)
+    nk = torch.nn.RMSNorm(128, eps=1e-6, device=dev, dtype=dtype)
+    for S in (512, 300):
+        x = torch.randn(1, S, C, generator=torch.Generator().manual_seed(S)).to(dtype).to(dev)
+        rot = O.flux_rotary(O.flux_ids(S - 64, 8, 8)).to(dev)
+        outs = []
+        for flag in (True, False):
+            gemm_mod.USE_BLOCKED_ACTIVATIONS = flag
+            try:
+                assert fc1.takes_blocked(S) == flag
+                outs.append([fc1(x).clone(), ops.fused_gelu_mlp(x, fc1, fc2).clone(), ops.fused_qkv_norm_rottary(x, qkv, nq, nk, rot).clone(),
+                             ops.fused_swiglu_mlp(x, g1, g2).clone()])  # fmt: skip
+            finally:
+                gemm_mod.USE_BLOCKED_ACTIVATIONS = True
+        torch.cuda.synchronize()
+        for a, b in zip(*outs):
+            assert torch.equal(a.view(torch.int16), b.view(torch.int16))
