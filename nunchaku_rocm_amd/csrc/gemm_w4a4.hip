@@ -169,6 +169,10 @@ __device__ inline v4i g_load128(__amdgpu_buffer_rsrc_t r, uint32_t lane_off, uin
     return __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(r, (int)lane_off, (int)uniform_off, 0));
 }
 
+__device__ inline v2i g_load64(__amdgpu_buffer_rsrc_t r, uint32_t lane_off, uint32_t uniform_off) {
+    return __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(r, (int)lane_off, (int)uniform_off, 0));
+}
+
 __device__ inline v16i magic_acc() {
     v16i c;
 #pragma unroll
@@ -829,8 +833,13 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_i8_kernel(svdq_gemm_arg
 // PIPE = false: held to 168 registers, three workgroups per CU, a step's matrix instructions and FMAs in program order.
 // PIPE = true: two workgroups per CU, the matrix instructions of step b + 1 issued ahead of the FMAs of step b (two sets
 // of result registers): a workgroup on its own runs faster, which pays when few, long tiles leave CUs half empty.
-template <typename T, bool ACT_UNSIGNED, int EPI, bool PIPE>
+// F6ACT (act_blocked == 2; instantiated with ACT_UNSIGNED, i.e. without the offset correction): the activations arrive
+// as fp6 codes (sign | magnitude, what the matrix instruction wants of a signed value too) in lane order -- per 32 rows
+// and group 1 KB of the lanes' first 16 bytes and 512 bytes of their last 8 -- and go into the matrix instruction as
+// they are loaded: fp6 x fp6 (half the matrix-pipe time of fp8 x fp6), no nibble unpack, no offset to take out.
+template <typename T, bool ACT_UNSIGNED, int EPI, bool PIPE, bool F6ACT = false>
 __global__ __launch_bounds__(NTHREADS, PIPE ? 2 : 3) void gemm_w4a4_f8_kernel(svdq_gemm_args a) {
+    static_assert(!F6ACT || ACT_UNSIGNED, "fp6 activation codes carry their sign: there is no offset to correct");
     // Separate LDS objects: the compiler then knows that a block load into one staging buffer cannot touch what is being
     // read from the other (one object would make every LDS read wait for the loads in flight).
     __shared__ __align__(16) uint8_t sbuf0[F8_STAGE_BYTES];
@@ -872,24 +881,33 @@ __global__ __launch_bounds__(NTHREADS, PIPE ? 2 : 3) void gemm_w4a4_f8_kernel(sv
     // exactly what the lane holds as MFMA operand after the unpack, and the row's two activation scales.  A group past
     // the end (K / 64 odd) re-reads the last one: its weight codes, scale and offset term are stored as zero.
     v4i araw[2];
+    v8i a6[2][2];  // F6ACT: [stage parity][group], loaded one stage ahead into the set the running stage does not read
     uint16_t qa[2];
     const int mrow = min(m0 + wm * 32 + l32, a.M - 1);
     // Activations either as the (M, K / 2) matrix (a lane fetches the 16 bytes of its own row: 32 rows to a load
     // instruction) or in lane order (act_blocked: per 32 rows and group 1 KB = lane l's 16 bytes at 16 l, groups in a
     // row): the same two loads per stage, base + lane offset + group * step, with other constants.
-    const bool ablk = a.act_blocked != 0;
+    const bool ablk = F6ACT || a.act_blocked != 0;
+    const uint32_t sAct = F6ACT ? 1536u : ablk ? 1024u : 32u;
     const __amdgpu_buffer_rsrc_t rAct =
-        g_buffer((const uint8_t *)a.act + (ablk ? (size_t)((m0 >> 5) + wm) * G * 1024 : (size_t)m0 * a.ld_act));
+        g_buffer((const uint8_t *)a.act + (ablk ? (size_t)((m0 >> 5) + wm) * G * sAct : (size_t)m0 * a.ld_act));
     const __amdgpu_buffer_rsrc_t rAS = g_buffer(a.ascales);
     const uint32_t oAct = ablk ? (uint32_t)lane * 16u : (uint32_t)(mrow - m0) * (uint32_t)a.ld_act + half * 16;
-    const uint32_t sAct = ablk ? 1024u : 32u;
+    const uint32_t oExt = 1024u + (uint32_t)lane * 8u;
     const uint32_t oA = 2u * (uint32_t)mrow;
-    auto load_regs = [&](int s) {
+    auto load_regs = [&](int s, auto set_tag) {
+        constexpr int SET = decltype(set_tag)::value;
 #pragma unroll
         for (int gg = 0; gg < 2; gg++) {
             const int gi = min(2 * s + gg, G - 1);
             qa[gg] = g_load16(rAS, oA, (uint32_t)gi * (uint32_t)a.ld_ascales * 2u);
-            araw[gg] = g_load128(rAct, oAct, (uint32_t)gi * sAct);
+            if constexpr (F6ACT) {
+                const v4i lo = g_load128(rAct, oAct, (uint32_t)gi * sAct);
+                const v2i hi = g_load64(rAct, oExt, (uint32_t)gi * sAct);
+                a6[SET][gg] = (v8i){lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], 0, 0};
+            } else {
+                araw[gg] = g_load128(rAct, oAct, (uint32_t)gi * sAct);
+            }
         }
     };
 
@@ -927,7 +945,7 @@ __global__ __launch_bounds__(NTHREADS, PIPE ? 2 : 3) void gemm_w4a4_f8_kernel(sv
         __builtin_amdgcn_s_waitcnt(waitcnt_imm(63, 0));
     }
 
-    load_regs(0);
+    load_regs(0, std::integral_constant<int, 0>{});
 #pragma unroll
     for (int i = 0; i < 4; i++) dma(0, sbuf0, 0, i);
     fetch_epilogue_operands<EPI>(a, sepi, n0, wm, lane);
@@ -943,13 +961,18 @@ __global__ __launch_bounds__(NTHREADS, PIPE ? 2 : 3) void gemm_w4a4_f8_kernel(sv
         // two's complement nibble -> a + 8 is a flip of the nibble's top bit; -> a - 7 = -(7 - a) is a flip of the other
         // three plus the fp8 sign bit: written per plane so that mask and flip are one three-input bit operation
         v8i a8[2];
+        if constexpr (F6ACT) {
+            a8[0] = a6[ST & 1][0];
+            a8[1] = a6[ST & 1][1];
+        } else {
 #pragma unroll
-        for (int gg = 0; gg < 2; gg++) {
-            typedef unsigned v4u __attribute__((ext_vector_type(4)));
-            const v4u u = __builtin_bit_cast(v4u, araw[gg]);
-            const unsigned fe = ACT_UNSIGNED ? 0u : 0x08080808u, fo = ACT_UNSIGNED ? 0u : 0x87878787u;
-            const v4u e = (u & 0x0F0F0F0Fu) ^ fe, o = ((u >> 4) & 0x0F0F0F0Fu) ^ fo;
-            a8[gg] = (v8i){(int)e[0], (int)e[1], (int)e[2], (int)e[3], (int)o[0], (int)o[1], (int)o[2], (int)o[3]};
+            for (int gg = 0; gg < 2; gg++) {
+                typedef unsigned v4u __attribute__((ext_vector_type(4)));
+                const v4u u = __builtin_bit_cast(v4u, araw[gg]);
+                const unsigned fe = ACT_UNSIGNED ? 0u : 0x08080808u, fo = ACT_UNSIGNED ? 0u : 0x87878787u;
+                const v4u e = (u & 0x0F0F0F0Fu) ^ fe, o = ((u >> 4) & 0x0F0F0F0Fu) ^ fo;
+                a8[gg] = (v8i){(int)e[0], (int)e[1], (int)e[2], (int)e[3], (int)o[0], (int)o[1], (int)o[2], (int)o[3]};
+            }
         }
         // Operands of the scale products as[m] * ws[n] for a 32x32x8 matrix instruction on 16-bit values: lanes 0-31 hold K
         // slots 0-3, two to a register.  The weight side is the dword (ws of the first group, ws of the second group) as it
@@ -975,7 +998,7 @@ __global__ __launch_bounds__(NTHREADS, PIPE ? 2 : 3) void gemm_w4a4_f8_kernel(sv
         // stage re-fetches itself (harmless, and keeps the stage one basic block); its rows go to the next ring slot all
         // the same, which nobody reads.
         const int sn = min(s + 1, nstages - 1), slotn = (s + 1) & (AUX_SLOTS - 1);
-        load_regs(sn);
+        load_regs(sn, std::integral_constant<int, (ST + 1) & 1>{});
         auto read_w8 = [&](int b) -> v8i {  // six registers of fp6 codes (the matrix instruction ignores the last two)
             const int gg = b >> 2, bn = b & 3;
             const v4i lo = *(const v4i *)(base + lane * 16 + (bn * WPL_BLOCKS + gg) * BLK_BYTES);
@@ -987,7 +1010,10 @@ __global__ __launch_bounds__(NTHREADS, PIPE ? 2 : 3) void gemm_w4a4_f8_kernel(sv
         // beside the vector FMAs; the fp32 rank-1 matrix instruction shares the vector ALUs and does not
         auto scales = [&](int b) -> v16f { return mfma32_16bit_k8<T>((v2i){(int)wsd[b & 3], 0}, sa[b >> 2], z16); };
         auto group = [&](int b, const v8i &w) -> v16f {
-            return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(w, a8[b >> 2], z16, 2, 0, 0, F6_SCALE, 0, F8_SCALE);
+            if constexpr (F6ACT)
+                return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(w, a8[b >> 2], z16, 2, 2, 0, F6_SCALE, 0, F6_SCALE);
+            else
+                return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(w, a8[b >> 2], z16, 2, 0, 0, F6_SCALE, 0, F8_SCALE);
         };
         if constexpr (!PIPE) {
             v8i w8[2];
@@ -1205,31 +1231,38 @@ static bool two_workgroups_per_cu(long tiles) {
     return cost(2, 2.16, last2) < cost(3, 3.0, last3);
 }
 
-template <typename T, bool U, bool PIPE>
+template <typename T, bool U, bool PIPE, bool F6ACT>
 static void launch_gemm_f8p(const svdq_gemm_args &a, hipStream_t s) {
     const dim3 grid(((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN)), block(NTHREADS);
     switch (a.epilogue) {
         case SVDQ_EPI_PLAIN:
-            hipLaunchKernelGGL((gemm_w4a4_f8_kernel<T, U, SVDQ_EPI_PLAIN, PIPE>), grid, block, 0, s, a);
+            hipLaunchKernelGGL((gemm_w4a4_f8_kernel<T, U, SVDQ_EPI_PLAIN, PIPE, F6ACT>), grid, block, 0, s, a);
             break;
         case SVDQ_EPI_QK_NORM_ROPE:
-            hipLaunchKernelGGL((gemm_w4a4_f8_kernel<T, U, SVDQ_EPI_QK_NORM_ROPE, PIPE>), grid, block, 0, s, a);
+            hipLaunchKernelGGL((gemm_w4a4_f8_kernel<T, U, SVDQ_EPI_QK_NORM_ROPE, PIPE, F6ACT>), grid, block, 0, s, a);
             break;
         case SVDQ_EPI_GELU_QUANT:
-            hipLaunchKernelGGL((gemm_w4a4_f8_kernel<T, U, SVDQ_EPI_GELU_QUANT, PIPE>), grid, block, 0, s, a);
+            hipLaunchKernelGGL((gemm_w4a4_f8_kernel<T, U, SVDQ_EPI_GELU_QUANT, PIPE, F6ACT>), grid, block, 0, s, a);
             break;
         case SVDQ_EPI_SWIGLU_QUANT:
-            hipLaunchKernelGGL((gemm_w4a4_f8_kernel<T, U, SVDQ_EPI_SWIGLU_QUANT, PIPE>), grid, block, 0, s, a);
+            hipLaunchKernelGGL((gemm_w4a4_f8_kernel<T, U, SVDQ_EPI_SWIGLU_QUANT, PIPE, F6ACT>), grid, block, 0, s, a);
             break;
     }
 }
 
 template <typename T, bool U>
 static void launch_gemm_f8(const svdq_gemm_args &a, hipStream_t s) {
-    if (two_workgroups_per_cu((long)((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN)))
-        launch_gemm_f8p<T, U, true>(a, s);
-    else
-        launch_gemm_f8p<T, U, false>(a, s);
+    const bool two = two_workgroups_per_cu((long)((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN));
+    if (a.act_blocked == 2) {  // fp6 codes carry their sign: one instantiation for signed and unsigned activations
+        if (two)
+            launch_gemm_f8p<T, true, true, true>(a, s);
+        else
+            launch_gemm_f8p<T, true, false, true>(a, s);
+    } else if (two) {
+        launch_gemm_f8p<T, U, true, false>(a, s);
+    } else {
+        launch_gemm_f8p<T, U, false, false>(a, s);
+    }
 }
 
 template <typename T, bool U>
@@ -1366,6 +1399,11 @@ static int gemm_w4a4_checked(const svdq_gemm_args &a, void *stream) {
     }
     if (a.wgt_planes && !al16(a.wgt_planes)) {
         set_error("svdq_gemm_w4a4: wgt_planes must be 16-byte aligned");
+        return SVDQ_E_INVALID;
+    }
+    if (a.act_blocked < 0 || a.act_blocked > 2) {
+        set_error("svdq_gemm_w4a4: act_blocked=%d (0: the (M, K / 2) matrix, 1: its bytes in lane order, 2: fp6 codes in lane order)",
+                  a.act_blocked);
         return SVDQ_E_INVALID;
     }
     if (a.act_blocked && !a.wgt_planes) {

@@ -207,6 +207,45 @@ def block_activations(act: torch.Tensor) -> torch.Tensor:
     return act.reshape(rows // 32, 32, kb // 32, 2, 16).permute(0, 2, 3, 1, 4).contiguous().reshape(rows, kb)
 
 
+def block_activations_f6(act: torch.Tensor, unsigned: bool = False) -> torch.Tensor:
+    """Packed activations ``(rows, K/2)`` (rows a multiple of 32, K of 64) -> ``(rows, 3K/4)`` bytes: the same values as
+    fp6 (e2m3) codes ``sign << 5 | magnitude`` in the order the GEMM's fp8 main loop reads them with ``act_blocked=2``
+    (what the quantizer writes with ``out_blocked=2``).  Per 32 rows and group of 64 values 1536 bytes: lane
+    ``32 h + r`` owns the 32 values ``k = 2 p + h`` of row ``r``'s group, code ``p`` in bits ``6 p .. 6 p + 5`` of 24
+    bytes, whose first 16 lie at byte ``16 lane`` and whose last 8 at byte ``1024 + 8 lane``.  Pure torch."""
+    rows, kb = act.shape
+    assert rows % 32 == 0 and kb % 32 == 0, "rows must be a multiple of 32 and K of 64"
+    a = act.to(torch.int16)
+    v = torch.stack([a & 15, a >> 4], dim=-1).reshape(rows, kb * 2)  # nibble values, low nibble = even k
+    if not unsigned:
+        v = (v ^ 8) - 8
+    code = torch.where(v < 0, 32 - v, v)  # sign << 5 | magnitude
+    code = code.reshape(rows // 32, 32, kb // 32, 32, 2).permute(0, 2, 4, 1, 3)  # [row block][group][h][r][p]
+    bits = (code.unsqueeze(-1) >> torch.arange(6, device=act.device)) & 1  # [...][p][bit]
+    bits = bits.reshape(*code.shape[:-1], 24, 8)
+    by = (bits << torch.arange(8, device=act.device)).sum(-1).to(torch.uint8)  # [rb][g][h][r][24]
+    by = by.reshape(rows // 32, kb // 32, 64, 24)
+    out = torch.cat([by[..., :16].reshape(rows // 32, kb // 32, 1024), by[..., 16:].reshape(rows // 32, kb // 32, 512)], dim=-1)
+    return out.reshape(rows, kb * 3 // 2)
+
+
+def unblock_activations_f6(blocked: torch.Tensor, unsigned: bool = False) -> torch.Tensor:
+    """Inverse of :func:`block_activations_f6`: ``(rows, 3K/4)`` fp6 codes in lane order -> packed ``(rows, K/2)``.
+    (A signed zero decodes to zero whatever its sign bit.)"""
+    rows, kb3 = blocked.shape
+    assert rows % 32 == 0 and kb3 % 48 == 0, "rows must be a multiple of 32 and K of 64"
+    g = kb3 // 48
+    b = blocked.reshape(rows // 32, g, 1536)
+    by = torch.cat([b[..., :1024].reshape(rows // 32, g, 64, 16), b[..., 1024:].reshape(rows // 32, g, 64, 8)], dim=-1)
+    bits = (by.to(torch.int16).unsqueeze(-1) >> torch.arange(8, device=blocked.device)) & 1
+    bits = bits.reshape(rows // 32, g, 64, 32, 6)
+    code = (bits << torch.arange(6, device=blocked.device)).sum(-1)  # [rb][g][lane][p]
+    v = torch.where(code >= 32, -(code - 32), code)
+    v = v.reshape(rows // 32, g, 2, 32, 32).permute(0, 3, 1, 4, 2).reshape(rows, g * 32, 2)  # [row][byte][nibble]
+    v = v & 15
+    return (v[..., 0] | (v[..., 1] << 4)).to(torch.uint8)
+
+
 def unblock_activations(blocked: torch.Tensor) -> torch.Tensor:
     """Inverse of :func:`block_activations`."""
     rows, kb = blocked.shape

@@ -34,6 +34,8 @@ USE_BLOCKED_ACTIVATIONS = True
 # instructions want it (made once per weight and cached, as large as the weight): 1 KB per load instruction instead of
 # 8-byte pieces of 32 rows.  False = read the transposed (R2, N) copy (same results).
 USE_BLOCKED_LORA_DOWN = True
+# values of ``act_blocked`` / ``out_blocked`` beyond False / True
+ACT_CODES_F6 = 2
 
 # True sends the requantizing epilogues' LoRA-down partial sums to the buffer built into the library
 # (svdq_gemm_w4a4_static_scratch) instead of a torch allocation per call: for callers that may not allocate, e.g. while
@@ -108,7 +110,7 @@ def svdq_gemm_w4a4_cuda(
     out_v: torch.Tensor | None = None,
     attn_tokens: int = 0,
     fuse_swiglu: bool = False,
-    act_blocked: bool = False,
+    act_blocked: bool | int = False,
     qout_blocked: bool = False,
 ):
     """
@@ -123,6 +125,9 @@ def svdq_gemm_w4a4_cuda(
     * ``act_blocked`` / ``qout_blocked`` (no counterpart in the reference): ``act`` holds its codes in the order the fp8
       main loop reads them, as the quantizer writes them with ``out_blocked=True`` / the requantizing epilogue writes
       ``qout`` that way for the GEMM that consumes it.  Needs a weight with a working copy (see ``USE_WEIGHT_PLANES``).
+      ``act_blocked=2`` (``ACT_CODES_F6``): ``act`` is ``(rows, 3K/4)`` bytes of fp6 codes in lane order, as the quantizer
+      writes them with ``out_blocked=2``: the matrix instruction takes them as they are (no offset term for signed
+      activations, fp6 x fp6); ``act_unsigned`` is then not looked at.
 
     Raises ``NotImplementedError`` for the arguments the reference's ROCm backend rejects as well (``poolout``,
     ``out_vk``, ``out_linearattn``, ``out_q/k/v``) and for the NVFP4-only ones (``fp4``, ``wcscales``, ``alpha != 1``,
@@ -144,8 +149,9 @@ def svdq_gemm_w4a4_cuda(
     assert ascales is not None and wscales is not None, "W4A4 GEMM requires both scale tensors"
 
     act = act.reshape(-1, act.shape[-1])
-    M, K, N = act.shape[0], act.shape[1] * 2, wgt.shape[0]
-    assert wgt.shape[1] * 2 == K, f"weight K mismatch: {wgt.shape[1] * 2} vs {K}"
+    act_blocked = int(act_blocked)
+    M, K, N = act.shape[0], wgt.shape[1] * 2, wgt.shape[0]
+    assert act.shape[1] == (K * 3 // 4 if act_blocked == ACT_CODES_F6 else K // 2), f"weight K mismatch: {K} vs act {tuple(act.shape)}"
     dev = _lib.require_cuda(act, wgt, out, qout, ascales, wscales, oscales, lora_act_in, lora_up, lora_down,
                             lora_act_out, norm_q, norm_k, rotary_emb, bias, smooth_factor)  # fmt: skip
 

@@ -90,6 +90,77 @@ def test_gemm_reads_either_order(dev, M, N, K, R, unsigned):
         gemm_mod.USE_WEIGHT_PLANES = old
 
 
+def test_fp6_layout_helpers_invert_each_other():
+    from nunchaku_rocm_amd.layout import block_activations_f6, unblock_activations_f6
+
+    a = torch.randint(0, 256, (96, 160), dtype=torch.uint8, generator=torch.Generator().manual_seed(0))
+    for unsigned in (False, True):
+        b = block_activations_f6(a, unsigned)
+        assert b.shape == (96, 240)
+        assert torch.equal(unblock_activations_f6(b, unsigned), a)
+    # code p of lane 32 h + r of (row block rb, group g) = value k = 2 p + h of row 32 rb + r's group, sign | magnitude
+    b = block_activations_f6(a, False).reshape(-1)
+    rb, g, h, r, p = 1, 2, 1, 5, 21  # bit 126: straddles the lane's first 16 bytes and its last 8
+    base = (rb * 5 + g) * 1536
+    lane = 32 * h + r
+    vec = torch.cat([b[base + 16 * lane :][:16], b[base + 1024 + 8 * lane :][:8]]).tolist()
+    code = (int.from_bytes(bytes(vec), "little") >> (6 * p)) & 63
+    byte = int(a[32 * rb + r, 32 * g + p])  # k = 2 p + 1: the high nibble of byte p of the group
+    v = ((byte >> 4) ^ 8) - 8
+    assert code == (32 - v if v < 0 else v)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("unsigned", [False, True])
+@pytest.mark.parametrize("M,N,K,R", [(256, 264, 256, 16), (96, 128, 320, 0), (4608, 3072, 3072, 32), (1024, 640, 1216, 32)])
+def test_gemm_takes_fp6_codes(dev, M, N, K, R, unsigned, dtype):
+    """act_blocked=2: the activations as fp6 codes in lane order.  The group sums are the same integers; unsigned
+    activations give the same bits as the nibble matrix, signed ones differ by what the nibble path's 16-bit offset
+    terms round (so they are compared with the oracle's bar instead, and bit for bit at unit scales)."""
+    from nunchaku_rocm_amd import ops
+    from nunchaku_rocm_amd.layout import block_activations_f6
+    from nunchaku_rocm_amd.ops import gemm as gemm_mod
+
+    print(f"case M={M} N={N} K={K} R={R} unsigned={unsigned} {dtype}", flush=True)
+    g = torch.Generator().manual_seed(M + N + K)
+    act = torch.randint(0, 256, (M, K // 2), generator=g, dtype=torch.uint8)
+    t = dict(wgt=torch.randint(0, 256, (N, K // 2), generator=g, dtype=torch.uint8),
+             ascales=(torch.rand(K // 64, M, generator=g) * 0.02 + 0.01).to(dtype),
+             wscales=(torch.rand(K // 64, N, generator=g) * 0.02 + 0.01).to(dtype), bias=torch.randn(N, generator=g).to(dtype))  # fmt: skip
+    if R:
+        t.update(lora_act_in=torch.randn(M, R, generator=g), lora_up=(torch.randn(N, R, generator=g) * 0.1).to(dtype))
+    t = {k: v.to(dev) for k, v in t.items()}
+    codes = block_activations_f6(act, unsigned).to(dev)
+    old = gemm_mod.USE_WEIGHT_PLANES
+    gemm_mod.USE_WEIGHT_PLANES = "all"
+    try:
+        nat = torch.empty(M - 5, N, dtype=dtype, device=dev)
+        ops.svdq_gemm_w4a4_cuda(act=act.to(dev), out=nat, act_unsigned=unsigned, **t)
+        f6 = torch.full((M - 5, N), float("nan"), dtype=dtype, device=dev)
+        ops.svdq_gemm_w4a4_cuda(act=codes, out=f6, act_unsigned=unsigned, act_blocked=2, **t)
+        torch.cuda.synchronize()
+        if unsigned:
+            assert torch.equal(nat.view(torch.int16), f6.view(torch.int16))
+        else:
+            ref = nat.float()
+            err = (f6.float() - ref).abs().max().item() / ref.abs().max().item()
+            assert err < (4e-3 if dtype == torch.bfloat16 else 1e-3), err
+        # unit scales, no LoRA, no bias: integer results below 2^24, exact either way
+        ones = {k: torch.ones_like(t[k]) for k in ("ascales", "wscales")}
+        small = torch.randint(0, 256, (M, K // 2), generator=g, dtype=torch.uint8) & 0x11  # values 0 / 1: sums stay exact in T
+        o1 = torch.empty(M, N, dtype=dtype, device=dev)
+        o2 = torch.empty(M, N, dtype=dtype, device=dev)
+        ops.svdq_gemm_w4a4_cuda(act=small.to(dev), wgt=t["wgt"], out=o1, act_unsigned=unsigned, **ones)
+        ops.svdq_gemm_w4a4_cuda(act=block_activations_f6(small, unsigned).to(dev), wgt=t["wgt"], out=o2, act_unsigned=unsigned, act_blocked=2, **ones)
+        torch.cuda.synchronize()
+        assert torch.equal(o1.view(torch.int16), o2.view(torch.int16))
+        gemm_mod.USE_WEIGHT_PLANES = "none"  # the int8 main loop reads the matrix only
+        with pytest.raises(ValueError):
+            ops.svdq_gemm_w4a4_cuda(act=codes, out=f6, act_unsigned=unsigned, act_blocked=2, **t)
+    finally:
+        gemm_mod.USE_WEIGHT_PLANES = old
+
+
 @pytest.mark.parametrize("swiglu", [False, True])
 def test_requantizing_epilogues_write_either_order(dev, swiglu):
     from nunchaku_rocm_amd import ops
