@@ -35,6 +35,14 @@ constexpr uint32_t pack_bias() {
     return c;
 }
 
+// sum_i (0x4B400000 << 6 i) mod 2^32 over the five codes that lie wholly in the low dword of a 48-bit piece of eight
+// six-bit codes (the sixth contributes its low two bits only, where the constant has none)
+constexpr uint32_t pack6_bias() {
+    uint32_t c = 0;
+    for (int i = 0; i < 5; i++) c += (uint32_t)RNE_MAGIC_BITS << (6 * i);
+    return c;
+}
+
 // per-group vectors a lane fetches for the group's 64 channels (one channel per lane), shared through LDS later
 struct QVecs {
     uint16_t sm, ns, nh;  // smooth factor, norm scale, norm shift
@@ -86,6 +94,21 @@ __global__ __launch_bounds__(Q_WAVES * 64, QR == 32 ? 1 : (NORM ? 4 : 2)) void q
         const int m = m0 + Q_ROWS * h + ml;
         bout[h] = (uint8_t *)a.out + (size_t)(m >> 5) * ngroups * 1024 + (((kq >> 1) * 32 + (m & 31)) * 16 + (kq & 1) * 8);
     }
+    // out_blocked == 2: fp6 codes (sign << 5 | magnitude) where the GEMM's lane 32 kh + row % 32 of the row block and
+    // group finds its 32 values k = 2 p + kh as 24 bytes, code p at bits 6 p: the first 16 bytes at 16 lane, the last 8 at
+    // 1024 + 8 lane of the (row block, group)'s 1536.  This lane's even channels are codes 8 kq .. 8 kq + 7 of kh = 0, its odd
+    // ones the same codes of kh = 1: two 48-bit pieces at byte 6 kq of those 24, each stored as an aligned dword and a
+    // 16-bit half (low dword + high half for even kq, low half + high dword for odd kq).
+    const bool f6 = a.out_blocked == 2;
+    uint8_t *__restrict__ const f6base = (uint8_t *)a.out + (size_t)(m0 >> 5) * ngroups * 1536;
+    uint32_t f6o32[NH], f6o16[NH];
+#pragma unroll
+    for (int h = 0; h < NH; h++) {
+        const uint32_t r = (uint32_t)(m0 + Q_ROWS * h + ml) & 31u;
+        f6o32[h] = kq == 0 ? 16u * r : kq == 1 ? 16u * r + 8u : kq == 2 ? 16u * r + 12u : 1024u + 8u * r + 4u;
+        f6o16[h] = kq == 0 ? 16u * r + 4u : kq == 1 ? 16u * r + 6u : kq == 2 ? 1024u + 8u * r : 1024u + 8u * r + 2u;
+    }
+    const uint32_t f6d32 = kq < 3 ? 512u : 256u, f6d16 = kq < 2 ? 512u : 256u;  // from kh = 0 to kh = 1
     constexpr int GSTEP = Q_WAVES * GROUP;  // elements between consecutive groups of one wavefront
     const float qmax = UNSIGNED ? 15.0f : 7.0f;
     const float rmagic = UNSIGNED ? RNE_MAGIC : RNE_MAGIC + 8.0f;  // signed codes are packed as c + 8, then ^ 8
@@ -286,6 +309,42 @@ __global__ __launch_bounds__(Q_WAVES * 64, QR == 32 ? 1 : (NORM ? 4 : 2)) void q
             // adds pack eight of them per dword (the constant upper bits add up to pack_bias()).  Signed codes need
             // no clamp: |x| <= gmax gives |x * (1 / (gmax / 7))| <= 7 (1 + 3 * 2^-24), which rounds to <= 7; unsigned codes
             // only need the lower clamp (negative values), the upper bound holds the same way.
+            if (f6) {
+                // the same products and the same rounding, on |q| with the sign carried as bit 5 of the code: the magic
+                // constant gets 32 more when q is negative (an even number of units: ties fall as they did)
+                uint32_t plo[2] = {0u - pack6_bias(), 0u - pack6_bias()}, phi[2] = {0u, 0u};  // [0]: even channels, [1]: odd
+#pragma unroll
+                for (int j = 0; j < 16; j++) {
+                    const float q = v[j] * rq;
+                    uint32_t b;
+                    if (UNSIGNED) {
+                        b = __float_as_uint(__builtin_fmaxf(q, 0.0f) + RNE_MAGIC);
+                    } else {
+                        const uint32_t mg = ((uint32_t)((int)__float_as_uint(q) >> 31) & 32u) | (uint32_t)RNE_MAGIC_BITS;
+                        b = __float_as_uint(__builtin_fabsf(q) + __uint_as_float(mg));
+                    }
+                    const int c = j >> 1, e = j & 1;  // code c of piece e
+                    if (c < 5)
+                        asm("v_lshl_add_u32 %0, %1, %2, %0" : "+v"(plo[e]) : "v"(b), "n"(6 * c));
+                    else if (c == 5) {
+                        plo[e] += b << 30;
+                        phi[e] = b >> 2;
+                    } else
+                        asm("v_lshl_add_u32 %0, %1, %2, %0" : "+v"(phi[e]) : "v"(b), "n"(6 * c - 32));
+                }
+                if (row_ok) {
+                    if (kq == 0) (scales + (size_t)i * Q_WAVES * a.ld_scales)[Q_ROWS * h + ml] = T::from_f32(scale);
+                    uint8_t *blk = f6base + (size_t)(wave + Q_WAVES * i) * 1536;
+#pragma unroll
+                    for (int e = 0; e < 2; e++) {
+                        const uint32_t d32 = (kq & 1) ? __builtin_amdgcn_alignbit(phi[e], plo[e], 16) : plo[e];
+                        const uint32_t d16 = (kq & 1) ? plo[e] : phi[e];
+                        *(uint32_t *)(blk + f6o32[h] + (e ? f6d32 : 0u)) = d32;
+                        *(uint16_t *)(blk + f6o16[h] + (e ? f6d16 : 0u)) = (uint16_t)d16;
+                    }
+                }
+                continue;
+            }
             uint32_t w0 = 0u - pack_bias(), w1 = 0u - pack_bias();
 #pragma unroll
             for (int j = 0; j < 8; j++) {
@@ -640,6 +699,11 @@ extern "C" int svdq_quantize_act(const svdq_quantize_args *args, void *stream) {
     }
     if (a.ld_x % 8 || ((uintptr_t)a.x & 15) || (a.R > 0 && ((uintptr_t)a.lora_down_t & 15))) {
         set_error("svdq_quantize_act: x rows and lora_down_t must be 16-byte aligned (ld_x=%d)", a.ld_x);
+        return SVDQ_E_INVALID;
+    }
+    if (a.out_blocked < 0 || a.out_blocked > 2) {
+        set_error("svdq_quantize_act: out_blocked=%d (0: the (M, K / 2) matrix, 1: its bytes in lane order, 2: fp6 codes in lane order)",
+                  a.out_blocked);
         return SVDQ_E_INVALID;
     }
     if ((!a.out_blocked && a.ld_out % 8) || ((uintptr_t)a.out & (a.out_blocked ? 15 : 7))) {

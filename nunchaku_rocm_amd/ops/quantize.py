@@ -60,7 +60,7 @@ def quantize_w4a4_act_fuse_lora(
     unsigned: bool = False,
     norm: tuple | None = None,
     norm_eps: float = 1e-6,
-    out_blocked: bool = False,
+    out_blocked: bool | int = False,
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """
     Backend-level quantizer with the reference's full option set (reference:
@@ -76,6 +76,8 @@ def quantize_w4a4_act_fuse_lora(
     ``out_blocked=True`` (no counterpart in the reference): ``output`` keeps its shape but holds the codes in the order
     the GEMM's fp8 main loop reads them (``svdq_quantize_args.out_blocked``; pass it on with ``act_blocked=True``); it
     must be contiguous with a multiple of 32 rows.  :func:`nunchaku_rocm_amd.layout.unblock_activations` undoes it.
+    ``out_blocked=2``: ``output`` is ``(rows, 3K/4)`` bytes of fp6 codes (sign << 5 | magnitude, the same integers) in
+    lane order, for the GEMM's ``act_blocked=2`` (:func:`nunchaku_rocm_amd.layout.unblock_activations_f6`).
     """
     if fp4:
         raise NotImplementedError("NVFP4 quantization is not implemented (int4 only)")
@@ -88,8 +90,10 @@ def quantize_w4a4_act_fuse_lora(
     if K % 64:
         raise ValueError(f"K={K} must be a multiple of the group size 64")
     rank = lora_down.shape[1] if lora_down is not None else 0
+    out_blocked = int(out_blocked)
+    kb = K * 3 // 4 if out_blocked == 2 else K // 2  # bytes of codes per row
     if output is None:
-        output = torch.empty(M, K // 2, dtype=torch.uint8, device=inp.device)
+        output = torch.empty(_ceil_divide(M, 32) * 32 if out_blocked else M, kb, dtype=torch.uint8, device=inp.device)
     if oscales is None:
         oscales = torch.empty(K // 64, M, dtype=inp.dtype, device=inp.device)
     if lora_act_out is None and lora_down is not None:
@@ -99,8 +103,8 @@ def quantize_w4a4_act_fuse_lora(
         inp = inp.contiguous()
     if output.element_size() != 1 or output.stride(1) != 1 or output.shape[0] < M:
         raise ValueError("output must be a (>= M, K/2) byte tensor with unit inner stride")
-    if out_blocked and (not output.is_contiguous() or output.shape[0] % 32 or output.shape[1] != K // 2 or output.data_ptr() % 16):
-        raise ValueError("out_blocked needs a contiguous (rows, K/2) output with rows a multiple of 32")
+    if out_blocked and (not output.is_contiguous() or output.shape[0] % 32 or output.shape[1] != kb or output.data_ptr() % 16):
+        raise ValueError("out_blocked needs a contiguous (rows, K/2) output (2: (rows, 3K/4)) with rows a multiple of 32")
     if oscales.dtype != inp.dtype or oscales.stride(1) != 1 or oscales.shape[1] < M or oscales.shape[0] < K // 64:
         raise ValueError("oscales must be (K/64, >= M) of the input dtype with unit inner stride")
     if rank and (lora_act_out.dtype != torch.float32 or lora_act_out.stride(1) != 1 or lora_act_out.shape[0] < M):
@@ -140,7 +144,7 @@ def quantize_w4a4_act_fuse_lora(
         is_unsigned=int(unsigned),
         prologue=_lib.PRE_GLU if fuse_glu else (_lib.PRE_GELU if fuse_gelu else _lib.PRE_NONE),
         shift=float(shift_value),
-        out_blocked=int(out_blocked),
+        out_blocked=out_blocked,
     )
     with torch.cuda.device(inp.device):
         _lib.check(_lib.load().svdq_quantize_act(args, _lib.stream_of(inp)))
@@ -183,7 +187,7 @@ def svdq_quantize_w4a4_act_fuse_lora_cuda(
     pad_size: int = 256,
     norm: tuple | None = None,
     norm_eps: float = 1e-6,
-    out_blocked: bool = False,
+    out_blocked: bool | int = False,
 ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """
     Quantize activations to int4 (per-group-64 absmax, after dividing by ``smooth``) and compute the LoRA
@@ -197,7 +201,8 @@ def svdq_quantize_w4a4_act_fuse_lora_cuda(
     Unlike the reference wrapper (which dereferences ``lora_down.shape`` unconditionally), ``lora_down=None`` is
     accepted and returns ``lora_act_out`` with zero columns.  ``norm`` / ``norm_eps``: the LayerNorm + modulate
     prologue described in :func:`quantize_w4a4_act_fuse_lora` (an addition; ``None`` = the reference's behaviour).
-    ``out_blocked``: see there as well (an addition; ``False`` = the reference's ``(M_pad, C/2)`` matrix).
+    ``out_blocked``: see there as well (an addition; ``False`` = the reference's ``(M_pad, C/2)`` matrix; ``2`` =
+    ``(M_pad, 3C/4)`` fp6 codes).
     """
     if fp4:
         raise NotImplementedError("NVFP4 quantization is not implemented (int4 only)")
@@ -207,7 +212,8 @@ def svdq_quantize_w4a4_act_fuse_lora_cuda(
     rank = lora_down.shape[1] if lora_down is not None else 0
     batch_size_pad = _ceil_divide(batch_size, pad_size) * pad_size
     if output is None:
-        output = torch.empty(batch_size_pad, channels // 2, dtype=torch.uint8, device=input.device)
+        kb = (channels // 2 if fuse_glu else channels) * 3 // 4 if int(out_blocked) == 2 else channels // 2
+        output = torch.empty(batch_size_pad, kb, dtype=torch.uint8, device=input.device)
     if oscales is None:
         assert channels % 64 == 0
         oscales = torch.empty(channels // 64, batch_size_pad, dtype=input.dtype, device=input.device)

@@ -57,6 +57,73 @@ def test_quantizer_writes_the_same_codes_elsewhere(dev, M, K, R, norm, dtype):
         assert torch.equal(blk[2].cpu()[:M], nat[2].cpu()[:M])
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,K,R,norm,unsigned", [(300, 256, 16, False, False), (4608, 3072, 32, False, False), (272, 320, 32, True, False),
+                                                 (100, 64, 0, False, False), (1000, 1024, 32, False, True), (4608, 3072, 32, True, False)])
+def test_quantizer_writes_fp6_codes(dev, M, K, R, norm, unsigned, dtype):
+    """out_blocked=2: the same integers as the (M, K/2) matrix holds, as sign | magnitude codes in lane order; scales and
+    LoRA-down product unchanged; rows past M untouched."""
+    from nunchaku_rocm_amd import ops
+    from nunchaku_rocm_amd.layout import unblock_activations_f6
+
+    print(f"case M={M} K={K} R={R} norm={norm} unsigned={unsigned} {dtype}", flush=True)
+    g = torch.Generator().manual_seed(M + K)
+    x = torch.randn(M, K, generator=g).to(dtype).to(dev)
+    x[3, :64] = 0  # a group of zeros: scale 0, codes 0
+    smooth = (torch.rand(K, generator=g) + 0.5).to(dtype).to(dev)
+    ld = (torch.randn(K, R, generator=g) * 0.1).to(dtype).to(dev) if R else None
+    nm = ((torch.randn(K, generator=g) * 0.1 + 1).to(dtype).to(dev), (torch.randn(K, generator=g) * 0.1).to(dtype).to(dev)) if norm else None
+    kw = dict(lora_down=ld, smooth=smooth, norm=nm)
+    if unsigned:
+        kw.update(shift_value=0.171875, unsigned=True, fuse_gelu=True)
+        fn = ops.quantize_w4a4_act_fuse_lora
+        nat = fn(x, **kw)
+        rows = (M + 31) // 32 * 32
+    else:
+        fn = ops.svdq_quantize_w4a4_act_fuse_lora_cuda
+        nat = fn(x, **kw)
+        rows = nat[0].shape[0]
+    out_b = torch.full((rows, K * 3 // 4), 0xEE, dtype=torch.uint8, device=dev)
+    blk = fn(x, output=out_b, out_blocked=2, **kw)
+    torch.cuda.synchronize()
+    dec = unblock_activations_f6(blk[0].cpu(), unsigned)
+    assert torch.equal(dec[:M], nat[0].cpu()[:M])
+    # rows past M of a 32-row block that has rows: untouched bytes decode to whatever 0xEE means; whole untouched blocks stay 0xEE
+    full = (M + 31) // 32 * 32
+    assert (blk[0].cpu()[full:] == 0xEE).all()
+    assert torch.equal(blk[1].cpu()[:, :M].view(torch.int16), nat[1].cpu()[:, :M].view(torch.int16))
+    if R:
+        assert torch.equal(blk[2].cpu()[:M], nat[2].cpu()[:M])
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_quantizer_then_gemm_through_fp6_codes(dev, dtype):
+    """The pair as the modules run it: quantizer (out_blocked=2) -> GEMM (act_blocked=2) against the pair through the
+    (M, K/2) matrix, at the oracle's bar for the GEMM output."""
+    from nunchaku_rocm_amd import ops
+
+    M, K, N, R = 1000, 1024, 768, 32
+    lin = {k: v.to(dev) for k, v in O.make_svdq_linear(K, N, seed=5, dtype=dtype).items()}
+    x = torch.randn(M, K, generator=torch.Generator().manual_seed(9)).to(dtype).to(dev)
+    from nunchaku_rocm_amd.ops import gemm as gemm_mod
+
+    outs = []
+    old = gemm_mod.USE_WEIGHT_PLANES
+    gemm_mod.USE_WEIGHT_PLANES = "all"
+    try:
+        for mode in (0, 2):
+            q, s, la = ops.svdq_quantize_w4a4_act_fuse_lora_cuda(x, lora_down=lin["proj_down"], smooth=lin["smooth_factor"], out_blocked=mode)
+            out = torch.empty(M, N, dtype=dtype, device=dev)
+            ops.svdq_gemm_w4a4_cuda(act=q, wgt=lin["qweight"], out=out, ascales=s, wscales=lin["wscales"], lora_act_in=la,
+                                    lora_up=lin["proj_up"], bias=lin["bias"], act_blocked=mode)
+            outs.append(out.float())
+        torch.cuda.synchronize()
+    finally:
+        gemm_mod.USE_WEIGHT_PLANES = old
+    err = (outs[0] - outs[1]).abs().max().item() / outs[0].abs().max().item()
+    assert err < (4e-3 if dtype == torch.bfloat16 else 1e-3), err
+
+
 @pytest.mark.parametrize("unsigned", [False, True])
 @pytest.mark.parametrize("M,N,K,R", [(256, 264, 256, 16), (96, 128, 320, 0), (4608, 3072, 3072, 32)])
 def test_gemm_reads_either_order(dev, M, N, K, R, unsigned):
