@@ -28,6 +28,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 INT8_MFMA_PEAK_TOPS = 5000.0  # MI355X dense int8 MFMA, published
+FP6_MFMA_PEAK_TOPS = 10100.0  # MI355X dense fp6 / fp4 MFMA, published
 BF16_MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 / fp16 MFMA, published
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # HBM bytes of one QKV GEMM launch: 2.00 x FETCH_SIZE + 1.00 x WRITE_SIZE (KiB per dispatch) of the grid-663552 launches
@@ -157,20 +158,21 @@ def main():
     # copy per parameter)
     lin = {k: torch.nn.Parameter(v.to(dev), requires_grad=False) for k, v in O.make_svdq_linear(K, N, R, seed=0).items()}
     x = O.make_activations(M, K, seed=1).to(dev)
-    qx = torch.empty(M, K // 2, dtype=torch.uint8, device=dev)
+    qx = torch.empty(M, K * 3 // 4, dtype=torch.uint8, device=dev)  # fp6 codes in the GEMM's lane order
     asc = torch.empty(K // 64, M, dtype=torch.bfloat16, device=dev)
     la = torch.empty(M, R, dtype=torch.float32, device=dev)
     out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
 
-    # The two operator calls of SVDQW4A4Linear.forward, with the hand-over it uses: the quantizer writes the codes in the
-    # order the GEMM's lanes read them (out_blocked / act_blocked; same codes, same results, about 3 % of the GEMM launch).
-    # The GEMM on the reference's (M, K/2) matrix is timed next to it in the per-kernel table.
+    # The two operator calls of SVDQW4A4Linear.forward, with the hand-over it uses: the quantizer writes the codes as fp6
+    # (sign | magnitude) in the order the GEMM's lanes read them (out_blocked = act_blocked = 2: the same integers, taken by
+    # the matrix instruction as they are; about 8 % of the GEMM launch).  The GEMM on the reference's (M, K/2) matrix is
+    # timed next to it in the per-kernel table.
     def quant():
-        ops.svdq_quantize_w4a4_act_fuse_lora_cuda(x, qx, asc, lin["proj_down"], la, lin["smooth_factor"], out_blocked=True)
+        ops.svdq_quantize_w4a4_act_fuse_lora_cuda(x, qx, asc, lin["proj_down"], la, lin["smooth_factor"], out_blocked=2)
 
     def gemm():
         ops.svdq_gemm_w4a4_cuda(act=qx, wgt=lin["qweight"], out=out, ascales=asc, wscales=lin["wscales"],
-                                lora_act_in=la, lora_up=lin["proj_up"], bias=lin["bias"], act_blocked=True)  # fmt: skip
+                                lora_act_in=la, lora_up=lin["proj_up"], bias=lin["bias"], act_blocked=2)  # fmt: skip
 
     def step():
         quant()
@@ -245,10 +247,10 @@ def main():
                                                   "ms_act_as_matrix": round(n_ms, 5)}  # fmt: skip
         for Ms in (1024, 8192):
             xs = O.make_activations(Ms, K, seed=1).to(dev)
-            q2, a2, l2 = ops.svdq_quantize_w4a4_act_fuse_lora_cuda(xs, lora_down=lin["proj_down"], smooth=lin["smooth_factor"], out_blocked=True)
+            q2, a2, l2 = ops.svdq_quantize_w4a4_act_fuse_lora_cuda(xs, lora_down=lin["proj_down"], smooth=lin["smooth_factor"], out_blocked=2)
             o2 = torch.empty(Ms, N, dtype=torch.bfloat16, device=dev)
             ms = _time_kernel(lambda: ops.svdq_gemm_w4a4_cuda(act=q2, wgt=lin["qweight"], out=o2, ascales=a2, wscales=lin["wscales"],
-                                                              lora_act_in=l2, lora_up=lin["proj_up"], bias=lin["bias"], act_blocked=True))  # fmt: skip
+                                                              lora_act_in=l2, lora_up=lin["proj_up"], bias=lin["bias"], act_blocked=2))  # fmt: skip
             kernels[f"gemm_w4a4 M{Ms} K3072 N9216"] = {"ms": round(ms, 5), "TOP/s": round(2.0 * Ms * N * K / ms / 1e9, 1),
                                                        "frac_int8_mfma": round(2.0 * Ms * N * K / ms / 1e9 / INT8_MFMA_PEAK_TOPS, 4)}  # fmt: skip
             del xs, q2, a2, l2, o2
@@ -264,7 +266,7 @@ def main():
             return m
 
         fc1, fc2 = module(3072, 12288, 42), module(12288, 3072, 43, True)
-        q1, a1, l1 = fc1.quantize(x, blocked=True)
+        q1, a1, l1 = fc1.quantize(x, blocked=2)
         qo = torch.empty(M, 6144, dtype=torch.uint8, device=dev)
         oo = torch.empty(192, M, dtype=torch.bfloat16, device=dev)
         lo = torch.empty(M, 32, dtype=torch.float32, device=dev)
@@ -273,7 +275,7 @@ def main():
         def fc1_fused():
             ops.svdq_gemm_w4a4_cuda(act=q1, wgt=fc1.qweight, qout=qo, ascales=a1, wscales=fc1.wscales, oscales=oo, lora_act_in=l1,
                                     lora_up=fc1.proj_up, lora_down=fc2.proj_down, lora_act_out=lo, bias=fc1.bias,
-                                    smooth_factor=fc2.smooth_factor, act_blocked=True, qout_blocked=True)  # fmt: skip
+                                    smooth_factor=fc2.smooth_factor, act_blocked=2, qout_blocked=True)  # fmt: skip
 
         ms = _time_kernel(fc1_fused)
         f = 2.0 * M * 12288 * 3072
@@ -284,7 +286,7 @@ def main():
         rot = O.flux_rotary(O.flux_ids(512, 64, 64)).to(dev)
         ms = _time_kernel(lambda: ops.svdq_gemm_w4a4_cuda(act=qx, wgt=lin["qweight"], out=out, ascales=asc, wscales=lin["wscales"],
                                                           lora_act_in=la, lora_up=lin["proj_up"], bias=lin["bias"], norm_q=nq, norm_k=nq, rotary_emb=rot,
-                                                          act_blocked=True))  # fmt: skip
+                                                          act_blocked=2))  # fmt: skip
         kernels["gemm_w4a4+qknorm+rope M4608 K3072 N9216"] = {"ms": round(ms, 5), "TOP/s": round(ops_per_gemm / ms / 1e9, 1), "frac_int8_mfma": round(ops_per_gemm / ms / 1e9 / INT8_MFMA_PEAK_TOPS, 4)}  # fmt: skip
         # AWQ GEMV, adaLN shape.  In the model every adaLN layer has its own weight, so a launch finds its 32 MB in HBM, not in
         # the 256 MB memory-side cache: the launches of the timed graph walk over 12 weight sets (384 MB) in turn ("cold",
@@ -380,11 +382,11 @@ def main():
         "vs_baseline": None,
         "dtype": "i8",
         "data": "synthetic",
-        "config": {"workload": "FLUX.1 QKV SVDQuant linear: activation quantizer + W4A4 GEMM, M=4608 K=3072 N=9216 group 64 LoRA rank 32 (the reference's FLUX.1 QKV benchmark shape); the two operator calls of SVDQW4A4Linear.forward, codes handed over in the GEMM's lane order",
+        "config": {"workload": "FLUX.1 QKV SVDQuant linear: activation quantizer + W4A4 GEMM, M=4608 K=3072 N=9216 group 64 LoRA rank 32 (the reference's FLUX.1 QKV benchmark shape); the two operator calls of SVDQW4A4Linear.forward, codes handed over as fp6 in the GEMM's lane order",
                    "M": M, "K": K, "N": N, "rank": R, "group": 64},  # fmt: skip
         "roofline": {
             "bound": "mfma",
-            "kernel": "gemm_w4a4_f8_kernel<BF16, signed activations, plain epilogue, three workgroups per CU>",
+            "kernel": "gemm_w4a4_f8_kernel<BF16, fp6 activation codes, plain epilogue, three workgroups per CU>",
             "achieved": round(achieved, 2),
             "peak": INT8_MFMA_PEAK_TOPS,
             "unit": "TOP/s",
@@ -395,8 +397,11 @@ def main():
             "avg_launch_ms": round(gemm_ms, 5),
             "quantizer_launch_ms": round(quant_ms, 5),
             "step_over_kernels": round(step_ms / (gemm_ms + quant_ms), 4),
-            "note": "2*M*N*K integer ops per launch; the pre-split weights run through the fp8 MFMA on int4-valued codes, "
-                    "whose published dense peak equals the int8 one (5.0 POP/s); avg_launch_ms = back-to-back launches "
+            "frac_of_fp6_mfma_peak": round(achieved / FP6_MFMA_PEAK_TOPS, 4),
+            "note": "2*M*N*K integer ops per launch against the int8 MFMA peak the target is stated in (5.0 POP/s); the group "
+                    "products run on the fp6 x fp6 form of v_mfma_scale_f32_32x32x64_f8f6f4 on int4-valued codes (exact integer "
+                    "sums), whose own published dense peak is 10.1 POP/s (frac_of_fp6_mfma_peak), next to one 16-bit MFMA "
+                    "and 16 fp32 FMAs per 32x32 block and group for the scales; avg_launch_ms = back-to-back launches "
                     "between HIP events on the launch stream",
         },
         "kernels": kernels,

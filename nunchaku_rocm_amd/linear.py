@@ -114,21 +114,24 @@ class SVDQW4A4Linear(nn.Module):
         output = self.forward_quant(quantized_x, ascales, lora_act_out, output, act_blocked=blocked)
         return output.reshape(batch_size, seq_len, -1)
 
-    def takes_blocked(self, rows: int, pad_size: int = 256) -> bool:
-        """Whether this layer's GEMM wants its quantized input in the fp8 main loop's own order (``blocked=True`` in
-        :meth:`quantize`, ``act_blocked=True`` in :meth:`forward_quant`) for ``rows`` rows padded to ``pad_size``."""
+    def takes_blocked(self, rows: int, pad_size: int = 256, requantized: bool = False) -> int:
+        """How this layer's GEMM wants its quantized input for ``rows`` rows padded to ``pad_size``: the value for
+        ``blocked=`` in :meth:`quantize` and ``act_blocked=`` in :meth:`forward_quant` (0 = the reference's matrix, 1 =
+        its bytes in the fp8 main loop's own order, 2 = fp6 codes in that order).  ``requantized``: the input comes out
+        of a requantizing GEMM epilogue instead of the quantizer."""
         from .ops.gemm import takes_blocked_activations
 
-        return takes_blocked_activations(self.qweight, self.wscales, -(-rows // pad_size) * pad_size)
+        return takes_blocked_activations(self.qweight, self.wscales, -(-rows // pad_size) * pad_size, requantized)
 
-    def quantize(self, x: torch.Tensor, pad_size: int = 256, norm: tuple | None = None, blocked: bool = False):
+    def quantize(self, x: torch.Tensor, pad_size: int = 256, norm: tuple | None = None, blocked: bool | int = False):
         """``blocked`` (an addition to the reference's signature): the codes in the order the GEMM's fp8 main loop reads
-        them, for :meth:`forward_quant` with ``act_blocked=True``; ``False`` = the reference's ``(M_pad, K/2)`` matrix."""
+        them (``True``) or as fp6 codes in that order (``2``), for :meth:`forward_quant` with the same ``act_blocked``;
+        ``False`` = the reference's ``(M_pad, K/2)`` matrix."""
         return svdq_quantize_w4a4_act_fuse_lora_cuda(
             x, lora_down=self.proj_down, smooth=self.smooth_factor, fp4=False, pad_size=pad_size, norm=norm, out_blocked=blocked
         )
 
-    def forward_quant(self, quantized_x, ascales, lora_act, output: torch.Tensor | None = None, act_blocked: bool = False) -> torch.Tensor:
+    def forward_quant(self, quantized_x, ascales, lora_act, output: torch.Tensor | None = None, act_blocked: bool | int = False) -> torch.Tensor:
         if output is None:
             output = torch.empty(quantized_x.shape[0], self.out_features, dtype=self.proj_up.dtype, device=quantized_x.device)
         svdq_gemm_w4a4_cuda(

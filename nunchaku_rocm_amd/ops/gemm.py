@@ -26,8 +26,11 @@ USE_BLOCKED_ROTARY = True
 # The modules and composite operators (SVDQW4A4Linear.forward, fused_gelu_mlp, fused_qkv_norm_rottary, fused_swiglu_mlp)
 # pass quantized activations from the quantizer, or from a requantizing epilogue, to the GEMM in the order the fp8 main
 # loop's lanes read them (out_blocked / act_blocked / qout_blocked): 1 KB per load instruction instead of 16-byte pieces
-# of 32 rows, about 3 % of a GEMM launch.  The operators themselves (svdq_quantize_w4a4_act_fuse_lora_cuda,
-# svdq_gemm_w4a4_cuda) keep the reference's (M, K/2) matrix unless asked.  False = the matrix everywhere (same results).
+# of 32 rows.  True: from the quantizer as fp6 codes (ACT_CODES_F6: the matrix instruction takes them as they are --
+# fp6 x fp6, no nibble unpack, no offset term for signed activations; 8 % of a GEMM launch), from a requantizing epilogue
+# as the matrix's bytes in lane order (3 %).  1: the matrix's bytes in lane order everywhere (same results as the
+# matrix, bit for bit).  False: the reference's (M, K/2) matrix everywhere.  The operators themselves
+# (svdq_quantize_w4a4_act_fuse_lora_cuda, svdq_gemm_w4a4_cuda) keep the matrix unless asked.
 USE_BLOCKED_ACTIVATIONS = True
 
 # The GELU + requantization epilogue reads the next layer's LoRA-down weight through a copy in the order its matrix
@@ -69,10 +72,14 @@ def working_copy(wgt: torch.Tensor, wscales: torch.Tensor) -> torch.Tensor | Non
     return planes
 
 
-def takes_blocked_activations(wgt: torch.Tensor, wscales: torch.Tensor, rows: int) -> bool:
-    """Whether a GEMM on this weight should be fed activations in the fp8 main loop's own order (``act_blocked``): the
-    switch is on, the weight has a working copy, and the (padded) row count is a multiple of 32."""
-    return USE_BLOCKED_ACTIVATIONS and rows % 32 == 0 and working_copy(wgt, wscales) is not None
+def takes_blocked_activations(wgt: torch.Tensor, wscales: torch.Tensor, rows: int, requantized: bool = False) -> int:
+    """How a GEMM on this weight should be fed its activations: 0 = the (M, K/2) matrix, 1 = its bytes in the fp8 main
+    loop's own order, 2 (``ACT_CODES_F6``) = fp6 codes in that order -- the value for ``out_blocked`` / ``act_blocked``.
+    Non-zero when the switch is on, the weight has a working copy and the (padded) row count is a multiple of 32;
+    ``requantized``: the activations come out of a requantizing GEMM epilogue (which writes bytes), not the quantizer."""
+    if not USE_BLOCKED_ACTIVATIONS or rows % 32 or working_copy(wgt, wscales) is None:
+        return 0
+    return ACT_CODES_F6 if USE_BLOCKED_ACTIVATIONS is True and not requantized else 1
 
 
 HEAD_DIM = 128
