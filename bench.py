@@ -267,7 +267,7 @@ def main():
 
         fc1, fc2 = module(3072, 12288, 42), module(12288, 3072, 43, True)
         q1, a1, l1 = fc1.quantize(x, blocked=2)
-        qo = torch.empty(M, 6144, dtype=torch.uint8, device=dev)
+        qo = torch.empty(M, 12288 * 3 // 4, dtype=torch.uint8, device=dev)  # fp6 codes in fc2's lane order
         oo = torch.empty(192, M, dtype=torch.bfloat16, device=dev)
         lo = torch.empty(M, 32, dtype=torch.float32, device=dev)
         y2 = torch.empty(M, 3072, dtype=torch.bfloat16, device=dev)
@@ -275,12 +275,12 @@ def main():
         def fc1_fused():
             ops.svdq_gemm_w4a4_cuda(act=q1, wgt=fc1.qweight, qout=qo, ascales=a1, wscales=fc1.wscales, oscales=oo, lora_act_in=l1,
                                     lora_up=fc1.proj_up, lora_down=fc2.proj_down, lora_act_out=lo, bias=fc1.bias,
-                                    smooth_factor=fc2.smooth_factor, act_blocked=2, qout_blocked=True)  # fmt: skip
+                                    smooth_factor=fc2.smooth_factor, act_blocked=2, qout_blocked=2)  # fmt: skip
 
         ms = _time_kernel(fc1_fused)
         f = 2.0 * M * 12288 * 3072
         kernels["gemm_w4a4+gelu+requant fc1 M4608 K3072 N12288"] = {"ms": round(ms, 5), "TOP/s": round(f / ms / 1e9, 1), "frac_int8_mfma": round(f / ms / 1e9 / INT8_MFMA_PEAK_TOPS, 4)}  # fmt: skip
-        ms = _time_kernel(lambda: fc2.forward_quant(qo, oo, lo, y2, act_blocked=True))
+        ms = _time_kernel(lambda: fc2.forward_quant(qo, oo, lo, y2, act_blocked=2))
         kernels["gemm_w4a4 fc2 (unsigned act) M4608 K12288 N3072"] = {"ms": round(ms, 5), "TOP/s": round(f / ms / 1e9, 1), "frac_int8_mfma": round(f / ms / 1e9 / INT8_MFMA_PEAK_TOPS, 4)}  # fmt: skip
         nq = (torch.rand(128, device=dev) + 0.5).to(torch.bfloat16)
         rot = O.flux_rotary(O.flux_ids(512, 64, 64)).to(dev)

@@ -222,6 +222,33 @@ __device__ inline void fetch_epilogue_operands(const svdq_gemm_args &a, uint8_t 
     }
 }
 
+// Requantized activations as fp6 codes in the consuming GEMM's lane order (qout_blocked == 2).  A lane of the epilogue
+// owns, of its row's group of 64 values, the runs k = 8 t + 4 half .. + 3 (t = 0 .. 7): codes p = 4 t + 2 half, + 1 of the
+// consuming lane of K half 0 (its even k) and the same codes of the lane of K half 1 (its odd k), i.e. one 12-bit piece
+// per t and consuming lane, at bit 24 t + 12 half of that lane's 192.  f6_pack_unit places four pieces (96 bits);
+// f6_swap_unit trades the two half-filled units with lane ^ 32 (all lanes of the wavefront must be active) -- every lane
+// ends up with all of one consuming lane's 24 bytes -- and f6_store writes their first 16 at 16 l and their last 8 at
+// 1024 + 8 l of the (row block, group)'s 1536, l = 32 half + row % 32.
+__device__ inline void f6_pack_unit(uint32_t p0, uint32_t p1, uint32_t p2, uint32_t p3, uint32_t sh, uint32_t (&d)[3]) {
+    const uint64_t lo = ((uint64_t)p0 | ((uint64_t)p1 << 24)) << sh, hi = ((uint64_t)p2 | ((uint64_t)p3 << 24)) << sh;
+    d[0] = (uint32_t)lo;
+    d[1] = (uint32_t)(lo >> 32) | ((uint32_t)hi << 16);
+    d[2] = (uint32_t)(hi >> 16);
+}
+__device__ inline void f6_swap_unit(const uint32_t (&v0)[3], const uint32_t (&v1)[3], uint32_t *r) {
+#pragma unroll
+    for (int i = 0; i < 3; i++) {
+        const auto sw = __builtin_amdgcn_permlane32_swap(v0[i], v1[i], false, false);
+        r[i] = sw[0] | sw[1];
+    }
+}
+__device__ inline void f6_store(const uint32_t (&r)[6], uint8_t *blk, int lane, bool ok) {
+    if (ok) {
+        *(v4i *)(blk + 16 * lane) = (v4i){(int)r[0], (int)r[1], (int)r[2], (int)r[3]};
+        *(v2i *)(blk + 1024 + 8 * lane) = (v2i){(int)r[4], (int)r[5]};
+    }
+}
+
 // Everything after the main loop, for one wavefront: acc[bn][i] holds out[m = mw0 + 8 (i >> 2) + 4 half + (i & 3)]
 // [n = n0 + 32 bn + lane % 32] without LoRA-up and bias -- or, with ROWS_IN_LANES (a main loop that passes the weights as
 // the matrix instruction's first operand), out[m = mw0 + lane % 32][n = n0 + 32 bn + 8 (i >> 2) + 4 half + (i & 3)],
@@ -494,6 +521,29 @@ __device__ __forceinline__ void tile_epilogue(const svdq_gemm_args &a, v16f (&ac
             const float safe = (scale == 0.0f) ? 1.0f : scale;
             const float rq = 1.0f / safe;
             if (half == 0 && m < a.M && n0 + 64 * gi < a.N) ((uint16_t *)a.oscales)[(size_t)g * a.ld_oscales + m] = T::from_f32(scale);
+            if (a.qout_blocked == 2) {
+                uint32_t vec[6];
+#pragma unroll
+                for (int b2 = 0; b2 < 2; b2++) {
+                    const int bn = 2 * gi + b2;
+                    uint32_t pc[2][4];
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        uint32_t c[4];
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            c[e] = __float_as_uint(__builtin_amdgcn_fmed3f(acc[bn][4 * j + e] * rq, 0.0f, 15.0f) + RNE_MAGIC) & 0xFu;
+                        pc[0][j] = c[0] | (c[2] << 6);
+                        pc[1][j] = c[1] | (c[3] << 6);
+                    }
+                    uint32_t d0[3], d1[3];
+                    f6_pack_unit(pc[0][0], pc[0][1], pc[0][2], pc[0][3], 12u * half, d0);
+                    f6_pack_unit(pc[1][0], pc[1][1], pc[1][2], pc[1][3], 12u * half, d1);
+                    f6_swap_unit(d0, d1, vec + 3 * b2);
+                }
+                f6_store(vec, (uint8_t *)a.qout + ((size_t)(m >> 5) * (a.N / GROUP) + g) * 1536, 32 * half + (m & 31), m < a.M);
+                continue;
+            }
 #pragma unroll
             for (int b2 = 0; b2 < 2; b2++) {
                 const int bn = 2 * gi + b2;
@@ -594,6 +644,32 @@ __device__ __forceinline__ void tile_epilogue(const svdq_gemm_args &a, v16f (&ac
         const float safe = (scale == 0.0f) ? 1.0f : scale;
         const float rq = 1.0f / safe;
         if (half == 0 && m < a.M) ((uint16_t *)a.oscales)[(size_t)(yt0 / GROUP) * a.ld_oscales + m] = T::from_f32(scale);
+        if (a.qout_blocked == 2) {
+            // sign | magnitude: the magnitude rounds as the value does; the magic constant gets 32 more for a negative one
+            uint32_t vec[6];
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                uint32_t pc[2][4];
+#pragma unroll
+                for (int t = 0; t < 4; t++) {  // piece 4 u + t: block bn = 2 u + t / 2, register run j = t % 2
+                    uint32_t c[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const float q = __builtin_amdgcn_fmed3f(y[2 * u + (t >> 1)][4 * (t & 1) + e] * rq, -8.0f, 7.0f);
+                        const uint32_t mg = ((uint32_t)((int)__float_as_uint(q) >> 31) & 32u) | (uint32_t)RNE_MAGIC_BITS;
+                        c[e] = __float_as_uint(__builtin_fabsf(q) + __uint_as_float(mg)) & 0x3Fu;
+                    }
+                    pc[0][t] = c[0] | (c[2] << 6);
+                    pc[1][t] = c[1] | (c[3] << 6);
+                }
+                uint32_t d0[3], d1[3];
+                f6_pack_unit(pc[0][0], pc[0][1], pc[0][2], pc[0][3], 12u * half, d0);
+                f6_pack_unit(pc[1][0], pc[1][1], pc[1][2], pc[1][3], 12u * half, d1);
+                f6_swap_unit(d0, d1, vec + 3 * u);
+            }
+            f6_store(vec, (uint8_t *)a.qout + ((size_t)(m >> 5) * (H / GROUP) + yt0 / GROUP) * 1536, 32 * half + (m & 31), m < a.M);
+            return;
+        }
 #pragma unroll
         for (int bn = 0; bn < NBN; bn++) {
             uint32_t mine[2];
@@ -1478,6 +1554,11 @@ static int gemm_w4a4_checked(const svdq_gemm_args &a, void *stream) {
         }
         if (a.epilogue == SVDQ_EPI_SWIGLU_QUANT && a.out) {
             set_error("svdq_gemm_w4a4: the SwiGLU epilogue writes qout/oscales only; out must be NULL");
+            return SVDQ_E_INVALID;
+        }
+        if (a.qout_blocked < 0 || a.qout_blocked > 2) {
+            set_error("svdq_gemm_w4a4: qout_blocked=%d (0: the (M, N / 2) matrix, 1: its bytes in lane order, 2: fp6 codes in lane order)",
+                      a.qout_blocked);
             return SVDQ_E_INVALID;
         }
         if (!a.qout || !a.oscales || ((uintptr_t)a.qout & (a.qout_blocked ? 15 : 7)) ||

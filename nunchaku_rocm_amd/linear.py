@@ -114,14 +114,14 @@ class SVDQW4A4Linear(nn.Module):
         output = self.forward_quant(quantized_x, ascales, lora_act_out, output, act_blocked=blocked)
         return output.reshape(batch_size, seq_len, -1)
 
-    def takes_blocked(self, rows: int, pad_size: int = 256, requantized: bool = False) -> int:
+    def takes_blocked(self, rows: int, pad_size: int = 256) -> int:
         """How this layer's GEMM wants its quantized input for ``rows`` rows padded to ``pad_size``: the value for
-        ``blocked=`` in :meth:`quantize` and ``act_blocked=`` in :meth:`forward_quant` (0 = the reference's matrix, 1 =
-        its bytes in the fp8 main loop's own order, 2 = fp6 codes in that order).  ``requantized``: the input comes out
-        of a requantizing GEMM epilogue instead of the quantizer."""
+        ``blocked=`` in :meth:`quantize` (or ``qout_blocked=`` of the GEMM whose epilogue produces the input) and
+        ``act_blocked=`` in :meth:`forward_quant`: 0 = the reference's matrix, 1 = its bytes in the fp8 main loop's own
+        order, 2 = fp6 codes in that order."""
         from .ops.gemm import takes_blocked_activations
 
-        return takes_blocked_activations(self.qweight, self.wscales, -(-rows // pad_size) * pad_size, requantized)
+        return takes_blocked_activations(self.qweight, self.wscales, -(-rows // pad_size) * pad_size)
 
     def quantize(self, x: torch.Tensor, pad_size: int = 256, norm: tuple | None = None, blocked: bool | int = False):
         """``blocked`` (an addition to the reference's signature): the codes in the order the GEMM's fp8 main loop reads

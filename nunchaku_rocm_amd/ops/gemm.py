@@ -26,11 +26,11 @@ USE_BLOCKED_ROTARY = True
 # The modules and composite operators (SVDQW4A4Linear.forward, fused_gelu_mlp, fused_qkv_norm_rottary, fused_swiglu_mlp)
 # pass quantized activations from the quantizer, or from a requantizing epilogue, to the GEMM in the order the fp8 main
 # loop's lanes read them (out_blocked / act_blocked / qout_blocked): 1 KB per load instruction instead of 16-byte pieces
-# of 32 rows.  True: from the quantizer as fp6 codes (ACT_CODES_F6: the matrix instruction takes them as they are --
-# fp6 x fp6, no nibble unpack, no offset term for signed activations; 8 % of a GEMM launch), from a requantizing epilogue
-# as the matrix's bytes in lane order (3 %).  1: the matrix's bytes in lane order everywhere (same results as the
-# matrix, bit for bit).  False: the reference's (M, K/2) matrix everywhere.  The operators themselves
-# (svdq_quantize_w4a4_act_fuse_lora_cuda, svdq_gemm_w4a4_cuda) keep the matrix unless asked.
+# of 32 rows.  True: as fp6 codes (ACT_CODES_F6: the matrix instruction takes them as they are -- fp6 x fp6, no nibble
+# unpack, no offset term for signed activations; 8 % of a GEMM launch on signed, 4 % on unsigned activations).  1: the
+# matrix's bytes in lane order (3 %; the same results as the matrix, bit for bit).  False: the reference's (M, K/2)
+# matrix everywhere.  The operators themselves (svdq_quantize_w4a4_act_fuse_lora_cuda, svdq_gemm_w4a4_cuda) keep the
+# matrix unless asked.
 USE_BLOCKED_ACTIVATIONS = True
 
 # The GELU + requantization epilogue reads the next layer's LoRA-down weight through a copy in the order its matrix
@@ -72,14 +72,14 @@ def working_copy(wgt: torch.Tensor, wscales: torch.Tensor) -> torch.Tensor | Non
     return planes
 
 
-def takes_blocked_activations(wgt: torch.Tensor, wscales: torch.Tensor, rows: int, requantized: bool = False) -> int:
+def takes_blocked_activations(wgt: torch.Tensor, wscales: torch.Tensor, rows: int) -> int:
     """How a GEMM on this weight should be fed its activations: 0 = the (M, K/2) matrix, 1 = its bytes in the fp8 main
-    loop's own order, 2 (``ACT_CODES_F6``) = fp6 codes in that order -- the value for ``out_blocked`` / ``act_blocked``.
-    Non-zero when the switch is on, the weight has a working copy and the (padded) row count is a multiple of 32;
-    ``requantized``: the activations come out of a requantizing GEMM epilogue (which writes bytes), not the quantizer."""
+    loop's own order, 2 (``ACT_CODES_F6``) = fp6 codes in that order -- the value for ``out_blocked`` / ``qout_blocked`` of
+    the producer and ``act_blocked`` of this GEMM.  Non-zero when the switch is on, the weight has a working copy and the
+    (padded) row count is a multiple of 32."""
     if not USE_BLOCKED_ACTIVATIONS or rows % 32 or working_copy(wgt, wscales) is None:
         return 0
-    return ACT_CODES_F6 if USE_BLOCKED_ACTIVATIONS is True and not requantized else 1
+    return ACT_CODES_F6 if USE_BLOCKED_ACTIVATIONS is True else 1
 
 
 HEAD_DIM = 128
@@ -118,7 +118,7 @@ def svdq_gemm_w4a4_cuda(
     attn_tokens: int = 0,
     fuse_swiglu: bool = False,
     act_blocked: bool | int = False,
-    qout_blocked: bool = False,
+    qout_blocked: bool | int = False,
 ):
     """
     ``out = deq(act) @ deq(wgt).T + lora_act_in @ lora_up.T + bias`` on packed int4 operands with per-group-64 scales,
@@ -134,7 +134,8 @@ def svdq_gemm_w4a4_cuda(
       ``qout`` that way for the GEMM that consumes it.  Needs a weight with a working copy (see ``USE_WEIGHT_PLANES``).
       ``act_blocked=2`` (``ACT_CODES_F6``): ``act`` is ``(rows, 3K/4)`` bytes of fp6 codes in lane order, as the quantizer
       writes them with ``out_blocked=2``: the matrix instruction takes them as they are (no offset term for signed
-      activations, fp6 x fp6); ``act_unsigned`` is then not looked at.
+      activations, fp6 x fp6); ``act_unsigned`` is then not looked at.  ``qout_blocked=2``: the requantizing epilogue writes
+      ``qout`` as ``(rows, 3NQ/4)`` bytes of such codes.
 
     Raises ``NotImplementedError`` for the arguments the reference's ROCm backend rejects as well (``poolout``,
     ``out_vk``, ``out_linearattn``, ``out_q/k/v``) and for the NVFP4-only ones (``fp4``, ``wcscales``, ``alpha != 1``,
@@ -283,7 +284,8 @@ def svdq_gemm_w4a4_cuda(
     elif want_quant:
         NQ = N // 2 if fuse_swiglu else N
         qout2d = qout.reshape(-1, qout.shape[-1])
-        if qout2d.element_size() != 1 or qout2d.shape[0] < M or qout2d.shape[1] != NQ // 2 or qout2d.stride(1) != 1:
+        qb = NQ * 3 // 4 if int(qout_blocked) == ACT_CODES_F6 else NQ // 2  # bytes of codes per row
+        if qout2d.element_size() != 1 or qout2d.shape[0] < M or qout2d.shape[1] != qb or qout2d.stride(1) != 1:
             raise ValueError(f"qout shape/dtype {tuple(qout.shape)} {qout.dtype}")
         if oscales.dtype != T or oscales.dim() != 2 or oscales.shape[0] != NQ // 64 or oscales.shape[1] < M or oscales.stride(1) != 1:
             raise ValueError(f"oscales shape {tuple(oscales.shape)}")
@@ -316,7 +318,7 @@ def svdq_gemm_w4a4_cuda(
         if qout_blocked:
             if not qout2d.is_contiguous() or qout2d.shape[0] % 32 or qout2d.data_ptr() % 16:
                 raise ValueError("qout_blocked needs a contiguous qout with a multiple of 32 rows")
-            args.qout_blocked = 1
+            args.qout_blocked = int(qout_blocked)
         args.shift = 0.0 if fuse_swiglu else GELU_SHIFT
 
     with torch.cuda.device(dev):

@@ -242,16 +242,21 @@ def test_requantizing_epilogues_write_either_order(dev, swiglu):
              bias=torch.randn(N, generator=g).to(dtype), smooth_factor=(torch.rand(NQ, generator=g) + 0.5).to(dtype),
              lora_down=(torch.randn(NQ, R2, generator=g) * 0.1).to(dtype))  # fmt: skip
     t = {k: v.to(dev) for k, v in t.items()}
+    from nunchaku_rocm_amd.layout import unblock_activations_f6
+
     res = []
-    for blocked in (False, True):
-        qout = torch.full((M, NQ // 2), 0xEE, dtype=torch.uint8, device=dev)
+    for blocked in (False, True, 2):
+        qout = torch.full((M, NQ * 3 // 4 if blocked == 2 else NQ // 2), 0xEE, dtype=torch.uint8, device=dev)
         osc = torch.zeros(NQ // 64, M, dtype=dtype, device=dev)
         lao = torch.zeros(M, R2, dtype=torch.float32, device=dev)
         ops.svdq_gemm_w4a4_cuda(qout=qout, oscales=osc, lora_act_out=lao, fuse_swiglu=swiglu, qout_blocked=blocked, **t)
         torch.cuda.synchronize()
-        res.append((unblock_activations(qout.cpu()) if blocked else qout.cpu(), osc.cpu().view(torch.int16), lao.cpu()))
-    for a, b in zip(*res):
-        assert torch.equal(a, b)
+        # the GELU epilogue's codes are unsigned, the SwiGLU epilogue's signed
+        codes = unblock_activations_f6(qout.cpu(), not swiglu) if blocked == 2 else unblock_activations(qout.cpu()) if blocked else qout.cpu()
+        res.append((codes, osc.cpu().view(torch.int16), lao.cpu()))
+    for other in res[1:]:
+        for a, b in zip(res[0], other):
+            assert torch.equal(a, b)
     assert (res[0][0] != 0xEE).any()
 
 
@@ -278,8 +283,7 @@ def test_modules_compute_the_same_bits_either_way(dev, dtype):
         for flag in (True, 1, False):
             gemm_mod.USE_BLOCKED_ACTIVATIONS = flag
             try:
-                assert fc1.takes_blocked(S) == (2 if flag is True else int(flag))
-                assert fc2.takes_blocked(S, requantized=True) == int(bool(flag))
+                assert fc1.takes_blocked(S) == fc2.takes_blocked(S) == (2 if flag is True else int(flag))
                 outs.append([fc1(x).clone(), ops.fused_gelu_mlp(x, fc1, fc2).clone(), ops.fused_qkv_norm_rottary(x, qkv, nq, nk, rot).clone(),
                              ops.fused_swiglu_mlp(x, g1, g2).clone()])  # fmt: skip
             finally:
