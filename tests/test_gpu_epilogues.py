@@ -180,16 +180,23 @@ def test_fused_ops_on_flux_block_shapes(dev):
     assert err <= TOL
 
 
+@pytest.mark.parametrize("handover", [0, 2], ids=["matrix", "fp6-codes"])
 @pytest.mark.parametrize("zero_mean_weights", [False, True])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_fc1_codes_at_the_flux_size(dev, dtype, zero_mean_weights, main_loop):
+def test_fc1_codes_at_the_flux_size(dev, dtype, zero_mean_weights, main_loop, handover):
     """FLUX.1 fc1 (M = 4608, K = 3072, N = 12288) with GELU + requantization: the int4 codes and scales it hands to fc2,
     as codes, on 192 sampled rows (2.4 M codes, 37 K scales) against the oracle, held to the reference's bar for both
     main loops, both 16-bit types and both weight distributions (codes uniform in [-8, 7], mean -0.5, as the benchmark
     draws them, and codes of zero mean as absmax-quantized checkpoints have).  The fp8 main loop offsets signed
     activations; the offset term it adds per group has no systematic part (a + 8 against the even-k weights, a - 7 against
-    the odd-k ones) and is taken out every four stages, so its accumulators stay near the true partial sums."""
+    the odd-k ones) and is taken out every four stages, so its accumulators stay near the true partial sums.
+    ``handover`` 2: activations in and out as fp6 codes in lane order, as the modules pass them (fp8 loop only; there
+    is then no offset at all)."""
     from nunchaku_rocm_amd import ops
+    from nunchaku_rocm_amd.layout import unblock_activations_f6
+
+    if handover and main_loop != "all":
+        return  # the int8 main loop reads the (M, K/2) matrix only (its refusal: test_gpu_gemm.py, test_gpu_blocked.py)
 
     M, C, H4 = 4608, 3072, 12288
     l1 = O.make_svdq_linear(C, H4, seed=42, dtype=dtype)
@@ -200,21 +207,23 @@ def test_fc1_codes_at_the_flux_size(dev, dtype, zero_mean_weights, main_loop):
     x = O.make_activations(M, C, seed=41).to(dtype)
     d1 = {k: v.to(dev) for k, v in l1.items()}
     d2 = {k: v.to(dev) for k, v in l2.items()}
-    q1, a1, la1 = ops.svdq_quantize_w4a4_act_fuse_lora_cuda(x.to(dev), lora_down=d1["proj_down"], smooth=d1["smooth_factor"])
-    qo = torch.zeros(M, H4 // 2, dtype=torch.uint8, device=dev)
+    q1, a1, la1 = ops.svdq_quantize_w4a4_act_fuse_lora_cuda(x.to(dev), lora_down=d1["proj_down"], smooth=d1["smooth_factor"], out_blocked=handover)
+    qo = torch.zeros(M, H4 * 3 // 4 if handover else H4 // 2, dtype=torch.uint8, device=dev)
     oo = torch.zeros(H4 // 64, M, dtype=dtype, device=dev)
     lo = torch.zeros(M, 32, dtype=torch.float32, device=dev)
     ops.svdq_gemm_w4a4_cuda(act=q1, wgt=d1["qweight"], qout=qo, ascales=a1, wscales=d1["wscales"], oscales=oo,
                             lora_act_in=la1, lora_up=d1["proj_up"], lora_down=d2["proj_down"], lora_act_out=lo,
-                            bias=d1["bias"], smooth_factor=d2["smooth_factor"])  # fmt: skip
+                            bias=d1["bias"], smooth_factor=d2["smooth_factor"], act_blocked=handover, qout_blocked=handover)  # fmt: skip
     torch.cuda.synchronize()
     rows = torch.randperm(M, generator=torch.Generator().manual_seed(5))[:192].sort().values
     rp, rs, rl, _ = O.quantize_act(x[rows], l1["proj_down"], l1["smooth_factor"])
-    assert torch.equal(q1[rows].cpu(), rp)
+    q1m = unblock_activations_f6(q1.cpu()) if handover else q1.cpu()
+    qom = unblock_activations_f6(qo.cpu(), True) if handover else qo.cpu()
+    assert torch.equal(q1m[rows], rp)
     h = O.gemm_w4a4(rp, l1["qweight"], rs, l1["wscales"], l1["bias"], rl, l1["proj_up"])
     hp, hs, hl, hc = O.gelu_quant(h, l2["smooth_factor"], l2["proj_down"], dtype)
-    assert_requantized_like_the_reference(O.unpack_int4(qo[rows].cpu(), False), hc, oo[:, rows].cpu(), hs, dtype,
-                                          what=f"fc1 {main_loop} {dtype} zero-mean={zero_mean_weights}: ")
+    assert_requantized_like_the_reference(O.unpack_int4(qom[rows], False), hc, oo[:, rows].cpu(), hs, dtype,
+                                          what=f"fc1 {main_loop} {dtype} zero-mean={zero_mean_weights} handover={handover}: ")
     assert (lo[rows].cpu() - hl).abs().max() <= TOL * hl.abs().max()
 
 

@@ -46,7 +46,7 @@ def _gpu_gemm(p, dev, actual_m=None, unsigned=False, dtype=torch.bfloat16, canar
     M, N = p["act"].shape[0], p["wgt"].shape[0]
     am = M if actual_m is None else actual_m
     buf = torch.full((am + canary, N), float("nan"), dtype=dtype, device=dev)
-    d = lambda t: None if t is None else t.to(dev)  # noqa: E731
+    d = lambda t: t.to(dev) if isinstance(t, torch.Tensor) else t  # noqa: E731
     ops.svdq_gemm_w4a4_cuda(
         act=d(p["act"]), wgt=d(p["wgt"]), out=buf[:am], ascales=d(p["asc"]), wscales=d(p["wsc"]), bias=d(p.get("bias")),
         lora_act_in=d(p.get("la")), lora_up=d(p.get("lu")), act_unsigned=unsigned, **{k: d(v) for k, v in extra.items()},
@@ -99,6 +99,66 @@ def test_scaled_gemm_bias_lora(dev, M, N, K, R, actual_m, unsigned, dtype):
     assert ((out.float() - ref).abs() <= ref.abs() * ulp * 1.01 + 1e-3 * ref.abs().max()).all()
     out2 = _gpu_gemm(p, dev, actual_m=actual_m, unsigned=unsigned, dtype=dtype)
     assert torch.equal(out.view(torch.int16), out2.view(torch.int16))
+
+
+def _as_fp6_codes(p, unsigned):
+    """The problem with its activations as fp6 codes in lane order (rows padded with zero codes to a multiple of 32;
+    the padded rows' scales and LoRA activations are never used: the output has the original row count)."""
+    from nunchaku_rocm_amd.layout import block_activations_f6
+
+    M = p["act"].shape[0]
+    Mp = (M + 31) // 32 * 32
+    q = dict(p)
+    act = torch.zeros(Mp, p["act"].shape[1], dtype=torch.uint8)
+    act[:M] = p["act"]
+    q["act"] = block_activations_f6(act, unsigned)
+    q["asc"] = torch.nn.functional.pad(p["asc"], (0, Mp - M))
+    if p.get("la") is not None:
+        q["la"] = torch.nn.functional.pad(p["la"], (0, 0, 0, Mp - M))
+    return q
+
+
+@pytest.mark.parametrize("unsigned", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,N,K,R,actual_m", [(136, 264, 256, 16, 130), (256, 256, 512, 32, 256), (64, 128, 1024, 48, 64), (128, 512, 256, 0, 100),
+                                                   (72, 136, 512, 288, 72), (136, 264, 64, 16, 136), (130, 200, 192, 32, 130), (256, 128, 448, 0, 200)])
+def test_scaled_gemm_from_fp6_codes(dev, M, N, K, R, actual_m, unsigned, dtype, main_loop):
+    """The same bar with the activations handed over as fp6 codes in lane order (act_blocked = 2; fp8 main loop only)."""
+    print(f"case M={M} N={N} K={K} R={R} actual_m={actual_m} unsigned={unsigned} {dtype}", flush=True)
+    p = _rand_problem(M, N, K, R, dtype, seed=K + R)
+    if main_loop != "all":  # the int8 main loop reads the (M, K/2) matrix only: the operator must refuse
+        with pytest.raises(ValueError):
+            _gpu_gemm(_as_fp6_codes(p, unsigned), dev, actual_m=actual_m, unsigned=unsigned, dtype=dtype, act_blocked=2)
+        return
+    out = _gpu_gemm(_as_fp6_codes(p, unsigned), dev, actual_m=actual_m, unsigned=unsigned, dtype=dtype, act_blocked=2)
+    ref = O.gemm_w4a4(p["act"], p["wgt"], p["asc"], p["wsc"], p["bias"], p["la"], p["lu"], unsigned)[:actual_m]
+    assert O.max_rel_err(out, ref) <= TOL
+    ulp = 2**-7 if dtype == torch.bfloat16 else 2**-10
+    assert ((out.float() - ref).abs() <= ref.abs() * ulp * 1.01 + 1e-3 * ref.abs().max()).all()
+
+
+@pytest.mark.parametrize("unsigned", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_scale_products_from_fp6_codes_are_exact(dev, dtype, unsigned, main_loop):
+    """One group, extreme scales: with fp6 activation codes the signed product has no offset term either, so signed and
+    unsigned outputs are the oracle's fp32 product p * (as * ws) rounded once, bit for bit."""
+    if main_loop != "all":
+        return  # the refusal of the int8 main loop is checked in test_scaled_gemm_from_fp6_codes
+    M, N, K = 64, 128, 64
+    p = _rand_problem(M, N, K, 0, dtype, seed=5)
+    p["bias"] = None
+    if dtype == torch.float16:  # weight scales a working copy exists for (its 16-bit offset terms overflow at about 17)
+        asc = torch.tensor([2.0**-14, 3 * 2.0**-14, 1023 * 2.0**-14, 2.0**-4, 2.0**-5, 0.0, 2.0**-2, 2.0**-10], dtype=torch.float32)
+        wsc = torch.tensor([1.0, 1.5, 2.0, 4.0, 2.5, 16.0, 0.0, 2054.0 / 1024], dtype=torch.float32)
+    else:
+        asc = torch.tensor([2.0**-60, 1.5 * 2.0**-40, 2.0**-14, 1.0, 2.0**20, 0.0, 255 * 2.0**-30, 2.0**-50], dtype=torch.float32)
+        wsc = torch.tensor([1.0, 2.0**30, 2.0**-20, 1.9921875, 2.0**-30, 2.0**40, 0.0, 2.0**-55], dtype=torch.float32)
+    p["asc"] = asc.repeat(M // 8).reshape(1, M).to(dtype)
+    p["wsc"] = wsc.repeat_interleave(N // 8).reshape(1, N).to(dtype)
+    out = _gpu_gemm(_as_fp6_codes(p, unsigned), dev, unsigned=unsigned, dtype=dtype, act_blocked=2)
+    ref = O.gemm_w4a4(p["act"], p["wgt"], p["asc"], p["wsc"], act_unsigned=unsigned).to(dtype)
+    assert torch.isfinite(ref.float()).all() and (ref != 0).any()
+    assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
