@@ -81,11 +81,18 @@ typedef struct {
     const void *norm_shift;        /* (batches, K) T, same strides                                           */
     int32_t norm_rows_per_batch;   /* rows m sharing one scale / shift vector (multiple of 16); 0 = all rows */
     int32_t norm_ld, norm_stride;  /* in elements (the adaLN projection interleaves its six vectors: stride 6) */
-    /* non-zero: `out` is written in the lane order of the GEMM's fp8 main loop instead of as the (M, K / 2) matrix:  */
-    /* the 32 packed bytes of (row m, group g) go to out + ((m / 32) * (K / 64) + g) * 1024 + (32 * h + m % 32) * 16,  */
-    /* h = 0 / 1 for bytes 0-15 / 16-31 (ld_out is not used; `out` must hold ceil(M / 32) * 32 rows' worth).  The GEMM */
-    /* then takes it with svdq_gemm_args.act_blocked: each of its load instructions reads 1 KB in a row instead of     */
-    /* 16-byte pieces of 32 rows (about 3 % of a launch).  No counterpart in the reference.                            */
+    /* How `out` is written (no counterpart in the reference; 1 and 2 need `out` 16-byte aligned and holding            */
+    /* ceil(M / 32) * 32 rows' worth, ld_out is then not used):                                                         */
+    /*   0  the (M, K / 2) matrix of packed int4 codes;                                                                 */
+    /*   1  the same bytes in the lane order of the GEMM's fp8 main loop: the 32 packed bytes of (row m, group g) go to  */
+    /*      out + ((m / 32) * (K / 64) + g) * 1024 + (32 * h + m % 32) * 16, h = 0 / 1 for bytes 0-15 / 16-31; the GEMM  */
+    /*      takes it with svdq_gemm_args.act_blocked = 1 and reads 1 KB per load instruction instead of 16-byte pieces   */
+    /*      of 32 rows (about 3 % of a launch);                                                                          */
+    /*   2  the same integers as fp6 (e2m3) codes, sign << 5 | magnitude, in that lane order: 48 bytes per row and group. */
+    /*      Of (row m, group g), lane 32 h + m % 32 owns the values k = 2 p + h (p = 0 .. 31), code p in bits 6 p .. 6 p + 5 */
+    /*      of 24 bytes; their first 16 lie at out + ((m / 32) * (K / 64) + g) * 1536 + 16 * lane, their last 8 at          */
+    /*      ... + 1024 + 8 * lane.  The GEMM takes it with act_blocked = 2: the matrix instruction reads the codes as they  */
+    /*      are (fp6 x fp6, no nibble unpack, no offset term for signed activations; about 8 % of a launch).               */
     int32_t out_blocked;
 } svdq_quantize_args;
 
@@ -161,11 +168,11 @@ typedef struct {
     /* SVDQ_EPI_GELU_QUANT, optional: `lora_down_t` re-laid-out by svdq_block_lora_down (the epilogue then reads each of */
     /* its LoRA-down operands as 1 KB in a row instead of 8-byte pieces of 32 rows); NULL = not given                   */
     const void *lora_down_blocked;
-    /* non-zero: `act` is not the (M, K / 2) matrix but the same bytes in the fp8 main loop's lane order, as the        */
-    /* quantizer writes them with out_blocked (pre-split weights only)                                                  */
+    /* 1 / 2: `act` is not the (M, K / 2) matrix but what the quantizer writes with out_blocked = 1 / 2 (its bytes, or   */
+    /* fp6 codes, in the fp8 main loop's lane order; pre-split weights only; with 2 act_unsigned is not looked at)      */
     int32_t act_blocked;    /* (`act` must then hold ceil(M / 32) * 32 rows' worth, 16-byte aligned; ld_act unused) */
-    /* non-zero: the requantizing epilogues write `qout` in that same lane order, for the GEMM that consumes it        */
-    /* (ld_qout unused; `qout` must hold ceil(M / 32) * 32 rows' worth)                                                 */
+    /* 1 / 2: the requantizing epilogues write `qout` that way, for the GEMM that consumes it (ld_qout unused; `qout`   */
+    /* must hold ceil(M / 32) * 32 rows' worth: NQ / 2 bytes a row, 3 NQ / 4 with 2)                                    */
     int32_t qout_blocked;
 } svdq_gemm_args;
 
