@@ -35,7 +35,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # in profiles/bench_all_kernels_hbm_traffic.txt, the factors being what the same counters read on plain copy kernels of
 # known size in the same run (FETCH_SIZE reads half the bytes of 16-byte-per-lane loads); counters cannot be read from
 # inside this process
-GEMM_QKV_HBM_BYTES = (2.0 * 78599.6 + 82944.0) * 1024
+GEMM_QKV_HBM_BYTES = (2.0 * 102484.5 + 82944.0) * 1024
 
 
 def _events(n):
@@ -150,9 +150,13 @@ def main():
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
     # torch loads a kernel's code object at that kernel's first launch.  Under rocprofv3's counter collection such a first
-    # launch late in the run (torch.arange in the model set-up, 12 GB already allocated) has crashed the profiler on some
-    # boxes; launched once here, while the device is empty, it does not.
-    torch.arange(4, device=dev).sum().item()
+    # launch late in the run (the small index and table kernels of the model set-up, 12 GB already allocated) has crashed
+    # the profiler on some boxes; launched once here, while the device is empty, it does not.
+    if not args.no_extras:
+        from nunchaku_rocm_amd.flux_shaped import FluxShapedConfig, flux_ids, rope_table
+
+        torch.arange(4, device=dev).sum().item()
+        rope_table(flux_ids(8, 2, 2, device=dev), FluxShapedConfig().axes_dim, FluxShapedConfig().theta).sum().item()
     M, K, N, R = 4608, 3072, 9216, 32
     # weights as module parameters, which is what the operators see in a model (the GEMM keeps its re-laid-out working
     # copy per parameter)
