@@ -173,6 +173,15 @@ __device__ inline v2i g_load64(__amdgpu_buffer_rsrc_t r, uint32_t lane_off, uint
     return __builtin_bit_cast(v2i, __builtin_amdgcn_raw_buffer_load_b64(r, (int)lane_off, (int)uniform_off, 0));
 }
 
+// Block loads global -> LDS through a raw buffer: the 64 lanes' 16 (or 12) bytes at base + lane offset + scalar offset land at
+// lds + 16 * lane; base and scalar offset live in SGPRs, so the loop's block loads need no vector address arithmetic.
+__device__ inline void g_load16_lds(__amdgpu_buffer_rsrc_t r, uint8_t *lds, uint32_t lane_off, uint32_t uniform_off) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (SVDQ_AS3 void *)lds, 16, (int)lane_off, (int)uniform_off, 0, 0);
+}
+__device__ inline void g_load12_lds(__amdgpu_buffer_rsrc_t r, uint8_t *lds, uint32_t lane_off, uint32_t uniform_off) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (SVDQ_AS3 void *)lds, 12, (int)lane_off, (int)uniform_off, 0, 0);
+}
+
 __device__ inline v16i magic_acc() {
     v16i c;
 #pragma unroll
@@ -940,17 +949,16 @@ __global__ __launch_bounds__(NTHREADS, PIPE ? 2 : 3) void gemm_w4a4_f8_kernel(sv
     const int nblk = min(n0 / 32 + wm, (a.N + 31) / 32 - 1);
     const uint8_t *wbase = (const uint8_t *)a.wgt_planes + (size_t)nblk * nstages * (WPL_BLOCKS * BLK_BYTES);
     const uint8_t *xbase = (const uint8_t *)a.wgt_planes + planes_code_bytes(a.N, a.K) + (size_t)nblk * (nstages + 1) * AUX_BLK;
+    const __amdgpu_buffer_rsrc_t rW = g_buffer(wbase), rX = g_buffer(xbase);
     auto dma = [&](int s, uint8_t *dstbuf, int slot, int i) {  // i = 0, 1, 2: code blocks of stage s; i = 3: its scales and offset terms
         if (i < WPL_BLOCKS) {
-            const uint8_t *src = wbase + i * BLK_BYTES + ((uint32_t)lane * 16u + (uint32_t)s * (uint32_t)(WPL_BLOCKS * BLK_BYTES));
-            __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)src, (SVDQ_AS3 void *)(dstbuf + (wm * WPL_BLOCKS + i) * BLK_BYTES), 16, 0, 0);
+            g_load16_lds(rW, dstbuf + (wm * WPL_BLOCKS + i) * BLK_BYTES, (uint32_t)lane * 16u,
+                         (uint32_t)s * (uint32_t)(WPL_BLOCKS * BLK_BYTES) + (uint32_t)(i * BLK_BYTES));
         } else {
             // 64 lanes x 12 bytes = the rows of stage s and of stage s + 1 (the copy has one stage of padding), into the given
             // ring slot and the one after it: issued before the loop for stages 0 and 1 and then by every odd stage for the two
             // stages after it (an even slot and its neighbour)
-            const uint8_t *src = xbase + ((uint32_t)lane * (uint32_t)AUX_ROW + (uint32_t)s * (uint32_t)AUX_BLK);
-            __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)src,
-                                             (SVDQ_AS3 void *)(sring + wm * AUX_NBLK_BYTES + slot * AUX_LBLK), 12, 0, 0);
+            g_load12_lds(rX, sring + wm * AUX_NBLK_BYTES + slot * AUX_LBLK, (uint32_t)lane * (uint32_t)AUX_ROW, (uint32_t)s * (uint32_t)AUX_BLK);
         }
     };
     // registers: the 16 packed bytes of the lane's activation row (row wm * 32 + l32, K half lane / 32) of both groups,
