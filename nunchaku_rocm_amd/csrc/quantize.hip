@@ -15,6 +15,8 @@
 // is conflict free.  Lane (m = lane % 16, q = lane / 16) then owns the 16 consecutive channels [64 g + 16 q, +16)
 // of row m: a group's absmax needs two cross-lane steps, and the lane's two 16-byte halves are exactly the B operands
 // of two 16x16x32 MFMAs whose A operands come from the LoRA-down tile.
+#include <algorithm>
+
 #include "svdq_common.h"
 
 // the codes and scales are a bit-exact contract: no multiply-add contraction anywhere in this file
@@ -70,7 +72,14 @@ __global__ __launch_bounds__(Q_WAVES * 64, QR == 32 ? 1 : (NORM ? 4 : 2)) void q
     const int kq = lane >> 4;
     const int m0 = blockIdx.x * QR;
     const int ngroups = a.K / GROUP;
-    const int nmy = (ngroups - wave + Q_WAVES - 1) / Q_WAVES;  // groups g = wave + Q_WAVES * i
+    // The grid's second axis: nq >= 0 workgroup rows that only quantize, each its own slice of the groups (a shorter chain
+    // of group steps per wavefront where CUs would otherwise idle), then one row per chunk of 32 ranks.
+    const int rchunks = (a.R + Q_RCHUNK - 1) / Q_RCHUNK;
+    const int nq = HAS_LORA ? max((int)gridDim.y - rchunks, 0) : 0;
+    const bool qonly = (int)blockIdx.y < nq;
+    const int g_lo = qonly ? (ngroups * (int)blockIdx.y) / nq : 0, g_hi = qonly ? (ngroups * ((int)blockIdx.y + 1)) / nq : ngroups;
+    const int gw = g_lo + wave;  // this wavefront's groups: gw + Q_WAVES * i < g_hi
+    const int nmy = max((g_hi - gw + Q_WAVES - 1) / Q_WAVES, 0);
     // Block loads: lane l of load i fetches chunk (l % 8) ^ (l / 8) of tile row 8 i + l / 8 into LDS slot l of that
     // load's 1 KB, i.e. tile[row][chunk ^ (row & 7)].  Rows >= M re-read row M - 1 and ranks >= R rank R - 1 (valid
     // memory; nothing is stored for them).  Addresses = uniform base + 32-bit lane offset (+ uniform group step).
@@ -83,9 +92,9 @@ __global__ __launch_bounds__(Q_WAVES * 64, QR == 32 ? 1 : (NORM ? 4 : 2)) void q
     const int rd_lo = ml * Q_ROW_BYTES + (((2 * kq) ^ (ml & 7)) * 16), rd_hi = ml * Q_ROW_BYTES + (((2 * kq + 1) ^ (ml & 7)) * 16);
     uint8_t *const wbase = smem + wave * WAVE_BYTES;
     const uint16_t *__restrict__ smooth = (const uint16_t *)a.smooth;
-    uint8_t *__restrict__ outbase = (uint8_t *)a.out + (size_t)m0 * a.ld_out + wave * (GROUP / 2);
+    uint8_t *__restrict__ outbase = (uint8_t *)a.out + (size_t)m0 * a.ld_out + gw * (GROUP / 2);
     const uint32_t outoff = (uint32_t)ml * a.ld_out + kq * 8;
-    uint16_t *__restrict__ scales = (uint16_t *)a.scales + (size_t)wave * a.ld_scales + m0;
+    uint16_t *__restrict__ scales = (uint16_t *)a.scales + (size_t)gw * a.ld_scales + m0;
     // out_blocked: the 32 packed bytes of (row, group) go where the GEMM's lane (row % 32, half) of that 32-row block and
     // group finds them, [32-row block][group][64 lanes x 16 bytes]: this lane's 8 bytes are half kq / 2, offset 8 (kq % 2)
     uint8_t *__restrict__ bout[NH];
@@ -134,9 +143,9 @@ __global__ __launch_bounds__(Q_WAVES * 64, QR == 32 ? 1 : (NORM ? 4 : 2)) void q
     // With one more workgroup row than rank chunks, row 0 only quantizes and rows 1 .. project (the two kinds of work
     // then run side by side on different CUs instead of one after the other in every wavefront).
     {
-        const bool split = HAS_LORA && (int)gridDim.y > (a.R + Q_RCHUNK - 1) / Q_RCHUNK;
-        const int rc = split ? max((int)blockIdx.y - 1, 0) : (int)blockIdx.y;
-        const bool do_lora = HAS_LORA && !(split && blockIdx.y == 0);
+        const bool split = nq > 0;
+        const int rc = max((int)blockIdx.y - nq, 0);
+        const bool do_lora = HAS_LORA && !qonly;
         v4f acc0[NH], acc1[NH];
 #pragma unroll
         for (int h = 0; h < NH; h++) acc0[h] = acc1[h] = (v4f){0.f, 0.f, 0.f, 0.f};
@@ -148,11 +157,11 @@ __global__ __launch_bounds__(Q_WAVES * 64, QR == 32 ? 1 : (NORM ? 4 : 2)) void q
             for (int i = 0; i < 4; i++)
                 ldma[i] = (uint32_t)min(rc * Q_RCHUNK + 8 * i + drow, a.R - 1) * a.K * 2 + dchunk * 16;
         }
-        const bool do_quant = split ? blockIdx.y == 0 : rc == 0;
+        const bool do_quant = split ? qonly : rc == 0;
 
         constexpr int NX = (GLU ? 4 : 2) * NH;  // block loads of one activation stage
         auto group_off = [&](int i) {  // byte offset of group wave + Q_WAVES * i in a row; past the end: the last group
-            return (uint32_t)min(wave + Q_WAVES * i, ngroups - 1) * (GROUP * 2);
+            return (uint32_t)min(gw + Q_WAVES * i, ngroups - 1) * (GROUP * 2);
         };
         auto issue_x = [&](int i, QVecs &qv) {
             const uint32_t k0 = group_off(i);
@@ -334,7 +343,7 @@ __global__ __launch_bounds__(Q_WAVES * 64, QR == 32 ? 1 : (NORM ? 4 : 2)) void q
                 }
                 if (row_ok) {
                     if (kq == 0) (scales + (size_t)i * Q_WAVES * a.ld_scales)[Q_ROWS * h + ml] = T::from_f32(scale);
-                    uint8_t *blk = f6base + (size_t)(wave + Q_WAVES * i) * 1536;
+                    uint8_t *blk = f6base + (size_t)(gw + Q_WAVES * i) * 1536;
 #pragma unroll
                     for (int e = 0; e < 2; e++) {
                         const uint32_t d32 = (kq & 1) ? __builtin_amdgcn_alignbit(phi[e], plo[e], 16) : plo[e];
@@ -363,7 +372,7 @@ __global__ __launch_bounds__(Q_WAVES * 64, QR == 32 ? 1 : (NORM ? 4 : 2)) void q
             }
             if (row_ok) {
                 if (kq == 0) (scales + (size_t)i * Q_WAVES * a.ld_scales)[Q_ROWS * h + ml] = T::from_f32(scale);
-                uint8_t *dst = a.out_blocked ? bout[h] + (size_t)(wave + Q_WAVES * i) * 1024
+                uint8_t *dst = a.out_blocked ? bout[h] + (size_t)(gw + Q_WAVES * i) * 1024
                                              : outbase + (size_t)i * (GSTEP / 2) + (uint32_t)(Q_ROWS * h) * a.ld_out + outoff;
                 *(uint2 *)dst = make_uint2(w0, w1);
             }
@@ -605,18 +614,23 @@ static int device_cus() {
     return cus;
 }
 
-// Second grid axis: one workgroup row per chunk of 32 ranks, plus one that only quantizes where that still leaves about
+// Second grid axis: one workgroup row per chunk of 32 ranks, plus rows that only quantize where that still leaves about
 // one workgroup per CU: quantizing and projecting then run side by side on different CUs (K = 3072, R = 32: 6.4
 // against 7.9 us at M = 512, 7.1 against 8.5 at 2048, 12.3 against 13.4 at 4608 with 32-row workgroups; slower once the
-// CUs are taken: 9.9 against 9.5 us at M = 4096, 17.2 against 14.5 at 6144).
+// CUs are taken: 9.9 against 9.5 us at M = 4096, 17.2 against 14.5 at 6144).  While CUs are left over, up to three such
+// rows share the groups between them: a wavefront's chain of group steps gets shorter (M = 1024: 7.8 -> 5.1 us with
+// three, M = 512: 7.6 -> 4.9; slower again beyond one workgroup per CU: M = 1024 with four 6.4 us, M = 4608 with two
+// 14.2 against 12.8).
 static int quantize_grid_y(const svdq_quantize_args &a, int row_blocks, int rows) {
     if (a.R == 0) return 1;
     const int chunks = (a.R + Q_RCHUNK - 1) / Q_RCHUNK, cus = device_cus();
     // (with a prologue the workgroups that only project compute it a second time: only where half the CUs would idle
     // anyway; norm prologue, M = 512: 10.4 against 11.8 us, M = 4608: 25.5 against 20.7)
     const bool prologue = a.norm_stats || a.prologue != SVDQ_PRE_NONE;
-    const bool split = row_blocks * (chunks + 1) <= (prologue ? cus / 2 : cus + (rows == 32 ? cus / 8 : 0));
-    return chunks + (split ? 1 : 0);
+    const int limit = prologue ? cus / 2 : cus + (rows == 32 ? cus / 8 : 0);
+    if (row_blocks * (chunks + 1) > limit) return chunks;
+    const int nq = std::min({3, limit / row_blocks - chunks, a.K / GROUP});
+    return chunks + std::max(nq, 1);
 }
 
 template <typename T, bool U, int G, bool NORM>

@@ -62,6 +62,22 @@ def test_every_grid_layout_bit_exact(dev, M):
     assert (la[:M].double() - ref64).abs().max() <= 2e-5 * ref64.abs().max()
 
 
+@pytest.mark.parametrize("M,K", [(512, 3072), (1024, 3072), (96, 320), (48, 704), (2048, 192)])
+def test_quantize_only_rows_share_the_groups(dev, M, K):
+    """Where CUs are left over the launcher adds up to three workgroup rows that only quantize, each a slice of the
+    groups (quantize_grid_y): group counts that do and do not divide by the number of slices, fewer groups than
+    wavefronts in a slice, and the largest row count that still takes three slices on a 256-CU part."""
+    print(f"case M={M} K={K}", flush=True)
+    R = 32
+    x = O.make_activations(M, K, seed=M + K, dtype=torch.bfloat16)
+    lin = O.make_svdq_linear(K, 64, R=R, seed=K)
+    (out, osc, la), (rp, rs, rl, _) = _run(x, lin, dev, R)
+    assert torch.equal(out[:M], rp)
+    assert torch.equal(osc[:, :M].view(torch.int16), rs.view(torch.int16))
+    ref64 = x.double() @ lin["proj_down"][:, :R].double()
+    assert (la[:M].double() - ref64).abs().max() <= 2e-5 * ref64.abs().max()
+
+
 @pytest.mark.parametrize("smooth", [True, False])
 def test_unsigned_with_shift_bit_exact(dev, smooth):
     M, K = 96, 512
