@@ -168,15 +168,15 @@ def main():
     out = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
 
     # The two operator calls of SVDQW4A4Linear.forward, with the hand-over it uses: the quantizer writes the codes as fp6
-    # (sign | magnitude) in the order the GEMM's lanes read them (out_blocked = act_blocked = 2: the same integers, taken by
-    # the matrix instruction as they are; about 8 % of the GEMM launch).  The GEMM on the reference's (M, K/2) matrix is
+    # (sign | magnitude) in the order the GEMM's lanes read them, and the scales so that one load brings eight groups'
+    # (out_blocked = act_blocked = 3: the same integers and scales, the codes taken by the matrix instruction as they are).  The GEMM on the reference's (M, K/2) matrix is
     # timed next to it in the per-kernel table.
     def quant():
-        ops.svdq_quantize_w4a4_act_fuse_lora_cuda(x, qx, asc, lin["proj_down"], la, lin["smooth_factor"], out_blocked=2)
+        ops.svdq_quantize_w4a4_act_fuse_lora_cuda(x, qx, asc, lin["proj_down"], la, lin["smooth_factor"], out_blocked=3)
 
     def gemm():
         ops.svdq_gemm_w4a4_cuda(act=qx, wgt=lin["qweight"], out=out, ascales=asc, wscales=lin["wscales"],
-                                lora_act_in=la, lora_up=lin["proj_up"], bias=lin["bias"], act_blocked=2)  # fmt: skip
+                                lora_act_in=la, lora_up=lin["proj_up"], bias=lin["bias"], act_blocked=3)  # fmt: skip
 
     def step():
         quant()
@@ -251,10 +251,10 @@ def main():
                                                   "ms_act_as_matrix": round(n_ms, 5)}  # fmt: skip
         for Ms in (1024, 8192):
             xs = O.make_activations(Ms, K, seed=1).to(dev)
-            q2, a2, l2 = ops.svdq_quantize_w4a4_act_fuse_lora_cuda(xs, lora_down=lin["proj_down"], smooth=lin["smooth_factor"], out_blocked=2)
+            q2, a2, l2 = ops.svdq_quantize_w4a4_act_fuse_lora_cuda(xs, lora_down=lin["proj_down"], smooth=lin["smooth_factor"], out_blocked=3)
             o2 = torch.empty(Ms, N, dtype=torch.bfloat16, device=dev)
             ms = _time_kernel(lambda: ops.svdq_gemm_w4a4_cuda(act=q2, wgt=lin["qweight"], out=o2, ascales=a2, wscales=lin["wscales"],
-                                                              lora_act_in=l2, lora_up=lin["proj_up"], bias=lin["bias"], act_blocked=2))  # fmt: skip
+                                                              lora_act_in=l2, lora_up=lin["proj_up"], bias=lin["bias"], act_blocked=3))  # fmt: skip
             kernels[f"gemm_w4a4 M{Ms} K3072 N9216"] = {"ms": round(ms, 5), "TOP/s": round(2.0 * Ms * N * K / ms / 1e9, 1),
                                                        "frac_int8_mfma": round(2.0 * Ms * N * K / ms / 1e9 / INT8_MFMA_PEAK_TOPS, 4)}  # fmt: skip
             del xs, q2, a2, l2, o2
@@ -270,7 +270,7 @@ def main():
             return m
 
         fc1, fc2 = module(3072, 12288, 42), module(12288, 3072, 43, True)
-        q1, a1, l1 = fc1.quantize(x, blocked=2)
+        q1, a1, l1 = fc1.quantize(x, blocked=3)
         qo = torch.empty(M, 12288 * 3 // 4, dtype=torch.uint8, device=dev)  # fp6 codes in fc2's lane order
         oo = torch.empty(192, M, dtype=torch.bfloat16, device=dev)
         lo = torch.empty(M, 32, dtype=torch.float32, device=dev)
@@ -279,18 +279,18 @@ def main():
         def fc1_fused():
             ops.svdq_gemm_w4a4_cuda(act=q1, wgt=fc1.qweight, qout=qo, ascales=a1, wscales=fc1.wscales, oscales=oo, lora_act_in=l1,
                                     lora_up=fc1.proj_up, lora_down=fc2.proj_down, lora_act_out=lo, bias=fc1.bias,
-                                    smooth_factor=fc2.smooth_factor, act_blocked=2, qout_blocked=2)  # fmt: skip
+                                    smooth_factor=fc2.smooth_factor, act_blocked=3, qout_blocked=3)  # fmt: skip
 
         ms = _time_kernel(fc1_fused)
         f = 2.0 * M * 12288 * 3072
         kernels["gemm_w4a4+gelu+requant fc1 M4608 K3072 N12288"] = {"ms": round(ms, 5), "TOP/s": round(f / ms / 1e9, 1), "frac_int8_mfma": round(f / ms / 1e9 / INT8_MFMA_PEAK_TOPS, 4)}  # fmt: skip
-        ms = _time_kernel(lambda: fc2.forward_quant(qo, oo, lo, y2, act_blocked=2))
+        ms = _time_kernel(lambda: fc2.forward_quant(qo, oo, lo, y2, act_blocked=3))
         kernels["gemm_w4a4 fc2 (unsigned act) M4608 K12288 N3072"] = {"ms": round(ms, 5), "TOP/s": round(f / ms / 1e9, 1), "frac_int8_mfma": round(f / ms / 1e9 / INT8_MFMA_PEAK_TOPS, 4)}  # fmt: skip
         nq = (torch.rand(128, device=dev) + 0.5).to(torch.bfloat16)
         rot = O.flux_rotary(O.flux_ids(512, 64, 64)).to(dev)
         ms = _time_kernel(lambda: ops.svdq_gemm_w4a4_cuda(act=qx, wgt=lin["qweight"], out=out, ascales=asc, wscales=lin["wscales"],
                                                           lora_act_in=la, lora_up=lin["proj_up"], bias=lin["bias"], norm_q=nq, norm_k=nq, rotary_emb=rot,
-                                                          act_blocked=2))  # fmt: skip
+                                                          act_blocked=3))  # fmt: skip
         kernels["gemm_w4a4+qknorm+rope M4608 K3072 N9216"] = {"ms": round(ms, 5), "TOP/s": round(ops_per_gemm / ms / 1e9, 1), "frac_int8_mfma": round(ops_per_gemm / ms / 1e9 / INT8_MFMA_PEAK_TOPS, 4)}  # fmt: skip
         # AWQ GEMV, adaLN shape.  In the model every adaLN layer has its own weight, so a launch finds its 32 MB in HBM, not in
         # the 256 MB memory-side cache: the launches of the timed graph walk over 12 weight sets (384 MB) in turn ("cold",

@@ -32,7 +32,7 @@
 extern "C" {
 #endif
 
-#define SVDQ_ABI_VERSION 8
+#define SVDQ_ABI_VERSION 9
 
 enum { SVDQ_BF16 = 0, SVDQ_FP16 = 1 };
 enum { SVDQ_PRE_NONE = 0, SVDQ_PRE_GLU = 1, SVDQ_PRE_GELU = 2 }; /* svdq_quantize_args.prologue */
@@ -94,6 +94,11 @@ typedef struct {
     /*      ... + 1024 + 8 * lane.  The GEMM takes it with act_blocked = 2: the matrix instruction reads the codes as they  */
     /*      are (fp6 x fp6, no nibble unpack, no offset term for signed activations; about 8 % of a launch).               */
     int32_t out_blocked;
+    /* non-zero: `scales` is written for the GEMM's svdq_gemm_args.ascales_blocked: the eight scales of groups 8 j .. 8 j + 7 */
+    /* of a row side by side, element ((m / 32) * (K / 512) + g / 8) * 256 + (m % 32) * 8 + g % 8 (K must be a multiple of  */
+    /* 512; the buffer holds ceil(M / 32) * 32 * (K / 64) elements, 16-byte aligned; ld_scales is not used).  No          */
+    /* counterpart in the reference.                                                                                      */
+    int32_t scales_blocked;
 } svdq_quantize_args;
 
 int svdq_quantize_act(const svdq_quantize_args *args, void *stream);
@@ -174,6 +179,12 @@ typedef struct {
     /* 1 / 2: the requantizing epilogues write `qout` that way, for the GEMM that consumes it (ld_qout unused; `qout`   */
     /* must hold ceil(M / 32) * 32 rows' worth: NQ / 2 bytes a row, 3 NQ / 4 with 2)                                    */
     int32_t qout_blocked;
+    /* non-zero (act_blocked = 2 only, K a multiple of 512): `ascales` in the layout of svdq_quantize_args.scales_blocked -- */
+    /* one 16-byte load per lane brings the activation scales of four stages instead of two 2-byte loads per stage        */
+    /* (ld_ascales unused)                                                                                                */
+    int32_t ascales_blocked;
+    /* non-zero: the requantizing epilogues write `oscales` in that layout (NQ a multiple of 512; ld_oscales unused)      */
+    int32_t oscales_blocked;
 } svdq_gemm_args;
 
 int svdq_gemm_w4a4(const svdq_gemm_args *args, void *stream);

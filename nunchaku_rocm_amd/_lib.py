@@ -14,7 +14,7 @@ import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libsvdq_mi355x.so")
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 BF16, FP16 = 0, 1
 EPI_PLAIN, EPI_QK_NORM_ROPE, EPI_GELU_QUANT, EPI_SWIGLU_QUANT = 0, 1, 2, 3
@@ -61,7 +61,7 @@ class QuantizeArgs(ctypes.Structure):
         + [(n, _i32) for n in ("M", "K", "R", "ld_x", "ld_out", "ld_scales", "ld_lora_act", "dtype", "is_unsigned", "prologue")]
         + [("shift", _f32)]
         + [(n, _vp) for n in ("norm_stats", "norm_scale", "norm_shift")]
-        + [(n, _i32) for n in ("norm_rows_per_batch", "norm_ld", "norm_stride", "out_blocked")]
+        + [(n, _i32) for n in ("norm_rows_per_batch", "norm_ld", "norm_stride", "out_blocked", "scales_blocked")]
     )  # fmt: skip
 
 
@@ -76,7 +76,8 @@ class GemmArgs(ctypes.Structure):
         + [("ld_rotary", _i32), ("eps", _f32)]
         + [(n, _vp) for n in ("qout", "oscales", "smooth_next", "lora_down_t", "lora_act_out", "scratch")]
         + [(n, _i32) for n in ("R2", "ld_qout", "ld_oscales", "ld_lora_act_out")]
-        + [("shift", _f32), ("rotary_blocked", _vp), ("lora_down_blocked", _vp), ("act_blocked", _i32), ("qout_blocked", _i32)]
+        + [("shift", _f32), ("rotary_blocked", _vp), ("lora_down_blocked", _vp), ("act_blocked", _i32), ("qout_blocked", _i32),
+           ("ascales_blocked", _i32), ("oscales_blocked", _i32)]
     )  # fmt: skip
 
 

@@ -529,7 +529,9 @@ __device__ __forceinline__ void tile_epilogue(const svdq_gemm_args &a, v16f (&ac
             const float scale = gmax / 15.0f;
             const float safe = (scale == 0.0f) ? 1.0f : scale;
             const float rq = 1.0f / safe;
-            if (half == 0 && m < a.M && n0 + 64 * gi < a.N) ((uint16_t *)a.oscales)[(size_t)g * a.ld_oscales + m] = T::from_f32(scale);
+            if (half == 0 && m < a.M && n0 + 64 * gi < a.N)  // (oscales_blocked: the consuming GEMM's ascales_blocked layout)
+                ((uint16_t *)a.oscales)[a.oscales_blocked ? ((size_t)(m >> 5) * (a.N / (8 * GROUP)) + (g >> 3)) * 256 + (m & 31) * 8 + (g & 7)
+                                                          : (size_t)g * a.ld_oscales + m] = T::from_f32(scale);
             if (a.qout_blocked == 2) {
                 uint32_t vec[6];
 #pragma unroll
@@ -652,7 +654,11 @@ __device__ __forceinline__ void tile_epilogue(const svdq_gemm_args &a, v16f (&ac
         const float scale = gmax / 7.0f;
         const float safe = (scale == 0.0f) ? 1.0f : scale;
         const float rq = 1.0f / safe;
-        if (half == 0 && m < a.M) ((uint16_t *)a.oscales)[(size_t)(yt0 / GROUP) * a.ld_oscales + m] = T::from_f32(scale);
+        if (half == 0 && m < a.M) {
+            const int g = yt0 / GROUP;
+            ((uint16_t *)a.oscales)[a.oscales_blocked ? ((size_t)(m >> 5) * (H / (8 * GROUP)) + (g >> 3)) * 256 + (m & 31) * 8 + (g & 7)
+                                                      : (size_t)g * a.ld_oscales + m] = T::from_f32(scale);
+        }
         if (a.qout_blocked == 2) {
             // sign | magnitude: the magnitude rounds as the value does; the magic constant gets 32 more for a negative one
             uint32_t vec[6];
@@ -922,9 +928,12 @@ __global__ __launch_bounds__(NTHREADS, 2) void gemm_w4a4_i8_kernel(svdq_gemm_arg
 // as fp6 codes (sign | magnitude, what the matrix instruction wants of a signed value too) in lane order -- per 32 rows
 // and group 1 KB of the lanes' first 16 bytes and 512 bytes of their last 8 -- and go into the matrix instruction as
 // they are loaded: fp6 x fp6 (half the matrix-pipe time of fp8 x fp6), no nibble unpack, no offset to take out.
-template <typename T, bool ACT_UNSIGNED, int EPI, bool PIPE, bool F6ACT = false>
+// SB (ascales_blocked, with F6ACT; K / 64 a multiple of 8): the activation scales of the eight groups of four stages lie
+// side by side per row: one 16-byte load per lane every four stages instead of two 2-byte loads per stage.
+template <typename T, bool ACT_UNSIGNED, int EPI, bool PIPE, bool F6ACT = false, bool SB = false>
 __global__ __launch_bounds__(NTHREADS, PIPE ? 2 : 3) void gemm_w4a4_f8_kernel(svdq_gemm_args a) {
     static_assert(!F6ACT || ACT_UNSIGNED, "fp6 activation codes carry their sign: there is no offset to correct");
+    static_assert(!SB || F6ACT, "blocked activation scales come with fp6 activation codes");
     // Separate LDS objects: the compiler then knows that a block load into one staging buffer cannot touch what is being
     // read from the other (one object would make every LDS read wait for the loads in flight).
     __shared__ __align__(16) uint8_t sbuf0[F8_STAGE_BYTES];
@@ -979,12 +988,18 @@ __global__ __launch_bounds__(NTHREADS, PIPE ? 2 : 3) void gemm_w4a4_f8_kernel(sv
     const uint32_t oAct = ablk ? (uint32_t)lane * 16u : (uint32_t)(mrow - m0) * (uint32_t)a.ld_act + half * 16;
     const uint32_t oExt = 1024u + (uint32_t)lane * 8u;
     const uint32_t oA = 2u * (uint32_t)mrow;
+    // SB: dword ST of sc_cur = the row's scales of the two groups of stage ST of the current four stages; sc_nxt is loaded
+    // during their first stage (512 bytes per 32 rows and four stages)
+    v4i sc_cur = {0, 0, 0, 0}, sc_nxt = {0, 0, 0, 0};
+    const __amdgpu_buffer_rsrc_t rASb = g_buffer((const uint8_t *)a.ascales + (SB ? (size_t)((m0 >> 5) + wm) * (G >> 3) * 512 : 0));
+    const uint32_t oAb = (uint32_t)l32 * 16u;
+    if constexpr (SB) sc_cur = g_load128(rASb, oAb, 0);
     auto load_regs = [&](int s, auto set_tag) {
         constexpr int SET = decltype(set_tag)::value;
 #pragma unroll
         for (int gg = 0; gg < 2; gg++) {
             const int gi = min(2 * s + gg, G - 1);
-            qa[gg] = g_load16(rAS, oA, (uint32_t)gi * (uint32_t)a.ld_ascales * 2u);
+            if constexpr (!SB) qa[gg] = g_load16(rAS, oA, (uint32_t)gi * (uint32_t)a.ld_ascales * 2u);
             if constexpr (F6ACT) {
                 const v4i lo = g_load128(rAct, oAct, (uint32_t)gi * sAct);
                 const v2i hi = g_load64(rAct, oExt, (uint32_t)gi * sAct);
@@ -1062,7 +1077,15 @@ __global__ __launch_bounds__(NTHREADS, PIPE ? 2 : 3) void gemm_w4a4_f8_kernel(sv
         // slots 0-3, two to a register.  The weight side is the dword (ws of the first group, ws of the second group) as it
         // lies in the ring; the activation side carries as of the step's group in that group's slot and zero elsewhere
         // (also in lanes 32-63, whose weight-side values therefore do not matter).
-        const int qa0 = (int)qa[0], qa1 = (int)((uint32_t)qa[1] << 16);
+        int qa0, qa1;
+        if constexpr (SB) {
+            qa0 = sc_cur[ST] & 0xFFFF;
+            qa1 = sc_cur[ST] & (int)0xFFFF0000;
+            if constexpr (ST == 0) sc_nxt = g_load128(rASb, oAb, (uint32_t)min((s >> 2) + 1, (nstages >> 2) - 1) * 512u);
+        } else {
+            qa0 = (int)qa[0];
+            qa1 = (int)((uint32_t)qa[1] << 16);
+        }
         const v2i sa[2] = {(v2i){half ? 0 : qa0, 0}, (v2i){half ? 0 : qa1, 0}};
         __builtin_amdgcn_s_barrier();
         if constexpr (!ACT_UNSIGNED) {
@@ -1146,6 +1169,7 @@ __global__ __launch_bounds__(NTHREADS, PIPE ? 2 : 3) void gemm_w4a4_f8_kernel(sv
         stage(std::integral_constant<int, 1>{}, s + 1);
         stage(std::integral_constant<int, 2>{}, s + 2);
         stage(std::integral_constant<int, 3>{}, s + 3);
+        if constexpr (SB) sc_cur = sc_nxt;
         par ^= 1;
         rcur = (uint32_t)l32 * AUX_LROW + (uint32_t)(4 * par) * AUX_LBLK;
         rprev = (uint32_t)l32 * AUX_LROW + (uint32_t)(4 * (par ^ 1) + 2 * half) * AUX_LBLK;
@@ -1315,21 +1339,21 @@ static bool two_workgroups_per_cu(long tiles) {
     return cost(2, 2.16, last2) < cost(3, 3.0, last3);
 }
 
-template <typename T, bool U, bool PIPE, bool F6ACT>
+template <typename T, bool U, bool PIPE, bool F6ACT, bool SB = false>
 static void launch_gemm_f8p(const svdq_gemm_args &a, hipStream_t s) {
     const dim3 grid(((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN)), block(NTHREADS);
     switch (a.epilogue) {
         case SVDQ_EPI_PLAIN:
-            hipLaunchKernelGGL((gemm_w4a4_f8_kernel<T, U, SVDQ_EPI_PLAIN, PIPE, F6ACT>), grid, block, 0, s, a);
+            hipLaunchKernelGGL((gemm_w4a4_f8_kernel<T, U, SVDQ_EPI_PLAIN, PIPE, F6ACT, SB>), grid, block, 0, s, a);
             break;
         case SVDQ_EPI_QK_NORM_ROPE:
-            hipLaunchKernelGGL((gemm_w4a4_f8_kernel<T, U, SVDQ_EPI_QK_NORM_ROPE, PIPE, F6ACT>), grid, block, 0, s, a);
+            hipLaunchKernelGGL((gemm_w4a4_f8_kernel<T, U, SVDQ_EPI_QK_NORM_ROPE, PIPE, F6ACT, SB>), grid, block, 0, s, a);
             break;
         case SVDQ_EPI_GELU_QUANT:
-            hipLaunchKernelGGL((gemm_w4a4_f8_kernel<T, U, SVDQ_EPI_GELU_QUANT, PIPE, F6ACT>), grid, block, 0, s, a);
+            hipLaunchKernelGGL((gemm_w4a4_f8_kernel<T, U, SVDQ_EPI_GELU_QUANT, PIPE, F6ACT, SB>), grid, block, 0, s, a);
             break;
         case SVDQ_EPI_SWIGLU_QUANT:
-            hipLaunchKernelGGL((gemm_w4a4_f8_kernel<T, U, SVDQ_EPI_SWIGLU_QUANT, PIPE, F6ACT>), grid, block, 0, s, a);
+            hipLaunchKernelGGL((gemm_w4a4_f8_kernel<T, U, SVDQ_EPI_SWIGLU_QUANT, PIPE, F6ACT, SB>), grid, block, 0, s, a);
             break;
     }
 }
@@ -1338,10 +1362,16 @@ template <typename T, bool U>
 static void launch_gemm_f8(const svdq_gemm_args &a, hipStream_t s) {
     const bool two = two_workgroups_per_cu((long)((a.M + BM - 1) / BM) * ((a.N + BN - 1) / BN));
     if (a.act_blocked == 2) {  // fp6 codes carry their sign: one instantiation for signed and unsigned activations
-        if (two)
+        if (a.ascales_blocked) {
+            if (two)
+                launch_gemm_f8p<T, true, true, true, true>(a, s);
+            else
+                launch_gemm_f8p<T, true, false, true, true>(a, s);
+        } else if (two) {
             launch_gemm_f8p<T, true, true, true>(a, s);
-        else
+        } else {
             launch_gemm_f8p<T, true, false, true>(a, s);
+        }
     } else if (two) {
         launch_gemm_f8p<T, U, true, false>(a, s);
     } else {
@@ -1500,7 +1530,11 @@ static int gemm_w4a4_checked(const svdq_gemm_args &a, void *stream) {
                   a.ld_act, a.ld_wgt);
         return SVDQ_E_INVALID;
     }
-    if (a.ld_ascales < a.M || a.ld_wscales < a.N) {
+    if (a.ascales_blocked && (a.act_blocked != 2 || a.K % 512 || !al16(a.ascales))) {
+        set_error("svdq_gemm_w4a4: ascales_blocked needs act_blocked = 2, K %% 512 == 0 (K=%d) and 16-byte aligned ascales", a.K);
+        return a.act_blocked != 2 ? SVDQ_E_UNSUPPORTED : SVDQ_E_INVALID;
+    }
+    if ((!a.ascales_blocked && a.ld_ascales < a.M) || a.ld_wscales < a.N) {
         set_error("svdq_gemm_w4a4: scale rows shorter than M / N");
         return SVDQ_E_INVALID;
     }
@@ -1570,8 +1604,12 @@ static int gemm_w4a4_checked(const svdq_gemm_args &a, void *stream) {
             return SVDQ_E_INVALID;
         }
         if (!a.qout || !a.oscales || ((uintptr_t)a.qout & (a.qout_blocked ? 15 : 7)) ||
-            (!a.qout_blocked && (a.ld_qout % 8 || a.ld_qout < NQ / 2)) || a.ld_oscales < a.M) {
+            (!a.qout_blocked && (a.ld_qout % 8 || a.ld_qout < NQ / 2)) || (!a.oscales_blocked && a.ld_oscales < a.M)) {
             set_error("svdq_gemm_w4a4: qout (8-byte aligned rows) and oscales are required");
+            return SVDQ_E_INVALID;
+        }
+        if (a.oscales_blocked && (NQ % 512 || !al16(a.oscales))) {
+            set_error("svdq_gemm_w4a4: oscales_blocked needs %d requantized columns to be a multiple of 512 and 16-byte aligned oscales", NQ);
             return SVDQ_E_INVALID;
         }
         if (a.R2 < 0 || a.R2 % 16 ||

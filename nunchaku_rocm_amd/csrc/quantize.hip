@@ -95,6 +95,9 @@ __global__ __launch_bounds__(Q_WAVES * 64, QR == 32 ? 1 : (NORM ? 4 : 2)) void q
     uint8_t *__restrict__ outbase = (uint8_t *)a.out + (size_t)m0 * a.ld_out + gw * (GROUP / 2);
     const uint32_t outoff = (uint32_t)ml * a.ld_out + kq * 8;
     uint16_t *__restrict__ scales = (uint16_t *)a.scales + (size_t)gw * a.ld_scales + m0;
+    // scales_blocked: the eight scales of groups 8 j .. 8 j + 7 of a row side by side (16 bytes), 32 rows to a 512-byte block:
+    // group gw + 8 i of row m at ((m / 32) * (ngroups / 8) + gw / 8 + i) * 256 + (m % 32) * 8 + gw % 8
+    uint16_t *__restrict__ const scalesb = (uint16_t *)a.scales + ((size_t)(m0 >> 5) * (ngroups >> 3) + (gw >> 3)) * 256 + (gw & 7);
     // out_blocked: the 32 packed bytes of (row, group) go where the GEMM's lane (row % 32, half) of that 32-row block and
     // group finds them, [32-row block][group][64 lanes x 16 bytes]: this lane's 8 bytes are half kq / 2, offset 8 (kq % 2)
     uint8_t *__restrict__ bout[NH];
@@ -342,7 +345,12 @@ __global__ __launch_bounds__(Q_WAVES * 64, QR == 32 ? 1 : (NORM ? 4 : 2)) void q
                         asm("v_lshl_add_u32 %0, %1, %2, %0" : "+v"(phi[e]) : "v"(b), "n"(6 * c - 32));
                 }
                 if (row_ok) {
-                    if (kq == 0) (scales + (size_t)i * Q_WAVES * a.ld_scales)[Q_ROWS * h + ml] = T::from_f32(scale);
+                    if (kq == 0) {
+                        if (a.scales_blocked)
+                            scalesb[(size_t)i * 256 + ((m0 + Q_ROWS * h + ml) & 31) * 8] = T::from_f32(scale);
+                        else
+                            (scales + (size_t)i * Q_WAVES * a.ld_scales)[Q_ROWS * h + ml] = T::from_f32(scale);
+                    }
                     uint8_t *blk = f6base + (size_t)(gw + Q_WAVES * i) * 1536;
 #pragma unroll
                     for (int e = 0; e < 2; e++) {
@@ -371,7 +379,12 @@ __global__ __launch_bounds__(Q_WAVES * 64, QR == 32 ? 1 : (NORM ? 4 : 2)) void q
                 w1 ^= 0x88888888u;
             }
             if (row_ok) {
-                if (kq == 0) (scales + (size_t)i * Q_WAVES * a.ld_scales)[Q_ROWS * h + ml] = T::from_f32(scale);
+                if (kq == 0) {
+                    if (a.scales_blocked)
+                        scalesb[(size_t)i * 256 + ((m0 + Q_ROWS * h + ml) & 31) * 8] = T::from_f32(scale);
+                    else
+                        (scales + (size_t)i * Q_WAVES * a.ld_scales)[Q_ROWS * h + ml] = T::from_f32(scale);
+                }
                 uint8_t *dst = a.out_blocked ? bout[h] + (size_t)(gw + Q_WAVES * i) * 1024
                                              : outbase + (size_t)i * (GSTEP / 2) + (uint32_t)(Q_ROWS * h) * a.ld_out + outoff;
                 *(uint2 *)dst = make_uint2(w0, w1);
@@ -728,7 +741,11 @@ extern "C" int svdq_quantize_act(const svdq_quantize_args *args, void *stream) {
         set_error("svdq_quantize_act: unknown prologue %d", a.prologue);
         return SVDQ_E_INVALID;
     }
-    if (a.ld_x < (a.prologue == SVDQ_PRE_GLU ? 2 : 1) * a.K || (!a.out_blocked && a.ld_out < a.K / 2) || a.ld_scales < a.M ||
+    if (a.scales_blocked && (a.K % 512 || ((uintptr_t)a.scales & 15))) {
+        set_error("svdq_quantize_act: scales_blocked needs K %% 512 == 0 (K=%d) and 16-byte aligned scales", a.K);
+        return SVDQ_E_INVALID;
+    }
+    if (a.ld_x < (a.prologue == SVDQ_PRE_GLU ? 2 : 1) * a.K || (!a.out_blocked && a.ld_out < a.K / 2) || (!a.scales_blocked && a.ld_scales < a.M) ||
         (a.R > 0 && a.ld_lora_act < a.R)) {
         set_error("svdq_quantize_act: a leading dimension is smaller than its row");
         return SVDQ_E_INVALID;

@@ -246,6 +246,22 @@ def unblock_activations_f6(blocked: torch.Tensor, unsigned: bool = False) -> tor
     return (v[..., 0] | (v[..., 1] << 4)).to(torch.uint8)
 
 
+def block_scales(scales: torch.Tensor) -> torch.Tensor:
+    """Activation scales ``(K/64, rows)`` (K a multiple of 512, rows of 32) -> the same values in the order the GEMM reads
+    them with ``act_blocked=3`` (what the quantizer writes with ``out_blocked=3``): per 32 rows and eight groups 512
+    bytes, row ``r``'s eight scales side by side at element ``8 r``.  Same shape; pure torch."""
+    g, rows = scales.shape
+    assert g % 8 == 0 and rows % 32 == 0, "K must be a multiple of 512 and rows of 32"
+    return scales.reshape(g // 8, 8, rows // 32, 32).permute(2, 0, 3, 1).contiguous().reshape(g, rows)
+
+
+def unblock_scales(blocked: torch.Tensor) -> torch.Tensor:
+    """Inverse of :func:`block_scales`."""
+    g, rows = blocked.shape
+    assert g % 8 == 0 and rows % 32 == 0, "K must be a multiple of 512 and rows of 32"
+    return blocked.reshape(rows // 32, g // 8, 32, 8).permute(1, 3, 0, 2).contiguous().reshape(g, rows)
+
+
 def unblock_activations(blocked: torch.Tensor) -> torch.Tensor:
     """Inverse of :func:`block_activations`."""
     rows, kb = blocked.shape

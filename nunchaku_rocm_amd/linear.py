@@ -118,14 +118,16 @@ class SVDQW4A4Linear(nn.Module):
         """How this layer's GEMM wants its quantized input for ``rows`` rows padded to ``pad_size``: the value for
         ``blocked=`` in :meth:`quantize` (or ``qout_blocked=`` of the GEMM whose epilogue produces the input) and
         ``act_blocked=`` in :meth:`forward_quant`: 0 = the reference's matrix, 1 = its bytes in the fp8 main loop's own
-        order, 2 = fp6 codes in that order."""
+        order, 2 = fp6 codes in that order, 3 = those with the activation scales in that order too (``in_features`` a
+        multiple of 512)."""
         from .ops.gemm import takes_blocked_activations
 
         return takes_blocked_activations(self.qweight, self.wscales, -(-rows // pad_size) * pad_size)
 
     def quantize(self, x: torch.Tensor, pad_size: int = 256, norm: tuple | None = None, blocked: bool | int = False):
         """``blocked`` (an addition to the reference's signature): the codes in the order the GEMM's fp8 main loop reads
-        them (``True``) or as fp6 codes in that order (``2``), for :meth:`forward_quant` with the same ``act_blocked``;
+        them (``True``), as fp6 codes in that order (``2``) or those with the scales in that order too (``3``), for
+        :meth:`forward_quant` with the same ``act_blocked``;
         ``False`` = the reference's ``(M_pad, K/2)`` matrix."""
         return svdq_quantize_w4a4_act_fuse_lora_cuda(
             x, lora_down=self.proj_down, smooth=self.smooth_factor, fp4=False, pad_size=pad_size, norm=norm, out_blocked=blocked

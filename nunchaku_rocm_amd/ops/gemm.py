@@ -37,8 +37,10 @@ USE_BLOCKED_ACTIVATIONS = True
 # instructions want it (made once per weight and cached, as large as the weight): 1 KB per load instruction instead of
 # 8-byte pieces of 32 rows.  False = read the transposed (R2, N) copy (same results).
 USE_BLOCKED_LORA_DOWN = True
-# values of ``act_blocked`` / ``out_blocked`` beyond False / True
+# values of ``act_blocked`` / ``out_blocked`` / ``qout_blocked`` beyond False / True: fp6 codes in lane order, and the same with
+# the activation scales in the GEMM's own order as well (eight groups of a row side by side; K a multiple of 512)
 ACT_CODES_F6 = 2
+ACT_CODES_F6_SCALES = 3
 
 # True sends the requantizing epilogues' LoRA-down partial sums to the buffer built into the library
 # (svdq_gemm_w4a4_static_scratch) instead of a torch allocation per call: for callers that may not allocate, e.g. while
@@ -74,12 +76,15 @@ def working_copy(wgt: torch.Tensor, wscales: torch.Tensor) -> torch.Tensor | Non
 
 def takes_blocked_activations(wgt: torch.Tensor, wscales: torch.Tensor, rows: int) -> int:
     """How a GEMM on this weight should be fed its activations: 0 = the (M, K/2) matrix, 1 = its bytes in the fp8 main
-    loop's own order, 2 (``ACT_CODES_F6``) = fp6 codes in that order -- the value for ``out_blocked`` / ``qout_blocked`` of
-    the producer and ``act_blocked`` of this GEMM.  Non-zero when the switch is on, the weight has a working copy and the
+    loop's own order, 2 (``ACT_CODES_F6``) = fp6 codes in that order, 3 (``ACT_CODES_F6_SCALES``, K a multiple of 512) = those
+    with the activation scales in the loop's own order too -- the value for ``out_blocked`` / ``qout_blocked`` of the
+    producer and ``act_blocked`` of this GEMM.  Non-zero when the switch is on, the weight has a working copy and the
     (padded) row count is a multiple of 32."""
     if not USE_BLOCKED_ACTIVATIONS or rows % 32 or working_copy(wgt, wscales) is None:
         return 0
-    return ACT_CODES_F6 if USE_BLOCKED_ACTIVATIONS is True else 1
+    if USE_BLOCKED_ACTIVATIONS is True:
+        return ACT_CODES_F6_SCALES if (wgt.shape[1] * 2) % 512 == 0 else ACT_CODES_F6
+    return int(USE_BLOCKED_ACTIVATIONS)
 
 
 HEAD_DIM = 128
@@ -135,7 +140,9 @@ def svdq_gemm_w4a4_cuda(
       ``act_blocked=2`` (``ACT_CODES_F6``): ``act`` is ``(rows, 3K/4)`` bytes of fp6 codes in lane order, as the quantizer
       writes them with ``out_blocked=2``: the matrix instruction takes them as they are (no offset term for signed
       activations, fp6 x fp6); ``act_unsigned`` is then not looked at.  ``qout_blocked=2``: the requantizing epilogue writes
-      ``qout`` as ``(rows, 3NQ/4)`` bytes of such codes.
+      ``qout`` as ``(rows, 3NQ/4)`` bytes of such codes.  ``3`` (``ACT_CODES_F6_SCALES``; K, or the requantized width, a
+      multiple of 512): as ``2``, and ``ascales`` / ``oscales`` hold their values in the loop's own order as well
+      (``svdq_gemm_args.ascales_blocked`` / ``oscales_blocked``; contiguous, rows a multiple of 32).
 
     Raises ``NotImplementedError`` for the arguments the reference's ROCm backend rejects as well (``poolout``,
     ``out_vk``, ``out_linearattn``, ``out_q/k/v``) and for the NVFP4-only ones (``fp4``, ``wcscales``, ``alpha != 1``,
@@ -159,7 +166,7 @@ def svdq_gemm_w4a4_cuda(
     act = act.reshape(-1, act.shape[-1])
     act_blocked = int(act_blocked)
     M, K, N = act.shape[0], wgt.shape[1] * 2, wgt.shape[0]
-    assert act.shape[1] == (K * 3 // 4 if act_blocked == ACT_CODES_F6 else K // 2), f"weight K mismatch: {K} vs act {tuple(act.shape)}"
+    assert act.shape[1] == (K * 3 // 4 if act_blocked >= ACT_CODES_F6 else K // 2), f"weight K mismatch: {K} vs act {tuple(act.shape)}"
     dev = _lib.require_cuda(act, wgt, out, qout, ascales, wscales, oscales, lora_act_in, lora_up, lora_down,
                             lora_act_out, norm_q, norm_k, rotary_emb, bias, smooth_factor)  # fmt: skip
 
@@ -231,6 +238,8 @@ def svdq_gemm_w4a4_cuda(
             raise ValueError("act_blocked needs a weight with a working copy (the int8 main loop reads the (M, K/2) matrix)")
         if not act.is_contiguous() or M % 32 or act.data_ptr() % 16:
             raise ValueError("act_blocked needs a contiguous act with a multiple of 32 rows")
+        if act_blocked == ACT_CODES_F6_SCALES and (K % 512 or not ascales.is_contiguous() or ascales.shape != (K // 64, M) or ascales.data_ptr() % 16):
+            raise ValueError("act_blocked=3 needs K % 512 == 0 and contiguous (K/64, rows) ascales over the same rows as act")
     args = _lib.GemmArgs(
         act=act.data_ptr(),
         wgt=wgt.data_ptr(),
@@ -257,7 +266,8 @@ def svdq_gemm_w4a4_cuda(
         act_unsigned=int(act_unsigned),
         epilogue=_lib.EPI_PLAIN,
         eps=1e-6,
-        act_blocked=int(act_blocked),
+        act_blocked=min(act_blocked, ACT_CODES_F6),
+        ascales_blocked=int(act_blocked == ACT_CODES_F6_SCALES),
     )
     keep = [planes]  # tensors that must outlive the launch call
     lib = _lib.load()
@@ -284,7 +294,7 @@ def svdq_gemm_w4a4_cuda(
     elif want_quant:
         NQ = N // 2 if fuse_swiglu else N
         qout2d = qout.reshape(-1, qout.shape[-1])
-        qb = NQ * 3 // 4 if int(qout_blocked) == ACT_CODES_F6 else NQ // 2  # bytes of codes per row
+        qb = NQ * 3 // 4 if int(qout_blocked) >= ACT_CODES_F6 else NQ // 2  # bytes of codes per row
         if qout2d.element_size() != 1 or qout2d.shape[0] < M or qout2d.shape[1] != qb or qout2d.stride(1) != 1:
             raise ValueError(f"qout shape/dtype {tuple(qout.shape)} {qout.dtype}")
         if oscales.dtype != T or oscales.dim() != 2 or oscales.shape[0] != NQ // 64 or oscales.shape[1] < M or oscales.stride(1) != 1:
@@ -318,7 +328,11 @@ def svdq_gemm_w4a4_cuda(
         if qout_blocked:
             if not qout2d.is_contiguous() or qout2d.shape[0] % 32 or qout2d.data_ptr() % 16:
                 raise ValueError("qout_blocked needs a contiguous qout with a multiple of 32 rows")
-            args.qout_blocked = int(qout_blocked)
+            args.qout_blocked = min(int(qout_blocked), ACT_CODES_F6)
+            if int(qout_blocked) == ACT_CODES_F6_SCALES:
+                if NQ % 512 or not oscales.is_contiguous() or oscales.shape[1] != qout2d.shape[0] or oscales.data_ptr() % 16:
+                    raise ValueError("qout_blocked=3 needs a requantized width that is a multiple of 512 and contiguous oscales over qout's rows")
+                args.oscales_blocked = 1
         args.shift = 0.0 if fuse_swiglu else GELU_SHIFT
 
     with torch.cuda.device(dev):

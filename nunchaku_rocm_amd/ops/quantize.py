@@ -78,6 +78,9 @@ def quantize_w4a4_act_fuse_lora(
     must be contiguous with a multiple of 32 rows.  :func:`nunchaku_rocm_amd.layout.unblock_activations` undoes it.
     ``out_blocked=2``: ``output`` is ``(rows, 3K/4)`` bytes of fp6 codes (sign << 5 | magnitude, the same integers) in
     lane order, for the GEMM's ``act_blocked=2`` (:func:`nunchaku_rocm_amd.layout.unblock_activations_f6`).
+    ``out_blocked=3`` (K a multiple of 512): as ``2``, and ``oscales`` -- contiguous ``(K/64, rows)``, rows a multiple of
+    32 -- holds the scales in the GEMM's own order too (``svdq_quantize_args.scales_blocked``, for ``act_blocked=3``;
+    :func:`nunchaku_rocm_amd.layout.unblock_scales`).
     """
     if fp4:
         raise NotImplementedError("NVFP4 quantization is not implemented (int4 only)")
@@ -91,11 +94,11 @@ def quantize_w4a4_act_fuse_lora(
         raise ValueError(f"K={K} must be a multiple of the group size 64")
     rank = lora_down.shape[1] if lora_down is not None else 0
     out_blocked = int(out_blocked)
-    kb = K * 3 // 4 if out_blocked == 2 else K // 2  # bytes of codes per row
+    kb = K * 3 // 4 if out_blocked >= 2 else K // 2  # bytes of codes per row
     if output is None:
         output = torch.empty(_ceil_divide(M, 32) * 32 if out_blocked else M, kb, dtype=torch.uint8, device=inp.device)
     if oscales is None:
-        oscales = torch.empty(K // 64, M, dtype=inp.dtype, device=inp.device)
+        oscales = torch.empty(K // 64, output.shape[0] if out_blocked == 3 else M, dtype=inp.dtype, device=inp.device)
     if lora_act_out is None and lora_down is not None:
         lora_act_out = torch.empty(M, rank, dtype=torch.float32, device=inp.device)
 
@@ -105,6 +108,8 @@ def quantize_w4a4_act_fuse_lora(
         raise ValueError("output must be a (>= M, K/2) byte tensor with unit inner stride")
     if out_blocked and (not output.is_contiguous() or output.shape[0] % 32 or output.shape[1] != kb or output.data_ptr() % 16):
         raise ValueError("out_blocked needs a contiguous (rows, K/2) output (2: (rows, 3K/4)) with rows a multiple of 32")
+    if out_blocked == 3 and (K % 512 or not oscales.is_contiguous() or oscales.shape != (K // 64, output.shape[0]) or oscales.data_ptr() % 16):
+        raise ValueError("out_blocked=3 needs K % 512 == 0 and contiguous (K/64, rows) oscales over output's rows")
     if oscales.dtype != inp.dtype or oscales.stride(1) != 1 or oscales.shape[1] < M or oscales.shape[0] < K // 64:
         raise ValueError("oscales must be (K/64, >= M) of the input dtype with unit inner stride")
     if rank and (lora_act_out.dtype != torch.float32 or lora_act_out.stride(1) != 1 or lora_act_out.shape[0] < M):
@@ -144,7 +149,8 @@ def quantize_w4a4_act_fuse_lora(
         is_unsigned=int(unsigned),
         prologue=_lib.PRE_GLU if fuse_glu else (_lib.PRE_GELU if fuse_gelu else _lib.PRE_NONE),
         shift=float(shift_value),
-        out_blocked=out_blocked,
+        out_blocked=min(out_blocked, 2),
+        scales_blocked=int(out_blocked == 3),
     )
     with torch.cuda.device(inp.device):
         _lib.check(_lib.load().svdq_quantize_act(args, _lib.stream_of(inp)))
@@ -212,7 +218,7 @@ def svdq_quantize_w4a4_act_fuse_lora_cuda(
     rank = lora_down.shape[1] if lora_down is not None else 0
     batch_size_pad = _ceil_divide(batch_size, pad_size) * pad_size
     if output is None:
-        kb = (channels // 2 if fuse_glu else channels) * 3 // 4 if int(out_blocked) == 2 else channels // 2
+        kb = (channels // 2 if fuse_glu else channels) * 3 // 4 if int(out_blocked) >= 2 else channels // 2
         output = torch.empty(batch_size_pad, kb, dtype=torch.uint8, device=input.device)
     if oscales is None:
         assert channels % 64 == 0

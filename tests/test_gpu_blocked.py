@@ -96,6 +96,77 @@ def test_quantizer_writes_fp6_codes(dev, M, K, R, norm, unsigned, dtype):
         assert torch.equal(blk[2].cpu()[:M], nat[2].cpu()[:M])
 
 
+def test_scale_layout_helpers_invert_each_other():
+    from nunchaku_rocm_amd.layout import block_scales, unblock_scales
+
+    a = torch.arange(16 * 96, dtype=torch.float32).reshape(16, 96).to(torch.bfloat16)
+    b = block_scales(a)
+    assert b.shape == a.shape and torch.equal(unblock_scales(b), a)
+    m, g = 70, 11  # element ((m / 32) * (G / 8) + g / 8) * 256 + (m % 32) * 8 + g % 8
+    assert b.reshape(-1)[((m // 32) * 2 + g // 8) * 256 + (m % 32) * 8 + g % 8] == a[g, m]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M,K,N,R,norm", [(300, 512, 264, 16, False), (4608, 3072, 384, 32, False), (1000, 1536, 256, 32, True), (96, 1024, 128, 0, False)])
+def test_scales_in_the_gemms_order(dev, M, K, N, R, norm, dtype):
+    """out_blocked = act_blocked = 3: fp6 codes as with 2, and the activation scales where the GEMM's lanes read eight
+    groups with one load.  The quantizer writes the same scale bits elsewhere; the GEMM computes the same output bits
+    as with act_blocked = 2; K that is not a multiple of 512 is refused."""
+    from nunchaku_rocm_amd import ops
+    from nunchaku_rocm_amd.layout import block_scales, unblock_activations_f6, unblock_scales
+    from nunchaku_rocm_amd.ops import gemm as gemm_mod
+
+    print(f"case M={M} K={K} N={N} R={R} norm={norm} {dtype}", flush=True)
+    lin = {k: v.to(dev) for k, v in O.make_svdq_linear(K, N, R=max(R, 16), seed=K + N, dtype=dtype).items()}
+    g = torch.Generator().manual_seed(M + K)
+    x = torch.randn(M, K, generator=g).to(dtype).to(dev)
+    ld = lin["proj_down"][:, :R].contiguous() if R else None
+    lu = lin["proj_up"][:, :R].contiguous() if R else None
+    nm = ((torch.randn(K, generator=g) * 0.1 + 1).to(dtype).to(dev), (torch.randn(K, generator=g) * 0.1).to(dtype).to(dev)) if norm else None
+    q2, s2, la2 = ops.svdq_quantize_w4a4_act_fuse_lora_cuda(x, lora_down=ld, smooth=lin["smooth_factor"], norm=nm, out_blocked=2)
+    s3 = torch.full_like(s2, 7.0)
+    q3, s3, la3 = ops.svdq_quantize_w4a4_act_fuse_lora_cuda(x, oscales=s3, lora_down=ld, smooth=lin["smooth_factor"], norm=nm, out_blocked=3)
+    torch.cuda.synchronize()
+    full = (M + 31) // 32 * 32
+    assert torch.equal(unblock_activations_f6(q2.cpu())[:M], unblock_activations_f6(q3.cpu())[:M])
+    assert torch.equal(unblock_scales(s3.cpu())[:, :M].view(torch.int16), s2.cpu()[:, :M].view(torch.int16))
+    assert (unblock_scales(s3.cpu())[:, full:] == 7.0).all()  # rows of untouched 32-row blocks keep what the buffer held
+    old = gemm_mod.USE_WEIGHT_PLANES
+    gemm_mod.USE_WEIGHT_PLANES = "all"
+    try:
+        outs = []
+        for mode, q, s, la in ((2, q2, s2, la2), (3, q3, s3, la3), (3, q2, block_scales(s2), la2)):
+            out = torch.full((M, N), float("nan"), dtype=dtype, device=dev)
+            ops.svdq_gemm_w4a4_cuda(act=q, wgt=lin["qweight"], out=out, ascales=s, wscales=lin["wscales"], lora_act_in=la if R else None,
+                                    lora_up=lu, bias=lin["bias"], act_blocked=mode)  # fmt: skip
+            outs.append(out)
+        torch.cuda.synchronize()
+        assert torch.equal(outs[0].view(torch.int16), outs[1].view(torch.int16))
+        assert torch.equal(outs[0].view(torch.int16), outs[2].view(torch.int16))
+    finally:
+        gemm_mod.USE_WEIGHT_PLANES = old
+
+
+def test_scales_in_the_gemms_order_need_k_of_512(dev):
+    from nunchaku_rocm_amd import ops
+    from nunchaku_rocm_amd.ops import gemm as gemm_mod
+
+    M, K, N = 64, 320, 128
+    lin = {k: v.to(dev) for k, v in O.make_svdq_linear(K, N, seed=1).items()}
+    x = torch.randn(M, K, generator=torch.Generator().manual_seed(2)).to(torch.bfloat16).to(dev)
+    with pytest.raises(ValueError):
+        ops.svdq_quantize_w4a4_act_fuse_lora_cuda(x, lora_down=lin["proj_down"], smooth=lin["smooth_factor"], out_blocked=3)
+    q, s, la = ops.svdq_quantize_w4a4_act_fuse_lora_cuda(x, lora_down=lin["proj_down"], smooth=lin["smooth_factor"], out_blocked=2)
+    old = gemm_mod.USE_WEIGHT_PLANES
+    gemm_mod.USE_WEIGHT_PLANES = "all"
+    try:
+        with pytest.raises(ValueError):
+            ops.svdq_gemm_w4a4_cuda(act=q, wgt=lin["qweight"], out=torch.empty(M, N, dtype=torch.bfloat16, device=dev), ascales=s,
+                                    wscales=lin["wscales"], act_blocked=3)  # fmt: skip
+    finally:
+        gemm_mod.USE_WEIGHT_PLANES = old
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_quantizer_then_gemm_through_fp6_codes(dev, dtype):
     """The pair as the modules run it: quantizer (out_blocked=2) -> GEMM (act_blocked=2) against the pair through the
@@ -234,7 +305,7 @@ def test_requantizing_epilogues_write_either_order(dev, swiglu):
     from nunchaku_rocm_amd.layout import unblock_activations
     from nunchaku_rocm_amd.ops import gemm as gemm_mod
 
-    M, N, K, R2, dtype = 288, 512, 256, 32, torch.bfloat16
+    M, N, K, R2, dtype = 288, 1024, 256, 32, torch.bfloat16  # 1024 / 512 requantized columns: eight groups of scales
     NQ = N // 2 if swiglu else N
     g = torch.Generator().manual_seed(11)
     t = dict(act=torch.randint(0, 256, (M, K // 2), generator=g, dtype=torch.uint8), wgt=torch.randint(0, 256, (N, K // 2), generator=g, dtype=torch.uint8),
@@ -244,16 +315,18 @@ def test_requantizing_epilogues_write_either_order(dev, swiglu):
     t = {k: v.to(dev) for k, v in t.items()}
     from nunchaku_rocm_amd.layout import unblock_activations_f6
 
+    from nunchaku_rocm_amd.layout import unblock_scales
+
     res = []
-    for blocked in (False, True, 2):
-        qout = torch.full((M, NQ * 3 // 4 if blocked == 2 else NQ // 2), 0xEE, dtype=torch.uint8, device=dev)
+    for blocked in (False, True, 2, 3):
+        qout = torch.full((M, NQ * 3 // 4 if blocked >= 2 else NQ // 2), 0xEE, dtype=torch.uint8, device=dev)
         osc = torch.zeros(NQ // 64, M, dtype=dtype, device=dev)
         lao = torch.zeros(M, R2, dtype=torch.float32, device=dev)
         ops.svdq_gemm_w4a4_cuda(qout=qout, oscales=osc, lora_act_out=lao, fuse_swiglu=swiglu, qout_blocked=blocked, **t)
         torch.cuda.synchronize()
         # the GELU epilogue's codes are unsigned, the SwiGLU epilogue's signed
-        codes = unblock_activations_f6(qout.cpu(), not swiglu) if blocked == 2 else unblock_activations(qout.cpu()) if blocked else qout.cpu()
-        res.append((codes, osc.cpu().view(torch.int16), lao.cpu()))
+        codes = unblock_activations_f6(qout.cpu(), not swiglu) if blocked >= 2 else unblock_activations(qout.cpu()) if blocked else qout.cpu()
+        res.append((codes, (unblock_scales(osc.cpu()) if blocked == 3 else osc.cpu()).view(torch.int16), lao.cpu()))
     for other in res[1:]:
         for a, b in zip(res[0], other):
             assert torch.equal(a, b)
@@ -283,7 +356,8 @@ def test_modules_compute_the_same_bits_either_way(dev, dtype):
         for flag in (True, 1, False):
             gemm_mod.USE_BLOCKED_ACTIVATIONS = flag
             try:
-                assert fc1.takes_blocked(S) == fc2.takes_blocked(S) == (2 if flag is True else int(flag))
+                assert fc1.takes_blocked(S) == (2 if flag is True else int(flag))  # K = 256
+                assert fc2.takes_blocked(S) == (3 if flag is True else int(flag))  # K = 1024: scales in the GEMM's order too
                 outs.append([fc1(x).clone(), ops.fused_gelu_mlp(x, fc1, fc2).clone(), ops.fused_qkv_norm_rottary(x, qkv, nq, nk, rot).clone(),
                              ops.fused_swiglu_mlp(x, g1, g2).clone()])  # fmt: skip
             finally:
