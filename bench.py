@@ -35,7 +35,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # in profiles/bench_all_kernels_hbm_traffic.txt, the factors being what the same counters read on plain copy kernels of
 # known size in the same run (FETCH_SIZE reads half the bytes of 16-byte-per-lane loads); counters cannot be read from
 # inside this process
-GEMM_QKV_HBM_BYTES = (2.0 * 103276.1 + 82944.0) * 1024
+GEMM_QKV_HBM_BYTES = (2.0 * 103140.0 + 82944.0) * 1024
 
 
 def _events(n):
@@ -386,11 +386,11 @@ def main():
         "vs_baseline": None,
         "dtype": "i8",
         "data": "synthetic",
-        "config": {"workload": "FLUX.1 QKV SVDQuant linear: activation quantizer + W4A4 GEMM, M=4608 K=3072 N=9216 group 64 LoRA rank 32 (the reference's FLUX.1 QKV benchmark shape); the two operator calls of SVDQW4A4Linear.forward, codes handed over as fp6 in the GEMM's lane order",
+        "config": {"workload": "FLUX.1 QKV SVDQuant linear: activation quantizer + W4A4 GEMM, M=4608 K=3072 N=9216 group 64 LoRA rank 32 (the reference's FLUX.1 QKV benchmark shape); the two operator calls of SVDQW4A4Linear.forward, codes handed over as fp6, and their scales, in the GEMM's lane order",
                    "M": M, "K": K, "N": N, "rank": R, "group": 64},  # fmt: skip
         "roofline": {
             "bound": "mfma",
-            "kernel": "gemm_w4a4_f8_kernel<BF16, fp6 activation codes, plain epilogue, three workgroups per CU>",
+            "kernel": "gemm_w4a4_f8_kernel<BF16, fp6 activation codes with their scales in the loop's order, plain epilogue, three workgroups per CU>",
             "achieved": round(achieved, 2),
             "peak": INT8_MFMA_PEAK_TOPS,
             "unit": "TOP/s",
