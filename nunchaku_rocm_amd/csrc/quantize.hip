@@ -37,14 +37,6 @@ constexpr uint32_t pack_bias() {
     return c;
 }
 
-// sum_i (0x4B400000 << 6 i) mod 2^32 over the five codes that lie wholly in the low dword of a 48-bit piece of eight
-// six-bit codes (the sixth contributes its low two bits only, where the constant has none)
-constexpr uint32_t pack6_bias() {
-    uint32_t c = 0;
-    for (int i = 0; i < 5; i++) c += (uint32_t)RNE_MAGIC_BITS << (6 * i);
-    return c;
-}
-
 // per-group vectors a lane fetches for the group's 64 channels (one channel per lane), shared through LDS later
 struct QVecs {
     uint16_t sm, ns, nh;  // smooth factor, norm scale, norm shift
@@ -112,6 +104,9 @@ __global__ __launch_bounds__(Q_WAVES * 64, QR == 32 ? 1 : (NORM ? 4 : 2)) void q
     // ones the same codes of kh = 1: two 48-bit pieces at byte 6 kq of those 24, each stored as an aligned dword and a
     // 16-bit half (low dword + high half for even kq, low half + high dword for odd kq).
     const bool f6 = a.out_blocked == 2;
+    typedef float v8f __attribute__((ext_vector_type(8)));
+    typedef float v16f __attribute__((ext_vector_type(16)));
+    typedef unsigned v6u __attribute__((ext_vector_type(6)));
     uint8_t *__restrict__ const f6base = (uint8_t *)a.out + (size_t)(m0 >> 5) * ngroups * 1536;
     uint32_t f6o32[NH], f6o16[NH];
 #pragma unroll
@@ -322,28 +317,27 @@ __global__ __launch_bounds__(Q_WAVES * 64, QR == 32 ? 1 : (NORM ? 4 : 2)) void q
             // no clamp: |x| <= gmax gives |x * (1 / (gmax / 7))| <= 7 (1 + 3 * 2^-24), which rounds to <= 7; unsigned codes
             // only need the lower clamp (negative values), the upper bound holds the same way.
             if (f6) {
-                // the same products and the same rounding, on |q| with the sign carried as bit 5 of the code: the magic
-                // constant gets 32 more when q is negative (an even number of units: ties fall as they did)
-                uint32_t plo[2] = {0u - pack6_bias(), 0u - pack6_bias()}, phi[2] = {0u, 0u};  // [0]: even channels, [1]: odd
+                // the same products, rounded to the same integers by the hardware's float -> fp6 conversion: e2m3 codes
+                // are sign | magnitude with steps of 1 / 8 up to 15 / 8, so q / 8 (the instruction's scale operand) rounds to
+                // nearest-even exactly as q does.  It converts 2 x 16 values, result code 2 i from the first source's
+                // element i and code 2 i + 1 from the second's: codes 0 .. 7 get the even channels, 8 .. 15 the odd ones
+                // (elements 8 .. 15 of the sources are not used and left undefined).
+                v8f c0, c1;
 #pragma unroll
                 for (int j = 0; j < 16; j++) {
-                    const float q = v[j] * rq;
-                    uint32_t b;
-                    if (UNSIGNED) {
-                        b = __float_as_uint(__builtin_fmaxf(q, 0.0f) + RNE_MAGIC);
-                    } else {
-                        const uint32_t mg = ((uint32_t)((int)__float_as_uint(q) >> 31) & 32u) | (uint32_t)RNE_MAGIC_BITS;
-                        b = __float_as_uint(__builtin_fabsf(q) + __uint_as_float(mg));
-                    }
-                    const int c = j >> 1, e = j & 1;  // code c of piece e
-                    if (c < 5)
-                        asm("v_lshl_add_u32 %0, %1, %2, %0" : "+v"(plo[e]) : "v"(b), "n"(6 * c));
-                    else if (c == 5) {
-                        plo[e] += b << 30;
-                        phi[e] = b >> 2;
-                    } else
-                        asm("v_lshl_add_u32 %0, %1, %2, %0" : "+v"(phi[e]) : "v"(b), "n"(6 * c - 32));
+                    float q = v[j] * rq;
+                    if (UNSIGNED) q = __builtin_fmaxf(q, 0.0f);
+                    const int c = j >> 1, o = (j & 1) * 4 + (c >> 1);
+                    if (c & 1)
+                        c1[o] = q;
+                    else
+                        c0[o] = q;
                 }
+                const v16f cv0 = __builtin_shufflevector(c0, c0, 0, 1, 2, 3, 4, 5, 6, 7, -1, -1, -1, -1, -1, -1, -1, -1);
+                const v16f cv1 = __builtin_shufflevector(c1, c1, 0, 1, 2, 3, 4, 5, 6, 7, -1, -1, -1, -1, -1, -1, -1, -1);
+                const v6u d = __builtin_amdgcn_cvt_scalef32_2xpk16_fp6_f32(cv0, cv1, 8.0f);
+                const uint32_t plo[2] = {d[0], __builtin_amdgcn_alignbit(d[2], d[1], 16)};  // [0]: even channels, [1]: odd
+                const uint32_t phi[2] = {d[1], d[2] >> 16};                                 // (only their low 16 bits are used)
                 if (row_ok) {
                     if (kq == 0) {
                         if (a.scales_blocked)
