@@ -68,3 +68,29 @@ def test_unpackers_refuse_cpu_tensors_and_fp4():
         layout.unpack_weight_packed_nibbles(torch.zeros(128, 64, dtype=torch.int8), 128, 128)
     with pytest.raises(NotImplementedError):
         layout.unpack_scale(torch.zeros(8, 128, dtype=torch.bfloat16), 128, group_size=16)
+
+
+def test_hand_over_layouts_on_the_host():
+    """The pure-torch converters of the layouts the quantizer, the requantizing epilogues and the GEMM pass between
+    them: inverses of each other, and the documented position of one element each."""
+    g = torch.Generator().manual_seed(0)
+    a = torch.randint(0, 256, (96, 160), dtype=torch.uint8, generator=g)
+    b = layout.block_activations(a)
+    assert b.shape == a.shape and torch.equal(layout.unblock_activations(b), a)
+    rb, grp, h, r = 2, 3, 1, 7  # lane 32 h + r of (row block, group) = bytes 16 h .. of row 32 rb + r
+    assert torch.equal(b.reshape(-1)[((rb * 5 + grp) * 64 + 32 * h + r) * 16 :][:16], a[32 * rb + r, 32 * grp + 16 * h :][:16])
+    for unsigned in (False, True):
+        c = layout.block_activations_f6(a, unsigned)
+        assert c.shape == (96, 240) and torch.equal(layout.unblock_activations_f6(c, unsigned), a)
+    c = layout.block_activations_f6(a, False).reshape(-1)
+    rb, grp, h, r, p = 1, 2, 0, 9, 21  # code p of lane 32 h + r: value k = 2 p + h, sign << 5 | magnitude, at bits 6 p of 24 bytes
+    lane = 32 * h + r
+    base = (rb * 5 + grp) * 1536
+    vec = bytes(torch.cat([c[base + 16 * lane :][:16], c[base + 1024 + 8 * lane :][:8]]).tolist())
+    v = ((int(a[32 * rb + r, 32 * grp + p]) & 15) ^ 8) - 8  # k = 2 p: the low nibble of byte p of the group
+    assert (int.from_bytes(vec, "little") >> (6 * p)) & 63 == (32 - v if v < 0 else v)
+    s = torch.arange(16 * 96, dtype=torch.float32).reshape(16, 96)
+    t = layout.block_scales(s)
+    assert t.shape == s.shape and torch.equal(layout.unblock_scales(t), s)
+    m, grp = 70, 11  # element ((m / 32) * (G / 8) + g / 8) * 256 + (m % 32) * 8 + g % 8
+    assert t.reshape(-1)[((m // 32) * 2 + grp // 8) * 256 + (m % 32) * 8 + grp % 8] == s[grp, m]
