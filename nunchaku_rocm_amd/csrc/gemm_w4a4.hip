@@ -10,9 +10,9 @@
 // orientation every row-wise epilogue wants; the int8 kernel has them the other way round (its scale FMAs want the weight
 // scale per lane) and turns its results through LDS after the loop.  K is staged through LDS 128 at
 // a time (two scale groups), two stages; operands that several wavefronts read go global -> LDS directly
-// (global_load_lds, no registers), one stage ahead, into a lane-linear layout (LDS slot l of a 1 KB block = the 16 bytes
-// MFMA lane l needs), so the operand reads are bank-conflict free by construction; one raw s_barrier per stage with
-// explicit s_waitcnt.
+// (buffer_load ... lds in the fp8 kernel, global_load_lds in the int8 kernel; no registers), one stage ahead, into a
+// lane-linear layout (LDS slot l of a 1 KB block = the 16 bytes MFMA lane l needs), so the operand reads are bank-conflict
+// free by construction; one raw s_barrier per stage with explicit s_waitcnt.
 //
 //  * gemm_w4a4_f8_kernel (pre-split weights, svdq_split_weight_planes; the default for module weights): an activation
 //    is carried as the fp8 (e4m3) code of value * 2^-9, a weight as the fp6 (e2m3) code of value / 8, 24 bytes per lane
@@ -27,6 +27,10 @@
 //    to 168 vector registers and 48.5 KB of LDS so that three workgroups share a CU (three wavefronts per SIMD): a
 //    wavefront issues scale product, group product and the sixteen FMAs of a step in program order (single result
 //    buffers) and the other two wavefronts of the SIMD fill the matrix pipe and the vector ALU meanwhile.
+//    Fed by this library's own quantizer or requantizing epilogues (act_blocked = 2) the activations arrive as fp6 codes
+//    sign | magnitude in the loop's lane order and go into the matrix instruction as loaded: fp6 x fp6 (half the matrix
+//    time per group), no unpack, no offset, one instantiation for signed and unsigned activations; their scales can come
+//    in the loop's order too (ascales_blocked: one 16-byte load per lane every four stages).
 //  * gemm_w4a4_i8_kernel (packed weights): a 16-byte LDS read holds 32 nibbles; the even and the odd nibbles are split
 //    into two int8 planes with shift/mask only (signed values land in the high nibble of each byte, i.e. times 16;
 //    unsigned activations in the low nibble, times 1).  Both operands use the same split, so the K order inside a group
