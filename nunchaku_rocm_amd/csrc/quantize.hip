@@ -7,14 +7,19 @@
 // add, clamp, low nibble first.  The LoRA-down product consumes the raw 16-bit activations (before shift and
 // smoothing) on the 16x16x32 MFMA with fp32 accumulation.
 //
-// Work split: one workgroup = 16 rows x all of K, four wavefronts taking scale groups round-robin with two groups
-// in flight each.  A group's operands (16 rows x 128 bytes of activations, 32 ranks x 128 bytes of the transposed
+// Work split: one workgroup = 16 (or 32) rows x all of K, eight wavefronts taking scale groups round-robin with two
+// groups in flight each; on the grid's second axis, one workgroup row per chunk of 32 LoRA ranks and, where CUs are
+// left over, up to three rows that only quantize a slice of the groups each.  A group's operands (16 rows x 128 bytes of activations, 32 ranks x 128 bytes of the transposed
 // LoRA-down weight (R, K)) are fetched straight into LDS (global_load_lds_dwordx4) by loads whose 64 lanes cover eight
 // full 128-byte rows -- read lane-per-row from global memory, the same bytes cost the memory pipeline four times as
 // many cycles -- and land in a tile whose 16-byte chunks are XOR-swizzled by the row so that the transposed read-back
 // is conflict free.  Lane (m = lane % 16, q = lane / 16) then owns the 16 consecutive channels [64 g + 16 q, +16)
 // of row m: a group's absmax needs two cross-lane steps, and the lane's two 16-byte halves are exactly the B operands
 // of two 16x16x32 MFMAs whose A operands come from the LoRA-down tile.
+//
+// Output: the reference's (M, K / 2) matrix of packed nibbles and (K / 64, M) scales, or -- for the GEMM of this library --
+// the same bytes in its lanes' order, or the same integers as fp6 codes in that order (from the hardware's float -> fp6
+// conversion), with the scales in that order as well.
 #include <algorithm>
 
 #include "svdq_common.h"
