@@ -54,6 +54,44 @@ def test_gemm_random_shapes(dev):
         assert O.max_rel_err(buf[:am].cpu(), ref) <= 1e-2
 
 
+def test_hand_over_random_shapes(dev, main_loop):
+    """Quantizer -> GEMM as the modules chain them, on random shapes and every hand-over the shape allows (the matrix,
+    its bytes in lane order, fp6 codes, fp6 codes with the scales in the GEMM's order): codes and scales decoded from
+    the quantizer's output bit-equal to the oracle's, GEMM output at the oracle's bar."""
+    from nunchaku_rocm_amd import ops
+    from nunchaku_rocm_amd.layout import unblock_activations, unblock_activations_f6, unblock_scales
+
+    if main_loop != "all":
+        return  # the int8 main loop reads the matrix only (its refusal of the other forms: test_gpu_blocked.py)
+    rnd = random.Random(777)
+    for case in range(24):
+        M = rnd.choice([1, 31, 32, 33, 100, 257, 300, 512, 1000])
+        K = 64 * rnd.choice([1, 2, 3, 5, 8, 8, 16, 16, 24])
+        N = 8 * rnd.randint(1, 48)
+        R = rnd.choice([0, 16, 32, 48])
+        dtype = rnd.choice([torch.bfloat16, torch.float16])
+        mode = rnd.choice([0, 1, 2, 3] if K % 512 == 0 else [0, 1, 2])
+        print(f"case {case}: M={M} K={K} N={N} R={R} mode={mode} {dtype}", flush=True)
+        lin = O.make_svdq_linear(K, N, R=max(R, 16), seed=case, dtype=dtype)
+        x = O.make_activations(M, K, seed=200 + case, dtype=dtype)
+        ld = lin["proj_down"][:, :R].contiguous() if R else None
+        lu = lin["proj_up"][:, :R].contiguous() if R else None
+        d = lambda t: None if t is None else t.to(dev)  # noqa: E731
+        q, s, la = ops.svdq_quantize_w4a4_act_fuse_lora_cuda(x.to(dev), lora_down=d(ld), smooth=lin["smooth_factor"].to(dev), out_blocked=mode)
+        out = torch.full((M + 2, N), float("nan"), dtype=dtype, device=dev)
+        ops.svdq_gemm_w4a4_cuda(act=q, wgt=lin["qweight"].to(dev), out=out[:M], ascales=s, wscales=lin["wscales"].to(dev),
+                                lora_act_in=la if R else None, lora_up=d(lu), bias=lin["bias"].to(dev), act_blocked=mode)  # fmt: skip
+        torch.cuda.synchronize()
+        rp, rs, rl, _ = O.quantize_act(x, ld, lin["smooth_factor"])
+        codes = unblock_activations_f6(q.cpu()) if mode >= 2 else unblock_activations(q.cpu()) if mode else q.cpu()
+        assert torch.equal(codes[:M], rp), "codes"
+        scales = unblock_scales(s.cpu()) if mode == 3 else s.cpu()
+        assert torch.equal(scales[:, :M].view(torch.int16), rs.view(torch.int16)), "scales"
+        assert bool(out[M:].isnan().all()), "rows past actual_m were written"
+        ref = O.gemm_w4a4(rp, lin["qweight"], rs, lin["wscales"], lin["bias"], rl if R else None, lu)
+        assert O.max_rel_err(out[:M].cpu(), ref) <= 1e-2
+
+
 def test_quantizer_random_shapes(dev):
     from nunchaku_rocm_amd.ops.quantize import quantize_w4a4_act_fuse_lora
 
