@@ -86,6 +86,30 @@ def test_unit_scales_exact_integer_gemm(dev, unsigned, dtype, K):
 
 @pytest.mark.parametrize("unsigned", [False, True])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("K", [256, 192, 64, 1024])
+def test_unit_scales_exact_integer_gemm_from_fp6_codes(dev, unsigned, dtype, K, main_loop):
+    """The same through the fp6 x fp6 instruction (activations as fp6 codes in lane order, full range of both operands;
+    K = 64 makes the output one group's accumulator, K = 1024 takes the blocked scales too): exact integers, the
+    oracle's bits."""
+    if main_loop != "all":
+        return  # the int8 main loop reads the matrix only
+    M, N = 136, 264
+    p = _rand_problem(M, N, K, 0, dtype, seed=2)
+    p["asc"] = torch.ones_like(p["asc"])
+    p["wsc"] = torch.ones_like(p["wsc"])
+    p["bias"] = None
+    ref = O.gemm_w4a4(p["act"], p["wgt"], p["asc"], p["wsc"], act_unsigned=unsigned).to(dtype)
+    q = _as_fp6_codes(p, unsigned)
+    out = _gpu_gemm(q, dev, actual_m=M, unsigned=unsigned, dtype=dtype, act_blocked=2)
+    assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
+    if K % 512 == 0:
+        q["asc"] = torch.ones_like(q["asc"])  # all ones, pad rows included: the same bytes in either order
+        out = _gpu_gemm(q, dev, actual_m=M, unsigned=unsigned, dtype=dtype, act_blocked=3)
+        assert torch.equal(out.view(torch.int16), ref.view(torch.int16))
+
+
+@pytest.mark.parametrize("unsigned", [False, True])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("M,N,K,R,actual_m", [(136, 264, 256, 16, 130), (256, 256, 512, 32, 256), (64, 128, 1024, 48, 64), (128, 512, 256, 0, 100),
                                                    (160, 256, 256, 160, 150), (72, 136, 512, 288, 72),  # ranks grown at run time (32 + sum of LoRA ranks)
                                                    (136, 264, 64, 16, 136), (130, 200, 192, 32, 130), (256, 128, 448, 0, 200)])  # K / 64 odd
