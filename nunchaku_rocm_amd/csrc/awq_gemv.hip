@@ -17,6 +17,7 @@
 //
 // One workgroup = 32 channels x all of K; its eight wavefronts take groups round-robin with up to six weight loads per
 // lane in flight (all of a wavefront's groups at K = 3072); partial sums are added through LDS in a fixed order.
+// A batched launch with five to eight rows gives a workgroup 64 channels where that leaves two workgroups per CU.
 #include <type_traits>
 
 #include "svdq_common.h"
@@ -86,20 +87,26 @@ __device__ inline float dpp_f32(float x) {
 // slot pc ^ r, rows 128 bytes apart would otherwise meet in the same banks) | s of the groups (64 bytes each) | z;
 // after the tables of all wavefronts: xs[w][group][8] fp32 = sums of the activations per (half, row) (RP <= 4) or per
 // row (RP = 8).  The partial sums of the final reduction reuse the wavefront's own x tiles.
-template <int RP>
-constexpr int awq_wave_bytes() { return AWQ_PF * RP * 128 + 2 * AWQ_PF * 64; }
+template <int RP, int CB = 1>
+constexpr int awq_wave_bytes() { return AWQ_PF * RP * 128 + 2 * AWQ_PF * 64 * CB; }
 
 //
 // BATCH: one launch serves `count` weights of one shape (the adaLN projections of a model all take the same vector and
 // differ only in their tensors): workgroup b works on problem b / (N / 32), whose five pointers it reads from `table`;
 // everything else comes from `a`.  A 32 MB weight by itself is read at 60 % of the HBM peak at best (launch ramp and
 // tail of a 6 us kernel); several in one launch stream like one long read.
-template <typename T, int RP, bool BATCH>
+//
+// CB = 2 (RP = 8 only): the workgroup takes 64 channels, every wavefront both 32-channel blocks of its groups, so that
+// the activation tiles, their sums and the MFMA A operand reads are paid once per 64 channels (at eight rows they are
+// as many bytes out of L2 as the weights are out of HBM).  Half as many workgroups: for launches with enough of them.
+template <typename T, int RP, bool BATCH, int CB = 1>
 __global__ __launch_bounds__(AWQ_WAVES * 64) __attribute__((amdgpu_waves_per_eu(RP <= 4 ? 6 : 4))) void awq_gemv_rows_kernel(svdq_awq_gemv_args a, const svdq_awq_gemv_args *table) {
+    static_assert(CB == 1 || (CB == 2 && RP == 8), "two channel blocks per wavefront only with eight rows");
+    constexpr int NBW = AWQ_NB * CB;  // channels per workgroup
     extern __shared__ __align__(16) uint8_t lds8[];
     int blk = blockIdx.x;
     if constexpr (BATCH) {
-        const int nblk = a.N / AWQ_NB, pi = blk / nblk;  // uniform: scalar loads
+        const int nblk = a.N / NBW, pi = blk / nblk;  // uniform: scalar loads
         blk -= pi * nblk;
         a.x = table[pi].x;
         a.qweight = table[pi].qweight;
@@ -108,11 +115,11 @@ __global__ __launch_bounds__(AWQ_WAVES * 64) __attribute__((amdgpu_waves_per_eu(
         a.out = table[pi].out;
     }
     constexpr bool SMALL = RP <= 4;
-    constexpr int WB = awq_wave_bytes<RP>(), XPIECES = AWQ_PF * 8 * RP, XPASSES = (XPIECES + 63) / 64;
+    constexpr int WB = awq_wave_bytes<RP, CB>(), XPIECES = AWQ_PF * 8 * RP, XPASSES = (XPIECES + 63) / 64;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int ngroups = a.K / GROUP;
-    const int nb0 = blk * AWQ_NB;
+    const int nb0 = blk * NBW;
     uint8_t *xw = lds8 + wave * WB, *szw = xw + AWQ_PF * RP * 128;
     float *xsw = (float *)(lds8 + AWQ_WAVES * WB) + wave * (AWQ_PF * 8);
 
@@ -130,9 +137,9 @@ __global__ __launch_bounds__(AWQ_WAVES * 64) __attribute__((amdgpu_waves_per_eu(
 
     uint32_t mask = 0x000F000Fu;
     asm volatile("" : "+v"(mask));  // keep the mask in a VGPR: v_and_or_b32 takes only one literal
-    float acc[SMALL ? RP : 4];
+    float acc[SMALL ? RP : 4 * CB];
 #pragma unroll
-    for (int i = 0; i < (SMALL ? RP : 4); i++) acc[i] = 0.0f;
+    for (int i = 0; i < (SMALL ? RP : 4 * CB); i++) acc[i] = 0.0f;
 
     // One batch: NV groups c = base + 8 u of this wavefront (NV < AWQ_PF only in the last batch of a ragged K)
     auto batch = [&](auto nv_tag, int base) {
@@ -146,18 +153,28 @@ __global__ __launch_bounds__(AWQ_WAVES * 64) __attribute__((amdgpu_waves_per_eu(
             if (XPIECES % 64 == 0 || i + 1 < XPASSES || q < XPIECES)
                 __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)((const uint8_t *)a.x + off), (SVDQ_AS3 void *)(xw + 1024 * i), 16, 0, 0);
         }
-        {   // scales: lanes 0 .. 4 PF - 1 = (group, 16-byte piece of its 32 channels); zeros: the next 4 PF lanes
+        if constexpr (CB == 2) {  // lanes 0 .. 8 PF - 1 = (group, 16-byte piece of its 64 channels), scales then zeros
+            const int c = min(base + AWQ_WAVES * (lane >> 3), ngroups - 1);
+            const uint32_t off = ((uint32_t)c * (uint32_t)a.ld_scales + nb0 + 8 * (lane & 7)) * 2;
+            if (lane < 8 * AWQ_PF) {
+                __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)((const uint8_t *)a.scales + off), (SVDQ_AS3 void *)szw, 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)((const uint8_t *)a.zeros + off), (SVDQ_AS3 void *)(szw + AWQ_PF * 128), 16, 0, 0);
+            }
+        } else {   // scales: lanes 0 .. 4 PF - 1 = (group, 16-byte piece of its 32 channels); zeros: the next 4 PF lanes
             const bool z = lane >= 4 * AWQ_PF;
             const int t = lane - (z ? 4 * AWQ_PF : 0), c = min(base + AWQ_WAVES * (t >> 2), ngroups - 1);
             const uint32_t off = ((uint32_t)c * (uint32_t)a.ld_scales + nb0 + 8 * (t & 3)) * 2;
             if (lane < 8 * AWQ_PF)
                 __builtin_amdgcn_global_load_lds((const SVDQ_AS1 void *)((const uint8_t *)(z ? a.zeros : a.scales) + off), (SVDQ_AS3 void *)szw, 16, 0, 0);
         }
-        v4i wreg[NV];
+        v4i wreg[NV * CB];  // channel block cb of group u in wreg[CB u + cb] (eight packed rows = 16 K bytes further on)
 #pragma unroll
         for (int u = 0; u < NV; u++)
-            wreg[u] = awq_wload((const v4i *)((const uint8_t *)a.qweight + (woff + (uint32_t)(base + AWQ_WAVES * u) * (GROUP * 2))));
-        __builtin_amdgcn_s_waitcnt(waitcnt_imm(NV, 15));  // activations, scales and zeros have landed
+#pragma unroll
+            for (int cb = 0; cb < CB; cb++)
+                wreg[CB * u + cb] = awq_wload((const v4i *)((const uint8_t *)a.qweight + (woff + (uint32_t)cb * 16u * (uint32_t)a.K +
+                                                                                          (uint32_t)(base + AWQ_WAVES * u) * (GROUP * 2))));
+        __builtin_amdgcn_s_waitcnt(waitcnt_imm(NV * CB, 15));  // activations, scales and zeros have landed
         // sums of the activations: every lane adds up its own piece, then the lanes of a (half) row are added
 #pragma unroll
         for (int i = 0; i < XPASSES; i++) {
@@ -177,11 +194,37 @@ __global__ __launch_bounds__(AWQ_WAVES * 64) __attribute__((amdgpu_waves_per_eu(
         }
 #pragma unroll
         for (int u = 0; u < NV; u++) {
-            const v4i w = wreg[u];
-            const float s = T::to_f32(((const uint16_t *)szw)[u * 32 + ch]);
-            const float zz = T::to_f32(((const uint16_t *)szw)[(AWQ_PF + u) * 32 + ch]) - AwqMagic<T>::off * s;
+            const v4i w = wreg[CB * u];
+            const float s = T::to_f32(((const uint16_t *)szw)[u * NBW + ch]);
+            const float zz = T::to_f32(((const uint16_t *)szw)[(AWQ_PF + u) * NBW + ch]) - AwqMagic<T>::off * s;
             const uint8_t *at = aop + u * (RP * 128);
-            if constexpr (SMALL) {
+            if constexpr (CB == 2) {
+                v4i xa[4];
+#pragma unroll
+                for (int pl = 0; pl < 4; pl++) xa[pl] = *(const v4i *)(at + aslot[pl]);
+                const v4f xv = *(const v4f *)(xsw + u * 8 + 4 * half);
+#pragma unroll
+                for (int cb = 0; cb < CB; cb++) {
+                    const v4i wc = wreg[CB * u + cb];
+                    const float sc = T::to_f32(((const uint16_t *)szw)[u * NBW + 32 * cb + ch]);
+                    const float zc = T::to_f32(((const uint16_t *)szw)[(AWQ_PF + u) * NBW + 32 * cb + ch]) - AwqMagic<T>::off * sc;
+                    v16f d;
+#pragma unroll
+                    for (int i = 0; i < 16; i++) d[i] = 0.0f;
+#pragma unroll
+                    for (int pl = 0; pl < 4; pl++) {
+                        v4i wb;
+#pragma unroll
+                        for (int e = 0; e < 4; e++) wb[e] = nibble_plane(wc[e], 4 * pl, mask, AwqMagic<T>::bits);
+                        d = mfma32_16bit<T>(xa[pl], wb, d);
+                    }
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        acc[4 * cb + e] = __builtin_fmaf(sc, d[e], acc[4 * cb + e]);
+                        acc[4 * cb + e] = __builtin_fmaf(zc, xv[e], acc[4 * cb + e]);
+                    }
+                }
+            } else if constexpr (SMALL) {
                 v4f d0 = {0.0f, 0.0f, 0.0f, 0.0f}, d1 = d0;
 #pragma unroll
                 for (int pl = 0; pl < 4; pl++) {
@@ -237,10 +280,12 @@ __global__ __launch_bounds__(AWQ_WAVES * 64) __attribute__((amdgpu_waves_per_eu(
         for (int r = 0; r < RP; r++) red[(half * RP + r) * AWQ_NB + ch] = acc[r];
     } else {
 #pragma unroll
-        for (int e = 0; e < 4; e++) red[(4 * half + e) * AWQ_NB + ch] = acc[e];
+        for (int cb = 0; cb < CB; cb++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) red[(4 * half + e) * NBW + 32 * cb + ch] = acc[4 * cb + e];
     }
     __syncthreads();
-    if (tid < a.M * AWQ_NB) {
+    if (tid < a.M * NBW) {
         float s = 0.0f;
 #pragma unroll
         for (int w = 0; w < AWQ_WAVES; w++) {
@@ -250,7 +295,7 @@ __global__ __launch_bounds__(AWQ_WAVES * 64) __attribute__((amdgpu_waves_per_eu(
             else
                 s += rw[tid];
         }
-        ((uint16_t *)a.out)[(size_t)(tid / AWQ_NB) * a.ld_out + nb0 + tid % AWQ_NB] = T::from_f32(s);
+        ((uint16_t *)a.out)[(size_t)(tid / NBW) * a.ld_out + nb0 + tid % NBW] = T::from_f32(s);
     }
 }
 
@@ -409,6 +454,12 @@ template <typename T, bool BATCH>
 static void launch_awq_rows(const svdq_awq_gemv_args &a, const svdq_awq_gemv_args *table, int count, hipStream_t s) {
     const dim3 grid((unsigned)(a.N / AWQ_NB) * (unsigned)count), block(AWQ_WAVES * 64);
     constexpr size_t XS_BYTES = (size_t)AWQ_WAVES * AWQ_PF * 8 * sizeof(float);
+    // 64-channel workgroups once the launch still has two and more of them for each of the 256 CUs
+    if constexpr (BATCH) if (a.M > 4 && a.N % (2 * AWQ_NB) == 0 && (size_t)(a.N / (2 * AWQ_NB)) * (size_t)count >= 512) {
+        constexpr size_t LDS2 = (size_t)AWQ_WAVES * awq_wave_bytes<8, 2>() + XS_BYTES;
+        hipLaunchKernelGGL((awq_gemv_rows_kernel<T, 8, BATCH, 2>), dim3(grid.x / 2), block, LDS2, s, a, table);
+        return;
+    }
     if (a.M <= 1)
         hipLaunchKernelGGL((awq_gemv_rows_kernel<T, 1, BATCH>), grid, block, AWQ_WAVES * awq_wave_bytes<1>() + XS_BYTES, s, a, table);
     else if (a.M <= 2)

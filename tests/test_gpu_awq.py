@@ -42,10 +42,13 @@ def test_flux_adaln_shape(dev, m):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("m,N,K,count", [(1, 18432, 3072, 3), (2, 96, 576, 5), (8, 256, 1088, 2), (3, 64, 64, 7), (5, 9216, 3072, 1)])
+@pytest.mark.parametrize("m,N,K,count", [(1, 18432, 3072, 3), (2, 96, 576, 5), (8, 256, 1088, 2), (3, 64, 64, 7), (5, 9216, 3072, 1),
+                                         (8, 4096, 1088, 8), (5, 18432, 3072, 2), (7, 2048, 192, 16), (6, 1056, 640, 16)])
 def test_batched_launch_matches_single_launches(dev, m, N, K, count, dtype):
     """``count`` weights of one shape on the same input in one launch (the adaLN projections of a model): every output
-    bit as from the single launches, and the oracle's result."""
+    bit as from the single launches, and the oracle's result.  The last four cases have more than four rows and 512
+    and more workgroups of 64 channels, where the launch gives a workgroup 64 channels (N = 1056 is no multiple of 64
+    and keeps 32)."""
     from nunchaku_rocm_amd import ops
 
     print(f"case m={m} N={N} K={K} count={count} {dtype}", flush=True)
