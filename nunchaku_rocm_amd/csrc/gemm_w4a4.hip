@@ -986,8 +986,9 @@ __global__ __launch_bounds__(NTHREADS, PIPE ? 2 : 3) void gemm_w4a4_f8_kernel(sv
     // row): the same two loads per stage, base + lane offset + group * step, with other constants.
     const bool ablk = F6ACT || a.act_blocked != 0;
     const uint32_t sAct = F6ACT ? 1536u : ablk ? 1024u : 32u;
-    const __amdgpu_buffer_rsrc_t rAct =
-        g_buffer((const uint8_t *)a.act + (ablk ? (size_t)((m0 >> 5) + wm) * G * sAct : (size_t)m0 * a.ld_act));
+    // a tile's row blocks past the last one that exists (M no multiple of 128) re-read the last: their rows are never stored
+    const int rblk = min((m0 >> 5) + wm, ((a.M + 31) >> 5) - 1);
+    const __amdgpu_buffer_rsrc_t rAct = g_buffer((const uint8_t *)a.act + (ablk ? (size_t)rblk * G * sAct : (size_t)m0 * a.ld_act));
     const __amdgpu_buffer_rsrc_t rAS = g_buffer(a.ascales);
     const uint32_t oAct = ablk ? (uint32_t)lane * 16u : (uint32_t)(mrow - m0) * (uint32_t)a.ld_act + half * 16;
     const uint32_t oExt = 1024u + (uint32_t)lane * 8u;
@@ -995,7 +996,7 @@ __global__ __launch_bounds__(NTHREADS, PIPE ? 2 : 3) void gemm_w4a4_f8_kernel(sv
     // SB: dword ST of sc_cur = the row's scales of the two groups of stage ST of the current four stages; sc_nxt is loaded
     // during their first stage (512 bytes per 32 rows and four stages)
     v4i sc_cur = {0, 0, 0, 0}, sc_nxt = {0, 0, 0, 0};
-    const __amdgpu_buffer_rsrc_t rASb = g_buffer((const uint8_t *)a.ascales + (SB ? (size_t)((m0 >> 5) + wm) * (G >> 3) * 512 : 0));
+    const __amdgpu_buffer_rsrc_t rASb = g_buffer((const uint8_t *)a.ascales + (SB ? (size_t)rblk * (G >> 3) * 512 : 0));
     const uint32_t oAb = (uint32_t)l32 * 16u;
     if constexpr (SB) sc_cur = g_load128(rASb, oAb, 0);
     auto load_regs = [&](int s, auto set_tag) {
